@@ -1,0 +1,256 @@
+/*
+ * openrlhf_amd.h — C ABI of libopenrlhf_amd.so: hand-written gfx950 (MI355X) kernels for the
+ * token-level RL numerics of OpenRLHF.
+ *
+ * The reference has no FFI layer for this path: its boundary is the Python signature of a set of
+ * torch functions. Each entry point below replaces the device work of one of them and cites it
+ * as `file:line` relative to the OpenRLHF source tree. A Python binding (ctypes) passes
+ * `tensor.data_ptr()`, element counts and the HIP stream; nothing here knows about torch.
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless the comment says "host";
+ *  - every function returns ORLHF_OK (0) or a negative error code, never throws, and leaves a
+ *    thread-local message readable with orlhf_last_error();
+ *  - kernels are launched asynchronously on `stream` (a hipStream_t; NULL = default stream) and
+ *    the call does not synchronise; the library keeps no device state between calls and
+ *    allocates no device memory: outputs, saved row statistics and workspaces are the caller's;
+ *  - per-token tensors come in one of two row layouts, selected by `cu_seqlens`:
+ *      padded : cu_seqlens == NULL, contiguous [n_rows, n_cols]; row b token t at b*n_cols + t;
+ *      packed : cu_seqlens != NULL, int64 [n_rows + 1] on the device; row b holds tokens
+ *               cu_seqlens[b] .. cu_seqlens[b+1]-1 of one flat array and n_cols is an upper
+ *               bound of the longest row (it only sizes the launch);
+ *  - masks are read as float weights (the reference multiplies by the mask): ORLHF_MASK_U8 for
+ *    torch.bool / torch.uint8, ORLHF_MASK_F32, ORLHF_MASK_I64, or ORLHF_MASK_NONE (all ones,
+ *    pointer ignored);
+ *  - reductions are two-stage and deterministic (no floating-point atomics): the same inputs give
+ *    the same bits on every run.
+ */
+#ifndef OPENRLHF_AMD_H
+#define OPENRLHF_AMD_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ORLHF_ABI_VERSION 1
+
+#define ORLHF_OK 0
+#define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
+#define ORLHF_ERR_LAUNCH (-2)      /* hipGetLastError() after a launch reported a failure       */
+#define ORLHF_ERR_UNSUPPORTED (-3) /* a combination the kernels do not implement                */
+
+enum orlhf_dtype { ORLHF_F32 = 0, ORLHF_BF16 = 1, ORLHF_F16 = 2 };
+enum orlhf_mask_dtype { ORLHF_MASK_NONE = 0, ORLHF_MASK_U8 = 1, ORLHF_MASK_F32 = 2, ORLHF_MASK_I64 = 3 };
+enum orlhf_kl_estimator { ORLHF_KL_K1 = 0, ORLHF_KL_K2 = 1, ORLHF_KL_K3 = 2 };
+enum orlhf_agg_mode {
+  ORLHF_AGG_TOKEN_MEAN = 0, /* sum(x*m) / (sum(m) | batch_num_tokens) * dp_size                  */
+  ORLHF_AGG_SEQ_MEAN = 1,   /* mean over non-empty rows of sum(x*m)/(sum(m)+1e-8)               */
+  ORLHF_AGG_ROW_MEAN = 2    /* per-row sum(x*m)/sum(m), output [n_rows] (masked_mean, dim=-1)   */
+};
+enum orlhf_policy_type { ORLHF_POLICY_PPO = 0, ORLHF_POLICY_GSPO = 1 };
+enum orlhf_is_correction { ORLHF_IS_NONE = 0, ORLHF_IS_TIS = 1, ORLHF_IS_ICEPOP = 2, ORLHF_IS_SEQ_MASK_TIS = 3 };
+enum orlhf_group_estimator {
+  ORLHF_GROUP_IDENTITY = 0, /* gae, reinforce: rewards unchanged                                 */
+  ORLHF_GROUP_RLOO = 1,     /* r - (sum - r)/(n-1)                                               */
+  ORLHF_GROUP_BASELINE = 2, /* reinforce_baseline, dr_grpo: r - mean                             */
+  ORLHF_GROUP_NORM = 3      /* group_norm: (r - mean)/(std_unbiased + 1e-9)                      */
+};
+
+typedef void* orlhf_stream_t; /* hipStream_t */
+
+/* Library ABI version (ORLHF_ABI_VERSION of the build). No reference counterpart. */
+int orlhf_version(void);
+/* Message of the last failing call on this host thread ("" if none). No reference counterpart. */
+const char* orlhf_last_error(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Vocabulary-row kernels
+ * ---------------------------------------------------------------------------------------- */
+
+/* `flags` of orlhf_logprob_entropy_fwd: reserved, must be 0. */
+
+/*
+ * Fused log-softmax + gather + entropy over full vocabulary rows, one streaming pass.
+ *   logprob[i] = z[i,label_i] - logsumexp_j z[i,j],  z = logits / temperature
+ *   entropy[i] = logsumexp_j x[i,j] - sum_j softmax(x)[i,j] * x[i,j],  x = logits (unscaled)
+ * Replaces log_probs_from_logits (openrlhf/models/utils.py:139-163, incl. _logsumexp_by_chunk
+ * :129-136 and the flash-attn cross_entropy_loss call :147-150) and compute_entropy
+ * (openrlhf/models/utils.py:182-186) as called from Actor.forward
+ * (openrlhf/models/actor.py:265-296: entropy before the temperature division, log-prob after).
+ *   logits    [n_rows, vocab], element stride 1, `row_stride` elements between rows
+ *   labels    int64 [n_rows]; label -100 gives logprob 0 (flash-attn ignore_index), any other
+ *             label outside [0, vocab) gives NaN; neither reads out of bounds
+ *   logprob   float [n_rows] or NULL;  entropy float [n_rows] or NULL (not both NULL)
+ *   row_stats float [n_rows, 4] or NULL: {lse(z), lse(x), E_softmax(x)[x], 0}, what the backward
+ *             needs; fp32 accumulation and fp32 outputs for every input dtype
+ */
+int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                              int64_t row_stride, const int64_t* labels, double temperature,
+                              float* logprob, float* entropy, float* row_stats, int flags,
+                              orlhf_stream_t stream);
+
+/*
+ * Backward of the above in one streaming pass, written in the logits dtype:
+ *   grad[i,j] = g_logprob[i] * (1[j==label_i] - softmax(z)[i,j]) / temperature
+ *             + g_entropy[i] * softmax(x)[i,j] * (E[x] - x[i,j])
+ * `grad_logits` may alias `logits` (in-place: each 16-byte chunk is read, then overwritten by the
+ * same lane). Replaces torch autograd through openrlhf/models/utils.py:139-163 and :182-186.
+ * g_logprob / g_entropy: float [n_rows] or NULL (treated as 0). Rows whose upstream gradients
+ * are both exactly 0 are written as zeros without reading their logits.
+ */
+int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, int dtype, int64_t n_rows,
+                              int64_t vocab, int64_t row_stride, int64_t grad_row_stride,
+                              const int64_t* labels, double temperature, const float* g_logprob,
+                              const float* g_entropy, const float* row_stats,
+                              orlhf_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Per-token kernels: KL, masked aggregation, PPO policy loss, value loss
+ * ---------------------------------------------------------------------------------------- */
+
+/*
+ * out = clamp(k(lp - base), -10, 10); k1: d, k2: d*d/2, k3: exp(-d) - 1 + d; fp32 out.
+ * Replaces compute_approx_kl (openrlhf/models/utils.py:64-95). `dtype` is the type of both
+ * inputs (the reference up-casts with .float()). n = number of elements (flat).
+ */
+int orlhf_approx_kl_fwd(const void* log_probs, const void* log_probs_base, int dtype, int64_t n,
+                        int estimator, float* out, orlhf_stream_t stream);
+/* g_lp = g_out * d(out)/d(lp) (0 where the clamp is active, closed interval passes);
+ * g_base (nullable) = -g_lp. Autograd of openrlhf/models/utils.py:78-95. */
+int orlhf_approx_kl_bwd(const void* log_probs, const void* log_probs_base, int dtype, int64_t n,
+                        int estimator, const float* g_out, float* g_lp, float* g_base,
+                        orlhf_stream_t stream);
+
+/* Normaliser of a token/sequence aggregate (openrlhf/models/loss.py:29-39,
+ * openrlhf/utils/loss_utils.py:15-105). norm_dev != NULL: read the denominator from that device
+ * float; else norm_value if it is not NaN; else the local sum over the mask (token mode) or the
+ * local count of non-empty rows (sequence mode). */
+typedef struct orlhf_norm {
+  double dp_size;
+  double norm_value;     /* NaN = not given */
+  const float* norm_dev; /* device scalar or NULL */
+} orlhf_norm;
+
+/* Bytes of workspace the per-token reductions need for an [n_rows, n_cols] problem. */
+int64_t orlhf_token_workspace_bytes(int64_t n_rows, int64_t n_cols);
+
+/*
+ * Masked aggregation of a per-token fp32 matrix.
+ *   TOKEN_MEAN / SEQ_MEAN: aggregate_loss (openrlhf/models/loss.py:11-39) and masked_mean with
+ *   dim=None (openrlhf/models/utils.py:166-169); out = 1 float.
+ *   ROW_MEAN: masked_mean with dim=-1; out = n_rows floats; `norm` ignored.
+ * row_coef (float [n_rows], nullable) receives d(out)/d(x[b,t]) / mask[b,t] for the backward.
+ * An all-zero mask gives NaN (0/0) in TOKEN_MEAN/ROW_MEAN exactly as the reference does.
+ */
+int orlhf_masked_aggregate_fwd(const float* x, const void* mask, int mask_dtype, int64_t n_rows,
+                               int64_t n_cols, const int64_t* cu_seqlens, int mode,
+                               const orlhf_norm* norm, void* workspace, float* out,
+                               float* row_coef, orlhf_stream_t stream);
+/* g_x[b,t] = g(b) * row_coef[b] * mask[b,t]; g(b) = g_out[0] (scalar modes) or g_out[b]. */
+int orlhf_masked_aggregate_bwd(const float* g_out, const void* mask, int mask_dtype,
+                               int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens, int mode,
+                               const float* row_coef, float* g_x, orlhf_stream_t stream);
+
+typedef struct orlhf_policy_params {
+  float clip_eps_low, clip_eps_high;
+  float dual_clip;    /* <= 0: no dual clip */
+  int policy_type;    /* orlhf_policy_type */
+  int is_correction;  /* orlhf_is_correction (needs rollout_log_probs) */
+  float is_low, is_high;
+  int token_level;    /* 1: TOKEN_MEAN, 0: SEQ_MEAN (GSPO forces 0, loss.py:143-144) */
+  orlhf_norm norm;
+} orlhf_policy_params;
+
+/*
+ * PolicyLoss.forward (openrlhf/models/loss.py:157-230): PPO / GSPO surrogate with low/high clip,
+ * dual clip, TIS / ICEPOP / seq-mask-TIS importance correction and token- or sequence-level
+ * aggregation. All per-token inputs fp32 in the row layout above; rollout_log_probs nullable.
+ *   out4     float [4]: loss, clip_ratio, ppo_kl, vllm_kl (NaN when no correction is applied)
+ *   row_coef float [n_rows]: aggregation weight per row (for the backward)
+ *   row_aux  float [n_rows, 2]: {GSPO sequence ratio or seq-mask-TIS 0/1 row flag,
+ *            1/max(sum(mask), 1)}; written only in those two modes, always required
+ */
+int orlhf_policy_loss_fwd(const float* log_probs, const float* old_log_probs,
+                          const float* advantages, const void* mask, int mask_dtype,
+                          const float* rollout_log_probs, int64_t n_rows, int64_t n_cols,
+                          const int64_t* cu_seqlens, const orlhf_policy_params* params,
+                          void* workspace, float* out4, float* row_coef, float* row_aux,
+                          orlhf_stream_t stream);
+/* grad wrt log_probs only (everything else is detached in the callers). g_out: device scalar.
+ * workspace (orlhf_token_workspace_bytes) is used by GSPO only and may be NULL otherwise. */
+int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs, const float* old_log_probs,
+                          const float* advantages, const void* mask, int mask_dtype,
+                          const float* rollout_log_probs, int64_t n_rows, int64_t n_cols,
+                          const int64_t* cu_seqlens, const orlhf_policy_params* params,
+                          const float* row_coef, const float* row_aux, void* workspace,
+                          float* g_log_probs, orlhf_stream_t stream);
+
+/*
+ * ValueLoss.forward (openrlhf/models/loss.py:244-269): 0.5 * aggregate(max((vc-R)^2, (v-R)^2)),
+ * vc = old + clamp(v - old, -eps, eps); has_clip == 0 gives 0.5 * aggregate((v-R)^2).
+ */
+int orlhf_value_loss_fwd(const float* values, const float* old_values, const float* returns,
+                         const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                         const int64_t* cu_seqlens, int has_clip, float clip_eps, int token_level,
+                         const orlhf_norm* norm, void* workspace, float* out, float* row_coef,
+                         orlhf_stream_t stream);
+int orlhf_value_loss_bwd(const float* g_out, const float* values, const float* old_values,
+                         const float* returns, const void* mask, int mask_dtype, int64_t n_rows,
+                         int64_t n_cols, const int64_t* cu_seqlens, int has_clip, float clip_eps,
+                         const float* row_coef, float* g_values, orlhf_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Advantage kernels (forward only; the reference runs them under torch.no_grad())
+ * ---------------------------------------------------------------------------------------- */
+
+/*
+ * compute_reward (openrlhf/models/utils.py:98-126): reward[b,t] = -max(kl_coef,0)*kl[b,t]
+ * + clamp(r[b]) at the row's last position whose (int64)mask is maximal (= last 1; last column
+ * for an all-zero row). eos_index (int64 [n_rows], nullable) receives that column.
+ */
+int orlhf_compute_reward(const float* r, float kl_coef, const float* kl, const void* mask,
+                         int mask_dtype, int64_t n_rows, int64_t n_cols,
+                         const int64_t* cu_seqlens, int has_clip, float clip_low, float clip_high,
+                         float* reward, int64_t* eos_index, orlhf_stream_t stream);
+
+/*
+ * get_advantages_and_returns (openrlhf/trainer/ppo_utils/experience_maker.py:332-377):
+ * v = m*values, r = m*rewards, delta_t = r_t + gamma*v_{t+1} - v_t, A_t = delta_t +
+ * gamma*lambd*A_{t+1}, returns = A + v; every column takes part and nothing is re-masked.
+ * Parallel reverse scan per row, fp64 carries.
+ */
+int orlhf_gae_scan(const float* values, const float* rewards, const void* mask, int mask_dtype,
+                   int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens, float gamma,
+                   float lambd, float* advantages, float* returns, orlhf_stream_t stream);
+
+/* get_cumulative_returns (experience_maker.py:379-411): G_t = m_t*r_t + gamma*G_{t+1}. */
+int orlhf_discounted_returns(const float* rewards, const void* mask, int mask_dtype,
+                             int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
+                             float gamma, float* returns, orlhf_stream_t stream);
+
+/*
+ * Group baseline / normalisation of scalar rewards (experience_maker.py:246-272).
+ * rewards / out / group_std are in experience order; indices[i] (int64, nullable = identity) is
+ * the prompt-order slot of sample i, so group g holds slots g*n .. g*n+n-1. group_std
+ * (nullable) receives the unbiased std of each sample's group (NaN for n == 1, as torch.std).
+ */
+int orlhf_group_normalize(const float* rewards, const int64_t* indices, int64_t n_prompts,
+                          int64_t n_samples, int estimator, float* out, float* group_std,
+                          void* workspace /* n_prompts*n_samples floats */, orlhf_stream_t stream);
+
+/*
+ * Global masked whitening (experience_maker.py:314-328) over a flat array of n elements:
+ * mean = sum(x*m)/sum(m); var = sum((x-mean)^2*m)/sum(m); rstd = rsqrt(max(var,1e-8)) or 1 when
+ * std_norm == 0; out = (x - mean)*rstd at EVERY position, masked or not. out may alias x.
+ * stats (float [2], nullable) receives mean and rstd. workspace: orlhf_whiten_workspace_bytes(n).
+ */
+int64_t orlhf_whiten_workspace_bytes(int64_t n);
+int orlhf_masked_whiten(const float* x, const void* mask, int mask_dtype, int64_t n, int std_norm,
+                        void* workspace, float* out, float* stats, orlhf_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OPENRLHF_AMD_H */

@@ -1,0 +1,189 @@
+"""ctypes binding of libopenrlhf_amd.so (the C ABI declared in include/openrlhf_amd.h).
+
+There is no CPU or pure-torch fallback: if the shared library has not been built, or a tensor
+is not on a GPU, the call raises. Build with ``python -m openrlhf_amd.csrc.build``.
+"""
+import ctypes
+import math
+import os
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int64, c_void_p
+
+import torch
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libopenrlhf_amd.so")
+
+# enums of include/openrlhf_amd.h
+F32, BF16, F16 = 0, 1, 2
+MASK_NONE, MASK_U8, MASK_F32, MASK_I64 = 0, 1, 2, 3
+KL_K1, KL_K2, KL_K3 = 0, 1, 2
+AGG_TOKEN_MEAN, AGG_SEQ_MEAN, AGG_ROW_MEAN = 0, 1, 2
+POLICY_PPO, POLICY_GSPO = 0, 1
+IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
+GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
+
+ABI_VERSION = 1
+
+
+class Norm(Structure):
+    _fields_ = [("dp_size", c_double), ("norm_value", c_double), ("norm_dev", c_void_p)]
+
+
+class PolicyParams(Structure):
+    _fields_ = [
+        ("clip_eps_low", c_float),
+        ("clip_eps_high", c_float),
+        ("dual_clip", c_float),
+        ("policy_type", c_int),
+        ("is_correction", c_int),
+        ("is_low", c_float),
+        ("is_high", c_float),
+        ("token_level", c_int),
+        ("norm", Norm),
+    ]
+
+
+P = c_void_p
+I64 = c_int64
+
+# name -> (restype, argtypes); every symbol the header declares
+SIGNATURES = {
+    "orlhf_version": (c_int, []),
+    "orlhf_last_error": (c_char_p, []),
+    "orlhf_logprob_entropy_fwd": (c_int, [P, c_int, I64, I64, I64, P, c_double, P, P, P, c_int, P]),
+    "orlhf_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P]),
+    "orlhf_approx_kl_fwd": (c_int, [P, P, c_int, I64, c_int, P, P]),
+    "orlhf_approx_kl_bwd": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
+    "orlhf_token_workspace_bytes": (I64, [I64, I64]),
+    "orlhf_masked_aggregate_fwd": (c_int, [P, P, c_int, I64, I64, P, c_int, POINTER(Norm), P, P, P, P]),
+    "orlhf_masked_aggregate_bwd": (c_int, [P, P, c_int, I64, I64, P, c_int, P, P, P]),
+    "orlhf_policy_loss_fwd": (c_int, [P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P]),
+    "orlhf_policy_loss_bwd": (c_int, [P, P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P]),
+    "orlhf_value_loss_fwd": (c_int, [P, P, P, P, c_int, I64, I64, P, c_int, c_float, c_int, POINTER(Norm), P, P, P, P]),
+    "orlhf_value_loss_bwd": (c_int, [P, P, P, P, P, c_int, I64, I64, P, c_int, c_float, P, P, P]),
+    "orlhf_compute_reward": (c_int, [P, c_float, P, P, c_int, I64, I64, P, c_int, c_float, c_float, P, P, P]),
+    "orlhf_gae_scan": (c_int, [P, P, P, c_int, I64, I64, P, c_float, c_float, P, P, P]),
+    "orlhf_discounted_returns": (c_int, [P, P, c_int, I64, I64, P, c_float, P, P]),
+    "orlhf_group_normalize": (c_int, [P, P, I64, I64, c_int, P, P, P, P]),
+    "orlhf_whiten_workspace_bytes": (I64, [I64]),
+    "orlhf_masked_whiten": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
+}
+
+_lib = None
+
+
+class KernelError(RuntimeError):
+    """A C-ABI entry point returned a negative status."""
+
+
+def load(path=None):
+    """Loads the shared library once and declares every prototype. Raises if it is missing."""
+    global _lib
+    if _lib is not None and path is None:
+        return _lib
+    path = path or LIB_PATH
+    if not os.path.exists(path):
+        raise ImportError(
+            f"{path} is missing: the HIP extension is not built. "
+            "Run `python -m openrlhf_amd.csrc.build` (needs hipcc); there is no CPU fallback."
+        )
+    lib = ctypes.CDLL(path)
+    missing = [name for name in SIGNATURES if not hasattr(lib, name)]
+    if missing:
+        raise ImportError(f"{path} lacks symbols declared in include/openrlhf_amd.h: {missing}; rebuild it")
+    for name, (restype, argtypes) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = restype
+        fn.argtypes = argtypes
+    got = lib.orlhf_version()
+    if got != ABI_VERSION:
+        raise ImportError(f"{path}: ABI version {got}, binding expects {ABI_VERSION}")
+    _lib = lib
+    return lib
+
+
+def check(status, what):
+    if status != 0:
+        msg = load().orlhf_last_error().decode("utf-8", "replace")
+        raise KernelError(f"{what} failed with status {status}: {msg}")
+
+
+def call(name, *args):
+    """Calls entry point `name` and raises KernelError on a non-zero status."""
+    check(getattr(load(), name)(*args), name)
+
+
+# ------------------------------------------------------------------ tensor plumbing
+_DTYPES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+
+def dtype_code(t):
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; expected float32, bfloat16 or float16") from None
+
+
+def require_gpu(*tensors):
+    """All given tensors must live on one GPU; returns its device."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError(
+                "openrlhf_amd runs on the GPU only (hand-written HIP kernels, no CPU fallback); "
+                f"got a tensor on {t.device}"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors on different devices: {dev} and {t.device}")
+    if dev is None:
+        raise RuntimeError("no tensor given")
+    return dev
+
+
+def ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def stream_of(device):
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def mask_arg(mask):
+    """(tensor kept alive, pointer, mask dtype code) for a mask of any torch dtype."""
+    if mask is None:
+        return None, None, MASK_NONE
+    if mask.dtype in (torch.bool, torch.uint8):
+        m = mask.contiguous()
+        return m, m.data_ptr(), MASK_U8
+    if mask.dtype == torch.float32:
+        m = mask.contiguous()
+        return m, m.data_ptr(), MASK_F32
+    if mask.dtype == torch.int64:
+        m = mask.contiguous()
+        return m, m.data_ptr(), MASK_I64
+    m = mask.to(torch.float32).contiguous()  # other int / float types: exact for 0/1 masks
+    return m, m.data_ptr(), MASK_F32
+
+
+def make_norm(dp_size, value, keep):
+    """orlhf_norm from a Python number, a 0-dim tensor or None. Device tensors are passed by
+    pointer (no host synchronisation); `keep` collects tensors that must outlive the call."""
+    n = Norm()
+    n.dp_size = float(dp_size)
+    n.norm_value = math.nan
+    n.norm_dev = None
+    if value is None:
+        return n
+    if isinstance(value, torch.Tensor):
+        if value.is_cuda:
+            v = value.detach().reshape(-1)[:1].to(torch.float32).contiguous()
+            keep.append(v)
+            n.norm_dev = v.data_ptr()
+        else:
+            n.norm_value = float(value)
+    else:
+        n.norm_value = float(value)
+    return n

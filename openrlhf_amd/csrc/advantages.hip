@@ -1,0 +1,411 @@
+// Advantage kernels for gfx950: terminal-reward placement, GAE / discounted returns as a
+// parallel reverse-time scan, group baselines and global masked whitening. Forward only.
+//
+// The scan: A_t = delta_t + c * A_{t+1} is a linear recurrence with a constant coefficient, so a
+// lane that owns kScanItems consecutive tokens reduces them to an affine map C -> b + a*C of the
+// carry C entering from later tokens. Maps compose associatively; a wave composes its 64 maps with
+// log2(64) cross-lane steps, the 4 waves of the workgroup chain through LDS, and a row longer than
+// one tile (kBlock * kScanItems tokens) walks its tiles from the end carrying one number. Carries
+// and the in-lane recurrence are fp64, inputs and outputs fp32.
+#include "common.h"
+
+namespace orlhf {
+
+
+// ---------------------------------------------------------------- compute_reward
+template <int MASK_DT>
+__device__ __forceinline__ int64_t mask_as_int(const void* mask, int64_t i) {
+  if (MASK_DT == ORLHF_MASK_NONE) return 1;
+  if (MASK_DT == ORLHF_MASK_U8) return (int64_t)((const uint8_t*)mask)[i];
+  if (MASK_DT == ORLHF_MASK_F32) return (int64_t)((const float*)mask)[i];  // .long() truncates
+  return ((const int64_t*)mask)[i];
+}
+
+template <int MASK_DT>
+__global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const float* __restrict__ r,
+                                                                float neg_coef, const float* __restrict__ kl,
+                                                                const void* __restrict__ mask, int has_clip,
+                                                                float clip_lo, float clip_hi,
+                                                                float* __restrict__ reward,
+                                                                int64_t* __restrict__ eos_index) {
+  __shared__ int64_t lds_val[kWavesPerBlock];
+  __shared__ int64_t lds_idx[kWavesPerBlock];
+  for (int64_t b = blockIdx.x; b < rows.n_rows; b += gridDim.x) {
+    int64_t start, len;
+    row_span(rows, b, start, len);
+    if (len <= 0) {
+      if (threadIdx.x == 0 && eos_index != nullptr) eos_index[b] = -1;
+      continue;
+    }
+    // last position where (int64)mask is maximal == argmax over the flipped row
+    int64_t best_v = INT64_MIN, best_i = -1;
+    for (int64_t t = threadIdx.x; t < len; t += kBlock) {
+      const int64_t v = mask_as_int<MASK_DT>(mask, start + t);
+      if (v > best_v || (v == best_v && t > best_i)) {
+        best_v = v;
+        best_i = t;
+      }
+    }
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+      const int64_t ov = __shfl_xor(best_v, o, kWave);
+      const int64_t oi = __shfl_xor(best_i, o, kWave);
+      if (ov > best_v || (ov == best_v && oi > best_i)) {
+        best_v = ov;
+        best_i = oi;
+      }
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      lds_val[threadIdx.x / kWave] = best_v;
+      lds_idx[threadIdx.x / kWave] = best_i;
+    }
+    __syncthreads();
+    best_v = lds_val[0];
+    best_i = lds_idx[0];
+#pragma unroll
+    for (int w = 1; w < kWavesPerBlock; ++w) {
+      if (lds_val[w] > best_v || (lds_val[w] == best_v && lds_idx[w] > best_i)) {
+        best_v = lds_val[w];
+        best_i = lds_idx[w];
+      }
+    }
+    __syncthreads();
+    float rb = r[b];
+    if (has_clip) rb = (rb != rb) ? rb : fminf(fmaxf(rb, clip_lo), clip_hi);
+    for (int64_t t = threadIdx.x; t < len; t += kBlock) {
+      const float last = (t == best_i) ? rb : 0.0f;
+      reward[start + t] = last + neg_coef * kl[start + t];
+    }
+    if (threadIdx.x == 0 && eos_index != nullptr) eos_index[b] = best_i;
+  }
+}
+
+// ---------------------------------------------------------------- reverse scan (GAE, returns)
+constexpr int kScanItems = 8;
+constexpr int kScanTile = kBlock * kScanItems;
+
+struct Affine {  // C -> b + a * C
+  double a, b;
+};
+// apply `inner` first (later tokens), then `outer` (earlier tokens)
+__device__ __forceinline__ Affine compose(const Affine& outer, const Affine& inner) {
+  Affine r;
+  r.a = outer.a * inner.a;
+  r.b = outer.b + outer.a * inner.b;
+  return r;
+}
+
+template <int MASK_DT, bool GAE>
+__global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const float* __restrict__ values,
+                                                              const float* __restrict__ rewards,
+                                                              const void* __restrict__ mask, double gamma,
+                                                              double coef, float* __restrict__ adv,
+                                                              float* __restrict__ ret) {
+  __shared__ Affine lds_wave[kWavesPerBlock];
+  __shared__ double lds_carry;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+
+  double pw[kScanItems + 1];  // coef^k
+  pw[0] = 1.0;
+#pragma unroll
+  for (int k = 1; k <= kScanItems; ++k) pw[k] = pw[k - 1] * coef;
+
+  for (int64_t b = blockIdx.x; b < rows.n_rows; b += gridDim.x) {
+    int64_t start, len;
+    row_span(rows, b, start, len);
+    if (len <= 0) continue;
+    const int64_t n_tiles = (len + kScanTile - 1) / kScanTile;
+    double tile_carry = 0.0;  // A at the first token of the previous (later) tile
+    for (int64_t tile = n_tiles - 1; tile >= 0; --tile) {
+      const int64_t t0 = tile * kScanTile + (int64_t)threadIdx.x * kScanItems;
+      // masked inputs of this lane's tokens, plus the value of the token after them
+      float v[kScanItems + 1], rw[kScanItems];
+#pragma unroll
+      for (int j = 0; j < kScanItems; ++j) {
+        const int64_t t = t0 + j;
+        if (t < len) {
+          const float m = load_mask<MASK_DT>(mask, start + t);
+          rw[j] = m * rewards[start + t];
+          v[j] = GAE ? m * values[start + t] : 0.0f;
+        } else {
+          rw[j] = 0.0f;
+          v[j] = 0.0f;
+        }
+      }
+      {
+        const int64_t t = t0 + kScanItems;
+        v[kScanItems] = (GAE && t < len) ? load_mask<MASK_DT>(mask, start + t) * values[start + t] : 0.0f;
+      }
+      // in-lane recurrence with zero carry-in
+      double local[kScanItems];
+      double run = 0.0;
+#pragma unroll
+      for (int j = kScanItems - 1; j >= 0; --j) {
+        const double delta = GAE ? ((double)rw[j] + gamma * (double)v[j + 1]) - (double)v[j] : (double)rw[j];
+        run = delta + coef * run;
+        local[j] = run;
+      }
+      // inclusive suffix composition over the wave: lane i ends with the map of lanes i..63
+      Affine f;
+      f.a = pw[kScanItems];
+      f.b = local[0];
+#pragma unroll
+      for (int d = 1; d < kWave; d <<= 1) {
+        Affine o;
+        o.a = __shfl_down(f.a, d, kWave);
+        o.b = __shfl_down(f.b, d, kWave);
+        if (lane + d < kWave) f = compose(f, o);
+      }
+      if (lane == 0) lds_wave[wave] = f;
+      __syncthreads();
+      // carry entering this wave = maps of the later waves applied to the tile carry
+      double wave_carry = tile_carry;
+      for (int w = kWavesPerBlock - 1; w > wave; --w) wave_carry = lds_wave[w].b + lds_wave[w].a * wave_carry;
+      // carry entering this lane = A at the first token of lane+1
+      Affine nxt;
+      nxt.a = __shfl_down(f.a, 1, kWave);
+      nxt.b = __shfl_down(f.b, 1, kWave);
+      const double carry = (lane == kWave - 1) ? wave_carry : nxt.b + nxt.a * wave_carry;
+#pragma unroll
+      for (int j = 0; j < kScanItems; ++j) {
+        const int64_t t = t0 + j;
+        if (t < len) {
+          const double a_t = local[j] + pw[kScanItems - j] * carry;
+          if (GAE) {
+            adv[start + t] = (float)a_t;
+            ret[start + t] = (float)(a_t + (double)v[j]);
+          } else {
+            ret[start + t] = (float)a_t;
+          }
+        }
+      }
+      if (threadIdx.x == 0) lds_carry = local[0] + pw[kScanItems] * carry;
+      __syncthreads();
+      tile_carry = lds_carry;
+    }
+  }
+}
+
+// ---------------------------------------------------------------- group normalisation
+__global__ __launch_bounds__(kBlock) void scatter_kernel(const float* __restrict__ src,
+                                                         const int64_t* __restrict__ indices, int64_t n,
+                                                         float* __restrict__ dst) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t slot = indices ? indices[i] : i;
+    if (slot >= 0 && slot < n) dst[slot] = src[i];
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void group_normalize_kernel(const float* __restrict__ ordered,
+                                                                 const int64_t* __restrict__ indices, int64_t n_total,
+                                                                 int64_t n_samples, int estimator,
+                                                                 float* __restrict__ out,
+                                                                 float* __restrict__ group_std) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n_total; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t slot = indices ? indices[i] : i;
+    if (slot < 0 || slot >= n_total) {
+      out[i] = NAN;
+      if (group_std) group_std[i] = NAN;
+      continue;
+    }
+    const float* grp = ordered + (slot / n_samples) * n_samples;
+    double sum = 0.0;
+    for (int64_t k = 0; k < n_samples; ++k) sum += (double)grp[k];
+    const double mean = sum / (double)n_samples;
+    double ss = 0.0;
+    for (int64_t k = 0; k < n_samples; ++k) {
+      const double d = (double)grp[k] - mean;
+      ss += d * d;
+    }
+    const double std_unbiased = sqrt(ss / (double)(n_samples - 1));  // NaN for n == 1, like torch.std
+    const double x = (double)ordered[slot];
+    double y = x;
+    if (estimator == ORLHF_GROUP_RLOO)
+      y = x - (sum - x) / (double)(n_samples - 1);
+    else if (estimator == ORLHF_GROUP_BASELINE)
+      y = x - mean;
+    else if (estimator == ORLHF_GROUP_NORM)
+      y = (x - mean) / (std_unbiased + 1e-9);
+    out[i] = (float)y;
+    if (group_std) group_std[i] = (float)std_unbiased;
+  }
+}
+
+// ---------------------------------------------------------------- global masked whitening
+constexpr int kWhitenBlocks = 1024;
+
+template <int MASK_DT>
+__global__ __launch_bounds__(kBlock) void whiten_partial_kernel(const float* __restrict__ x,
+                                                                const void* __restrict__ mask, int64_t n,
+                                                                double* __restrict__ partial) {
+  __shared__ double lds[kWavesPerBlock];
+  double sx = 0.0, sxx = 0.0, sm = 0.0;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const double m = (double)load_mask<MASK_DT>(mask, i);
+    const double v = (double)x[i];
+    sx += v * m;
+    sxx += v * v * m;
+    sm += m;
+  }
+  sx = block_sum(sx, lds);
+  sxx = block_sum(sxx, lds);
+  sm = block_sum(sm, lds);
+  if (threadIdx.x == 0) {
+    partial[blockIdx.x * 3 + 0] = sx;
+    partial[blockIdx.x * 3 + 1] = sxx;
+    partial[blockIdx.x * 3 + 2] = sm;
+  }
+}
+
+// partial -> {mean, rstd} as floats right after the partials
+__global__ __launch_bounds__(kBlock) void whiten_final_kernel(const double* __restrict__ partial, int n_partial,
+                                                              int std_norm, float* __restrict__ mean_rstd,
+                                                              float* __restrict__ stats_out) {
+  __shared__ double lds[kWavesPerBlock];
+  double sx = 0.0, sxx = 0.0, sm = 0.0;
+  for (int i = threadIdx.x; i < n_partial; i += kBlock) {
+    sx += partial[i * 3 + 0];
+    sxx += partial[i * 3 + 1];
+    sm += partial[i * 3 + 2];
+  }
+  sx = block_sum(sx, lds);
+  sxx = block_sum(sxx, lds);
+  sm = block_sum(sm, lds);
+  if (threadIdx.x == 0) {
+    const double mean = sx / sm;
+    // sum((x-mean)^2 m)/sum(m) expanded; fp64 keeps the cancellation harmless
+    double var = sxx / sm - mean * mean;
+    double rstd = 1.0;
+    if (std_norm) rstd = 1.0 / sqrt(var > 1e-8 ? var : (var != var ? var : 1e-8));
+    mean_rstd[0] = (float)mean;
+    mean_rstd[1] = (float)rstd;
+    if (stats_out != nullptr) {
+      stats_out[0] = (float)mean;
+      stats_out[1] = (float)rstd;
+    }
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* __restrict__ x, int64_t n,
+                                                              const float* __restrict__ mean_rstd,
+                                                              float* __restrict__ out) {
+  const float mean = mean_rstd[0], rstd = mean_rstd[1];
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    out[i] = (x[i] - mean) * rstd;
+}
+
+
+
+template <bool GAE>
+static void launch_scan(int mask_dtype, Rows rows, const float* values, const float* rewards, const void* mask,
+                        double gamma, double coef, float* adv, float* ret, hipStream_t s) {
+  const dim3 grid((unsigned)(rows.n_rows < 65536 ? rows.n_rows : 65536)), block(kBlock);
+  switch (mask_dtype) {
+    case ORLHF_MASK_NONE: hipLaunchKernelGGL((reverse_scan_kernel<ORLHF_MASK_NONE, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, ret); break;
+    case ORLHF_MASK_U8: hipLaunchKernelGGL((reverse_scan_kernel<ORLHF_MASK_U8, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, ret); break;
+    case ORLHF_MASK_F32: hipLaunchKernelGGL((reverse_scan_kernel<ORLHF_MASK_F32, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, ret); break;
+    default: hipLaunchKernelGGL((reverse_scan_kernel<ORLHF_MASK_I64, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, ret); break;
+  }
+}
+
+}  // namespace orlhf
+
+using namespace orlhf;
+
+extern "C" int orlhf_compute_reward(const float* r, float kl_coef, const float* kl, const void* mask,
+                                    int mask_dtype, int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
+                                    int has_clip, float clip_low, float clip_high, float* reward,
+                                    int64_t* eos_index, orlhf_stream_t stream) {
+  if (int rc = check_rows("compute_reward", n_rows, n_cols, mask, mask_dtype)) return rc;
+  if (n_rows == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(r && reward && (kl || n_cols == 0), "compute_reward: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const float neg_coef = -(kl_coef > 0.0f ? kl_coef : 0.0f);
+  const dim3 grid((unsigned)(n_rows < 65536 ? n_rows : 65536)), block(kBlock);
+  switch (mask_dtype) {
+    case ORLHF_MASK_NONE: hipLaunchKernelGGL(compute_reward_kernel<ORLHF_MASK_NONE>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, clip_high, reward, eos_index); break;
+    case ORLHF_MASK_U8: hipLaunchKernelGGL(compute_reward_kernel<ORLHF_MASK_U8>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, clip_high, reward, eos_index); break;
+    case ORLHF_MASK_F32: hipLaunchKernelGGL(compute_reward_kernel<ORLHF_MASK_F32>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, clip_high, reward, eos_index); break;
+    default: hipLaunchKernelGGL(compute_reward_kernel<ORLHF_MASK_I64>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, clip_high, reward, eos_index); break;
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_compute_reward");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_gae_scan(const float* values, const float* rewards, const void* mask, int mask_dtype,
+                              int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens, float gamma, float lambd,
+                              float* advantages, float* returns, orlhf_stream_t stream) {
+  if (int rc = check_rows("gae_scan", n_rows, n_cols, mask, mask_dtype)) return rc;
+  if (n_rows * n_cols == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(values && rewards && advantages && returns, "gae_scan: NULL pointer");
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  launch_scan<true>(mask_dtype, rows, values, rewards, mask, (double)gamma, (double)gamma * (double)lambd,
+                    advantages, returns, (hipStream_t)stream);
+  ORLHF_CHECK_LAUNCH("orlhf_gae_scan");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_discounted_returns(const float* rewards, const void* mask, int mask_dtype, int64_t n_rows,
+                                        int64_t n_cols, const int64_t* cu_seqlens, float gamma, float* returns,
+                                        orlhf_stream_t stream) {
+  if (int rc = check_rows("discounted_returns", n_rows, n_cols, mask, mask_dtype)) return rc;
+  if (n_rows * n_cols == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(rewards && returns, "discounted_returns: NULL pointer");
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  launch_scan<false>(mask_dtype, rows, nullptr, rewards, mask, (double)gamma, (double)gamma, nullptr, returns,
+                     (hipStream_t)stream);
+  ORLHF_CHECK_LAUNCH("orlhf_discounted_returns");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_group_normalize(const float* rewards, const int64_t* indices, int64_t n_prompts,
+                                     int64_t n_samples, int estimator, float* out, float* group_std,
+                                     void* workspace, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_prompts >= 0 && n_samples >= 1, "group_normalize: n_prompts=%lld n_samples=%lld",
+                  (long long)n_prompts, (long long)n_samples);
+  ORLHF_CHECK_ARG(estimator >= ORLHF_GROUP_IDENTITY && estimator <= ORLHF_GROUP_NORM,
+                  "group_normalize: unknown estimator %d", estimator);
+  const int64_t n = n_prompts * n_samples;
+  if (n == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(rewards && out && workspace, "group_normalize: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  float* ordered = (float*)workspace;
+  hipLaunchKernelGGL(scatter_kernel, dim3(flat_grid(n, 4096)), dim3(kBlock), 0, s, rewards, indices, n, ordered);
+  ORLHF_CHECK_LAUNCH("orlhf_group_normalize(scatter)");
+  hipLaunchKernelGGL(group_normalize_kernel, dim3(flat_grid(n, 4096)), dim3(kBlock), 0, s, ordered, indices, n,
+                     n_samples, estimator, out, group_std);
+  ORLHF_CHECK_LAUNCH("orlhf_group_normalize");
+  return ORLHF_OK;
+}
+
+extern "C" int64_t orlhf_whiten_workspace_bytes(int64_t) {
+  return (int64_t)kWhitenBlocks * 3 * (int64_t)sizeof(double) + 64;
+}
+
+extern "C" int orlhf_masked_whiten(const float* x, const void* mask, int mask_dtype, int64_t n, int std_norm,
+                                   void* workspace, float* out, float* stats, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n >= 0, "masked_whiten: n=%lld", (long long)n);
+  ORLHF_CHECK_ARG(valid_mask_dtype(mask_dtype), "masked_whiten: unknown mask dtype %d", mask_dtype);
+  if (n == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(x && out && workspace, "masked_whiten: NULL pointer");
+  ORLHF_CHECK_ARG(mask_dtype == ORLHF_MASK_NONE || mask != nullptr, "masked_whiten: mask is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  double* partial = (double*)workspace;
+  float* mean_rstd = (float*)(partial + (int64_t)kWhitenBlocks * 3);
+  const int nb = flat_grid(n, kWhitenBlocks);
+  const dim3 grid(nb), block(kBlock);
+  switch (mask_dtype) {
+    case ORLHF_MASK_NONE: hipLaunchKernelGGL(whiten_partial_kernel<ORLHF_MASK_NONE>, grid, block, 0, s, x, mask, n, partial); break;
+    case ORLHF_MASK_U8: hipLaunchKernelGGL(whiten_partial_kernel<ORLHF_MASK_U8>, grid, block, 0, s, x, mask, n, partial); break;
+    case ORLHF_MASK_F32: hipLaunchKernelGGL(whiten_partial_kernel<ORLHF_MASK_F32>, grid, block, 0, s, x, mask, n, partial); break;
+    default: hipLaunchKernelGGL(whiten_partial_kernel<ORLHF_MASK_I64>, grid, block, 0, s, x, mask, n, partial); break;
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(partial)");
+  hipLaunchKernelGGL(whiten_final_kernel, dim3(1), block, 0, s, partial, nb, std_norm, mean_rstd, stats);
+  ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(final)");
+  hipLaunchKernelGGL(whiten_apply_kernel, dim3(flat_grid(n, 65536)), block, 0, s, x, n, mean_rstd, out);
+  ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(apply)");
+  return ORLHF_OK;
+}

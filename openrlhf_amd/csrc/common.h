@@ -1,0 +1,136 @@
+// Shared device/host helpers for the gfx950 (CDNA4, wave64) token-numerics kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/openrlhf_amd.h"
+
+namespace orlhf {
+
+constexpr int kWave = 64;       // CDNA wavefront width
+constexpr int kBlock = 256;     // 4 wave64 per workgroup: one wave per SIMD of a CU
+constexpr int kWavesPerBlock = kBlock / kWave;
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr double kLn2d = 0.6931471805599453;
+
+// ---------------------------------------------------------------- error state
+// Thread-local message behind orlhf_last_error(); set by every failing entry point.
+void set_error(const char* fmt, ...);
+int fail(int code, const char* fmt, ...);
+
+#define ORLHF_CHECK_ARG(cond, ...)                              \
+  do {                                                          \
+    if (!(cond)) return ::orlhf::fail(ORLHF_ERR_INVALID_ARG, __VA_ARGS__); \
+  } while (0)
+
+#define ORLHF_CHECK_LAUNCH(name)                                                     \
+  do {                                                                               \
+    hipError_t e_ = hipGetLastError();                                               \
+    if (e_ != hipSuccess)                                                            \
+      return ::orlhf::fail(ORLHF_ERR_LAUNCH, "%s: launch failed: %s", name, hipGetErrorString(e_)); \
+  } while (0)
+
+// ---------------------------------------------------------------- wave / block reductions
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
+  return v;
+}
+
+// Sum over a whole kBlock-thread workgroup; every thread gets the result. `lds` holds
+// kWavesPerBlock doubles and may be reused after the call returns (trailing barrier).
+__device__ __forceinline__ double block_sum(double v, double* lds) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wave] = v;
+  __syncthreads();
+  double r = 0.0;
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) r += lds[w];
+  __syncthreads();
+  return r;
+}
+
+// ---------------------------------------------------------------- dtype helpers
+__device__ __forceinline__ float as_float(uint32_t w) { return __builtin_bit_cast(float, w); }
+__device__ __forceinline__ uint32_t as_uint(float f) { return __builtin_bit_cast(uint32_t, f); }
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __builtin_bit_cast(float, w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __builtin_bit_cast(float, w & 0xffff0000u); }
+
+// Two fp32 -> packed bf16 pair, round-to-nearest-even (v_cvt_pk_bf16_f32 on gfx950).
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ uint32_t pack_f16(float a, float b) {
+  f32x2 v = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+}
+
+// Raw v_exp_f32 (2^x); inputs below -126 flush to zero, which is what the callers want.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Mask element as a float weight; the reference multiplies by the mask, so a float mask
+// acts as a weight and a bool mask as 0/1.
+template <int MASK_DT>
+__device__ __forceinline__ float load_mask(const void* mask, int64_t i) {
+  if (MASK_DT == ORLHF_MASK_NONE) return 1.0f;
+  if (MASK_DT == ORLHF_MASK_U8) return (float)((const uint8_t*)mask)[i];
+  if (MASK_DT == ORLHF_MASK_F32) return ((const float*)mask)[i];
+  return (float)((const int64_t*)mask)[i];
+}
+
+inline bool valid_mask_dtype(int m) { return m >= ORLHF_MASK_NONE && m <= ORLHF_MASK_I64; }
+
+// ---------------------------------------------------------------- per-token row layouts
+// padded: contiguous [n_rows, n_cols]; packed: row b = tokens cu[b] .. cu[b+1]-1 of a flat array.
+struct Rows {
+  int64_t n_rows, n_cols;
+  const int64_t* cu;  // packed layout when non-null
+};
+
+__device__ __forceinline__ void row_span(const Rows& r, int64_t b, int64_t& start, int64_t& len) {
+  if (r.cu != nullptr) {
+    start = r.cu[b];
+    len = r.cu[b + 1] - start;
+  } else {
+    start = b * r.n_cols;
+    len = r.n_cols;
+  }
+}
+
+inline int check_rows(const char* what, int64_t n_rows, int64_t n_cols, const void* mask, int mask_dtype) {
+  if (n_rows < 0 || n_cols < 0)
+    return fail(ORLHF_ERR_INVALID_ARG, "%s: n_rows=%lld n_cols=%lld", what, (long long)n_rows, (long long)n_cols);
+  if (!valid_mask_dtype(mask_dtype)) return fail(ORLHF_ERR_INVALID_ARG, "%s: unknown mask dtype %d", what, mask_dtype);
+  if (mask_dtype != ORLHF_MASK_NONE && mask == nullptr && n_rows * n_cols > 0)
+    return fail(ORLHF_ERR_INVALID_ARG, "%s: mask is NULL but mask dtype is %d", what, mask_dtype);
+  return ORLHF_OK;
+}
+
+inline int flat_grid(int64_t n, int cap = 65536) {
+  const int64_t g = (n + kBlock - 1) / kBlock;
+  return (int)(g < cap ? (g > 0 ? g : 1) : cap);
+}
+
+}  // namespace orlhf

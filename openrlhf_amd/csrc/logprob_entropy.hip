@@ -1,0 +1,715 @@
+// Vocabulary-row kernels for gfx950: fused log-softmax + gather + entropy forward and its
+// streaming backward. Both are pure HBM streams (read V elements per row; the backward also
+// writes V elements), so the design goal is bytes in flight, not arithmetic:
+//   * one 256-thread workgroup (4 wave64, one per SIMD) owns one vocabulary row;
+//   * every lane issues ORLHF_ROW_UNROLL independent 16-byte loads before it touches the data
+//     (8 x 4 KiB = 32 KiB per workgroup in flight with the default unroll);
+//   * the softmax statistics are accumulated against a per-wave reference maximum taken from the
+//     first 16-byte chunk of each lane instead of a running maximum: 1 fma + 1 v_exp_f32 + 2
+//     accumulates per element. A row whose sums come out non-finite (an element more than ~88
+//     nats above the reference, or inf/NaN logits) is re-read once with a classic per-lane online
+//     maximum, so the result never depends on the shortcut;
+//   * sums are kept in fp32 in 4 independent accumulators per lane, reduced over the wave with
+//     cross-lane shuffles and over the 4 waves through LDS; the per-row epilogue runs in fp64.
+#include "common.h"
+
+#ifndef ORLHF_ROW_UNROLL
+#define ORLHF_ROW_UNROLL 8
+#endif
+#ifndef ORLHF_NT_LOAD
+#define ORLHF_NT_LOAD 1
+#endif
+#ifndef ORLHF_NT_STORE
+#define ORLHF_NT_STORE 1
+#endif
+#ifndef ORLHF_FWD_WAVES_PER_EU
+#define ORLHF_FWD_WAVES_PER_EU 0
+#endif
+
+namespace orlhf {
+
+// ---------------------------------------------------------------- element traits
+template <int DT>
+struct Elt;
+
+template <>
+struct Elt<ORLHF_BF16> {
+  static constexpr int kSize = 2;
+  static constexpr int kPerVec = 8;
+  static __device__ __forceinline__ void unpack(const u32x4& r, float (&x)[8]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      x[2 * k] = bf16_lo(r[k]);
+      x[2 * k + 1] = bf16_hi(r[k]);
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float (&x)[8]) {
+    u32x4 r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) r[k] = pack_bf16(x[2 * k], x[2 * k + 1]);
+    return r;
+  }
+  static __device__ __forceinline__ float load1(const char* p) {
+    return __builtin_bit_cast(float, (uint32_t)(*(const uint16_t*)p) << 16);
+  }
+  static __device__ __forceinline__ void store1(char* p, float v) {
+    *(uint16_t*)p = (uint16_t)(pack_bf16(v, 0.0f) & 0xffffu);
+  }
+  static __device__ __forceinline__ float round(float v) { return bf16_lo(pack_bf16(v, 0.0f)); }
+};
+
+template <>
+struct Elt<ORLHF_F16> {
+  static constexpr int kSize = 2;
+  static constexpr int kPerVec = 8;
+  static __device__ __forceinline__ void unpack(const u32x4& r, float (&x)[8]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const uint32_t w = r[k];  // by value: a vector lane is not addressable
+      f16x2 h = __builtin_bit_cast(f16x2, w);
+      x[2 * k] = (float)h[0];
+      x[2 * k + 1] = (float)h[1];
+    }
+  }
+  static __device__ __forceinline__ u32x4 pack(const float (&x)[8]) {
+    u32x4 r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) r[k] = pack_f16(x[2 * k], x[2 * k + 1]);
+    return r;
+  }
+  static __device__ __forceinline__ float load1(const char* p) { return (float)(*(const _Float16*)p); }
+  static __device__ __forceinline__ void store1(char* p, float v) { *(_Float16*)p = (_Float16)v; }
+  static __device__ __forceinline__ float round(float v) { return (float)(_Float16)v; }
+};
+
+template <>
+struct Elt<ORLHF_F32> {
+  static constexpr int kSize = 4;
+  static constexpr int kPerVec = 4;
+  static __device__ __forceinline__ void unpack(const u32x4& r, float (&x)[4]) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) x[k] = as_float(r[k]);  // by value: a vector lane is not addressable
+  }
+  static __device__ __forceinline__ u32x4 pack(const float (&x)[4]) {
+    u32x4 r;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) r[k] = as_uint(x[k]);
+    return r;
+  }
+  static __device__ __forceinline__ float load1(const char* p) { return *(const float*)p; }
+  static __device__ __forceinline__ void store1(char* p, float v) { *(float*)p = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+
+__device__ __forceinline__ u32x4 load_vec(const char* p) {
+#if ORLHF_NT_LOAD
+  return __builtin_nontemporal_load((const u32x4*)p);
+#else
+  return *(const u32x4*)p;
+#endif
+}
+__device__ __forceinline__ void store_vec(char* p, const u32x4& v) {
+#if ORLHF_NT_STORE
+  __builtin_nontemporal_store(v, (u32x4*)p);
+#else
+  *(u32x4*)p = v;
+#endif
+}
+
+// ---------------------------------------------------------------- row geometry + traversal
+// A row is split into a scalar head (elements before the first 16-byte boundary), a body of
+// 16-byte vectors and a scalar tail, so any vocab size, row stride and base alignment works.
+// `scalar_only` (host decision: input and output rows are misaligned differently) turns the
+// whole row into the scalar part.
+struct RowGeom {
+  uint32_t head, nvec, tail;  // element / vector counts; a row is < 2 GiB (host check)
+};
+
+template <int DT>
+__device__ __forceinline__ RowGeom row_geom(const char* row, int64_t vocab, bool scalar_only) {
+  using E = Elt<DT>;
+  RowGeom g;
+  if (scalar_only) {
+    g.head = (uint32_t)vocab;
+    g.nvec = 0;
+    g.tail = 0;
+    return g;
+  }
+  const uint32_t mis = (uint32_t)((uintptr_t)row & 15u);
+  uint32_t head = mis ? (16u - mis) / E::kSize : 0u;
+  if (head > (uint32_t)vocab) head = (uint32_t)vocab;
+  g.head = head;
+  g.nvec = ((uint32_t)vocab - head) / E::kPerVec;
+  g.tail = (uint32_t)vocab - head - g.nvec * E::kPerVec;
+  return g;
+}
+
+// Visits every element of a row exactly once. f.vec(x, v) gets the kPerVec consecutive elements
+// of body vector v (element index head + v*kPerVec); f.one(x, e) gets element e. With STORE the
+// (modified) values are written to out_row at the same element positions in the same dtype.
+// All in-row offsets are 32-bit: the row base stays in scalar registers.
+template <int DT, bool STORE, typename F>
+__device__ __forceinline__ void traverse_row(const char* row, char* out_row, const RowGeom& g,
+                                             F& f) {
+  using E = Elt<DT>;
+  constexpr uint32_t U = ORLHF_ROW_UNROLL;
+  constexpr uint32_t EPV = E::kPerVec;
+  const uint32_t tid = threadIdx.x;
+  const char* body = row + g.head * E::kSize;
+  char* obody = STORE ? out_row + g.head * E::kSize : nullptr;
+
+  const uint32_t nbatch = g.nvec / (kBlock * U);
+  uint32_t v0 = tid;
+  for (uint32_t b = 0; b < nbatch; ++b, v0 += kBlock * U) {
+    u32x4 buf[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) buf[u] = load_vec(body + (v0 + u * kBlock) * 16u);
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      float x[EPV];
+      E::unpack(buf[u], x);
+      f.vec(x, v0 + u * kBlock);
+      if (STORE) store_vec(obody + (v0 + u * kBlock) * 16u, E::pack(x));
+    }
+  }
+  if (v0 < g.nvec) {  // last, partial batch: same loads in flight, predicated per vector
+    u32x4 buf[U];
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      const uint32_t v = v0 + u * kBlock;
+      if (v < g.nvec) buf[u] = load_vec(body + v * 16u);
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < U; ++u) {
+      const uint32_t v = v0 + u * kBlock;
+      if (v < g.nvec) {
+        float x[EPV];
+        E::unpack(buf[u], x);
+        f.vec(x, v);
+        if (STORE) store_vec(obody + v * 16u, E::pack(x));
+      }
+    }
+  }
+  // scalar head + tail (at most 2*(kPerVec-1) elements unless scalar_only)
+  const uint32_t nscalar = g.head + g.tail;
+  for (uint32_t k = tid; k < nscalar; k += kBlock) {
+    const uint32_t e = k < g.head ? k : g.head + g.nvec * EPV + (k - g.head);
+    float x = E::load1(row + e * E::kSize);
+    f.one(x, e);
+    if (STORE) E::store1(out_row + e * E::kSize, x);
+  }
+}
+
+// ---------------------------------------------------------------- forward accumulators
+// Modes: which statistics a row needs.
+//   kLpOnly   : sum exp(z - m)                      z = x / T
+//   kEntOnly  : sum exp(x - m), sum exp(x - m) * x
+//   kBothT1   : T == 1, one shared set
+//   kBothT    : T != 1, scaled set for the log-prob and unscaled set for the entropy
+enum FwdMode { kLpOnly = 0, kEntOnly = 1, kBothT1 = 2, kBothT = 3 };
+
+template <int MODE>
+struct ModeTraits {
+  static constexpr bool kScaledSet = (MODE == kLpOnly || MODE == kBothT);  // separate x/T set
+  static constexpr bool kPlainSet = (MODE != kLpOnly);                     // unscaled set (+ sum e*x)
+};
+
+constexpr int kAcc = 4;  // independent accumulators per lane
+
+// Fast path: exponent = x*c - M with a wave-uniform reference M (no running maximum).
+template <int MODE>
+struct FastAcc {
+  float cT, negMT, c1, negM1;
+  float sT[kAcc], s1[kAcc], t1[kAcc];
+  __device__ __forceinline__ void init(float m_ref, float c_scaled, float c_plain) {
+    cT = c_scaled;
+    c1 = c_plain;
+    negMT = -(m_ref * c_scaled);
+    negM1 = -(m_ref * c_plain);
+#pragma unroll
+    for (int k = 0; k < kAcc; ++k) sT[k] = s1[k] = t1[k] = 0.0f;
+  }
+  __device__ __forceinline__ void elem(float x, int k) {
+    if (ModeTraits<MODE>::kScaledSet) sT[k] += fast_exp2(fmaf(x, cT, negMT));
+    if (ModeTraits<MODE>::kPlainSet) {
+      const float e = fast_exp2(fmaf(x, c1, negM1));
+      s1[k] += e;
+      t1[k] = fmaf(e, x, t1[k]);
+    }
+  }
+  template <int N>
+  __device__ __forceinline__ void vec(float (&x)[N], uint32_t) {
+#pragma unroll
+    for (int j = 0; j < N; ++j) elem(x[j], j % kAcc);
+  }
+  __device__ __forceinline__ void one(float& x, uint32_t) { elem(x, 0); }
+  __device__ __forceinline__ void fold(float& st, float& s, float& t) const {
+    st = (sT[0] + sT[1]) + (sT[2] + sT[3]);
+    s = (s1[0] + s1[1]) + (s1[2] + s1[3]);
+    t = (t1[0] + t1[1]) + (t1[2] + t1[3]);
+  }
+};
+
+// Safe path: per-lane running maximum m (raw logit units), sums relative to it.
+template <int MODE>
+struct SafeAcc {
+  float cT, c1;
+  float m, sT, s1, t1;
+  __device__ __forceinline__ void init(float c_scaled, float c_plain) {
+    cT = c_scaled;
+    c1 = c_plain;
+    m = -INFINITY;
+    sT = s1 = t1 = 0.0f;
+  }
+  __device__ __forceinline__ void raise(float cm) {
+    if (cm > m) {  // also true for the first finite element (m == -inf)
+      if (m != -INFINITY) {
+        const float d = m - cm;  // < 0, or -inf when cm == +inf
+        if (ModeTraits<MODE>::kScaledSet) sT *= fast_exp2(d * cT);
+        if (ModeTraits<MODE>::kPlainSet) {
+          const float r = fast_exp2(d * c1);
+          s1 *= r;
+          t1 *= r;
+        }
+      }
+      m = cm;
+    }
+  }
+  __device__ __forceinline__ void elem(float x) {
+    if (m == -INFINITY) {
+      // only -inf (or NaN) seen so far: exp() contributes 0 to the sums, but the reference's
+      // softmax(x)*x is 0 * -inf = NaN for such an element (a NaN logit poisons everything).
+      if (ModeTraits<MODE>::kPlainSet) t1 = NAN;
+      if (x != x) sT = s1 = NAN;
+      return;
+    }
+    // x == m covers m == +inf (inf - inf would be NaN): such an element counts as exp(0),
+    // which makes logsumexp +inf and the entropy NaN, as in the reference
+    const float d = (x == m) ? 0.0f : x - m;
+    if (ModeTraits<MODE>::kScaledSet) sT += fast_exp2(d * cT);
+    if (ModeTraits<MODE>::kPlainSet) {
+      const float e = fast_exp2(d * c1);
+      s1 += e;
+      t1 = fmaf(e, x, t1);
+    }
+  }
+  template <int N>
+  __device__ __forceinline__ void vec(float (&x)[N], uint32_t) {
+    float cm = x[0];
+#pragma unroll
+    for (int j = 1; j < N; ++j) cm = fmaxf(cm, x[j]);
+    raise(cm);
+#pragma unroll
+    for (int j = 0; j < N; ++j) elem(x[j]);
+  }
+  __device__ __forceinline__ void one(float& x, uint32_t) {
+    raise(x);
+    elem(x);
+  }
+};
+
+// Workgroup-combined sums. Fast pass: exponents were x*c - M, MT / M1 hold M (log2 units).
+// Safe pass: exponents were (x - m)*c, MT and M1 both hold the row maximum m (logit units).
+struct RowSums {
+  float MT, sT, M1, s1, t1;
+};
+
+__device__ __forceinline__ bool sums_usable(float s) { return s > 0.0f && s < INFINITY; }
+
+// ---------------------------------------------------------------- forward kernel
+template <int DT, int MODE>
+__global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
+    const char* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
+    const int64_t* __restrict__ labels, double temperature, float* __restrict__ logprob,
+    float* __restrict__ entropy, float* __restrict__ row_stats, int scalar_only) {
+  using E = Elt<DT>;
+  using MT = ModeTraits<MODE>;
+  __shared__ float lds[kWavesPerBlock][8];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1);
+  const int wave = tid / kWave;
+  const float c_plain = kLog2e;
+  const float c_scaled = (float)(1.4426950408889634 / temperature);
+
+  for (int64_t row_i = blockIdx.x; row_i < n_rows; row_i += gridDim.x) {
+    const char* row = logits + row_i * row_stride_bytes;
+    const RowGeom g = row_geom<DT>(row, vocab, scalar_only != 0);
+
+    // ---- reference maximum of this wave: first vector (or first scalar) of each lane
+    float m_ref = -INFINITY;
+    if (g.nvec > 0) {
+      const uint32_t v = (uint32_t)tid < g.nvec ? (uint32_t)tid : g.nvec - 1;
+      float x[E::kPerVec];
+      E::unpack(load_vec(row + g.head * E::kSize + v * 16u), x);
+#pragma unroll
+      for (int j = 0; j < E::kPerVec; ++j) m_ref = fmaxf(m_ref, x[j]);
+    } else {
+      const uint32_t e = (uint32_t)tid < (uint32_t)vocab ? (uint32_t)tid : (uint32_t)vocab - 1;
+      m_ref = E::load1(row + e * E::kSize);
+    }
+    m_ref = wave_max(m_ref);
+
+    // ---- fast pass
+    RowSums sums;
+    {
+      FastAcc<MODE> acc;
+      acc.init(m_ref, c_scaled, c_plain);
+      traverse_row<DT, false>(row, nullptr, g, acc);
+      float st, s, t;
+      acc.fold(st, s, t);
+      st = wave_sum(st);
+      s = wave_sum(s);
+      t = wave_sum(t);
+      if (lane == 0) {
+        lds[wave][0] = -acc.negMT;
+        lds[wave][1] = st;
+        lds[wave][2] = -acc.negM1;
+        lds[wave][3] = s;
+        lds[wave][4] = t;
+      }
+      __syncthreads();
+      float MTm = lds[0][0], M1m = lds[0][2];
+#pragma unroll
+      for (int w = 1; w < kWavesPerBlock; ++w) {
+        MTm = fmaxf(MTm, lds[w][0]);
+        M1m = fmaxf(M1m, lds[w][2]);
+      }
+      sums.MT = MTm;
+      sums.M1 = M1m;
+      sums.sT = sums.s1 = sums.t1 = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        const float rT = fast_exp2(lds[w][0] - MTm);
+        const float r1 = fast_exp2(lds[w][2] - M1m);
+        sums.sT = fmaf(lds[w][1], rT, sums.sT);
+        sums.s1 = fmaf(lds[w][3], r1, sums.s1);
+        sums.t1 = fmaf(lds[w][4], r1, sums.t1);
+      }
+      __syncthreads();
+    }
+    bool ok = true;
+    if (MT::kScaledSet) ok = ok && sums_usable(sums.sT);
+    if (MT::kPlainSet) ok = ok && sums_usable(sums.s1) && (fabsf(sums.t1) < INFINITY);
+
+    // ---- safe pass (workgroup-uniform branch; rare)
+    if (!ok) {
+      SafeAcc<MODE> acc;
+      acc.init(c_scaled, c_plain);
+      traverse_row<DT, false>(row, nullptr, g, acc);
+      const float m_w = wave_max(acc.m);
+      // rescale each lane to the wave maximum; a lane that saw nothing finite keeps its
+      // sums (0 or NaN markers) untouched
+      float st = acc.sT, s = acc.s1, t = acc.t1;
+      if (acc.m != -INFINITY && m_w != acc.m) {
+        const float d = acc.m - m_w;
+        st *= fast_exp2(d * c_scaled);
+        const float r = fast_exp2(d * c_plain);
+        s *= r;
+        t *= r;
+      }
+      st = wave_sum(st);
+      s = wave_sum(s);
+      t = wave_sum(t);
+      if (lane == 0) {
+        lds[wave][0] = m_w;
+        lds[wave][1] = st;
+        lds[wave][3] = s;
+        lds[wave][4] = t;
+      }
+      __syncthreads();
+      float m_all = lds[0][0];
+#pragma unroll
+      for (int w = 1; w < kWavesPerBlock; ++w) m_all = fmaxf(m_all, lds[w][0]);
+      sums.sT = sums.s1 = sums.t1 = 0.0f;
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        const float mw = lds[w][0];
+        float rT = 1.0f, r1 = 1.0f;
+        if (mw != -INFINITY && mw != m_all) {
+          rT = fast_exp2((mw - m_all) * c_scaled);
+          r1 = fast_exp2((mw - m_all) * c_plain);
+        }
+        sums.sT += lds[w][1] * rT;
+        sums.s1 += lds[w][3] * r1;
+        sums.t1 += lds[w][4] * r1;
+      }
+      sums.MT = sums.M1 = m_all;
+      __syncthreads();
+    }
+
+    // ---- per-row epilogue in fp64
+    if (tid == 0) {
+      double lse_t = 0.0, lse_1 = 0.0, ex = 0.0;
+      if (MT::kScaledSet) {
+        const double base = ok ? (double)sums.MT * kLn2d : (double)sums.MT / temperature;
+        lse_t = base + log((double)sums.sT);
+      }
+      if (MT::kPlainSet) {
+        const double base = ok ? (double)sums.M1 * kLn2d : (double)sums.M1;
+        lse_1 = base + log((double)sums.s1);
+        ex = (double)sums.t1 / (double)sums.s1;
+        if (!MT::kScaledSet) lse_t = lse_1;  // T == 1 (or entropy only)
+      }
+      if (MODE != kEntOnly && logprob != nullptr) {
+        const int64_t label = labels[row_i];
+        float lp;
+        if (label >= 0 && label < vocab) {
+          const double xl = (double)E::load1(row + label * E::kSize);
+          lp = (float)(xl / temperature - lse_t);
+        } else {
+          lp = (label == -100) ? 0.0f : NAN;
+        }
+        logprob[row_i] = lp;
+      }
+      if (MT::kPlainSet && entropy != nullptr) entropy[row_i] = (float)(lse_1 - ex);
+      if (row_stats != nullptr) {
+        f32x4 st = {(float)lse_t, (float)(MT::kPlainSet ? lse_1 : lse_t), (float)ex, 0.0f};
+        *(f32x4*)(row_stats + row_i * 4) = st;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- backward kernel
+enum BwdMode { kBwdLp = 0, kBwdEnt = 1, kBwdBothT1 = 2, kBwdBothT = 3 };
+
+template <int MODE>
+struct GradFn {
+  float cT, negLT, c1, negL1;  // exponents: x*c - lse*log2e
+  float a_lp;                  // -g_lp / T          (coefficient of softmax(z))
+  float gh, k1;                // entropy term p*(k1 - gh*x); k1 = gh*E (- g_lp when T == 1)
+  float onehot;                // g_lp / T
+  uint32_t label_vec;          // body vector holding the label (0xffffffff: none)
+  uint32_t label_lane;         // its position inside that vector
+  uint32_t label_elem;         // the label as an element index (0xffffffff: out of range)
+  __device__ __forceinline__ float elem(float x) const {
+    if (MODE == kBwdLp) return fast_exp2(fmaf(x, cT, negLT)) * a_lp;
+    if (MODE == kBwdEnt || MODE == kBwdBothT1) return fast_exp2(fmaf(x, c1, negL1)) * fmaf(-gh, x, k1);
+    const float pt = fast_exp2(fmaf(x, cT, negLT));
+    const float p1 = fast_exp2(fmaf(x, c1, negL1));
+    return fmaf(pt, a_lp, p1 * fmaf(-gh, x, k1));
+  }
+  template <int N>
+  __device__ __forceinline__ void vec(float (&x)[N], uint32_t v) const {
+#pragma unroll
+    for (int j = 0; j < N; ++j) x[j] = elem(x[j]);
+    if (MODE != kBwdEnt && v == label_vec) {
+#pragma unroll
+      for (int j = 0; j < N; ++j) x[j] += ((uint32_t)j == label_lane) ? onehot : 0.0f;
+    }
+  }
+  __device__ __forceinline__ void one(float& x, uint32_t e) const {
+    x = elem(x);
+    if (MODE != kBwdEnt && e == label_elem) x += onehot;
+  }
+  __device__ __forceinline__ void set_label(int64_t label, int64_t vocab, const RowGeom& g, int epv) {
+    label_vec = label_lane = label_elem = 0xffffffffu;
+    if (label < 0 || label >= vocab) return;
+    label_elem = (uint32_t)label;
+    if (label_elem >= g.head && label_elem < g.head + g.nvec * (uint32_t)epv) {
+      label_vec = (label_elem - g.head) / (uint32_t)epv;
+      label_lane = (label_elem - g.head) % (uint32_t)epv;
+    }
+  }
+};
+
+// Zero-fills a row without reading it.
+template <int DT>
+__device__ __forceinline__ void zero_row(char* out_row, const RowGeom& g) {
+  using E = Elt<DT>;
+  const uint32_t tid = threadIdx.x;
+  char* obody = out_row + g.head * E::kSize;
+  const u32x4 z = {0u, 0u, 0u, 0u};
+  for (uint32_t v = tid; v < g.nvec; v += kBlock) store_vec(obody + v * 16u, z);
+  const uint32_t nscalar = g.head + g.tail;
+  for (uint32_t k = tid; k < nscalar; k += kBlock) {
+    const uint32_t e = k < g.head ? k : g.head + g.nvec * E::kPerVec + (k - g.head);
+    E::store1(out_row + e * E::kSize, 0.0f);
+  }
+}
+
+template <int DT, int MODE>
+__global__ __launch_bounds__(kBlock) void logprob_entropy_bwd_kernel(
+    const char* logits, char* grad, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
+    int64_t grad_stride_bytes, const int64_t* __restrict__ labels, double temperature,
+    const float* __restrict__ g_logprob, const float* __restrict__ g_entropy,
+    const float* __restrict__ row_stats, int scalar_only) {
+  const double inv_t = 1.0 / temperature;
+  for (int64_t row_i = blockIdx.x; row_i < n_rows; row_i += gridDim.x) {
+    const char* row = logits + row_i * row_stride_bytes;
+    char* out_row = grad + row_i * grad_stride_bytes;
+    // the geometry follows the OUTPUT row when only zeros are written, the input row otherwise
+    // (the host guarantees both have the same 16-byte phase unless scalar_only is set)
+    const RowGeom g = row_geom<DT>(row, vocab, scalar_only != 0);
+
+    const float glp = (MODE != kBwdEnt) ? g_logprob[row_i] : 0.0f;
+    const float gh = (MODE != kBwdLp) ? g_entropy[row_i] : 0.0f;
+    if (glp == 0.0f && gh == 0.0f) {
+      zero_row<DT>(out_row, g);
+      continue;
+    }
+    const f32x4 st = *(const f32x4*)(row_stats + row_i * 4);
+    GradFn<MODE> fn;
+    fn.cT = (float)(1.4426950408889634 * inv_t);
+    fn.c1 = kLog2e;
+    fn.negLT = -(float)((double)st[0] * 1.4426950408889634);
+    fn.negL1 = -(float)((double)st[1] * 1.4426950408889634);
+    fn.a_lp = -(float)((double)glp * inv_t);
+    fn.onehot = (float)((double)glp * inv_t);
+    fn.gh = gh;
+    fn.k1 = gh * st[2] - (MODE == kBwdBothT1 ? glp : 0.0f);
+    fn.set_label((MODE != kBwdEnt) ? labels[row_i] : -1, vocab, g, Elt<DT>::kPerVec);
+    traverse_row<DT, true>(row, out_row, g, fn);
+  }
+}
+
+// ---------------------------------------------------------------- host side
+static int grid_for_rows(int64_t n_rows) {
+  // one workgroup per row; cap the grid and stride over rows beyond it
+  const int64_t cap = 1 << 20;
+  return (int)(n_rows < cap ? n_rows : cap);
+}
+
+template <int DT>
+static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                      const int64_t* labels, double temperature, float* logprob, float* entropy,
+                      float* row_stats, hipStream_t stream) {
+  using E = Elt<DT>;
+  const bool want_lp = logprob != nullptr;
+  const bool want_ent = entropy != nullptr;
+  const bool t1 = (temperature == 1.0);
+  const int mode = !want_ent ? kLpOnly : (!want_lp ? kEntOnly : (t1 ? kBothT1 : kBothT));
+  const char* p = (const char*)logits;
+  const int64_t stride_bytes = row_stride * E::kSize;
+  const int scalar_only = 0;
+  const dim3 grid(grid_for_rows(n_rows)), block(kBlock);
+#define ORLHF_FWD(M)                                                                          \
+  hipLaunchKernelGGL((logprob_entropy_fwd_kernel<DT, M>), grid, block, 0, stream, p, n_rows,  \
+                     vocab, stride_bytes, labels, temperature, logprob, entropy, row_stats,   \
+                     scalar_only)
+  switch (mode) {
+    case kLpOnly: ORLHF_FWD(kLpOnly); break;
+    case kEntOnly: ORLHF_FWD(kEntOnly); break;
+    case kBothT1: ORLHF_FWD(kBothT1); break;
+    default: ORLHF_FWD(kBothT); break;
+  }
+#undef ORLHF_FWD
+  ORLHF_CHECK_LAUNCH("orlhf_logprob_entropy_fwd");
+  return ORLHF_OK;
+}
+
+template <int DT>
+static int launch_bwd(const void* logits, void* grad, int64_t n_rows, int64_t vocab,
+                      int64_t row_stride, int64_t grad_row_stride, const int64_t* labels,
+                      double temperature, const float* g_logprob, const float* g_entropy,
+                      const float* row_stats, hipStream_t stream) {
+  using E = Elt<DT>;
+  const bool has_lp = g_logprob != nullptr;
+  const bool has_ent = g_entropy != nullptr;
+  const bool t1 = (temperature == 1.0);
+  const int mode = !has_ent ? kBwdLp : (!has_lp ? kBwdEnt : (t1 ? kBwdBothT1 : kBwdBothT));
+  const char* p = (const char*)logits;
+  char* gp = (char*)grad;
+  const int64_t stride_bytes = row_stride * E::kSize;
+  const int64_t gstride_bytes = grad_row_stride * E::kSize;
+  // vector path needs input and output rows on the same 16-byte phase
+  const bool same_phase = (((uintptr_t)p ^ (uintptr_t)gp) & 15u) == 0 &&
+                          ((stride_bytes - gstride_bytes) & 15) == 0;
+  const int scalar_only = same_phase ? 0 : 1;
+  const dim3 grid(grid_for_rows(n_rows)), block(kBlock);
+#define ORLHF_BWD(M)                                                                          \
+  hipLaunchKernelGGL((logprob_entropy_bwd_kernel<DT, M>), grid, block, 0, stream, p, gp,      \
+                     n_rows, vocab, stride_bytes, gstride_bytes, labels, temperature,         \
+                     g_logprob, g_entropy, row_stats, scalar_only)
+  switch (mode) {
+    case kBwdLp: ORLHF_BWD(kBwdLp); break;
+    case kBwdEnt: ORLHF_BWD(kBwdEnt); break;
+    case kBwdBothT1: ORLHF_BWD(kBwdBothT1); break;
+    default: ORLHF_BWD(kBwdBothT); break;
+  }
+#undef ORLHF_BWD
+  ORLHF_CHECK_LAUNCH("orlhf_logprob_entropy_bwd");
+  return ORLHF_OK;
+}
+
+}  // namespace orlhf
+
+using namespace orlhf;
+
+extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows,
+                                         int64_t vocab, int64_t row_stride, const int64_t* labels,
+                                         double temperature, float* logprob, float* entropy,
+                                         float* row_stats, int flags, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_rows >= 0 && vocab > 0, "logprob_entropy_fwd: n_rows=%lld vocab=%lld",
+                  (long long)n_rows, (long long)vocab);
+  ORLHF_CHECK_ARG(row_stride >= vocab, "logprob_entropy_fwd: row_stride %lld < vocab %lld",
+                  (long long)row_stride, (long long)vocab);
+  ORLHF_CHECK_ARG(vocab < (1ll << 29), "logprob_entropy_fwd: vocab %lld too large (row must stay below 2 GiB)",
+                  (long long)vocab);
+  ORLHF_CHECK_ARG(logprob != nullptr || entropy != nullptr,
+                  "logprob_entropy_fwd: logprob and entropy are both NULL");
+  ORLHF_CHECK_ARG(temperature > 0.0 && temperature == temperature,
+                  "logprob_entropy_fwd: temperature must be > 0");
+  ORLHF_CHECK_ARG(flags == 0, "logprob_entropy_fwd: unknown flags 0x%x", flags);
+  if (n_rows == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(logits != nullptr, "logprob_entropy_fwd: logits is NULL");
+  ORLHF_CHECK_ARG(logprob == nullptr || labels != nullptr, "logprob_entropy_fwd: labels is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case ORLHF_F32:
+      ORLHF_CHECK_ARG(((uintptr_t)logits & 3u) == 0, "logprob_entropy_fwd: logits not 4-byte aligned");
+      return launch_fwd<ORLHF_F32>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
+                                   entropy, row_stats, s);
+    case ORLHF_BF16:
+      ORLHF_CHECK_ARG(((uintptr_t)logits & 1u) == 0, "logprob_entropy_fwd: logits not 2-byte aligned");
+      return launch_fwd<ORLHF_BF16>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
+                                    entropy, row_stats, s);
+    case ORLHF_F16:
+      ORLHF_CHECK_ARG(((uintptr_t)logits & 1u) == 0, "logprob_entropy_fwd: logits not 2-byte aligned");
+      return launch_fwd<ORLHF_F16>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
+                                   entropy, row_stats, s);
+    default:
+      return fail(ORLHF_ERR_INVALID_ARG, "logprob_entropy_fwd: unknown dtype %d", dtype);
+  }
+}
+
+extern "C" int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, int dtype,
+                                         int64_t n_rows, int64_t vocab, int64_t row_stride,
+                                         int64_t grad_row_stride, const int64_t* labels,
+                                         double temperature, const float* g_logprob,
+                                         const float* g_entropy, const float* row_stats,
+                                         orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_rows >= 0 && vocab > 0, "logprob_entropy_bwd: n_rows=%lld vocab=%lld",
+                  (long long)n_rows, (long long)vocab);
+  ORLHF_CHECK_ARG(row_stride >= vocab && grad_row_stride >= vocab,
+                  "logprob_entropy_bwd: row strides %lld/%lld < vocab %lld", (long long)row_stride,
+                  (long long)grad_row_stride, (long long)vocab);
+  ORLHF_CHECK_ARG(vocab < (1ll << 29), "logprob_entropy_bwd: vocab %lld too large (row must stay below 2 GiB)",
+                  (long long)vocab);
+  ORLHF_CHECK_ARG(g_logprob != nullptr || g_entropy != nullptr,
+                  "logprob_entropy_bwd: g_logprob and g_entropy are both NULL");
+  ORLHF_CHECK_ARG(temperature > 0.0 && temperature == temperature,
+                  "logprob_entropy_bwd: temperature must be > 0");
+  if (n_rows == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(logits != nullptr && grad_logits != nullptr && row_stats != nullptr,
+                  "logprob_entropy_bwd: NULL logits / grad_logits / row_stats");
+  ORLHF_CHECK_ARG(g_logprob == nullptr || labels != nullptr, "logprob_entropy_bwd: labels is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  const int esize = dtype == ORLHF_F32 ? 4 : 2;
+  ORLHF_CHECK_ARG((((uintptr_t)logits | (uintptr_t)grad_logits) & (uintptr_t)(esize - 1)) == 0,
+                  "logprob_entropy_bwd: pointers not aligned to the element size");
+  switch (dtype) {
+    case ORLHF_F32:
+      return launch_bwd<ORLHF_F32>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride,
+                                   labels, temperature, g_logprob, g_entropy, row_stats, s);
+    case ORLHF_BF16:
+      return launch_bwd<ORLHF_BF16>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride,
+                                    labels, temperature, g_logprob, g_entropy, row_stats, s);
+    case ORLHF_F16:
+      return launch_bwd<ORLHF_F16>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride,
+                                   labels, temperature, g_logprob, g_entropy, row_stats, s);
+    default:
+      return fail(ORLHF_ERR_INVALID_ARG, "logprob_entropy_bwd: unknown dtype %d", dtype);
+  }
+}

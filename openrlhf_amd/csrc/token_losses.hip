@@ -1,0 +1,697 @@
+// Per-token kernels for gfx950: approximate KL, masked token / sequence aggregation, the PPO
+// (and GSPO) policy surrogate and the clipped value loss, each with its backward.
+//
+// Layout: a [n_rows, n_cols] problem is cut into chunks of kChunk tokens of one row; a workgroup
+// evaluates one chunk elementwise (coalesced 4-byte loads, 4 tokens per lane) and reduces the
+// quantities it needs to one fp64 partial per (row, chunk). A second, single-workgroup kernel
+// folds the partials per row and over rows in a fixed order and writes the scalars plus a
+// per-row aggregation weight that the backward kernels multiply with. No atomics anywhere:
+// the result is bit-reproducible. All of these are HBM-bound streams of 4-17 bytes per token.
+#include "common.h"
+
+namespace orlhf {
+
+constexpr int kTokPerLane = 4;
+constexpr int kChunk = kBlock * kTokPerLane;  // tokens of one row per workgroup
+constexpr int kMaxQ = 6;                      // quantities reduced per token
+constexpr int kMaxGridY = 32768;
+
+
+static inline int64_t chunks_of(int64_t n_cols) { return n_cols > 0 ? (n_cols + kChunk - 1) / kChunk : 1; }
+
+struct NormArg {
+  double dp_size, value;
+  const float* dev;
+};
+
+static inline NormArg norm_arg(const orlhf_norm* n) {
+  NormArg a;
+  a.dp_size = n ? n->dp_size : 1.0;
+  a.value = n ? n->norm_value : (double)NAN;
+  a.dev = n ? n->norm_dev : nullptr;
+  return a;
+}
+
+// ---------------------------------------------------------------- token functors
+// Each functor evaluates one token: q[] are the quantities to reduce (already multiplied by the
+// mask weight where the reference multiplies), and grad() is d(token loss)/d(input).
+
+struct AggTok {  // aggregate_loss / masked_mean: x*m and m
+  static constexpr int kQ = 2;
+  const float* x;
+  __device__ __forceinline__ void eval(int64_t, int64_t i, float m, float* q) const {
+    q[0] = x[i] * m;
+    q[1] = m;
+  }
+};
+
+struct PolicyTok {
+  static constexpr int kQ = 5;
+  const float *lp, *old, *adv, *rollout;
+  const float* row_aux;  // [n_rows, 2]
+  float lo, hi;          // 1 - eps_low, 1 + eps_high
+  float dual;            // <= 0: off
+  int gspo;
+  int is_mode;
+  float is_lo, is_hi;
+
+  // loss of one token and its derivative wrt the probability ratio
+  __device__ __forceinline__ void surrogate(float ratio, float a, float& loss, float& dratio,
+                                            float& clipped) const {
+    const float s1 = ratio * a;
+    const float rc = fminf(fmaxf(ratio, lo), hi);
+    const float in_clip = (ratio >= lo && ratio <= hi) ? 1.0f : 0.0f;  // clamp passes grad on [lo, hi]
+    const float s2 = rc * a;
+    // torch.min: gradient to the smaller operand, split evenly on ties
+    const float w1 = s1 < s2 ? 1.0f : (s1 > s2 ? 0.0f : 0.5f);
+    const float w2 = 1.0f - w1;
+    float val = fminf(s1, s2);
+    float dval = w1 * a + w2 * a * in_clip;  // d(min)/d(ratio)
+    if (dual > 0.0f && a < 0.0f) {
+      const float floor_v = dual * a;
+      // torch.max(clip1, c*A): gradient to clip1 only where it is the larger one
+      const float wk = val > floor_v ? 1.0f : (val < floor_v ? 0.0f : 0.5f);
+      val = fmaxf(val, floor_v);
+      dval *= wk;
+    }
+    if (s1 != s1 || s2 != s2) val = NAN;  // torch.min / torch.max propagate NaN, fminf does not
+    loss = -val;
+    dratio = -dval;
+    clipped = s2 < s1 ? 1.0f : 0.0f;
+  }
+
+  __device__ __forceinline__ float is_weight(int64_t b, int64_t i) const {
+    if (is_mode == ORLHF_IS_NONE || gspo) return 1.0f;
+    const float w = expf(old[i] - rollout[i]);
+    if (is_mode == ORLHF_IS_TIS) return fminf(fmaxf(w, is_lo), is_hi);
+    if (is_mode == ORLHF_IS_ICEPOP) return (w >= is_lo && w <= is_hi) ? w : 0.0f;
+    return row_aux[b * 2] * w;  // seq-mask-tis: row keep flag times the unclamped token weight
+  }
+
+  // ratio and d(ratio)/d(lp) of the token's own log-prob (GSPO: handled by the caller)
+  __device__ __forceinline__ void ppo_ratio(float raw, float& ratio, float& dr) const {
+    const float c = fminf(fmaxf(raw, -20.0f), 20.0f);
+    ratio = expf(c);
+    dr = (raw >= -20.0f && raw <= 20.0f) ? ratio : 0.0f;
+  }
+
+  __device__ __forceinline__ void eval(int64_t b, int64_t i, float m, float* q) const {
+    const float raw = lp[i] - old[i];
+    float ratio, dr;
+    if (gspo) {
+      ratio = row_aux[b * 2] * m;
+    } else {
+      ppo_ratio(raw, ratio, dr);
+    }
+    float loss, dratio, clipped;
+    surrogate(ratio, adv[i], loss, dratio, clipped);
+    loss *= is_weight(b, i);
+    q[0] = loss * m;
+    q[1] = m;
+    q[2] = clipped * m;
+    q[3] = -raw * m;
+    q[4] = (is_mode != ORLHF_IS_NONE && !gspo) ? (rollout[i] - old[i]) * m : 0.0f;
+  }
+
+  // PPO: d(token loss)/d(lp[i]).  GSPO: d(token loss)/d(ratio) * m (summed per row by the caller).
+  __device__ __forceinline__ float grad(int64_t b, int64_t i, float m) const {
+    const float raw = lp[i] - old[i];
+    float ratio, dr;
+    if (gspo) {
+      ratio = row_aux[b * 2] * m;
+      dr = m;
+    } else {
+      ppo_ratio(raw, ratio, dr);
+    }
+    float loss, dratio, clipped;
+    surrogate(ratio, adv[i], loss, dratio, clipped);
+    return is_weight(b, i) * dratio * dr;
+  }
+};
+
+struct ValueTok {
+  static constexpr int kQ = 2;
+  const float *v, *old, *ret;
+  int has_clip;
+  float eps;
+  __device__ __forceinline__ void both(int64_t i, float& loss, float& dv) const {
+    const float x = v[i], r = ret[i];
+    const float e2 = x - r;
+    const float b2 = e2 * e2;
+    if (!has_clip) {
+      loss = b2;
+      dv = 2.0f * e2;
+      return;
+    }
+    const float o = old[i];
+    const float d = x - o;
+    const float dc = fminf(fmaxf(d, -eps), eps);
+    const float in_clip = (d >= -eps && d <= eps) ? 1.0f : 0.0f;
+    const float e1 = (o + dc) - r;
+    const float a2 = e1 * e1;
+    // torch.max: gradient to the larger operand, split evenly on ties
+    const float wa = a2 > b2 ? 1.0f : (a2 < b2 ? 0.0f : 0.5f);
+    loss = fmaxf(a2, b2);
+    if (a2 != a2 || b2 != b2) loss = NAN;
+    dv = wa * 2.0f * e1 * in_clip + (1.0f - wa) * 2.0f * e2;
+  }
+  __device__ __forceinline__ void eval(int64_t, int64_t i, float m, float* q) const {
+    float loss, dv;
+    both(i, loss, dv);
+    q[0] = loss * m;
+    q[1] = m;
+  }
+  __device__ __forceinline__ float grad(int64_t, int64_t i, float) const {
+    float loss, dv;
+    both(i, loss, dv);
+    return dv;
+  }
+};
+
+struct RatioTok {  // row prepass: sum(lr*m), sum(m) with lr = a - b
+  static constexpr int kQ = 2;
+  const float *a, *b;
+  __device__ __forceinline__ void eval(int64_t, int64_t i, float m, float* q) const {
+    q[0] = (a[i] - b[i]) * m;
+    q[1] = m;
+  }
+};
+
+struct GspoGradTok {  // backward row sum: m * d(token loss)/d(ratio_t) * d(ratio_t)/d(s_b)
+  static constexpr int kQ = 1;
+  PolicyTok p;
+  __device__ __forceinline__ void eval(int64_t b, int64_t i, float m, float* q) const {
+    q[0] = p.grad(b, i, m) * m;
+  }
+};
+
+// ---------------------------------------------------------------- stage 1: chunk partials
+template <int MASK_DT, typename Tok>
+__global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const void* __restrict__ mask,
+                                                              Tok tok, double* __restrict__ partial,
+                                                              int n_chunks) {
+  constexpr int NQ = Tok::kQ;
+  __shared__ double lds[kWavesPerBlock];
+  for (int64_t b = blockIdx.y; b < rows.n_rows; b += gridDim.y) {
+    int64_t start, len;
+    row_span(rows, b, start, len);
+    const int64_t c0 = (int64_t)blockIdx.x * kChunk;
+    double acc[NQ];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) acc[i] = 0.0;
+#pragma unroll
+    for (int k = 0; k < kTokPerLane; ++k) {
+      const int64_t t = c0 + threadIdx.x + k * kBlock;
+      if (t < len) {
+        const float m = load_mask<MASK_DT>(mask, start + t);
+        float q[NQ];
+        tok.eval(b, start + t, m, q);
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) acc[i] += (double)q[i];
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+      const double r = block_sum(acc[i], lds);
+      if (threadIdx.x == 0) partial[(b * n_chunks + blockIdx.x) * NQ + i] = r;
+    }
+  }
+}
+
+// ---------------------------------------------------------------- stage 2: rows -> scalars
+// Quantity 0 is the loss numerator, quantity 1 the mask weight; quantities 2.. are numerators of
+// plain masked means. out[0] = post_scale * aggregate(q0); out[k-1] = sum(qk)/sum(q1), k >= 2.
+// row_coef[b] = post_scale * d(aggregate)/d(row b's masked token sum).
+template <int NQ>
+__global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int n_chunks,
+                                                            const double* __restrict__ partial, int mode,
+                                                            NormArg norm, float post_scale, int n_out,
+                                                            float* __restrict__ out,
+                                                            float* __restrict__ row_coef) {
+  __shared__ double lds[kWavesPerBlock];
+  double tot[NQ];
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) tot[i] = 0.0;
+  double seq_sum = 0.0, seq_cnt = 0.0;
+  for (int64_t b = threadIdx.x; b < n_rows; b += kBlock) {
+    double rq[NQ];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) rq[i] = 0.0;
+    for (int c = 0; c < n_chunks; ++c) {
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) rq[i] += partial[(b * n_chunks + c) * NQ + i];
+    }
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) tot[i] += rq[i];
+    if (mode == ORLHF_AGG_SEQ_MEAN) {
+      if (rq[1] > 0.0) {
+        seq_sum += rq[0] / (rq[1] + 1e-8);
+        seq_cnt += 1.0;
+      } else if (rq[0] != rq[0]) {
+        seq_sum += rq[0];  // NaN * 0 stays NaN in the reference
+      }
+    } else if (mode == ORLHF_AGG_ROW_MEAN) {
+      out[b] = (float)(rq[0] / rq[1]);
+    }
+    if (row_coef != nullptr) row_coef[b] = (float)rq[1];  // finished below
+  }
+  if (mode == ORLHF_AGG_ROW_MEAN) {
+    if (row_coef != nullptr) {
+      __syncthreads();
+      for (int64_t b = threadIdx.x; b < n_rows; b += kBlock) row_coef[b] = 1.0f / row_coef[b];
+    }
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) tot[i] = block_sum(tot[i], lds);
+  seq_sum = block_sum(seq_sum, lds);
+  seq_cnt = block_sum(seq_cnt, lds);
+
+  const bool given = norm.dev != nullptr || norm.value == norm.value;
+  const double denom_given = norm.dev != nullptr ? (double)norm.dev[0] : norm.value;
+  double scale;  // d(loss)/d(numerator)
+  double loss;
+  if (mode == ORLHF_AGG_TOKEN_MEAN) {
+    scale = given ? norm.dp_size / denom_given : 1.0 / tot[1];
+    loss = given ? tot[0] / denom_given * norm.dp_size : tot[0] / tot[1];
+  } else {
+    scale = given ? norm.dp_size / denom_given : 1.0 / seq_cnt;
+    loss = given ? seq_sum / denom_given * norm.dp_size : seq_sum / seq_cnt;
+  }
+  if (threadIdx.x == 0) {
+    out[0] = (float)((double)post_scale * loss);
+    for (int i = 2; i < NQ && i - 1 < n_out; ++i) out[i - 1] = (float)(tot[i] / tot[1]);
+  }
+  if (row_coef != nullptr) {
+    for (int64_t b = threadIdx.x; b < n_rows; b += kBlock) {
+      const double cnt = (double)row_coef[b];
+      double c;
+      if (mode == ORLHF_AGG_TOKEN_MEAN)
+        c = scale;
+      else
+        c = cnt > 0.0 ? scale / (cnt + 1e-8) : 0.0;
+      row_coef[b] = (float)((double)post_scale * c);
+    }
+  }
+}
+
+// Row prepass results for GSPO (kind 0) and seq-mask-TIS (kind 1): row_aux[b] = {value, 1/max(cnt,1)}.
+__global__ __launch_bounds__(kBlock) void row_aux_kernel(int64_t n_rows, int n_chunks,
+                                                         const double* __restrict__ partial, int kind,
+                                                         float is_lo, float is_hi,
+                                                         float* __restrict__ row_aux) {
+  for (int64_t b = (int64_t)blockIdx.x * kBlock + threadIdx.x; b < n_rows; b += (int64_t)gridDim.x * kBlock) {
+    double s = 0.0, cnt = 0.0;
+    for (int c = 0; c < n_chunks; ++c) {
+      s += partial[(b * n_chunks + c) * 2];
+      cnt += partial[(b * n_chunks + c) * 2 + 1];
+    }
+    const float inv = (float)(1.0 / (cnt > 1.0 ? cnt : 1.0));
+    float v;
+    if (kind == 0) {
+      v = expf((float)(s / (cnt > 1.0 ? cnt : 1.0)));  // exp(sum(lr*m) / clamp(sum(m), 1))
+    } else {
+      const float w = expf((float)(s / cnt));  // exp(masked_mean): NaN for an empty row -> dropped
+      v = (w >= is_lo && w <= is_hi) ? 1.0f : 0.0f;
+    }
+    row_aux[b * 2] = v;
+    row_aux[b * 2 + 1] = inv;
+  }
+}
+
+// ---------------------------------------------------------------- backward, elementwise
+// g[b,t] = g_out * row_coef[b] * m * tok.grad(...)
+template <int MASK_DT, typename Tok>
+__global__ __launch_bounds__(kBlock) void rows_grad_kernel(Rows rows, const void* __restrict__ mask, Tok tok,
+                                                           const float* __restrict__ g_out, int g_per_row,
+                                                           const float* __restrict__ row_coef,
+                                                           float* __restrict__ g) {
+  for (int64_t b = blockIdx.y; b < rows.n_rows; b += gridDim.y) {
+    int64_t start, len;
+    row_span(rows, b, start, len);
+    const float w = (g_per_row ? g_out[b] : g_out[0]) * row_coef[b];
+    const int64_t c0 = (int64_t)blockIdx.x * kChunk;
+#pragma unroll
+    for (int k = 0; k < kTokPerLane; ++k) {
+      const int64_t t = c0 + threadIdx.x + k * kBlock;
+      if (t < len) {
+        const float m = load_mask<MASK_DT>(mask, start + t);
+        g[start + t] = w * m * tok.grad(b, start + t, m);
+      }
+    }
+  }
+}
+
+struct UnitGrad {  // aggregate backward: d(x*m)/dx / m = 1
+  __device__ __forceinline__ float grad(int64_t, int64_t, float) const { return 1.0f; }
+};
+
+// GSPO backward: g[b,t] = g_out * row_coef[b] * rowsum_b * s_b * m / max(cnt_b, 1)
+template <int MASK_DT>
+__global__ __launch_bounds__(kBlock) void gspo_grad_kernel(Rows rows, const void* __restrict__ mask,
+                                                           const double* __restrict__ partial, int n_chunks,
+                                                           const float* __restrict__ g_out,
+                                                           const float* __restrict__ row_coef,
+                                                           const float* __restrict__ row_aux,
+                                                           float* __restrict__ g) {
+  for (int64_t b = blockIdx.y; b < rows.n_rows; b += gridDim.y) {
+    int64_t start, len;
+    row_span(rows, b, start, len);
+    double rs = 0.0;
+    for (int c = 0; c < n_chunks; ++c) rs += partial[b * n_chunks + c];
+    const float w = g_out[0] * row_coef[b] * (float)rs * row_aux[b * 2] * row_aux[b * 2 + 1];
+    const int64_t c0 = (int64_t)blockIdx.x * kChunk;
+#pragma unroll
+    for (int k = 0; k < kTokPerLane; ++k) {
+      const int64_t t = c0 + threadIdx.x + k * kBlock;
+      if (t < len) g[start + t] = w * load_mask<MASK_DT>(mask, start + t);
+    }
+  }
+}
+
+// ---------------------------------------------------------------- approximate KL (flat)
+template <int DT>
+__device__ __forceinline__ float load_as_float(const void* p, int64_t i) {
+  if (DT == ORLHF_F32) return ((const float*)p)[i];
+  if (DT == ORLHF_BF16) return __builtin_bit_cast(float, (uint32_t)((const uint16_t*)p)[i] << 16);
+  return (float)((const _Float16*)p)[i];
+}
+
+__device__ __forceinline__ void kl_value(int est, float d, float& v, float& dv) {
+  if (est == ORLHF_KL_K1) {
+    v = d;
+    dv = 1.0f;
+  } else if (est == ORLHF_KL_K2) {
+    v = d * d / 2.0f;
+    dv = d;
+  } else {
+    const float e = expf(-d);
+    v = e - 1.0f + d;
+    dv = 1.0f - e;
+  }
+  if (v == v) {  // NaN passes through untouched, like torch.clamp
+    if (v < -10.0f || v > 10.0f) dv = 0.0f;  // clamp passes the gradient on the closed interval only
+    v = fminf(fmaxf(v, -10.0f), 10.0f);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void approx_kl_fwd_kernel(const void* __restrict__ lp,
+                                                               const void* __restrict__ base, int64_t n, int est,
+                                                               float* __restrict__ out) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    float v, dv;
+    kl_value(est, load_as_float<DT>(lp, i) - load_as_float<DT>(base, i), v, dv);
+    out[i] = v;
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void approx_kl_bwd_kernel(const void* __restrict__ lp,
+                                                               const void* __restrict__ base, int64_t n, int est,
+                                                               const float* __restrict__ g_out,
+                                                               float* __restrict__ g_lp, float* __restrict__ g_base) {
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    float v, dv;
+    kl_value(est, load_as_float<DT>(lp, i) - load_as_float<DT>(base, i), v, dv);
+    const float g = g_out[i] * dv;
+    if (g_lp != nullptr) g_lp[i] = g;
+    if (g_base != nullptr) g_base[i] = -g;
+  }
+}
+
+// ---------------------------------------------------------------- host helpers
+static inline dim3 row_grid(int64_t n_rows, int64_t n_cols) {
+  return dim3((unsigned)chunks_of(n_cols), (unsigned)(n_rows < kMaxGridY ? n_rows : kMaxGridY));
+}
+
+template <typename Tok>
+static void launch_partial(int mask_dt, Rows rows, const void* mask, const Tok& tok, double* partial,
+                           int n_chunks, hipStream_t s) {
+  const dim3 grid = row_grid(rows.n_rows, rows.n_cols), block(kBlock);
+  switch (mask_dt) {
+    case ORLHF_MASK_NONE:
+      hipLaunchKernelGGL((rows_partial_kernel<ORLHF_MASK_NONE, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks);
+      break;
+    case ORLHF_MASK_U8:
+      hipLaunchKernelGGL((rows_partial_kernel<ORLHF_MASK_U8, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks);
+      break;
+    case ORLHF_MASK_F32:
+      hipLaunchKernelGGL((rows_partial_kernel<ORLHF_MASK_F32, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks);
+      break;
+    default:
+      hipLaunchKernelGGL((rows_partial_kernel<ORLHF_MASK_I64, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks);
+      break;
+  }
+}
+
+template <typename Tok>
+static void launch_grad(int mask_dt, Rows rows, const void* mask, const Tok& tok, const float* g_out,
+                        int g_per_row, const float* row_coef, float* g, hipStream_t s) {
+  const dim3 grid = row_grid(rows.n_rows, rows.n_cols), block(kBlock);
+  switch (mask_dt) {
+    case ORLHF_MASK_NONE:
+      hipLaunchKernelGGL((rows_grad_kernel<ORLHF_MASK_NONE, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g);
+      break;
+    case ORLHF_MASK_U8:
+      hipLaunchKernelGGL((rows_grad_kernel<ORLHF_MASK_U8, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g);
+      break;
+    case ORLHF_MASK_F32:
+      hipLaunchKernelGGL((rows_grad_kernel<ORLHF_MASK_F32, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g);
+      break;
+    default:
+      hipLaunchKernelGGL((rows_grad_kernel<ORLHF_MASK_I64, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g);
+      break;
+  }
+}
+
+
+static PolicyTok policy_tok(const float* lp, const float* old, const float* adv, const float* rollout,
+                            const float* row_aux, const orlhf_policy_params* p) {
+  PolicyTok t;
+  t.lp = lp;
+  t.old = old;
+  t.adv = adv;
+  t.rollout = rollout;
+  t.row_aux = row_aux;
+  t.lo = 1.0f - p->clip_eps_low;
+  t.hi = 1.0f + p->clip_eps_high;
+  t.dual = p->dual_clip;
+  t.gspo = p->policy_type == ORLHF_POLICY_GSPO;
+  t.is_mode = p->is_correction;
+  t.is_lo = p->is_low;
+  t.is_hi = p->is_high;
+  return t;
+}
+
+static int check_policy(const char* what, const orlhf_policy_params* p, const float* rollout) {
+  if (p == nullptr) return fail(ORLHF_ERR_INVALID_ARG, "%s: params is NULL", what);
+  if (p->policy_type != ORLHF_POLICY_PPO && p->policy_type != ORLHF_POLICY_GSPO)
+    return fail(ORLHF_ERR_INVALID_ARG, "%s: unknown policy_type %d", what, p->policy_type);
+  if (p->is_correction < ORLHF_IS_NONE || p->is_correction > ORLHF_IS_SEQ_MASK_TIS)
+    return fail(ORLHF_ERR_INVALID_ARG, "%s: unknown is_correction %d", what, p->is_correction);
+  if (p->is_correction != ORLHF_IS_NONE && rollout == nullptr)
+    return fail(ORLHF_ERR_INVALID_ARG, "%s: importance correction needs rollout_log_probs", what);
+  if (p->dual_clip > 0.0f && !(p->dual_clip > 1.0f))
+    return fail(ORLHF_ERR_INVALID_ARG, "%s: dual_clip must be > 1.0, got %g", what, (double)p->dual_clip);
+  return ORLHF_OK;
+}
+
+}  // namespace orlhf
+
+using namespace orlhf;
+
+extern "C" int64_t orlhf_token_workspace_bytes(int64_t n_rows, int64_t n_cols) {
+  if (n_rows < 0 || n_cols < 0) return 0;
+  return (n_rows > 0 ? n_rows : 1) * chunks_of(n_cols) * kMaxQ * (int64_t)sizeof(double) + 256;
+}
+
+extern "C" int orlhf_approx_kl_fwd(const void* log_probs, const void* log_probs_base, int dtype, int64_t n,
+                                   int estimator, float* out, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n >= 0, "approx_kl_fwd: n=%lld", (long long)n);
+  ORLHF_CHECK_ARG(estimator >= ORLHF_KL_K1 && estimator <= ORLHF_KL_K3, "approx_kl_fwd: unknown estimator %d", estimator);
+  if (n == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(log_probs && log_probs_base && out, "approx_kl_fwd: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(flat_grid(n)), block(kBlock);
+  switch (dtype) {
+    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
+    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
+    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
+    default: return fail(ORLHF_ERR_INVALID_ARG, "approx_kl_fwd: unknown dtype %d", dtype);
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_approx_kl_fwd");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_approx_kl_bwd(const void* log_probs, const void* log_probs_base, int dtype, int64_t n,
+                                   int estimator, const float* g_out, float* g_lp, float* g_base,
+                                   orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n >= 0, "approx_kl_bwd: n=%lld", (long long)n);
+  ORLHF_CHECK_ARG(estimator >= ORLHF_KL_K1 && estimator <= ORLHF_KL_K3, "approx_kl_bwd: unknown estimator %d", estimator);
+  if (n == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(log_probs && log_probs_base && g_out && (g_lp || g_base), "approx_kl_bwd: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid(flat_grid(n)), block(kBlock);
+  switch (dtype) {
+    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
+    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
+    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
+    default: return fail(ORLHF_ERR_INVALID_ARG, "approx_kl_bwd: unknown dtype %d", dtype);
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_approx_kl_bwd");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_masked_aggregate_fwd(const float* x, const void* mask, int mask_dtype, int64_t n_rows,
+                                          int64_t n_cols, const int64_t* cu_seqlens, int mode,
+                                          const orlhf_norm* norm, void* workspace, float* out,
+                                          float* row_coef, orlhf_stream_t stream) {
+  if (int rc = check_rows("masked_aggregate_fwd", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(mode >= ORLHF_AGG_TOKEN_MEAN && mode <= ORLHF_AGG_ROW_MEAN, "masked_aggregate_fwd: unknown mode %d", mode);
+  ORLHF_CHECK_ARG(out != nullptr && workspace != nullptr, "masked_aggregate_fwd: NULL out / workspace");
+  ORLHF_CHECK_ARG(x != nullptr || n_rows * n_cols == 0, "masked_aggregate_fwd: x is NULL");
+  hipStream_t s = (hipStream_t)stream;
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const int n_chunks = (int)chunks_of(n_cols);
+  double* partial = (double*)workspace;
+  if (n_rows > 0) {
+    AggTok tok{x};
+    launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
+    ORLHF_CHECK_LAUNCH("orlhf_masked_aggregate_fwd(partial)");
+  }
+  hipLaunchKernelGGL(rows_final_kernel<2>, dim3(1), dim3(kBlock), 0, s, n_rows, n_chunks, partial, mode,
+                     norm_arg(norm), 1.0f, 1, out, row_coef);
+  ORLHF_CHECK_LAUNCH("orlhf_masked_aggregate_fwd(final)");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_masked_aggregate_bwd(const float* g_out, const void* mask, int mask_dtype, int64_t n_rows,
+                                          int64_t n_cols, const int64_t* cu_seqlens, int mode,
+                                          const float* row_coef, float* g_x, orlhf_stream_t stream) {
+  if (int rc = check_rows("masked_aggregate_bwd", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(mode >= ORLHF_AGG_TOKEN_MEAN && mode <= ORLHF_AGG_ROW_MEAN, "masked_aggregate_bwd: unknown mode %d", mode);
+  if (n_rows * n_cols == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(g_out && row_coef && g_x, "masked_aggregate_bwd: NULL pointer");
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  launch_grad(mask_dtype, rows, mask, UnitGrad{}, g_out, mode == ORLHF_AGG_ROW_MEAN, row_coef, g_x, (hipStream_t)stream);
+  ORLHF_CHECK_LAUNCH("orlhf_masked_aggregate_bwd");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_log_probs, const float* advantages,
+                                     const void* mask, int mask_dtype, const float* rollout_log_probs,
+                                     int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
+                                     const orlhf_policy_params* params, void* workspace, float* out4,
+                                     float* row_coef, float* row_aux, orlhf_stream_t stream) {
+  if (int rc = check_rows("policy_loss_fwd", n_rows, n_cols, mask, mask_dtype)) return rc;
+  if (int rc = check_policy("policy_loss_fwd", params, rollout_log_probs)) return rc;
+  ORLHF_CHECK_ARG(out4 && workspace && row_aux, "policy_loss_fwd: NULL out4 / workspace / row_aux");
+  ORLHF_CHECK_ARG((log_probs && old_log_probs && advantages) || n_rows * n_cols == 0, "policy_loss_fwd: NULL input");
+  hipStream_t s = (hipStream_t)stream;
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const int n_chunks = (int)chunks_of(n_cols);
+  double* partial = (double*)workspace;
+  const bool gspo = params->policy_type == ORLHF_POLICY_GSPO;
+  const bool use_is = params->is_correction != ORLHF_IS_NONE;
+  if (n_rows > 0 && (gspo || params->is_correction == ORLHF_IS_SEQ_MASK_TIS)) {
+    RatioTok pre;
+    if (gspo) {
+      pre.a = log_probs;
+      pre.b = use_is ? rollout_log_probs : old_log_probs;
+    } else {
+      pre.a = old_log_probs;
+      pre.b = rollout_log_probs;
+    }
+    launch_partial(mask_dtype, rows, mask, pre, partial, n_chunks, s);
+    ORLHF_CHECK_LAUNCH("orlhf_policy_loss_fwd(prepass)");
+    hipLaunchKernelGGL(row_aux_kernel, dim3(flat_grid(n_rows)), dim3(kBlock), 0, s, n_rows, n_chunks, partial,
+                       gspo ? 0 : 1, params->is_low, params->is_high, row_aux);
+    ORLHF_CHECK_LAUNCH("orlhf_policy_loss_fwd(row_aux)");
+  }
+  if (n_rows > 0) {
+    PolicyTok tok = policy_tok(log_probs, old_log_probs, advantages, rollout_log_probs, row_aux, params);
+    launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
+    ORLHF_CHECK_LAUNCH("orlhf_policy_loss_fwd(partial)");
+  }
+  const int mode = (params->token_level && !gspo) ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN;
+  const int n_out = (use_is && !gspo) ? 4 : 3;
+  hipLaunchKernelGGL(rows_final_kernel<5>, dim3(1), dim3(kBlock), 0, s, n_rows, n_chunks, partial, mode,
+                     norm_arg(&params->norm), 1.0f, n_out, out4, row_coef);
+  ORLHF_CHECK_LAUNCH("orlhf_policy_loss_fwd(final)");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs, const float* old_log_probs,
+                                     const float* advantages, const void* mask, int mask_dtype,
+                                     const float* rollout_log_probs, int64_t n_rows, int64_t n_cols,
+                                     const int64_t* cu_seqlens, const orlhf_policy_params* params,
+                                     const float* row_coef, const float* row_aux, void* workspace,
+                                     float* g_log_probs, orlhf_stream_t stream) {
+  if (int rc = check_rows("policy_loss_bwd", n_rows, n_cols, mask, mask_dtype)) return rc;
+  if (int rc = check_policy("policy_loss_bwd", params, rollout_log_probs)) return rc;
+  if (n_rows * n_cols == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(g_out && log_probs && old_log_probs && advantages && row_coef && row_aux && g_log_probs,
+                  "policy_loss_bwd: NULL pointer");
+  hipStream_t s = (hipStream_t)stream;
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  PolicyTok tok = policy_tok(log_probs, old_log_probs, advantages, rollout_log_probs, row_aux, params);
+  if (!tok.gspo) {
+    launch_grad(mask_dtype, rows, mask, tok, g_out, 0, row_coef, g_log_probs, s);
+    ORLHF_CHECK_LAUNCH("orlhf_policy_loss_bwd");
+    return ORLHF_OK;
+  }
+  ORLHF_CHECK_ARG(workspace != nullptr, "policy_loss_bwd: GSPO needs a workspace");
+  const int n_chunks = (int)chunks_of(n_cols);
+  double* partial = (double*)workspace;
+  GspoGradTok gt{tok};
+  launch_partial(mask_dtype, rows, mask, gt, partial, n_chunks, s);
+  ORLHF_CHECK_LAUNCH("orlhf_policy_loss_bwd(gspo partial)");
+  const dim3 grid = row_grid(n_rows, n_cols), block(kBlock);
+  switch (mask_dtype) {
+    case ORLHF_MASK_NONE: hipLaunchKernelGGL(gspo_grad_kernel<ORLHF_MASK_NONE>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, g_log_probs); break;
+    case ORLHF_MASK_U8: hipLaunchKernelGGL(gspo_grad_kernel<ORLHF_MASK_U8>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, g_log_probs); break;
+    case ORLHF_MASK_F32: hipLaunchKernelGGL(gspo_grad_kernel<ORLHF_MASK_F32>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, g_log_probs); break;
+    default: hipLaunchKernelGGL(gspo_grad_kernel<ORLHF_MASK_I64>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, g_log_probs); break;
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_policy_loss_bwd(gspo grad)");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_value_loss_fwd(const float* values, const float* old_values, const float* returns,
+                                    const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                                    const int64_t* cu_seqlens, int has_clip, float clip_eps, int token_level,
+                                    const orlhf_norm* norm, void* workspace, float* out, float* row_coef,
+                                    orlhf_stream_t stream) {
+  if (int rc = check_rows("value_loss_fwd", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(out && workspace, "value_loss_fwd: NULL out / workspace");
+  ORLHF_CHECK_ARG((values && returns && (old_values || !has_clip)) || n_rows * n_cols == 0, "value_loss_fwd: NULL input");
+  hipStream_t s = (hipStream_t)stream;
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const int n_chunks = (int)chunks_of(n_cols);
+  double* partial = (double*)workspace;
+  if (n_rows > 0) {
+    ValueTok tok{values, old_values, returns, has_clip, clip_eps};
+    launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
+    ORLHF_CHECK_LAUNCH("orlhf_value_loss_fwd(partial)");
+  }
+  hipLaunchKernelGGL(rows_final_kernel<2>, dim3(1), dim3(kBlock), 0, s, n_rows, n_chunks, partial,
+                     token_level ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN, norm_arg(norm), 0.5f, 1, out, row_coef);
+  ORLHF_CHECK_LAUNCH("orlhf_value_loss_fwd(final)");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_value_loss_bwd(const float* g_out, const float* values, const float* old_values,
+                                    const float* returns, const void* mask, int mask_dtype, int64_t n_rows,
+                                    int64_t n_cols, const int64_t* cu_seqlens, int has_clip, float clip_eps,
+                                    const float* row_coef, float* g_values, orlhf_stream_t stream) {
+  if (int rc = check_rows("value_loss_bwd", n_rows, n_cols, mask, mask_dtype)) return rc;
+  if (n_rows * n_cols == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(g_out && values && returns && (old_values || !has_clip) && row_coef && g_values,
+                  "value_loss_bwd: NULL pointer");
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  ValueTok tok{values, old_values, returns, has_clip, clip_eps};
+  launch_grad(mask_dtype, rows, mask, tok, g_out, 0, row_coef, g_values, (hipStream_t)stream);
+  ORLHF_CHECK_LAUNCH("orlhf_value_loss_bwd");
+  return ORLHF_OK;
+}

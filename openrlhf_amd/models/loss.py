@@ -1,0 +1,253 @@
+"""Losses with the signatures of ``openrlhf.models.loss`` on hand-written HIP kernels.
+
+Mirrors (paths relative to the OpenRLHF tree):
+  aggregate_loss   openrlhf/models/loss.py:11-39
+  SFTLoss          openrlhf/models/loss.py:87-113
+  PolicyLoss       openrlhf/models/loss.py:116-230
+  ValueLoss        openrlhf/models/loss.py:233-269
+
+Each loss is one elementwise + reduction launch pair forward and one elementwise launch
+backward instead of the reference's chain of ~20 eager kernels. Per-token inputs are consumed
+as fp32. ``batch_num_tokens`` / ``global_batch_size`` may be Python numbers or 0-dim tensors
+(device tensors are read on the device, no host synchronisation). Every loss also accepts the
+packed layout: flat per-token tensors plus ``cu_seqlens`` (int64 [B+1]).
+"""
+from typing import Optional
+
+import torch
+import torch.nn as nn
+
+from .. import _lib
+from .._lib import call, ptr, require_gpu, stream_of
+from .utils import _Aggregate, _cu_arg, _f32, _rows_of, _workspace, masked_mean  # noqa: F401
+
+
+def aggregate_loss(
+    loss: torch.Tensor,
+    loss_mask: torch.Tensor,
+    token_level_loss: bool = True,
+    dp_size: int = 1,
+    batch_num_tokens: Optional[float] = None,
+    global_batch_size: Optional[float] = None,
+    cu_seqlens: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """token_level_loss=True: sum(loss*mask) / (sum(mask) or batch_num_tokens) [* dp_size when
+    the global count is given]; False: mean over non-empty rows of sum(loss*mask)/(count+1e-8),
+    or that sum / global_batch_size * dp_size (openrlhf/models/loss.py:11-39)."""
+    if token_level_loss:
+        return _Aggregate.apply(loss, loss_mask, _lib.AGG_TOKEN_MEAN, dp_size, batch_num_tokens, cu_seqlens)
+    return _Aggregate.apply(loss, loss_mask, _lib.AGG_SEQ_MEAN, dp_size, global_batch_size, cu_seqlens)
+
+
+class SFTLoss(nn.Module):
+    """-log-prob aggregated over the loss mask (openrlhf/models/loss.py:87-113)."""
+
+    def __init__(self, token_level_loss: bool = True):
+        super().__init__()
+        self.token_level_loss = token_level_loss
+
+    def forward(self, per_token_logps, loss_mask, dp_size=1, batch_num_tokens=None, global_batch_size=None):
+        return aggregate_loss(
+            -per_token_logps, loss_mask, token_level_loss=self.token_level_loss, dp_size=dp_size,
+            batch_num_tokens=batch_num_tokens, global_batch_size=global_batch_size,
+        )
+
+
+_IS_CODES = {"tis": _lib.IS_TIS, "icepop": _lib.IS_ICEPOP, "seq-mask-tis": _lib.IS_SEQ_MASK_TIS}
+
+
+class _PolicyLossFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, log_probs, old_log_probs, advantages, action_mask, rollout_log_probs, cfg, dp_size,
+                norm_value, cu_seqlens):
+        dev = require_gpu(log_probs, old_log_probs, advantages, action_mask, rollout_log_probs)
+        lp, old, adv = _f32(log_probs), _f32(old_log_probs.detach()), _f32(advantages.detach())
+        if old.shape != lp.shape or adv.shape != lp.shape:
+            old, adv = old.expand_as(lp).contiguous(), adv.expand_as(lp).contiguous()
+        rollout = None if rollout_log_probs is None else _f32(rollout_log_probs.detach())
+        n_rows, n_cols = _rows_of(lp, cu_seqlens)
+        if action_mask is not None and action_mask.shape != lp.shape:
+            action_mask = action_mask.expand_as(lp)
+        mkeep, mptr, mcode = _lib.mask_arg(action_mask)
+        cu = _cu_arg(cu_seqlens, dev)
+        keep = []
+        params = _lib.PolicyParams()
+        params.clip_eps_low, params.clip_eps_high = cfg["clip_eps_low"], cfg["clip_eps_high"]
+        params.dual_clip = cfg["dual_clip"] if cfg["dual_clip"] is not None else 0.0
+        params.policy_type = cfg["policy_type"]
+        params.is_correction = cfg["is_correction"]
+        params.is_low, params.is_high = cfg["is_low"], cfg["is_high"]
+        params.token_level = 1 if cfg["token_level"] else 0
+        params.norm = _lib.make_norm(dp_size, norm_value, keep)
+        ws = _workspace(n_rows, n_cols, dev)
+        out4 = torch.empty(4, dtype=torch.float32, device=dev)
+        row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
+        row_aux = torch.empty(max(n_rows, 1) * 2, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            call("orlhf_policy_loss_fwd", ptr(lp), ptr(old), ptr(adv), mptr, mcode, ptr(rollout), n_rows, n_cols,
+                 ptr(cu), params, ptr(ws), ptr(out4), ptr(row_coef), ptr(row_aux), stream_of(dev))
+        ctx.params, ctx.keep, ctx.dims, ctx.mcode = params, keep, (n_rows, n_cols), mcode
+        ctx.lp_shape, ctx.lp_dtype = log_probs.shape, log_probs.dtype
+        ctx.save_for_backward(lp, old, adv, mkeep, rollout, cu, row_coef, row_aux)
+        loss, clip_ratio, ppo_kl, vllm_kl = out4[0], out4[1], out4[2], out4[3]
+        ctx.mark_non_differentiable(clip_ratio, ppo_kl, vllm_kl)
+        return loss, clip_ratio, ppo_kl, vllm_kl
+
+    @staticmethod
+    def backward(ctx, g_loss, _g1, _g2, _g3):
+        lp, old, adv, mkeep, rollout, cu, row_coef, row_aux = ctx.saved_tensors
+        dev = lp.device
+        n_rows, n_cols = ctx.dims
+        g = _f32(g_loss).reshape(-1)
+        g_lp = torch.empty(lp.shape, dtype=torch.float32, device=dev)
+        ws = _workspace(n_rows, n_cols, dev) if ctx.params.policy_type == _lib.POLICY_GSPO else None
+        with torch.cuda.device(dev):
+            call("orlhf_policy_loss_bwd", ptr(g), ptr(lp), ptr(old), ptr(adv), ptr(mkeep), ctx.mcode, ptr(rollout),
+                 n_rows, n_cols, ptr(cu), ctx.params, ptr(row_coef), ptr(row_aux), ptr(ws), ptr(g_lp),
+                 stream_of(dev))
+        return g_lp.view(ctx.lp_shape).to(ctx.lp_dtype), None, None, None, None, None, None, None, None
+
+
+class PolicyLoss(nn.Module):
+    """PPO / GSPO policy loss (openrlhf/models/loss.py:116-230): low/high ratio clip, optional
+    dual clip, optional TIS / ICEPOP / seq-mask-TIS importance correction against the rollout
+    engine's log-probs, token- or sequence-level aggregation. forward returns
+    (loss, clip_ratio, ppo_kl, vllm_kl-or-None)."""
+
+    def __init__(
+        self,
+        clip_eps_low: float = 0.2,
+        clip_eps_high: float = 0.2,
+        dual_clip: float = None,
+        token_level_loss: bool = True,
+        policy_loss_type: str = "ppo",
+        enable_vllm_is_correction: bool = False,
+        vllm_is_truncated_threshold: list = None,
+        vllm_is_correction_type: str = "tis",
+    ) -> None:
+        super().__init__()
+        self.clip_eps_low = clip_eps_low
+        self.clip_eps_high = clip_eps_high
+        self.token_level_loss = token_level_loss
+        self.dual_clip = dual_clip
+        self.policy_loss_type = policy_loss_type
+        self.enable_vllm_is_correction = enable_vllm_is_correction
+        self.vllm_is_truncated_threshold = vllm_is_truncated_threshold
+        self.vllm_is_correction_type = vllm_is_correction_type
+
+        if policy_loss_type == "gspo":  # GSPO is defined on per-sequence means
+            self.token_level_loss = False
+        if dual_clip is not None:
+            assert dual_clip > 1.0, f"dual_clip must be > 1.0, got {dual_clip}"
+        if self.vllm_is_correction_type not in _IS_CODES:
+            raise ValueError(
+                f"Invalid vllm_is_correction_type: {self.vllm_is_correction_type}, must be one of tis/icepop/seq-mask-tis"
+            )
+
+    def forward(
+        self,
+        log_probs: torch.Tensor,
+        old_log_probs: torch.Tensor,
+        advantages: torch.Tensor,
+        action_mask: Optional[torch.Tensor] = None,
+        rollout_log_probs: Optional[torch.Tensor] = None,
+        dp_size: int = 1,
+        batch_num_tokens: Optional[float] = None,
+        global_batch_size: Optional[float] = None,
+        cu_seqlens: Optional[torch.Tensor] = None,
+    ):
+        if self.policy_loss_type == "ppo":
+            policy_type = _lib.POLICY_PPO
+        elif self.policy_loss_type == "gspo":
+            policy_type = _lib.POLICY_GSPO
+        else:
+            raise ValueError(f"Invalid policy loss type: {self.policy_loss_type}")
+        use_is = bool(self.enable_vllm_is_correction)
+        if use_is and rollout_log_probs is None:
+            raise ValueError("enable_vllm_is_correction needs rollout_log_probs")
+        lo, hi = (self.vllm_is_truncated_threshold if use_is and policy_type == _lib.POLICY_PPO else (0.0, 0.0))
+        cfg = dict(
+            clip_eps_low=float(self.clip_eps_low),
+            clip_eps_high=float(self.clip_eps_high),
+            dual_clip=None if self.dual_clip is None else float(self.dual_clip),
+            policy_type=policy_type,
+            is_correction=_IS_CODES[self.vllm_is_correction_type] if use_is else _lib.IS_NONE,
+            is_low=float(lo),
+            is_high=float(hi),
+            token_level=bool(self.token_level_loss),
+        )
+        norm_value = batch_num_tokens if (self.token_level_loss and policy_type == _lib.POLICY_PPO) else global_batch_size
+        loss, clip_ratio, ppo_kl, vllm_kl = _PolicyLossFn.apply(
+            log_probs, old_log_probs, advantages, action_mask, rollout_log_probs if use_is else None, cfg,
+            dp_size, norm_value, cu_seqlens,
+        )
+        if not (use_is and policy_type == _lib.POLICY_PPO):
+            vllm_kl = None
+        return loss, clip_ratio, ppo_kl, vllm_kl
+
+
+class _ValueLossFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, values, old_values, returns, action_mask, clip_eps, token_level, dp_size, norm_value,
+                cu_seqlens):
+        dev = require_gpu(values, old_values, returns, action_mask)
+        v, ret = _f32(values), _f32(returns.detach())
+        old = None if old_values is None else _f32(old_values.detach())
+        n_rows, n_cols = _rows_of(v, cu_seqlens)
+        if action_mask is not None and action_mask.shape != v.shape:
+            action_mask = action_mask.expand_as(v)
+        mkeep, mptr, mcode = _lib.mask_arg(action_mask)
+        cu = _cu_arg(cu_seqlens, dev)
+        keep = []
+        norm = _lib.make_norm(dp_size, norm_value, keep)
+        ws = _workspace(n_rows, n_cols, dev)
+        out = torch.empty(1, dtype=torch.float32, device=dev)
+        row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
+        has_clip = clip_eps is not None
+        with torch.cuda.device(dev):
+            call("orlhf_value_loss_fwd", ptr(v), ptr(old), ptr(ret), mptr, mcode, n_rows, n_cols, ptr(cu),
+                 1 if has_clip else 0, float(clip_eps) if has_clip else 0.0, 1 if token_level else 0, norm,
+                 ptr(ws), ptr(out), ptr(row_coef), stream_of(dev))
+        ctx.clip, ctx.dims, ctx.mcode = (has_clip, float(clip_eps) if has_clip else 0.0), (n_rows, n_cols), mcode
+        ctx.v_shape, ctx.v_dtype = values.shape, values.dtype
+        ctx.save_for_backward(v, old, ret, mkeep, cu, row_coef)
+        return out.view(())
+
+    @staticmethod
+    def backward(ctx, g_out):
+        v, old, ret, mkeep, cu, row_coef = ctx.saved_tensors
+        dev = v.device
+        n_rows, n_cols = ctx.dims
+        g = _f32(g_out).reshape(-1)
+        g_v = torch.empty(v.shape, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            call("orlhf_value_loss_bwd", ptr(g), ptr(v), ptr(old), ptr(ret), ptr(mkeep), ctx.mcode, n_rows, n_cols,
+                 ptr(cu), 1 if ctx.clip[0] else 0, ctx.clip[1], ptr(row_coef), ptr(g_v), stream_of(dev))
+        return g_v.view(ctx.v_shape).to(ctx.v_dtype), None, None, None, None, None, None, None, None
+
+
+class ValueLoss(nn.Module):
+    """Clipped value loss (openrlhf/models/loss.py:233-269): 0.5 * aggregate(max((clip(v) - R)^2,
+    (v - R)^2)); no clip_eps gives 0.5 * aggregate((v - R)^2)."""
+
+    def __init__(self, clip_eps: float = None, token_level_loss: bool = True) -> None:
+        super().__init__()
+        self.clip_eps = clip_eps
+        self.token_level_loss = token_level_loss
+
+    def forward(
+        self,
+        values: torch.Tensor,
+        old_values: torch.Tensor,
+        returns: torch.Tensor,
+        action_mask: Optional[torch.Tensor] = None,
+        dp_size: int = 1,
+        batch_num_tokens: Optional[float] = None,
+        global_batch_size: Optional[float] = None,
+        cu_seqlens: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        norm_value = batch_num_tokens if self.token_level_loss else global_batch_size
+        return _ValueLossFn.apply(
+            values, old_values if self.clip_eps is not None else None, returns, action_mask, self.clip_eps,
+            self.token_level_loss, dp_size, norm_value, cu_seqlens,
+        )

@@ -1,0 +1,308 @@
+"""Token-level numerics with the call signatures of ``openrlhf.models.utils``.
+
+Mirrors (paths relative to the OpenRLHF tree):
+  compute_approx_kl        openrlhf/models/utils.py:64-95
+  compute_reward           openrlhf/models/utils.py:98-126
+  log_probs_from_logits    openrlhf/models/utils.py:139-163
+  masked_mean              openrlhf/models/utils.py:166-169
+  compute_entropy          openrlhf/models/utils.py:182-186
+plus ``logprobs_and_entropy_from_logits``, the one-pass form of what Actor.forward does with
+two calls (openrlhf/models/actor.py:269-285).
+
+Every function launches hand-written HIP kernels through the C ABI; tensors must be on the GPU.
+
+Deliberate differences from the reference, all on the value-preserving side:
+  * bf16 / fp16 logits are accumulated in fp32 and the result is returned in fp32 (the reference
+    computes and returns the input dtype for those);
+  * ``log_probs_from_logits`` does not divide the caller's logits in place when
+    ``temperature != 1``; the division is folded into the loads;
+  * ``compute_reward`` takes tensors only (the reference's list-of-tensors form of ``kl`` is not
+    used by any caller).
+"""
+from typing import Optional, Tuple, Union
+
+import torch
+
+from .. import _lib
+from .._lib import call, ptr, require_gpu, stream_of
+
+_KL_CODES = {"k1": _lib.KL_K1, "k2": _lib.KL_K2, "k3": _lib.KL_K3}
+
+
+# ------------------------------------------------------------------ vocabulary rows
+def _as_rows(logits: torch.Tensor):
+    """[..., V] -> (2-D tensor sharing storage when the layout allows, row stride in elements)."""
+    vocab = logits.shape[-1]
+    if logits.is_contiguous():
+        return logits.view(-1, vocab), vocab
+    if logits.dim() == 2 and logits.stride(1) == 1 and logits.stride(0) >= vocab:
+        return logits, logits.stride(0)
+    return logits.contiguous().view(-1, vocab), vocab
+
+
+class _LogprobEntropy(torch.autograd.Function):
+    """logits -> (log-prob of label, entropy), one vocabulary pass forward, one backward."""
+
+    @staticmethod
+    def forward(ctx, logits, labels, temperature, want_logprob, want_entropy, inplace_backward):
+        dev = require_gpu(logits, labels if want_logprob else None)
+        code = _lib.dtype_code(logits)
+        batch_shape = logits.shape[:-1]
+        rows, row_stride = _as_rows(logits)
+        n_rows, vocab = rows.shape
+        if want_logprob:
+            if labels.shape != batch_shape:
+                raise ValueError(f"labels shape {tuple(labels.shape)} != logits batch shape {tuple(batch_shape)}")
+            lab = labels.reshape(-1)
+            if lab.dtype != torch.int64:
+                lab = lab.long()
+            lab = lab.contiguous()
+        else:
+            lab = None
+        needs_grad = ctx.needs_input_grad[0]
+        opts = dict(device=dev, dtype=torch.float32)
+        logprob = torch.empty(n_rows, **opts) if want_logprob else None
+        entropy = torch.empty(n_rows, **opts) if want_entropy else None
+        stats = torch.empty(n_rows, 4, **opts) if needs_grad else None
+        with torch.cuda.device(dev):
+            call(
+                "orlhf_logprob_entropy_fwd", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
+                float(temperature), ptr(logprob), ptr(entropy), ptr(stats), 0, stream_of(dev),
+            )
+        ctx.temperature = float(temperature)
+        ctx.inplace = bool(inplace_backward)
+        ctx.row_stride = row_stride
+        ctx.shares_storage = rows.data_ptr() == logits.data_ptr() and (
+            logits.is_contiguous() or rows is logits
+        )
+        ctx.logits_shape = logits.shape
+        ctx.set_materialize_grads(False)
+        if needs_grad:
+            ctx.save_for_backward(rows, lab, stats)
+        out_lp = logprob.view(batch_shape) if want_logprob else None
+        out_ent = entropy.view(batch_shape) if want_entropy else None
+        return out_lp, out_ent
+
+    @staticmethod
+    def backward(ctx, g_logprob, g_entropy):
+        rows, lab, stats = ctx.saved_tensors
+        if g_logprob is None and g_entropy is None:
+            return None, None, None, None, None, None
+        dev = rows.device
+        n_rows, vocab = rows.shape
+        code = _lib.dtype_code(rows)
+        glp = None if g_logprob is None else g_logprob.reshape(-1).to(torch.float32).contiguous()
+        gent = None if g_entropy is None else g_entropy.reshape(-1).to(torch.float32).contiguous()
+        if ctx.inplace and ctx.shares_storage:
+            grad_rows, grad_stride = rows, ctx.row_stride
+        else:
+            grad_rows = torch.empty((n_rows, vocab), device=dev, dtype=rows.dtype)
+            grad_stride = vocab
+        with torch.cuda.device(dev):
+            call(
+                "orlhf_logprob_entropy_bwd", ptr(rows), ptr(grad_rows), code, n_rows, vocab,
+                ctx.row_stride, grad_stride, ptr(lab), ctx.temperature, ptr(glp), ptr(gent),
+                ptr(stats), stream_of(dev),
+            )
+        if grad_rows is rows:
+            # the logits storage now holds the gradient: bump the shared version counter (an
+            # in-place op on an empty view costs no launch) so that any later use of the saved
+            # logits by autograd raises instead of reading gradients as logits
+            rows.view(-1)[:0].zero_() if rows.is_contiguous() else rows[:0].zero_()
+        grad = grad_rows if grad_rows.shape == ctx.logits_shape else grad_rows.view(ctx.logits_shape)
+        return grad, None, None, None, None, None
+
+
+def logprobs_and_entropy_from_logits(
+    logits: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float = 1.0,
+    inplace_backward: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """(log_probs_from_logits(logits, labels, temperature), compute_entropy(logits)) from one
+    pass over the logits: the log-prob uses logits / temperature, the entropy the unscaled
+    logits, the order Actor.forward applies them in (openrlhf/models/actor.py:269-285).
+
+    ``inplace_backward=True`` writes d(loss)/d(logits) over the logits storage in backward
+    instead of allocating a second [N, V] tensor; the logits are unusable afterwards.
+    """
+    return _LogprobEntropy.apply(logits, labels, temperature, True, True, inplace_backward)
+
+
+def log_probs_from_logits(
+    logits: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0, inplace_backward: bool = False
+) -> torch.Tensor:
+    """log_softmax(logits / temperature) gathered at ``labels``
+    (openrlhf/models/utils.py:139-163), fp32 result."""
+    return _LogprobEntropy.apply(logits, labels, temperature, True, False, inplace_backward)[0]
+
+
+def compute_entropy(logits: torch.Tensor, inplace_backward: bool = False) -> torch.Tensor:
+    """logsumexp(x) - sum(softmax(x) * x) over the last dim (openrlhf/models/utils.py:182-186),
+    fp32 result."""
+    return _LogprobEntropy.apply(logits, None, 1.0, False, True, inplace_backward)[1]
+
+
+# ------------------------------------------------------------------ per-token helpers
+def _f32(t: torch.Tensor) -> torch.Tensor:
+    """Per-token tensors are consumed as contiguous fp32 (the callers' tensors already are)."""
+    if t.dtype != torch.float32:
+        t = t.float()
+    return t.contiguous()
+
+
+def _rows_of(t: torch.Tensor, cu_seqlens: Optional[torch.Tensor]):
+    """(n_rows, n_cols) of a padded [..., A] tensor, or of a packed flat tensor + cu_seqlens."""
+    if cu_seqlens is not None:
+        n_rows = cu_seqlens.numel() - 1
+        return n_rows, max(int(t.numel()), 1)
+    if t.dim() == 0:
+        return 1, 1
+    n_cols = t.shape[-1]
+    return (t.numel() // n_cols if n_cols > 0 else 0), n_cols
+
+
+def _cu_arg(cu_seqlens, dev):
+    if cu_seqlens is None:
+        return None
+    cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
+    return cu
+
+
+def _workspace(n_rows, n_cols, dev):
+    nbytes = _lib.load().orlhf_token_workspace_bytes(n_rows, n_cols)
+    return torch.empty(nbytes, dtype=torch.uint8, device=dev)
+
+
+class _ApproxKL(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, log_probs, log_probs_base, estimator):
+        dev = require_gpu(log_probs, log_probs_base)
+        if log_probs.dtype == log_probs_base.dtype and log_probs.dtype in _lib._DTYPES:
+            lp, base = log_probs.contiguous(), log_probs_base.contiguous()
+        else:
+            lp, base = _f32(log_probs), _f32(log_probs_base)
+        lp, base = torch.broadcast_tensors(lp, base)
+        lp, base = lp.contiguous(), base.contiguous()
+        out = torch.empty(lp.shape, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            call("orlhf_approx_kl_fwd", ptr(lp), ptr(base), _lib.dtype_code(lp), lp.numel(), estimator,
+                 ptr(out), stream_of(dev))
+        ctx.estimator = estimator
+        ctx.in_shapes = (log_probs.shape, log_probs_base.shape)
+        ctx.in_dtypes = (log_probs.dtype, log_probs_base.dtype)
+        ctx.save_for_backward(lp, base)
+        return out
+
+    @staticmethod
+    def backward(ctx, g_out):
+        lp, base = ctx.saved_tensors
+        dev = lp.device
+        g_out = _f32(g_out)
+        need_lp, need_base = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        g_lp = torch.empty(lp.shape, dtype=torch.float32, device=dev) if need_lp else None
+        g_base = torch.empty(lp.shape, dtype=torch.float32, device=dev) if need_base else None
+        if need_lp or need_base:
+            with torch.cuda.device(dev):
+                call("orlhf_approx_kl_bwd", ptr(lp), ptr(base), _lib.dtype_code(lp), lp.numel(),
+                     ctx.estimator, ptr(g_out), ptr(g_lp), ptr(g_base), stream_of(dev))
+
+        def fit(g, shape, dtype):
+            if g is None:
+                return None
+            if g.shape != shape:
+                g = g.sum_to_size(shape)
+            return g.to(dtype)
+
+        return fit(g_lp, ctx.in_shapes[0], ctx.in_dtypes[0]), fit(g_base, ctx.in_shapes[1], ctx.in_dtypes[1]), None
+
+
+def compute_approx_kl(
+    log_probs: torch.Tensor,
+    log_probs_base: torch.Tensor,
+    kl_estimator: str = "k1",
+) -> torch.Tensor:
+    """k1: d, k2: d^2/2, k3: exp(-d) - 1 + d with d = log_probs - log_probs_base, clamped to
+    [-10, 10], fp32 (openrlhf/models/utils.py:64-95). Differentiable."""
+    if kl_estimator not in _KL_CODES:
+        raise ValueError(f"Unknown kl_estimator: {kl_estimator}")
+    return _ApproxKL.apply(log_probs, log_probs_base, _KL_CODES[kl_estimator])
+
+
+class _Aggregate(torch.autograd.Function):
+    """Masked token-mean / sequence-mean / per-row mean of a per-token tensor."""
+
+    @staticmethod
+    def forward(ctx, x, mask, mode, dp_size, norm_value, cu_seqlens):
+        dev = require_gpu(x, mask)
+        xf = _f32(x)
+        n_rows, n_cols = _rows_of(xf, cu_seqlens)
+        if mask is not None and mask.shape != x.shape:
+            mask = mask.expand_as(x)
+        mkeep, mptr, mcode = _lib.mask_arg(mask)
+        cu = _cu_arg(cu_seqlens, dev)
+        keep = []
+        norm = _lib.make_norm(dp_size, norm_value, keep)
+        ws = _workspace(n_rows, n_cols, dev)
+        out = torch.empty(n_rows if mode == _lib.AGG_ROW_MEAN else 1, dtype=torch.float32, device=dev)
+        row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            call("orlhf_masked_aggregate_fwd", ptr(xf), mptr, mcode, n_rows, n_cols, ptr(cu), mode, norm,
+                 ptr(ws), ptr(out), ptr(row_coef), stream_of(dev))
+        ctx.mode, ctx.dims, ctx.mcode = mode, (n_rows, n_cols), mcode
+        ctx.x_shape, ctx.x_dtype = x.shape, x.dtype
+        ctx.save_for_backward(mkeep, cu, row_coef)
+        if mode == _lib.AGG_ROW_MEAN:
+            return out.view(x.shape[:-1]) if cu_seqlens is None else out
+        return out.view(())
+
+    @staticmethod
+    def backward(ctx, g_out):
+        mkeep, cu, row_coef = ctx.saved_tensors
+        dev = row_coef.device
+        n_rows, n_cols = ctx.dims
+        g = _f32(g_out).reshape(-1)
+        g_x = torch.empty(ctx.x_shape, dtype=torch.float32, device=dev)
+        with torch.cuda.device(dev):
+            call("orlhf_masked_aggregate_bwd", ptr(g), ptr(mkeep), ctx.mcode, n_rows, n_cols, ptr(cu), ctx.mode,
+                 ptr(row_coef), ptr(g_x), stream_of(dev))
+        return g_x.to(ctx.x_dtype), None, None, None, None, None
+
+
+def masked_mean(tensor: torch.Tensor, mask: Optional[torch.Tensor], dim: int = None) -> torch.Tensor:
+    """sum(tensor * mask) / sum(mask) over everything (dim=None) or over `dim`; no epsilon, so
+    an all-zero mask gives NaN (openrlhf/models/utils.py:166-169). mask=None is a plain mean."""
+    if dim is None:
+        return _Aggregate.apply(tensor, mask, _lib.AGG_TOKEN_MEAN, 1, None, None)
+    nd = tensor.dim()
+    d = dim if dim >= 0 else dim + nd
+    if d != nd - 1:
+        tensor = tensor.movedim(d, -1)
+        if mask is not None:
+            mask = mask.expand(torch.broadcast_shapes(mask.shape, tensor.movedim(-1, d).shape)).movedim(d, -1)
+    return _Aggregate.apply(tensor, mask, _lib.AGG_ROW_MEAN, 1, None, None)
+
+
+def compute_reward(
+    r: torch.Tensor,
+    kl_coef: float,
+    kl: torch.Tensor,
+    action_mask: Optional[torch.Tensor] = None,
+    reward_clip_range: Tuple[float, float] = None,
+    cu_seqlens: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Per-token reward: -max(kl_coef, 0) * kl everywhere plus the (clipped) scalar reward r[b]
+    at row b's last unmasked column (openrlhf/models/utils.py:98-126). Forward only."""
+    dev = require_gpu(r, kl, action_mask)
+    klf, rf = _f32(kl.detach()), _f32(r.detach()).reshape(-1)
+    n_rows, n_cols = _rows_of(klf, cu_seqlens)
+    if rf.numel() != n_rows:
+        raise ValueError(f"r has {rf.numel()} entries for {n_rows} rows")
+    mkeep, mptr, mcode = _lib.mask_arg(action_mask)
+    cu = _cu_arg(cu_seqlens, dev)
+    out = torch.empty_like(klf)
+    lo, hi = (reward_clip_range[0], reward_clip_range[1]) if reward_clip_range else (0.0, 0.0)
+    with torch.cuda.device(dev):
+        call("orlhf_compute_reward", ptr(rf), float(kl_coef), ptr(klf), mptr, mcode, n_rows, n_cols, ptr(cu),
+             1 if reward_clip_range else 0, float(lo), float(hi), ptr(out), None, stream_of(dev))
+    return out

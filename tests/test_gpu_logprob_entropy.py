@@ -1,0 +1,230 @@
+"""Parity of the fused log-prob + entropy kernels (forward and backward) with the CPU oracle.
+
+Tolerances (from the task statement): 1e-5 abs for fp32 logits; 2e-3 abs against the fp32
+up-cast oracle for bf16 logits. Gradients in the logits dtype are compared to the fp64 analytic
+gradient within the rounding of that dtype.
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import token_numerics as otn
+
+pytestmark = pytest.mark.gpu
+
+FP32_ATOL = 1e-5
+BF16_ATOL = 2e-3
+
+
+def _logits(rows, vocab, dtype, std, seed, spike_frac=0.0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(rows, vocab, generator=g) * std
+    if spike_frac > 0:
+        n_spike = max(1, int(rows * spike_frac))
+        r = torch.randperm(rows, generator=g)[:n_spike]
+        c = torch.randint(0, vocab, (n_spike,), generator=g)
+        x[r, c] += 15.0
+    labels = torch.randint(0, vocab, (rows,), generator=g)
+    return x.to(dtype), labels
+
+
+def _oracle64(x, labels, temperature):
+    x64 = x.double()
+    return otn.log_probs_from_logits(x64, labels, temperature), otn.compute_entropy(x64)
+
+
+def _analytic_grad64(x, labels, temperature, g_lp, g_ent):
+    x64 = x.double()
+    p_t = torch.softmax(x64 / temperature, -1)
+    p = torch.softmax(x64, -1)
+    onehot = torch.zeros_like(x64).scatter_(1, labels.unsqueeze(1), 1.0)
+    ex = (p * x64).sum(-1, keepdim=True)
+    return g_lp.double().unsqueeze(1) * (onehot - p_t) / temperature + g_ent.double().unsqueeze(1) * p * (ex - x64)
+
+
+@pytest.mark.parametrize(
+    "rows,vocab,dtype,std,temperature",
+    [
+        (64, 32000, torch.float32, 2.0, 1.0),      # config-1 vocabulary
+        (48, 151936, torch.bfloat16, 3.0, 1.0),    # config-2 vocabulary (headline)
+        (16, 262144, torch.bfloat16, 4.0, 0.6),    # config-5 vocabulary and temperature
+        (33, 50257, torch.float32, 2.0, 0.7),      # odd vocabulary, fp32, T != 1
+        (33, 50257, torch.bfloat16, 3.0, 1.0),     # odd vocabulary: scalar tail
+        (9, 1000, torch.float16, 2.0, 1.3),
+        (300, 7, torch.float32, 1.0, 1.0),         # rows shorter than one vector
+        (5, 129, torch.bfloat16, 1.0, 2.0),
+    ],
+)
+def test_forward_matches_oracle(cuda, rows, vocab, dtype, std, temperature):
+    from openrlhf_amd.models.utils import compute_entropy, log_probs_from_logits, logprobs_and_entropy_from_logits
+
+    x, labels = _logits(rows, vocab, dtype, std, seed=rows * 7919 + vocab, spike_frac=0.05)
+    ref_lp, ref_ent = _oracle64(x, labels, temperature)
+    xd, ld = x.to(cuda), labels.to(cuda)
+    lp, ent = logprobs_and_entropy_from_logits(xd, ld, temperature)
+    assert lp.dtype == torch.float32 and ent.dtype == torch.float32
+    atol = FP32_ATOL if dtype == torch.float32 else BF16_ATOL
+    assert (lp.cpu().double() - ref_lp).abs().max().item() <= atol
+    assert (ent.cpu().double() - ref_ent).abs().max().item() <= atol
+    # the two single-output entry points give the same bits as the fused one
+    assert torch.equal(log_probs_from_logits(xd, ld, temperature), lp)
+    assert torch.equal(compute_entropy(xd), ent) or (compute_entropy(xd) - ent).abs().max().item() <= 2e-6
+    # the input is not modified (no in-place temperature division)
+    assert torch.equal(xd.cpu(), x)
+
+
+def test_forward_3d_shape_and_fp32_reference_op_sequence(cuda):
+    """[B, T, V] input as Actor.forward passes it; compared with the fp32 oracle that follows the
+    reference's own op sequence (gather - chunked logsumexp)."""
+    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(4, 64, 32000, generator=g) * 2.0
+    labels = torch.randint(0, 32000, (4, 64), generator=g)
+    lp, ent = logprobs_and_entropy_from_logits(x.to(cuda), labels.to(cuda), 1.0)
+    assert lp.shape == (4, 64) and ent.shape == (4, 64)
+    assert (lp.cpu() - otn.log_probs_from_logits(x, labels)).abs().max().item() <= FP32_ATOL
+    assert (ent.cpu() - otn.compute_entropy(x)).abs().max().item() <= FP32_ATOL
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_unaligned_and_strided_rows(cuda, dtype):
+    """Row starts off the 16-byte grid (element offset 1..3, odd row stride)."""
+    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+
+    rows, vocab, stride = 12, 4099, 4099 + 5
+    g = torch.Generator().manual_seed(11)
+    base = (torch.randn(rows * stride + 3, generator=g) * 2).to(dtype)
+    labels = torch.randint(0, vocab, (rows,), generator=g)
+    for off in (0, 1, 3):
+        x = base[off : off + rows * stride].view(rows, stride)[:, :vocab]
+        ref_lp, ref_ent = _oracle64(x.contiguous(), labels, 1.0)
+        xd = base.to(cuda)[off : off + rows * stride].view(rows, stride)[:, :vocab]
+        assert not xd.is_contiguous()
+        lp, ent = logprobs_and_entropy_from_logits(xd, labels.to(cuda), 1.0)
+        atol = FP32_ATOL if dtype == torch.float32 else BF16_ATOL
+        assert (lp.cpu().double() - ref_lp).abs().max().item() <= atol
+        assert (ent.cpu().double() - ref_ent).abs().max().item() <= atol
+
+
+def test_closed_forms(cuda):
+    """Constant rows: entropy = ln V and logprob = -ln V; shift invariance; one dominant logit."""
+    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+
+    vocab = 151936
+    x = torch.full((3, vocab), 1.25, dtype=torch.bfloat16)
+    labels = torch.tensor([0, 77, vocab - 1])
+    lp, ent = logprobs_and_entropy_from_logits(x.to(cuda), labels.to(cuda), 1.0)
+    assert (ent.cpu() - math.log(vocab)).abs().max().item() <= 1e-5
+    assert (lp.cpu() + math.log(vocab)).abs().max().item() <= 1e-5
+    # shift invariance (exact in bf16 for these values)
+    g = torch.Generator().manual_seed(3)
+    y = (torch.randn(4, 4096, generator=g)).to(torch.bfloat16)
+    lab = torch.randint(0, 4096, (4,), generator=g)
+    a = logprobs_and_entropy_from_logits(y.float().to(cuda), lab.to(cuda))
+    b = logprobs_and_entropy_from_logits((y.float() + 8.0).to(cuda), lab.to(cuda))
+    assert (a[0] - b[0]).abs().max().item() <= 1e-5 and (a[1] - b[1]).abs().max().item() <= 1e-5
+    # one logit far above the rest: logprob -> 0, entropy -> 0
+    z = torch.zeros(2, 5000)
+    z[:, 123] = 60.0
+    lp, ent = logprobs_and_entropy_from_logits(z.to(cuda), torch.tensor([123, 123]).to(cuda))
+    assert lp.abs().max().item() <= 1e-6 and ent.abs().max().item() <= 1e-6
+
+
+def test_extreme_rows_take_the_safe_pass(cuda):
+    """Rows the reference-maximum shortcut cannot handle: a huge late spike, -inf (masked
+    vocabulary), +inf and NaN logits. Values follow torch's own logsumexp / softmax semantics."""
+    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+
+    vocab = 20000
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(6, vocab, generator=g)
+    x[0, vocab - 5] = 500.0                 # > 88 nats above anything seen early in the row
+    x[1, :1000] = -1.0e4                    # very low start: reference max far below the rest
+    x[2, ::3] = float("-inf")               # masked vocabulary entries
+    x[3, 17] = float("inf")
+    x[4, 9] = float("nan")
+    x[5] = x[5] * 30.0                      # wide dynamic range
+    labels = torch.tensor([vocab - 5, 5000, 1, 3, 4, 7])
+    ref_lp = otn.log_probs_from_logits(x.double(), labels)
+    ref_ent = otn.compute_entropy(x.double())
+    lp, ent = logprobs_and_entropy_from_logits(x.to(cuda), labels.to(cuda))
+    lp, ent = lp.cpu().double(), ent.cpu().double()
+    for i in (0, 1, 5):
+        assert abs(lp[i] - ref_lp[i]) <= FP32_ATOL * max(1.0, abs(ref_lp[i].item()) * 1e-1), (i, lp[i], ref_lp[i])
+        assert abs(ent[i] - ref_ent[i]) <= 1e-4, (i, ent[i], ref_ent[i])
+    # -inf entries: finite log-prob, NaN entropy (0 * -inf), like the reference
+    assert abs(lp[2] - ref_lp[2]) <= FP32_ATOL and math.isnan(ent[2]) and math.isnan(ref_ent[2])
+    # +inf entry: logsumexp = +inf
+    assert lp[3] == ref_lp[3] == float("-inf") and math.isnan(ent[3])
+    assert math.isnan(lp[4]) and math.isnan(ent[4])
+    # labels outside the vocabulary never read out of bounds
+    bad = torch.tensor([-100, -1, vocab, 0, 0, 0])
+    lp2, _ = logprobs_and_entropy_from_logits(x.to(cuda), bad.to(cuda))
+    assert lp2[0].item() == 0.0 and math.isnan(lp2[1].item()) and math.isnan(lp2[2].item())
+
+
+@pytest.mark.parametrize(
+    "rows,vocab,dtype,std,temperature,inplace",
+    [
+        (32, 32000, torch.float32, 2.0, 1.0, False),
+        (32, 32000, torch.float32, 2.0, 0.7, True),
+        (24, 151936, torch.bfloat16, 3.0, 1.0, True),
+        (24, 151936, torch.bfloat16, 3.0, 1.0, False),
+        (8, 262144, torch.bfloat16, 4.0, 0.6, True),
+        (17, 50257, torch.bfloat16, 3.0, 1.0, True),
+        (9, 1000, torch.float16, 2.0, 1.3, False),
+        (40, 7, torch.float32, 1.0, 1.0, True),
+    ],
+)
+def test_backward_matches_analytic_gradient(cuda, rows, vocab, dtype, std, temperature, inplace):
+    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+
+    x, labels = _logits(rows, vocab, dtype, std, seed=rows + vocab, spike_frac=0.05)
+    g = torch.Generator().manual_seed(rows)
+    g_lp = torch.randn(rows, generator=g)
+    g_ent = torch.randn(rows, generator=g)
+    g_lp[1] = 0.0
+    g_ent[1] = 0.0  # a fully masked token: its grad row must be exactly zero
+    ref = _analytic_grad64(x, labels, temperature, g_lp, g_ent)
+
+    xd = x.to(cuda).requires_grad_(True)
+    lp, ent = logprobs_and_entropy_from_logits(xd, labels.to(cuda), temperature, inplace_backward=inplace)
+    loss = (lp * g_lp.to(cuda)).sum() + (ent * g_ent.to(cuda)).sum()
+    loss.backward()
+    grad = xd.grad
+    assert grad.dtype == dtype and grad.shape == x.shape
+    if inplace:
+        assert grad.data_ptr() == xd.data_ptr()
+    err = (grad.cpu().double() - ref).abs()
+    if dtype == torch.float32:
+        assert err.max().item() <= 1e-5
+    else:
+        eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        assert (err <= eps * ref.abs() + 1e-6).all(), err.max().item()
+    assert grad[1].abs().max().item() == 0.0
+    # rows of d(logprob)/dx and d(entropy)/dx each sum to zero
+    assert grad.cpu().double().sum(-1).abs().max().item() <= (1e-4 if dtype == torch.float32 else 2e-2)
+
+
+def test_backward_single_outputs_and_reuse_guard(cuda):
+    """Log-prob-only and entropy-only backward; autograd refuses to reuse logits that an
+    in-place backward has overwritten."""
+    from openrlhf_amd.models.utils import compute_entropy, log_probs_from_logits
+
+    x, labels = _logits(10, 4096, torch.float32, 2.0, seed=1)
+    g = torch.randn(10, generator=torch.Generator().manual_seed(2))
+    zero = torch.zeros(10)
+    xd = x.to(cuda).requires_grad_(True)
+    (log_probs_from_logits(xd, labels.to(cuda), 0.8) * g.to(cuda)).sum().backward()
+    assert (xd.grad.cpu().double() - _analytic_grad64(x, labels, 0.8, g, zero)).abs().max().item() <= 1e-5
+    xd.grad = None
+    (compute_entropy(xd) * g.to(cuda)).sum().backward()
+    assert (xd.grad.cpu().double() - _analytic_grad64(x, labels, 1.0, zero, g)).abs().max().item() <= 1e-5
+
+    yd = x.to(cuda).requires_grad_(True)
+    out = log_probs_from_logits(yd, labels.to(cuda), 1.0, inplace_backward=True).sum()
+    out.backward(retain_graph=True)
+    with pytest.raises(RuntimeError):
+        out.backward()
