@@ -1,0 +1,242 @@
+"""Advantage functions of the experience maker on hand-written HIP kernels.
+
+Mirrors (paths relative to the OpenRLHF tree, all in
+openrlhf/trainer/ppo_utils/experience_maker.py):
+  compute_advantages_and_returns   :237-330  (group baseline :246-272, per-experience reward and
+                                              GAE / returns :275-312, global whitening :314-328)
+  get_advantages_and_returns       :332-377  (GAE)
+  get_cumulative_returns           :379-411  (discounted reward-to-go)
+
+The reference runs these on the controller's CPU with Python loops over time. Here every
+function is a GPU kernel launch; tensors that arrive on the CPU (the reference's experiences
+are CPU tensors) are copied to the current GPU, processed there and the results copied back to
+where the inputs lived, so callers see the same devices as before. There is no CPU compute path:
+without a GPU the functions raise.
+
+Only the numerics are mirrored. Length penalties (apply_length_penalties) and the Ray dispatch
+half of RemoteExperienceMaker are outside this package; ``compute_advantages_and_returns`` takes a
+``length_penalty_fn`` hook for the former.
+"""
+import itertools
+from typing import List, Optional, Tuple
+
+import torch
+
+from ... import _lib
+from ..._lib import call, ptr, stream_of
+from ...models.utils import _cu_arg, _f32, _rows_of, compute_reward
+
+_GROUP_CODES = {
+    "gae": _lib.GROUP_IDENTITY,
+    "reinforce": _lib.GROUP_IDENTITY,
+    "rloo": _lib.GROUP_RLOO,
+    "reinforce_baseline": _lib.GROUP_BASELINE,
+    "dr_grpo": _lib.GROUP_BASELINE,
+    "group_norm": _lib.GROUP_NORM,
+}
+_RETURN_ESTIMATORS = ("reinforce", "rloo", "reinforce_baseline", "group_norm", "dr_grpo")
+
+
+def _gpu_device() -> torch.device:
+    if not torch.cuda.is_available():
+        raise RuntimeError("openrlhf_amd needs a GPU: the advantage functions are HIP kernels, there is no CPU path")
+    return torch.device("cuda", torch.cuda.current_device())
+
+
+def _on_gpu(t: Optional[torch.Tensor], dev: torch.device) -> Optional[torch.Tensor]:
+    if t is None or t.is_cuda:
+        return t
+    return t.to(dev)
+
+
+def _device_for(*tensors) -> Tuple[torch.device, torch.device]:
+    """(GPU to compute on, device the results go back to)."""
+    home = next(t.device for t in tensors if t is not None)
+    gpu = next((t.device for t in tensors if t is not None and t.is_cuda), None)
+    return (gpu if gpu is not None else _gpu_device()), home
+
+
+@torch.no_grad()
+def get_advantages_and_returns(
+    values: torch.Tensor,
+    rewards: torch.Tensor,
+    action_mask: Optional[torch.Tensor],
+    gamma: float,
+    lambd: float,
+    cu_seqlens: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """GAE (experience_maker.py:332-377): with v = mask*values, r = mask*rewards,
+    delta_t = r_t + gamma*v_{t+1} - v_t, A_t = delta_t + gamma*lambd*A_{t+1}; returns = A + v.
+    Every column of the [B, A] block takes part and the outputs are not re-masked."""
+    dev, home = _device_for(values, rewards, action_mask)
+    v, r = _f32(_on_gpu(values, dev)), _f32(_on_gpu(rewards, dev))
+    mkeep, mptr, mcode = _lib.mask_arg(_on_gpu(action_mask, dev))
+    n_rows, n_cols = _rows_of(v, cu_seqlens)
+    cu = _cu_arg(cu_seqlens, dev)
+    adv, ret = torch.empty_like(v), torch.empty_like(v)
+    with torch.cuda.device(dev):
+        call("orlhf_gae_scan", ptr(v), ptr(r), mptr, mcode, n_rows, n_cols, ptr(cu), float(gamma), float(lambd),
+             ptr(adv), ptr(ret), stream_of(dev))
+    return adv.to(home), ret.to(home)
+
+
+@torch.no_grad()
+def get_cumulative_returns(
+    rewards: torch.Tensor,
+    action_mask: Optional[torch.Tensor],
+    gamma: float,
+    cu_seqlens: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """Discounted reward-to-go G_t = mask_t*r_t + gamma*G_{t+1} (experience_maker.py:379-411)."""
+    dev, home = _device_for(rewards, action_mask)
+    r = _f32(_on_gpu(rewards, dev))
+    mkeep, mptr, mcode = _lib.mask_arg(_on_gpu(action_mask, dev))
+    n_rows, n_cols = _rows_of(r, cu_seqlens)
+    cu = _cu_arg(cu_seqlens, dev)
+    ret = torch.empty_like(r)
+    with torch.cuda.device(dev):
+        call("orlhf_discounted_returns", ptr(r), mptr, mcode, n_rows, n_cols, ptr(cu), float(gamma), ptr(ret),
+             stream_of(dev))
+    return ret.to(home)
+
+
+@torch.no_grad()
+def group_normalize_rewards(
+    rewards: torch.Tensor,
+    indices: Optional[torch.Tensor],
+    n_samples_per_prompt: int,
+    estimator: str,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Group baseline / normalisation of scalar rewards (experience_maker.py:246-272).
+
+    rewards: [P*n] in experience order; indices[i] = position of sample i in prompt order (None:
+    already in prompt order), so samples whose positions fall in one block of n share a prompt.
+    rloo: r - mean of the other n-1; reinforce_baseline / dr_grpo: r - group mean; group_norm:
+    (r - mean) / (unbiased std + 1e-9); gae / reinforce: unchanged. Returns (shaped rewards in
+    experience order, the unbiased group std per sample or None when n == 1)."""
+    if estimator not in _GROUP_CODES:
+        raise Exception(f"Unkown advantage_estimator {estimator}")
+    dev, home = _device_for(rewards)
+    r = _f32(_on_gpu(rewards, dev)).reshape(-1)
+    n_total = r.numel()
+    n = int(n_samples_per_prompt)
+    if n < 1 or n_total % n != 0:
+        raise ValueError(f"{n_total} rewards do not split into groups of {n}")
+    idx = None if indices is None else _on_gpu(indices, dev).to(torch.int64).contiguous()
+    out = torch.empty_like(r)
+    std = torch.empty_like(r) if n > 1 else None
+    ws = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        call("orlhf_group_normalize", ptr(r), ptr(idx), n_total // n, n, _GROUP_CODES[estimator], ptr(out), ptr(std),
+             ptr(ws), stream_of(dev))
+    return out.to(home), (None if std is None else std.to(home))
+
+
+@torch.no_grad()
+def whiten_advantages(
+    advantages: List[torch.Tensor],
+    action_masks: List[torch.Tensor],
+    no_std_norm: bool = False,
+) -> List[torch.Tensor]:
+    """Global masked whitening over all experiences (experience_maker.py:314-328): mean and
+    biased variance over the unmasked tokens of every block, rstd = rsqrt(max(var, 1e-8)) (1 when
+    no_std_norm); (adv - mean) * rstd is applied to every column, masked or not."""
+    dev, home = _device_for(*advantages)
+    flat = torch.cat([_on_gpu(a, dev).flatten() for a in advantages]).float()
+    mask = torch.cat([_on_gpu(m, dev).flatten() for m in action_masks])
+    mkeep, mptr, mcode = _lib.mask_arg(mask)
+    n = flat.numel()
+    ws = torch.empty(_lib.load().orlhf_whiten_workspace_bytes(n), dtype=torch.uint8, device=dev)
+    out = torch.empty_like(flat)
+    with torch.cuda.device(dev):
+        call("orlhf_masked_whiten", ptr(flat), mptr, mcode, n, 0 if no_std_norm else 1, ptr(ws), ptr(out), None,
+             stream_of(dev))
+    pieces = out.split([a.numel() for a in advantages])
+    return [p.view(a.shape).to(home) for p, a in zip(pieces, advantages)]
+
+
+@torch.no_grad()
+def compute_advantages_and_returns(
+    experiences: list,
+    *,
+    advantage_estimator: str,
+    n_samples_per_prompt: int,
+    kl_coef: float,
+    gamma: float = 1.0,
+    lambd: float = 1.0,
+    reward_clip_range: Optional[Tuple[float, float]] = None,
+    no_std_norm: bool = False,
+    length_penalty_fn=None,
+) -> list:
+    """The numerics of RemoteExperienceMaker.compute_advantages_and_returns
+    (experience_maker.py:237-330) on a list of experience objects with the attributes the
+    reference reads and writes: index, rewards, kl, action_mask, values, info, advantages,
+    returns. Group baseline over prompts, per-token reward (compute_reward), GAE or discounted
+    returns, then global whitening for gae / reinforce / reinforce_baseline."""
+    if length_penalty_fn is not None:
+        length_penalty_fn(experiences)
+    exp_len = [len(e.index) for e in experiences]
+    indices = torch.tensor(list(itertools.chain.from_iterable(e.index for e in experiences)), dtype=torch.int64)
+    raw = torch.cat([e.rewards for e in experiences], dim=0)
+    shaped, group_std = group_normalize_rewards(raw, indices.to(raw.device), n_samples_per_prompt, advantage_estimator)
+    if group_std is not None:
+        for e, s in zip(experiences, group_std.split(exp_len)):
+            e.info["group_reward_std"] = s
+
+    for e, reward in zip(experiences, shaped.split(exp_len)):
+        token_reward = compute_reward(
+            _on_gpu(reward, _gpu_device()), kl_coef, _on_gpu(e.kl, _gpu_device()),
+            action_mask=_on_gpu(e.action_mask, _gpu_device()), reward_clip_range=reward_clip_range,
+        )
+        home = e.kl.device
+        if advantage_estimator == "gae":
+            adv, ret = get_advantages_and_returns(e.values.to(token_reward.device), token_reward,
+                                                  e.action_mask.to(token_reward.device), gamma, lambd)
+            e.advantages, e.returns = adv.to(home), ret.to(home)
+        elif advantage_estimator in _RETURN_ESTIMATORS:
+            g = gamma if advantage_estimator == "reinforce" else 1.0  # the reference forces gamma = 1 here
+            e.returns = get_cumulative_returns(token_reward, e.action_mask.to(token_reward.device), g).to(home)
+            e.advantages = e.returns.clone()
+        else:
+            raise Exception(f"Unkown advantage_estimator {advantage_estimator}")
+        e.info["return"] = token_reward.sum(dim=-1).to(home)
+        e.kl = None
+
+    if advantage_estimator in ("gae", "reinforce", "reinforce_baseline"):
+        whitened = whiten_advantages([e.advantages for e in experiences], [e.action_mask for e in experiences],
+                                     no_std_norm=no_std_norm)
+        for e, a in zip(experiences, whitened):
+            e.advantages = a
+    return experiences
+
+
+class AdvantageFunctions:
+    """The three advantage methods of RemoteExperienceMaker with their reference signatures, for
+    code that calls them as bound methods. ``strategy.args`` and ``kl_ctl`` are read the way the
+    reference reads them (experience_maker.py:240-330)."""
+
+    def __init__(self, strategy=None, kl_ctl=None, length_penalty_fn=None):
+        self.strategy = strategy
+        self.kl_ctl = kl_ctl
+        self.length_penalty_fn = length_penalty_fn
+        self.advantage_estimator = None if strategy is None else strategy.args.algo.advantage.estimator
+
+    def get_advantages_and_returns(self, values, rewards, action_mask, gamma, lambd):
+        return get_advantages_and_returns(values, rewards, action_mask, gamma, lambd)
+
+    def get_cumulative_returns(self, rewards, action_mask, gamma):
+        return get_cumulative_returns(rewards, action_mask, gamma)
+
+    def compute_advantages_and_returns(self, experiences):
+        args = self.strategy.args
+        return compute_advantages_and_returns(
+            experiences,
+            advantage_estimator=args.algo.advantage.estimator,
+            n_samples_per_prompt=args.rollout.n_samples_per_prompt,
+            kl_coef=self.kl_ctl.value,
+            gamma=args.algo.advantage.gamma,
+            lambd=args.algo.advantage.lambd,
+            reward_clip_range=args.reward.clip_range,
+            no_std_norm=args.algo.advantage.no_std_norm,
+            length_penalty_fn=self.length_penalty_fn,
+        )

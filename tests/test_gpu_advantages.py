@@ -1,0 +1,278 @@
+"""Parity of the advantage kernels (compute_reward, GAE, discounted returns, group baselines,
+whitening) with the CPU oracle. GAE tolerance: 1e-5 relative (to the largest magnitude in the
+block, so that exact cancellations do not dominate)."""
+import math
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from oracle import advantages as oa
+from oracle import token_numerics as otn
+
+pytestmark = pytest.mark.gpu
+RTOL = 1e-5
+
+
+def _rel_close(got, ref, rtol=RTOL):
+    got = got.detach().cpu().double()
+    ref = ref.detach().double()
+    assert got.shape == ref.shape
+    scale = max(ref.abs().max().item(), 1e-30) if ref.numel() else 1.0
+    err = (got - ref).abs().max().item() if ref.numel() else 0.0
+    assert err <= rtol * scale, (err, scale)
+
+
+def _mask(b, a, seed, kind="mixed"):
+    g = torch.Generator().manual_seed(seed)
+    m = torch.ones(b, a)
+    for i in range(b):
+        left = int(torch.randint(0, max(a // 3, 1), (1,), generator=g))
+        right = int(torch.randint(0, max(a // 3, 1), (1,), generator=g))
+        m[i, :left] = 0
+        if right:
+            m[i, a - right:] = 0
+        if kind == "mixed" and a > 16:
+            h = int(torch.randint(0, a - 3, (1,), generator=g))
+            m[i, h:h + 3] = 0
+    return m
+
+
+# ------------------------------------------------------------------ compute_reward
+@pytest.mark.parametrize("mask_dtype", [torch.bool, torch.float32, torch.int64])
+def test_compute_reward_matches_oracle_and_brute_force(cuda, mask_dtype):
+    from openrlhf_amd.models.utils import compute_reward
+
+    b, a = 40, 777
+    g = torch.Generator().manual_seed(1)
+    mask = _mask(b, a, 1)
+    mask[3] = 0  # all-zero row: the reward lands on the last column
+    mask[4] = 1
+    r = torch.randn(b, generator=g) * 8
+    kl = torch.randn(b, a, generator=g)
+    ref = otn.compute_reward(r, 0.05, kl, mask, reward_clip_range=(-10, 10))
+    out = compute_reward(r.to(cuda), 0.05, kl.to(cuda), action_mask=mask.to(mask_dtype).to(cuda), reward_clip_range=(-10, 10))
+    assert torch.equal(out.cpu(), ref)  # same fp32 operations: bit-exact
+    # the double loop given as a comment in the reference (models/utils.py:112-120)
+    brute = torch.zeros(b, a)
+    for i in range(b):
+        for t in reversed(range(a)):
+            if mask[i, t] > 0.5:
+                brute[i, t] = r[i].clamp(-10, 10)
+                break
+    rows = [i for i in range(b) if mask[i].sum() > 0]
+    assert torch.equal((out.cpu() - (-0.05) * kl)[rows].round(decimals=4), brute[rows].round(decimals=4))
+    assert abs(out[3, a - 1].item() - (r[3].clamp(-10, 10) - 0.05 * kl[3, a - 1]).item()) < 1e-6
+    # negative coefficient is treated as 0; no clip range
+    out2 = compute_reward(r.to(cuda), -1.0, kl.to(cuda), action_mask=mask.to(cuda))
+    assert torch.equal(out2.cpu(), otn.compute_reward(r, -1.0, kl, mask))
+
+
+# ------------------------------------------------------------------ GAE / returns
+@pytest.mark.parametrize("a", [1, 7, 8, 9, 255, 2047, 2048, 2049, 5000])
+@pytest.mark.parametrize("gamma,lambd", [(1.0, 0.95), (0.99, 0.9), (1.0, 1.0)])
+def test_gae_matches_sequential_oracle(cuda, a, gamma, lambd):
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import get_advantages_and_returns
+
+    b = 13
+    g = torch.Generator().manual_seed(a)
+    values = torch.randn(b, a, generator=g)
+    rewards = torch.randn(b, a, generator=g) * 0.1
+    mask = _mask(b, a, a)
+    adv64, ret64 = oa.get_advantages_and_returns(values.double(), rewards.double(), mask.double(), gamma, lambd)
+    adv, ret = get_advantages_and_returns(values.to(cuda), rewards.to(cuda), mask.to(cuda), gamma, lambd)
+    _rel_close(adv, adv64)
+    _rel_close(ret, ret64)
+    # CPU tensors in, CPU tensors out (the reference's experiences live on the CPU)
+    adv_c, ret_c = get_advantages_and_returns(values, rewards, mask.bool(), gamma, lambd)
+    assert adv_c.device.type == "cpu" and torch.equal(adv_c, adv.cpu()) and torch.equal(ret_c, ret.cpu())
+
+
+def test_gae_closed_forms(cuda):
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import get_advantages_and_returns
+
+    b, a = 5, 300
+    g = torch.Generator().manual_seed(3)
+    values = torch.randn(b, a, generator=g)
+    rewards = torch.randn(b, a, generator=g)
+    ones = torch.ones(b, a)
+    # lambda = gamma = 1: A_t = sum_{s >= t} r_s - v_t
+    adv, ret = get_advantages_and_returns(values.to(cuda), rewards.to(cuda), ones.to(cuda), 1.0, 1.0)
+    togo = rewards.double().flip(1).cumsum(1).flip(1)
+    _rel_close(adv, togo - values.double())
+    _rel_close(ret, togo)
+    # lambda = 0: one-step TD error
+    adv, _ = get_advantages_and_returns(values.to(cuda), rewards.to(cuda), ones.to(cuda), 0.9, 0.0)
+    nxt = torch.cat([values[:, 1:], torch.zeros(b, 1)], 1).double()
+    _rel_close(adv, rewards.double() + 0.9 * nxt - values.double())
+    # right padding gives exact zeros; masked prompt columns are NOT zero (nothing is re-masked)
+    mask = ones.clone()
+    mask[:, 250:] = 0
+    mask[:, :20] = 0
+    adv, ret = get_advantages_and_returns(values.to(cuda), rewards.to(cuda), mask.to(cuda), 1.0, 0.95)
+    assert adv[:, 250:].abs().max().item() == 0.0 and ret[:, 250:].abs().max().item() == 0.0
+    assert adv[:, :20].abs().min().item() > 0.0
+
+
+@pytest.mark.parametrize("a", [1, 100, 2048, 4097])
+def test_cumulative_returns(cuda, a):
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import get_cumulative_returns
+
+    b = 9
+    g = torch.Generator().manual_seed(a + 1)
+    rewards = torch.randn(b, a, generator=g)
+    mask = _mask(b, a, a + 1)
+    for gamma in (1.0, 0.97):
+        ref = oa.get_cumulative_returns(rewards.double(), mask.double(), gamma)
+        _rel_close(get_cumulative_returns(rewards.to(cuda), mask.to(cuda), gamma), ref)
+    # gamma = 1 and a single terminal reward: every column up to it holds that reward
+    one = torch.zeros(b, a)
+    one[:, -1] = 2.5
+    out = get_cumulative_returns(one.to(cuda), torch.ones(b, a).to(cuda), 1.0)
+    assert torch.equal(out.cpu(), torch.full((b, a), 2.5))
+
+
+def test_packed_scan_equals_padded(cuda):
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import get_advantages_and_returns, get_cumulative_returns
+
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(1, 6000, (21,), generator=g)
+    a = int(lens.max())
+    values = torch.randn(21, a, generator=g)
+    rewards = torch.randn(21, a, generator=g) * 0.1
+    valid = torch.arange(a)[None, :] < lens[:, None]
+    inner = (torch.rand(21, a, generator=g) > 0.1) & valid
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), lens.cumsum(0)]).to(cuda)
+    adv, ret = get_advantages_and_returns(values.to(cuda), rewards.to(cuda), inner.to(cuda), 1.0, 0.95)
+    adv_p, ret_p = get_advantages_and_returns(values[valid].to(cuda), rewards[valid].to(cuda), inner[valid].to(cuda),
+                                              1.0, 0.95, cu_seqlens=cu)
+    assert torch.equal(adv_p, adv[valid.to(cuda)]) and torch.equal(ret_p, ret[valid.to(cuda)])
+    assert adv[~valid.to(cuda)].abs().max().item() == 0.0  # what unpacking restores
+    g1 = get_cumulative_returns(rewards.to(cuda), inner.to(cuda), 0.99)
+    g2 = get_cumulative_returns(rewards[valid].to(cuda), inner[valid].to(cuda), 0.99, cu_seqlens=cu)
+    assert torch.equal(g2, g1[valid.to(cuda)])
+
+
+# ------------------------------------------------------------------ group baselines
+@pytest.mark.parametrize("estimator", ["gae", "reinforce", "rloo", "reinforce_baseline", "dr_grpo", "group_norm"])
+@pytest.mark.parametrize("n", [2, 8, 5])
+def test_group_normalize(cuda, estimator, n):
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import group_normalize_rewards
+
+    p = 64
+    g = torch.Generator().manual_seed(n)
+    rewards = (torch.rand(p * n, generator=g) < 0.3).float()  # Bernoulli(0.3): many all-equal groups
+    rewards[: 2 * n] = torch.randn(2 * n, generator=g)
+    perm = torch.randperm(p * n, generator=g)
+    ref, ref_std = oa.group_normalize(rewards.double(), perm, n, estimator)
+    out, std = group_normalize_rewards(rewards.to(cuda), perm.to(cuda), n, estimator)
+    assert (out.cpu().double() - ref).abs().max().item() <= 1e-5 * max(1.0, ref.abs().max().item())
+    assert (std.cpu().double() - ref_std).abs().max().item() <= 1e-6
+    # numpy-style cross-check of the unbiased std and of exact zeros for all-equal groups
+    ordered = torch.empty_like(rewards)
+    ordered[perm] = rewards
+    grid = ordered.view(p, n)
+    flat_group = (perm // n)
+    if estimator in ("reinforce_baseline", "dr_grpo", "group_norm", "rloo"):
+        equal = (grid.max(1).values == grid.min(1).values)[flat_group]
+        assert out.cpu()[equal].abs().max().item() == 0.0
+    if estimator == "rloo":
+        sums = torch.zeros(p).index_add_(0, flat_group, out.cpu())
+        assert sums.abs().max().item() <= 1e-5
+    if estimator in ("gae", "reinforce"):
+        assert torch.equal(out.cpu(), rewards)
+
+
+def test_group_normalize_single_sample_and_errors(cuda):
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import group_normalize_rewards
+
+    r = torch.randn(10)
+    out, std = group_normalize_rewards(r.to(cuda), None, 1, "reinforce")
+    assert std is None and torch.equal(out.cpu(), r)
+    with pytest.raises(Exception):
+        group_normalize_rewards(r.to(cuda), None, 2, "unknown")
+    with pytest.raises(ValueError):
+        group_normalize_rewards(r.to(cuda), None, 3, "rloo")
+
+
+# ------------------------------------------------------------------ whitening
+@pytest.mark.parametrize("no_std_norm", [False, True])
+def test_whitening(cuda, no_std_norm):
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import whiten_advantages
+
+    g = torch.Generator().manual_seed(11)
+    shapes = [(4, 300), (7, 1111), (1, 5)]
+    advs = [torch.randn(s, generator=g) * 3 + 1.5 for s in shapes]
+    masks = [_mask(s[0], s[1], i + 20) for i, s in enumerate(shapes)]
+    ref, mean, rstd = oa.whiten_advantages([a.double() for a in advs], [m.double() for m in masks], no_std_norm)
+    out = whiten_advantages([a.to(cuda) for a in advs], [m.to(cuda).bool() for m in masks], no_std_norm)
+    for o, r in zip(out, ref):
+        _rel_close(o, r)
+    flat = torch.cat([o.cpu().double().flatten() for o in out])
+    m = torch.cat([x.flatten() for x in masks]).double()
+    assert abs(((flat * m).sum() / m.sum()).item()) <= 1e-5
+    if not no_std_norm:
+        assert abs((((flat ** 2) * m).sum() / m.sum()).item() - 1.0) <= 1e-4
+    # masked columns are whitened too (not zeroed)
+    assert out[0].cpu()[masks[0] == 0].abs().min().item() > 0.0
+
+
+# ------------------------------------------------------------------ config 3 shape, end to end
+@pytest.mark.parametrize("estimator", ["gae", "reinforce_baseline", "group_norm", "rloo"])
+def test_compute_advantages_and_returns_pipeline(cuda, estimator):
+    """A down-scaled BASELINE config 3 / 4: experiences with CPU tensors as the reference's
+    controller holds them; k1 KL penalty 0.01, gamma 1, lambda 0.95; compared with the oracle's
+    composition of the same steps (experience_maker.py:237-330)."""
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import AdvantageFunctions
+
+    g = torch.Generator().manual_seed(33)
+    n_prompts, n = 12, 4
+    total = n_prompts * n
+    lens = torch.clamp(torch.exp(torch.randn(total, generator=g) * 0.8 + 5.5), 16, 2048).long()
+    perm = torch.randperm(total, generator=g)
+    exps, ref_exps = [], []
+    per_exp = 8
+    for lo in range(0, total, per_exp):
+        ids = list(range(lo, lo + per_exp))
+        a = int(lens[ids].max())
+        mask = (torch.arange(a)[None, :] < lens[ids][:, None])
+        mask[:, :3] = False
+        kl = torch.randn(per_exp, a, generator=g) * 0.05
+        values = torch.randn(per_exp, a, generator=g)
+        rewards = (torch.rand(per_exp, generator=g) < 0.5).float()
+        index = perm[ids].tolist()
+        for store in (exps, ref_exps):
+            store.append(SimpleNamespace(index=index, rewards=rewards.clone(), kl=kl.clone(), action_mask=mask.clone(),
+                                         values=values.clone(), info={}, advantages=None, returns=None))
+    args = SimpleNamespace(
+        algo=SimpleNamespace(advantage=SimpleNamespace(estimator=estimator, gamma=1.0, lambd=0.95, no_std_norm=False)),
+        rollout=SimpleNamespace(n_samples_per_prompt=n),
+        reward=SimpleNamespace(clip_range=(-10, 10)),
+    )
+    fn = AdvantageFunctions(strategy=SimpleNamespace(args=args), kl_ctl=SimpleNamespace(value=0.01))
+    out = fn.compute_advantages_and_returns(exps)
+
+    # oracle composition in fp64
+    raw = torch.cat([e.rewards for e in ref_exps]).double()
+    idx = torch.tensor([i for e in ref_exps for i in e.index])
+    shaped, gstd = oa.group_normalize(raw, idx, n, estimator)
+    advs, rets, infos = [], [], []
+    for e, r in zip(ref_exps, shaped.split([per_exp] * len(ref_exps))):
+        rew = otn.compute_reward(r, 0.01, e.kl.double(), e.action_mask, (-10, 10))
+        if estimator == "gae":
+            a_, r_ = oa.get_advantages_and_returns(e.values.double(), rew, e.action_mask, 1.0, 0.95)
+        else:
+            r_ = oa.get_cumulative_returns(rew, e.action_mask, 1.0)
+            a_ = r_.clone()
+        advs.append(a_)
+        rets.append(r_)
+        infos.append(rew.sum(-1))
+    if estimator in ("gae", "reinforce", "reinforce_baseline"):
+        advs, _, _ = oa.whiten_advantages(advs, [e.action_mask for e in ref_exps])
+    for e, a_, r_, i_ in zip(out, advs, rets, infos):
+        assert e.advantages.device.type == "cpu" and e.kl is None
+        _rel_close(e.advantages, a_, 2e-5)
+        _rel_close(e.returns, r_)
+        _rel_close(e.info["return"], i_, 1e-5)
+    std_all = torch.cat([e.info["group_reward_std"] for e in out])
+    assert (std_all.double() - gstd).abs().max().item() <= 1e-6

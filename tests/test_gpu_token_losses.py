@@ -1,0 +1,372 @@
+"""Parity of the per-token kernels (KL, masked aggregation, PolicyLoss, ValueLoss) with the CPU
+oracle. Values are compared with the fp64 oracle at 1e-5 abs (the stated tolerance for fp32
+inputs); gradients with torch autograd through the oracle (which carries torch's own min/max/clamp
+tie rules)."""
+import math
+
+import pytest
+import torch
+
+from oracle import losses as ol
+from oracle import token_numerics as otn
+
+pytestmark = pytest.mark.gpu
+ATOL = 1e-5
+
+
+def _tok(b, a, seed, holes=True):
+    """Per-token tensors in the reference's [B, A] layout with left prompt zeros, optional
+    mid-row holes and right padding in the mask."""
+    g = torch.Generator().manual_seed(seed)
+    lp = -torch.rand(b, a, generator=g) * 3
+    old = lp + torch.randn(b, a, generator=g) * 0.2
+    rollout = old + torch.randn(b, a, generator=g) * 0.1
+    adv = torch.randn(b, a, generator=g)
+    mask = torch.ones(b, a)
+    for i in range(b):
+        left = int(torch.randint(0, max(a // 4, 1), (1,), generator=g))
+        right = int(torch.randint(0, max(a // 3, 1), (1,), generator=g))
+        mask[i, :left] = 0
+        if right:
+            mask[i, a - right:] = 0
+        if holes and a > 8:
+            h = int(torch.randint(left, a - right - 1, (1,), generator=g)) if a - right - 1 > left else left
+            mask[i, h:h + 2] = 0
+    return lp, old, rollout, adv, mask
+
+
+def _close(got, ref, atol=ATOL):
+    got = got.detach().cpu().double()
+    ref = ref.detach().double()
+    assert got.shape == ref.shape, (got.shape, ref.shape)
+    assert torch.equal(got.isnan(), ref.isnan())  # NaN (0/0 on an empty mask) in the same places
+    diff = (got - ref).abs()[~ref.isnan()]
+    err = diff.max().item() if diff.numel() else 0.0
+    assert err <= atol, err
+
+
+# ------------------------------------------------------------------ compute_approx_kl
+@pytest.mark.parametrize("est", ["k1", "k2", "k3"])
+def test_approx_kl_values_and_grads(cuda, est):
+    from openrlhf_amd.models.utils import compute_approx_kl
+
+    g = torch.Generator().manual_seed(1)
+    lp = -torch.rand(7, 333, generator=g) * 5
+    base = lp + torch.randn(7, 333, generator=g) * 2.0
+    base[0, :5] = lp[0, :5] + torch.tensor([30.0, -30.0, 12.0, -4.5, 0.0])  # clamp at +-10 active
+    ref = otn.compute_approx_kl(lp.double(), base.double(), est)
+    lpd = lp.to(cuda).requires_grad_(True)
+    based = base.to(cuda).requires_grad_(True)
+    out = compute_approx_kl(lpd, based, est)
+    assert out.dtype == torch.float32
+    _close(out, ref, 1e-5 if est != "k3" else 2e-5)
+    w = torch.randn(7, 333, generator=g)
+    (out * w.to(cuda)).sum().backward()
+    lp_ref = lp.double().requires_grad_(True)
+    base_ref = base.double().requires_grad_(True)
+    (otn.compute_approx_kl(lp_ref, base_ref, est) * w.double()).sum().backward()
+    _close(lpd.grad, lp_ref.grad, 1e-4)
+    _close(based.grad, base_ref.grad, 1e-4)
+    # closed forms: k2, k3 >= 0; k1 itself is clamped
+    if est != "k1":
+        assert out.min().item() >= 0.0
+    assert out.max().item() <= 10.0 and out.min().item() >= -10.0
+
+
+def test_approx_kl_bf16_inputs_and_errors(cuda):
+    from openrlhf_amd.models.utils import compute_approx_kl
+
+    g = torch.Generator().manual_seed(2)
+    lp = (-torch.rand(4, 100, generator=g) * 5).to(torch.bfloat16)
+    base = (lp.float() + torch.randn(4, 100, generator=g) * 0.1).to(torch.bfloat16)
+    out = compute_approx_kl(lp.to(cuda), base.to(cuda), "k3")
+    _close(out, otn.compute_approx_kl(lp, base, "k3"), 1e-6)
+    with pytest.raises(ValueError):
+        compute_approx_kl(lp.to(cuda), base.to(cuda), "k4")
+    with pytest.raises(RuntimeError):
+        compute_approx_kl(lp, base, "k1")  # CPU tensors: no fallback
+
+
+# ------------------------------------------------------------------ masked_mean / aggregate_loss
+@pytest.mark.parametrize("mask_dtype", [torch.float32, torch.bool, torch.int64, torch.uint8, torch.bfloat16, None])
+def test_masked_mean_all_dims(cuda, mask_dtype):
+    from openrlhf_amd.models.utils import masked_mean
+
+    lp, _, _, adv, mask = _tok(9, 517, seed=3)
+    m = None if mask_dtype is None else mask.to(mask_dtype)
+    mref = None if m is None else mask.double()
+    md = None if m is None else m.to(cuda)
+    _close(masked_mean(adv.to(cuda), md), otn.masked_mean(adv.double(), mref))
+    _close(masked_mean(adv.to(cuda), md, dim=-1), otn.masked_mean(adv.double(), mref, dim=-1))
+    _close(masked_mean(adv.to(cuda), md, dim=1), otn.masked_mean(adv.double(), mref, dim=1))
+    _close(masked_mean(adv.to(cuda), md, dim=0), otn.masked_mean(adv.double(), mref, dim=0))
+
+
+def test_masked_mean_empty_mask_is_nan_and_weights(cuda):
+    from openrlhf_amd.models.utils import masked_mean
+
+    x = torch.arange(12.0).view(3, 4)
+    zero = torch.zeros(3, 4)
+    assert math.isnan(masked_mean(x.to(cuda), zero.to(cuda)).item())
+    row = masked_mean(x.to(cuda), torch.tensor([[1.0, 1, 0, 0], [0, 0, 0, 0], [0, 0, 0, 1]]).to(cuda), dim=-1).cpu()
+    assert row[0].item() == 0.5 and math.isnan(row[1].item()) and row[2].item() == 11.0
+    # a float mask is a weight, as in the reference's tensor * mask
+    w = torch.tensor([[0.5, 2.0, 0.0, 1.0]] * 3)
+    _close(masked_mean(x.to(cuda), w.to(cuda)), otn.masked_mean(x.double(), w.double()))
+
+
+def test_aggregate_loss_reference_identities(cuda):
+    """The assertions of the reference's tests/test_loss_aggregation.py:47-94 on the HIP path:
+    DP-split invariance of token-mean and of seq-mean, and exclusion of fully masked rows."""
+    from openrlhf_amd.models.loss import aggregate_loss
+
+    d = cuda
+    loss = torch.tensor([[1.0, 2.0, 0.0], [3.0, 4.0, 5.0], [7.0, 0.0, 0.0]], device=d)
+    mask = torch.tensor([[1.0, 1.0, 0.0], [1.0, 1.0, 1.0], [1.0, 0.0, 0.0]], device=d)
+    full = aggregate_loss(loss, mask)
+    n_tok = mask.sum()  # a device tensor, as get_loss_batch_info returns
+    r0 = aggregate_loss(loss[:2], mask[:2], dp_size=2, batch_num_tokens=n_tok)
+    r1 = aggregate_loss(loss[2:], mask[2:], dp_size=2, batch_num_tokens=n_tok)
+    assert torch.allclose((r0 + r1) / 2, full)
+    assert abs(full.item() - 22.0 / 6.0) < 1e-6
+
+    loss = torch.tensor([[1.0, 3.0, 9.0], [2.0, 4.0, 0.0], [8.0, 0.0, 0.0]], device=d)
+    mask = torch.tensor([[1.0, 1.0, 0.0], [1.0, 1.0, 0.0], [1.0, 0.0, 0.0]], device=d)
+    full = aggregate_loss(loss, mask, token_level_loss=False)
+    r0 = aggregate_loss(loss[:2], mask[:2], token_level_loss=False, dp_size=2, global_batch_size=torch.tensor(3.0))
+    r1 = aggregate_loss(loss[2:], mask[2:], token_level_loss=False, dp_size=2, global_batch_size=3.0)
+    assert torch.allclose((r0 + r1) / 2, full)
+    assert abs(full.item() - (2.0 + 3.0 + 8.0) / 3.0) < 1e-6
+
+    loss = torch.tensor([[1.0, 3.0], [5.0, 7.0]], device=d)
+    mask = torch.tensor([[1.0, 1.0], [0.0, 0.0]], device=d)
+    info = ol.loss_batch_info(mask.cpu())
+    assert info["global_batch_size"].item() == 1.0
+    seq = aggregate_loss(loss, mask, token_level_loss=False, **info)
+    assert torch.allclose(seq.cpu(), torch.tensor(2.0))
+
+
+@pytest.mark.parametrize("token_level,given", [(True, False), (True, True), (False, False), (False, True)])
+def test_aggregate_loss_values_and_grads(cuda, token_level, given):
+    from openrlhf_amd.models.loss import aggregate_loss
+
+    lp, _, _, adv, mask = _tok(37, 1500, seed=4)
+    mask[5] = 0  # one fully masked sequence
+    kw = {}
+    if given:
+        kw = dict(dp_size=4, batch_num_tokens=12345.0, global_batch_size=77.0)
+    ref_in = adv.double().requires_grad_(True)
+    ref = ol.aggregate_loss(ref_in, mask.double(), token_level_loss=token_level, **kw)
+    ref.backward()
+    x = adv.to(cuda).requires_grad_(True)
+    out = aggregate_loss(x, mask.to(cuda).bool(), token_level_loss=token_level, **kw)
+    _close(out, ref)
+    out.backward()
+    _close(x.grad, ref_in.grad, 1e-9 + 1e-6 * ref_in.grad.abs().max().item())
+
+
+# ------------------------------------------------------------------ PolicyLoss
+POLICY_CASES = [
+    dict(),
+    dict(clip_eps_low=0.1, clip_eps_high=0.3),
+    dict(dual_clip=3.0),
+    dict(token_level_loss=False),
+    dict(dual_clip=3.0, token_level_loss=False),
+    dict(enable_vllm_is_correction=True, vllm_is_truncated_threshold=[0.8, 1.2], vllm_is_correction_type="tis"),
+    dict(enable_vllm_is_correction=True, vllm_is_truncated_threshold=[0.9, 1.1], vllm_is_correction_type="icepop"),
+    dict(enable_vllm_is_correction=True, vllm_is_truncated_threshold=[0.995, 1.005], vllm_is_correction_type="seq-mask-tis"),
+    dict(policy_loss_type="gspo"),
+    dict(policy_loss_type="gspo", enable_vllm_is_correction=True, vllm_is_truncated_threshold=[0.5, 2.0]),
+]
+
+
+@pytest.mark.parametrize("cfg", POLICY_CASES)
+@pytest.mark.parametrize("given", [False, True])
+def test_policy_loss_matches_oracle(cuda, cfg, given):
+    from openrlhf_amd.models.loss import PolicyLoss
+
+    lp, old, rollout, adv, mask = _tok(23, 1300, seed=5)
+    old[0, :40] = lp[0, :40] - 25.0   # ratio clamp at +-20 active
+    old[1, :40] = lp[1, :40] + 25.0
+    adv[2, :50] = 0.0                 # ties between the two surrogates
+    old[3] = lp[3]                    # ratio exactly 1
+    mask[4] = 0                       # fully masked sequence
+    kw = dict(dp_size=2, batch_num_tokens=20000.0, global_batch_size=30.0) if given else {}
+    use_rollout = cfg.get("enable_vllm_is_correction", False)
+
+    ref_lp = lp.double().requires_grad_(True)
+    ref = ol.policy_loss(ref_lp, old.double(), adv.double(), mask.double(),
+                         rollout.double() if use_rollout else None, **cfg, **kw)
+    ref[0].backward()
+
+    fn = PolicyLoss(**cfg)
+    x = lp.to(cuda).requires_grad_(True)
+    out = fn(x, old.to(cuda), adv.to(cuda), action_mask=mask.to(cuda),
+             rollout_log_probs=rollout.to(cuda) if use_rollout else None, **kw)
+    assert len(out) == 4
+    _close(out[0], ref[0], 2e-5)
+    _close(out[1], ref[1])
+    _close(out[2], ref[2])
+    if ref[3] is None:
+        assert out[3] is None
+    else:
+        _close(out[3], ref[3])
+    out[0].backward()
+    scale = ref_lp.grad.abs().max().item()
+    _close(x.grad, ref_lp.grad, 1e-9 + 2e-5 * scale)
+
+
+def test_policy_loss_reference_identities(cuda):
+    """tests/test_loss_aggregation.py:97-148,196-204 of the reference, on the HIP path."""
+    from openrlhf_amd.models.loss import PolicyLoss
+
+    d = cuda
+    lp = torch.tensor([[-0.20, -0.40, -0.10], [-0.70, -0.30, -0.20], [-0.60, -0.10, -0.50]], device=d)
+    old = lp - torch.tensor([[0.03, -0.04, 0.01], [0.02, 0.05, -0.03], [0.04, 0.0, -0.02]], device=d)
+    adv = torch.tensor([[1.0, -0.5, 0.0], [0.3, -1.2, 0.5], [1.5, 0.0, -0.7]], device=d)
+    mask = torch.tensor([[1.0, 1.0, 0.0], [1.0, 1.0, 1.0], [1.0, 0.0, 1.0]], device=d)
+    fn = PolicyLoss(clip_eps_low=0.2, clip_eps_high=0.2)
+    full, *_ = fn(lp, old, adv, action_mask=mask)
+    n = mask.sum()
+    r0, *_ = fn(lp[:2], old[:2], adv[:2], action_mask=mask[:2], dp_size=2, batch_num_tokens=n)
+    r1, *_ = fn(lp[2:], old[2:], adv[2:], action_mask=mask[2:], dp_size=2, batch_num_tokens=n)
+    assert torch.allclose((r0 + r1) / 2, full)
+
+    lp = torch.tensor([[-0.2, -0.4]], device=d)
+    old = torch.tensor([[-0.3, -0.1]], device=d)
+    roll = torch.tensor([[-1.3, -1.1]], device=d)
+    fn = PolicyLoss(enable_vllm_is_correction=True, vllm_is_truncated_threshold=[0.1, 10.0], vllm_is_correction_type="tis")
+    _, _, ppo_kl, vllm_kl = fn(lp, old, torch.ones_like(lp), action_mask=torch.ones_like(lp), rollout_log_probs=roll)
+    assert torch.allclose(ppo_kl, (old - lp).mean())
+    assert torch.allclose(vllm_kl, (roll - old).mean())
+
+    lp = torch.tensor([[100.0]], device=d)
+    _, _, ppo_kl, _ = PolicyLoss()(lp, torch.zeros_like(lp), torch.ones_like(lp), action_mask=torch.ones_like(lp))
+    assert torch.allclose(ppo_kl, torch.tensor(-100.0, device=d))  # the metric is not clamped
+
+
+def test_policy_loss_closed_forms_and_errors(cuda):
+    from openrlhf_amd.models.loss import PolicyLoss
+
+    lp, old, _, adv, mask = _tok(6, 200, seed=6)
+    d = cuda
+    # lp == old: loss = -masked_mean(A), nothing clipped
+    loss, clip, kl, v = PolicyLoss()(lp.to(d), lp.to(d), adv.to(d), action_mask=mask.to(d))
+    _close(loss, -(adv.double() * mask.double()).sum() / mask.double().sum())
+    assert clip.item() == 0.0 and kl.item() == 0.0 and v is None
+    # dual clip: A < 0 and ratio > c  =>  token loss = -c * A
+    a = -torch.ones(1, 4)
+    big = torch.full((1, 4), math.log(10.0))
+    loss, *_ = PolicyLoss(dual_clip=3.0)(big.to(d), torch.zeros(1, 4).to(d), a.to(d), action_mask=torch.ones(1, 4).to(d))
+    assert abs(loss.item() - 3.0) < 1e-6
+    with pytest.raises(AssertionError):
+        PolicyLoss(dual_clip=1.0)
+    with pytest.raises(ValueError):
+        PolicyLoss(vllm_is_correction_type="nope")
+    with pytest.raises(ValueError):
+        PolicyLoss(policy_loss_type="nope")(lp.to(d), old.to(d), adv.to(d), action_mask=mask.to(d))
+
+
+def test_packed_layout_equals_padded(cuda):
+    """cu_seqlens layout: pack(right-padded rows) gives the same scalars and the same per-token
+    gradients as the padded [B, A] layout with its mask."""
+    from openrlhf_amd.models.loss import PolicyLoss, ValueLoss, aggregate_loss
+
+    g = torch.Generator().manual_seed(7)
+    lens = torch.randint(1, 3000, (19,), generator=g)
+    a = int(lens.max())
+    lp, old, _, adv, _ = _tok(19, a, seed=8, holes=False)
+    valid = (torch.arange(a)[None, :] < lens[:, None])
+    inner = (torch.rand(19, a, generator=g) > 0.2) & valid  # action mask inside the valid part
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), lens.cumsum(0)])
+
+    def pack(t):
+        return t[valid].to(cuda)
+
+    for cfg in (dict(), dict(token_level_loss=False, dual_clip=3.0), dict(policy_loss_type="gspo")):
+        fn = PolicyLoss(**cfg)
+        x = lp.to(cuda).requires_grad_(True)
+        ref = fn(x, old.to(cuda), adv.to(cuda), action_mask=inner.to(cuda))
+        ref[0].backward()
+        xp = pack(lp).requires_grad_(True)
+        out = fn(xp, pack(old), pack(adv), action_mask=pack(inner), cu_seqlens=cu.to(cuda))
+        out[0].backward()
+        for i in range(3):
+            assert abs(out[i].item() - ref[i].item()) <= 1e-6 * max(1.0, abs(ref[i].item()))
+        assert (xp.grad - x.grad[valid.to(cuda)]).abs().max().item() <= 1e-9
+    v = ValueLoss(0.2)
+    r1 = v(lp.to(cuda), old.to(cuda), adv.to(cuda), action_mask=inner.to(cuda))
+    r2 = v(pack(lp), pack(old), pack(adv), action_mask=pack(inner), cu_seqlens=cu.to(cuda))
+    assert abs(r1.item() - r2.item()) <= 1e-6 * max(1.0, abs(r1.item()))
+    s1 = aggregate_loss(adv.to(cuda), inner.to(cuda), token_level_loss=False)
+    s2 = aggregate_loss(pack(adv), pack(inner), token_level_loss=False, cu_seqlens=cu.to(cuda))
+    assert abs(s1.item() - s2.item()) <= 1e-6
+
+
+# ------------------------------------------------------------------ ValueLoss
+@pytest.mark.parametrize("clip_eps", [None, 0.2, 0.5])
+@pytest.mark.parametrize("token_level", [True, False])
+def test_value_loss_matches_oracle(cuda, clip_eps, token_level):
+    from openrlhf_amd.models.loss import ValueLoss
+
+    g = torch.Generator().manual_seed(9)
+    _, _, _, _, mask = _tok(31, 900, seed=9)
+    values = torch.randn(31, 900, generator=g)
+    old = values + torch.randn(31, 900, generator=g) * 0.3
+    ret = torch.randn(31, 900, generator=g)
+    old[0, :30] = values[0, :30]  # clipped == unclipped: tie in torch.max
+    ref_v = values.double().requires_grad_(True)
+    ref = ol.value_loss(ref_v, old.double(), ret.double(), mask.double(), clip_eps=clip_eps, token_level_loss=token_level)
+    ref.backward()
+    x = values.to(cuda).requires_grad_(True)
+    out = ValueLoss(clip_eps, token_level_loss=token_level)(x, old.to(cuda), ret.to(cuda), action_mask=mask.to(cuda))
+    _close(out, ref)
+    out.backward()
+    _close(x.grad, ref_v.grad, 1e-9 + 2e-5 * ref_v.grad.abs().max().item())
+    if clip_eps is not None:  # eps -> infinity equals the unclipped loss
+        big = ValueLoss(1e9, token_level_loss=token_level)(values.to(cuda), old.to(cuda), ret.to(cuda), action_mask=mask.to(cuda))
+        plain = ValueLoss(None, token_level_loss=token_level)(values.to(cuda), old.to(cuda), ret.to(cuda), action_mask=mask.to(cuda))
+        assert abs(big.item() - plain.item()) <= 1e-6 * max(1.0, plain.item())
+
+
+# ------------------------------------------------------------------ config 1 end to end
+def test_config1_plumbing(cuda):
+    """BASELINE config 1: fp32 logits [4, 256, 32000] ~ N(0, 2), labels uniform, action mask with
+    0-64 right-padding zeros per row; log_probs_from_logits -> k3 KL vs ref = lp + N(0, 0.05) ->
+    PolicyLoss(eps 0.2, token mean) with old = lp + N(0, 0.02), advantages ~ N(0, 1)."""
+    from openrlhf_amd.models.loss import PolicyLoss
+    from openrlhf_amd.models.utils import compute_approx_kl, log_probs_from_logits, masked_mean
+
+    g = torch.Generator().manual_seed(2024)
+    b, t, vocab = 4, 256, 32000
+    logits = torch.randn(b, t, vocab, generator=g) * 2.0
+    labels = torch.randint(0, vocab, (b, t), generator=g)
+    mask = torch.ones(b, t)
+    for i in range(b):
+        pad = int(torch.randint(0, 65, (1,), generator=g))
+        if pad:
+            mask[i, t - pad:] = 0
+    ref_noise = torch.randn(b, t, generator=g) * 0.05
+    old_noise = torch.randn(b, t, generator=g) * 0.02
+    adv = torch.randn(b, t, generator=g)
+
+    # oracle, fp64
+    x64 = logits.double().requires_grad_(True)
+    lp64 = otn.log_probs_from_logits(x64, labels)
+    kl64 = otn.compute_approx_kl(lp64, (lp64 + ref_noise.double()).detach(), "k3")
+    pl64 = ol.policy_loss(lp64, (lp64 + old_noise.double()).detach(), adv.double(), mask.double())
+    klm64 = otn.masked_mean(kl64, mask.double())
+    (pl64[0] + 0.01 * klm64).backward()
+
+    xd = logits.to(cuda).requires_grad_(True)
+    lp = log_probs_from_logits(xd, labels.to(cuda))
+    _close(lp, lp64, ATOL)
+    kl = compute_approx_kl(lp, (lp + ref_noise.to(cuda)).detach(), "k3")
+    _close(kl, kl64, ATOL)
+    out = PolicyLoss(0.2, 0.2)(lp, (lp + old_noise.to(cuda)).detach(), adv.to(cuda), action_mask=mask.to(cuda))
+    klm = masked_mean(kl, mask.to(cuda))
+    for got, ref in zip(out[:3], pl64[:3]):
+        _close(got, ref, ATOL)
+    _close(klm, klm64, ATOL)
+    (out[0] + 0.01 * klm).backward()
+    assert (xd.grad.cpu().double() - x64.grad).abs().max().item() <= 1e-7
