@@ -1,0 +1,243 @@
+"""Headline benchmark: fused log-prob + entropy forward + in-place backward over packed bf16
+logits at V = 151936 (BASELINE config 2), one GPU.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
+
+One step = one forward and one backward of ``logprobs_and_entropy_from_logits`` over the whole
+packed batch (16 sequences, lengths uniform in [512, 3072], ~28.7 K tokens, 8.7 GB of logits),
+called through the public Python API, i.e. through the C ABI into the HIP kernels. The backward
+overwrites the logits with their gradient, so every step gets logits nobody has touched: a ring
+of buffers is refilled from a pristine copy between timed segments (the refill is outside the
+timed segments; each segment is bracketed by torch.cuda.synchronize()).
+
+Prints ONE JSON line. `value` = tokens/s over the timed steps with inputs resident in HBM;
+`roofline` prices the dominant kernel (the backward: it moves 2/3 of the bytes) against the
+published 8 TB/s, from HIP-event durations taken on the launch stream inside the timed steps;
+`cpu_baseline` is the CPU oracle (the reference's op sequence on torch CPU) on a row sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+VOCAB = 151936
+N_SEQ = 16
+LEN_LO, LEN_HI = 512, 3072
+HBM_PEAK_GBS = 8000.0
+METRIC = "logprob+entropy fwd+bwd tokens/s at V=151936 bf16; achieved HBM GB/s vs peak"
+
+
+def _ensure_built():
+    from openrlhf_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from openrlhf_amd.csrc.build import build
+
+        build(verbose=False)
+    return _lib.load()
+
+
+def make_workload(dev, seed=1234):
+    """Config 2: packed bf16 logits ~ N(0, 3) with 1% of the rows given one +15 spike, labels
+    uniform, upstream grads ~ N(0, 1). Returns (pristine logits, labels, g_lp, g_ent, cu_seqlens)."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    lens = torch.randint(LEN_LO, LEN_HI + 1, (N_SEQ,), generator=g)
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), lens.cumsum(0)])
+    n = int(cu[-1])
+    gd = torch.Generator(device=dev).manual_seed(seed)
+    logits = torch.empty(n, VOCAB, dtype=torch.bfloat16, device=dev)
+    for lo in range(0, n, 2048):  # fp32 noise in slabs keeps the transient small
+        hi = min(lo + 2048, n)
+        logits[lo:hi] = (torch.randn(hi - lo, VOCAB, generator=gd, device=dev) * 3.0).to(torch.bfloat16)
+    n_spike = max(1, n // 100)
+    rows = torch.randperm(n, generator=g)[:n_spike].to(dev)
+    cols = torch.randint(0, VOCAB, (n_spike,), generator=g).to(dev)
+    logits[rows, cols] += 15.0
+    labels = torch.randint(0, VOCAB, (n,), generator=g).to(dev)
+    g_lp = torch.randn(n, generator=g).to(dev)
+    g_ent = torch.randn(n, generator=g).to(dev)
+    return logits, labels, g_lp, g_ent, cu
+
+
+def cpu_baseline(logits_rows, labels, g_lp, g_ent, repeats=3):
+    """The CPU oracle on a row sample: bf16 -> fp32 up-cast, entropy, gather - chunked logsumexp,
+    autograd backward (the reference's op sequence, openrlhf/models/actor.py:267-285)."""
+    from oracle import token_numerics as otn
+
+    x_bf16 = logits_rows.cpu()
+    labels, g_lp, g_ent = labels.cpu(), g_lp.cpu(), g_ent.cpu()
+    times = []
+    for _ in range(repeats + 1):
+        t0 = time.perf_counter()
+        x = x_bf16.to(torch.float32).requires_grad_(True)
+        ent = otn.compute_entropy(x)
+        lp = otn.log_probs_from_logits(x, labels, 1.0)
+        torch.autograd.backward([lp, ent], [g_lp, g_ent])
+        times.append(time.perf_counter() - t0)
+        del x, ent, lp
+    times = sorted(times[1:])  # first run is warm-up
+    med = times[len(times) // 2]
+    return x_bf16.shape[0] / med, med
+
+
+def measured_traffic(kernel, n_tok):
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary (FETCH_SIZE + WRITE_SIZE,
+    each scaled by what the counter reads for a copy of known size); None if it does not cover
+    this workload."""
+    path = os.path.join(ROOT, "profiles", "logprob_entropy_fwd_bwd_config2_hbm_traffic.txt")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    if f"tokens = {n_tok})" not in text:
+        return None
+    for line in text.splitlines():
+        parts = line.split()
+        if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == kernel:
+            return float(parts[2])
+    return None
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=12)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--ring", type=int, default=6, help="distinct logits buffers per timed segment")
+    ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU-baseline sample")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU only (the path shards by rows with no collective "
+                 "on it; see DESIGN.md); run with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
+
+    _ensure_built()
+    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    pristine, labels, g_lp, g_ent, cu = make_workload(dev)
+    n_tok = pristine.shape[0]
+    row_bytes = VOCAB * 2
+    ring = max(1, min(args.ring, args.steps + args.warmup))
+    bufs = [torch.empty_like(pristine) for _ in range(ring)]
+
+    fwd_ms, bwd_ms = [], []
+
+    def step(buf, timed):
+        x = buf.requires_grad_(True)
+        if timed:
+            e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+            e0.record()
+        lp, ent = logprobs_and_entropy_from_logits(x, labels, 1.0, inplace_backward=True)
+        if timed:
+            e1.record()
+        # autograd.grad hands the gradient to the caller the way the next backward node (the
+        # lm_head matmul) would receive it; .backward() on a leaf would add an accumulate step
+        (grad,) = torch.autograd.grad([lp, ent], [x], [g_lp, g_ent])
+        assert grad.data_ptr() == buf.data_ptr()  # written in place, nothing allocated
+        if timed:
+            e2.record()
+            return e0, e1, e2
+        return None
+
+    def run_segment(count, timed):
+        for b in bufs[:count]:
+            b.detach_().copy_(pristine)  # fresh logits; outside the timed segment
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        evs = [step(bufs[i], timed) for i in range(count)]
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        if timed:
+            for e0, e1, e2 in evs:
+                fwd_ms.append(e0.elapsed_time(e1))
+                bwd_ms.append(e1.elapsed_time(e2))
+        return dt
+
+    left = args.warmup
+    while left > 0:
+        c = min(left, ring)
+        run_segment(c, False)
+        left -= c
+    total, left = 0.0, args.steps
+    while left > 0:
+        c = min(left, ring)
+        total += run_segment(c, True)
+        left -= c
+
+    ms_per_step = total / args.steps * 1e3
+    tok_s = n_tok * args.steps / total
+    fwd_avg = sum(fwd_ms) / len(fwd_ms)
+    bwd_avg = sum(bwd_ms) / len(bwd_ms)
+    fwd_bytes = n_tok * (row_bytes + 8 + 24)       # logits + label + logprob, entropy, 4 row stats
+    bwd_bytes = n_tok * (2 * row_bytes + 8 + 24)   # read logits, write grad + label, 2 grads, 4 stats
+    bwd_gbs = bwd_bytes / (bwd_avg * 1e-3) / 1e9
+    fwd_gbs = fwd_bytes / (fwd_avg * 1e-3) / 1e9
+
+    out = {
+        "metric": METRIC,
+        "value": tok_s,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "BASELINE config 2: 16 sequences, lengths uniform in [512,3072], packed to one row; bf16 "
+                        "logits [T_total,151936] ~N(0,3), 1% of rows with one +15 spike, temperature 1.0; fused "
+                        "logprob+entropy forward and in-place backward, upstream grads ~N(0,1)",
+            "total_tokens": n_tok,
+            "vocab": VOCAB,
+            "logits_gb": n_tok * row_bytes / 1e9,
+            "entry": "openrlhf_amd.models.utils.logprobs_and_entropy_from_logits(inplace_backward=True)",
+        },
+        "achieved_hbm_gbs_fwd_bwd": (fwd_bytes + bwd_bytes) * args.steps / total / 1e9,
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "logprob_entropy_bwd_kernel<bf16, lp+entropy, T=1> (in place)",
+            "achieved": bwd_gbs,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": bwd_gbs / HBM_PEAK_GBS,
+            "traffic": measured_traffic("backward", n_tok),
+            "bytes_per_launch": bwd_bytes,
+            "avg_launch_ms": bwd_avg,
+            "other_kernels": {
+                "logprob_entropy_fwd_kernel<bf16, lp+entropy, T=1>": {
+                    "achieved": fwd_gbs, "frac": fwd_gbs / HBM_PEAK_GBS, "bytes_per_launch": fwd_bytes,
+                    "avg_launch_ms": fwd_avg,
+                }
+            },
+        },
+    }
+    if not args.no_cpu_baseline:
+        rows = min(args.cpu_rows, n_tok)
+        cpu_tok_s, cpu_s = cpu_baseline(pristine[:rows], labels[:rows], g_lp[:rows], g_ent[:rows])
+        out["cpu_baseline"] = {
+            "value": cpu_tok_s,
+            "unit": "tokens/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"first {rows} rows of the same workload at full V (bf16->fp32 up-cast, entropy, gather - "
+                      f"chunked logsumexp, autograd backward) on torch CPU, median of 3 runs of {cpu_s:.2f} s; "
+                      f"os.cpu_count()={os.cpu_count()}",
+        }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

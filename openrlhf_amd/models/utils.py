@@ -48,7 +48,9 @@ class _LogprobEntropy(torch.autograd.Function):
         dev = require_gpu(logits, labels if want_logprob else None)
         code = _lib.dtype_code(logits)
         batch_shape = logits.shape[:-1]
-        rows, row_stride = _as_rows(logits)
+        # a detached alias: shares storage and the version counter with `logits`, but is not a
+        # view autograd tracks, so handing it back as the (in-place) gradient is legal
+        rows, row_stride = _as_rows(logits.detach())
         n_rows, vocab = rows.shape
         if want_logprob:
             if labels.shape != batch_shape:
@@ -105,10 +107,10 @@ class _LogprobEntropy(torch.autograd.Function):
                 ptr(stats), stream_of(dev),
             )
         if grad_rows is rows:
-            # the logits storage now holds the gradient: bump the shared version counter (an
-            # in-place op on an empty view costs no launch) so that any later use of the saved
-            # logits by autograd raises instead of reading gradients as logits
-            rows.view(-1)[:0].zero_() if rows.is_contiguous() else rows[:0].zero_()
+            # the logits storage now holds the gradient: bump the shared version counter so that
+            # any later use of the saved logits by autograd raises instead of reading gradients
+            # as logits
+            torch.autograd.graph.increment_version(rows)
         grad = grad_rows if grad_rows.shape == ctx.logits_shape else grad_rows.view(ctx.logits_shape)
         return grad, None, None, None, None, None
 

@@ -1,0 +1,130 @@
+"""CPU-only checks: the shared library exports every symbol the public header declares, the
+ctypes binding covers them, argument validation returns error codes before anything touches a
+GPU, and the Python mirrors raise the reference's exception types. No kernel is launched."""
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "openrlhf_amd.h")
+
+
+def _declared():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(orlhf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_binding_and_library_agree(lib):
+    from openrlhf_amd import _lib
+
+    names = _declared()
+    assert len(names) >= 19
+    assert sorted(_lib.SIGNATURES) == names
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in the header but not exported"
+    assert lib.orlhf_version() == _lib.ABI_VERSION
+    src = open(HEADER).read()
+    assert f"#define ORLHF_ABI_VERSION {_lib.ABI_VERSION}" in src
+    # enum values of the binding match the header
+    for name, val in (("ORLHF_BF16", _lib.BF16), ("ORLHF_MASK_I64", _lib.MASK_I64), ("ORLHF_KL_K3", _lib.KL_K3),
+                      ("ORLHF_AGG_ROW_MEAN", _lib.AGG_ROW_MEAN), ("ORLHF_IS_SEQ_MASK_TIS", _lib.IS_SEQ_MASK_TIS),
+                      ("ORLHF_GROUP_NORM", _lib.GROUP_NORM), ("ORLHF_POLICY_GSPO", _lib.POLICY_GSPO)):
+        assert re.search(rf"{name} = {val}\b", src), name
+
+
+def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
+    from openrlhf_amd import _lib
+
+    def err():
+        return lib.orlhf_last_error().decode()
+
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 0, 0, None, 1.0, None, None, None, 0, None) == -1
+    assert "vocab" in err()
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 4, None, 1.0, None, None, None, 0, None) == -1
+    assert "row_stride" in err()
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 8, None, 1.0, None, None, None, 0, None) == -1
+    assert "both NULL" in err()
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 8, None, 0.0, 8, None, None, 0, None) == -1
+    assert "temperature" in err()
+    assert lib.orlhf_logprob_entropy_fwd(8, 9, 4, 8, 8, 8, 1.0, 8, None, None, 0, None) == -1
+    assert "dtype" in err()
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 0, 8, 8, None, 1.0, 8, None, None, 0, None) == 0  # empty: no launch
+    assert lib.orlhf_logprob_entropy_bwd(None, None, 1, 2, 8, 8, 8, None, 1.0, None, None, None, None) == -1
+    assert lib.orlhf_approx_kl_fwd(None, None, 0, 5, 7, None, None) == -1 and "estimator" in err()
+    assert lib.orlhf_approx_kl_fwd(None, None, 0, 0, 0, None, None) == 0
+    assert lib.orlhf_masked_aggregate_fwd(None, None, 9, 1, 1, None, 0, None, None, None, None, None) == -1
+    assert "mask dtype" in err()
+    p = _lib.PolicyParams()
+    p.policy_type = 5
+    assert lib.orlhf_policy_loss_fwd(None, None, None, None, 0, None, 0, 0, None, p, None, None, None, None, None) == -1
+    p.policy_type, p.dual_clip = 0, 0.5
+    assert lib.orlhf_policy_loss_fwd(None, None, None, None, 0, None, 0, 0, None, p, None, None, None, None, None) == -1
+    assert "dual_clip" in err()
+    p.dual_clip, p.is_correction = 0.0, 1
+    assert lib.orlhf_policy_loss_fwd(None, None, None, None, 0, None, 0, 0, None, p, None, None, None, None, None) == -1
+    assert "rollout" in err()
+    assert lib.orlhf_group_normalize(None, None, 3, 0, 0, None, None, None, None) == -1
+    assert lib.orlhf_group_normalize(None, None, 3, 2, 9, None, None, None, None) == -1
+    assert lib.orlhf_gae_scan(None, None, None, 0, -1, 4, None, 1.0, 1.0, None, None, None) == -1
+    assert lib.orlhf_token_workspace_bytes(4096, 16383) >= 4096 * 16 * 6 * 8
+    assert lib.orlhf_whiten_workspace_bytes(10) > 0
+
+
+def test_python_mirrors_raise_like_the_reference(lib):
+    from openrlhf_amd.models.loss import PolicyLoss, ValueLoss
+    from openrlhf_amd.models.utils import compute_approx_kl, log_probs_from_logits
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import group_normalize_rewards
+
+    x = torch.zeros(2, 3)
+    with pytest.raises(ValueError, match="Unknown kl_estimator"):
+        compute_approx_kl(x, x, "k5")
+    with pytest.raises(AssertionError):
+        PolicyLoss(dual_clip=0.9)
+    with pytest.raises(ValueError, match="Invalid vllm_is_correction_type"):
+        PolicyLoss(vllm_is_correction_type="bad")
+    with pytest.raises(ValueError, match="Invalid policy loss type"):
+        PolicyLoss(policy_loss_type="bad")(x, x, x)
+    assert PolicyLoss(policy_loss_type="gspo").token_level_loss is False
+    assert ValueLoss().clip_eps is None and ValueLoss(0.2).token_level_loss is True
+    with pytest.raises(Exception, match="Unkown advantage_estimator"):
+        group_normalize_rewards(torch.zeros(4), None, 2, "bad")
+    # no CPU fallback: CPU tensors are refused, loudly
+    with pytest.raises(RuntimeError, match="GPU only"):
+        log_probs_from_logits(torch.zeros(2, 8), torch.zeros(2, dtype=torch.long))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        PolicyLoss()(x, x, x, action_mask=x)
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    from openrlhf_amd import _lib
+
+    with pytest.raises(ImportError, match="not built"):
+        _lib.load(str(tmp_path / "nope.so"))
+
+
+def test_row_view_and_norm_plumbing():
+    from openrlhf_amd import _lib
+    from openrlhf_amd.models.utils import _as_rows, _rows_of
+
+    x = torch.zeros(2, 5, 16)
+    rows, stride = _as_rows(x)
+    assert rows.shape == (10, 16) and stride == 16 and rows.data_ptr() == x.data_ptr()
+    y = torch.zeros(6, 20)[:, :16]
+    rows, stride = _as_rows(y)
+    assert rows.shape == (6, 16) and stride == 20 and rows.data_ptr() == y.data_ptr()
+    z = torch.zeros(16, 6).t()
+    rows, stride = _as_rows(z)
+    assert rows.is_contiguous() and stride == 16
+    assert _rows_of(torch.zeros(3, 4, 7), None) == (12, 7)
+    assert _rows_of(torch.zeros(30), torch.tensor([0, 10, 30])) == (2, 30)
+    keep = []
+    n = _lib.make_norm(2, None, keep)
+    assert n.dp_size == 2.0 and n.norm_value != n.norm_value and not n.norm_dev
+    n = _lib.make_norm(1, torch.tensor(7.0), keep)
+    assert n.norm_value == 7.0 and not n.norm_dev
+    assert _lib.mask_arg(None)[2] == _lib.MASK_NONE
+    assert _lib.mask_arg(torch.ones(3, dtype=torch.bool))[2] == _lib.MASK_U8
+    assert _lib.mask_arg(torch.ones(3, dtype=torch.int32))[2] == _lib.MASK_F32
