@@ -11,6 +11,8 @@
 //     maximum, so the result never depends on the shortcut;
 //   * sums are kept in fp32 in 4 independent accumulators per lane, reduced over the wave with
 //     cross-lane shuffles and over the 4 waves through LDS; the per-row epilogue runs in fp64.
+#include <stdlib.h>
+
 #include "common.h"
 
 #ifndef ORLHF_ROW_UNROLL
@@ -567,7 +569,10 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_bwd_kernel(
 // ---------------------------------------------------------------- host side
 static int grid_for_rows(int64_t n_rows) {
   // one workgroup per row; cap the grid and stride over rows beyond it
-  const int64_t cap = 1 << 20;
+  int64_t cap = 1 << 20;
+#ifdef ORLHF_TUNING
+  if (const char* e = getenv("ORLHF_GRID_CAP")) cap = atoll(e);
+#endif
   return (int)(n_rows < cap ? n_rows : cap);
 }
 
