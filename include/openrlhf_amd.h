@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 1
+#define ORLHF_ABI_VERSION 2
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -85,11 +85,14 @@ const char* orlhf_last_error(void);
  *   logprob   float [n_rows] or NULL;  entropy float [n_rows] or NULL (not both NULL)
  *   row_stats float [n_rows, 4] or NULL: {lse(z), lse(x), E_softmax(x)[x], 0}, what the backward
  *             needs; fp32 accumulation and fp32 outputs for every input dtype
+ *   row_mask  uint8 [n_rows] or NULL: rows with 0 are not read; their outputs and statistics are
+ *             0. This is how the caller skips prompt and padding positions, whose log-probs
+ *             Actor.forward multiplies by 0 anyway (openrlhf/models/actor.py:294).
  */
 int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
                               int64_t row_stride, const int64_t* labels, double temperature,
-                              float* logprob, float* entropy, float* row_stats, int flags,
-                              orlhf_stream_t stream);
+                              float* logprob, float* entropy, float* row_stats,
+                              const uint8_t* row_mask, int flags, orlhf_stream_t stream);
 
 /*
  * Backward of the above in one streaming pass, written in the logits dtype:
@@ -98,13 +101,14 @@ int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows, int
  * `grad_logits` may alias `logits` (in-place: each 16-byte chunk is read, then overwritten by the
  * same lane). Replaces torch autograd through openrlhf/models/utils.py:139-163 and :182-186.
  * g_logprob / g_entropy: float [n_rows] or NULL (treated as 0). Rows whose upstream gradients
- * are both exactly 0 are written as zeros without reading their logits.
+ * are both exactly 0, and rows with row_mask 0 (same array as in the forward, or NULL), are
+ * written as zeros without reading their logits.
  */
 int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, int dtype, int64_t n_rows,
                               int64_t vocab, int64_t row_stride, int64_t grad_row_stride,
                               const int64_t* labels, double temperature, const float* g_logprob,
                               const float* g_entropy, const float* row_stats,
-                              orlhf_stream_t stream);
+                              const uint8_t* row_mask, orlhf_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Per-token kernels: KL, masked aggregation, PPO policy loss, value loss

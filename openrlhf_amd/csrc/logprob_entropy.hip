@@ -323,7 +323,8 @@ template <int DT, int MODE>
 __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
     const char* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
     const int64_t* __restrict__ labels, double temperature, float* __restrict__ logprob,
-    float* __restrict__ entropy, float* __restrict__ row_stats, int scalar_only) {
+    float* __restrict__ entropy, float* __restrict__ row_stats, const uint8_t* __restrict__ row_mask,
+    int scalar_only) {
   using E = Elt<DT>;
   using MT = ModeTraits<MODE>;
   __shared__ float lds[kWavesPerBlock][8];
@@ -335,6 +336,14 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
   const float c_scaled = (float)(1.4426950408889634 / temperature);
 
   for (int64_t row_i = blockIdx.x; row_i < n_rows; row_i += gridDim.x) {
+    if (row_mask != nullptr && row_mask[row_i] == 0) {  // row not wanted: outputs 0, logits not read
+      if (tid == 0) {
+        if (MODE != kEntOnly && logprob != nullptr) logprob[row_i] = 0.0f;
+        if (MT::kPlainSet && entropy != nullptr) entropy[row_i] = 0.0f;
+        if (row_stats != nullptr) *(f32x4*)(row_stats + row_i * 4) = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+      }
+      continue;
+    }
     const char* row = logits + row_i * row_stride_bytes;
     const RowGeom g = row_geom<DT>(row, vocab, scalar_only != 0);
 
@@ -536,7 +545,7 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_bwd_kernel(
     const char* logits, char* grad, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
     int64_t grad_stride_bytes, const int64_t* __restrict__ labels, double temperature,
     const float* __restrict__ g_logprob, const float* __restrict__ g_entropy,
-    const float* __restrict__ row_stats, int scalar_only) {
+    const float* __restrict__ row_stats, const uint8_t* __restrict__ row_mask, int scalar_only) {
   const double inv_t = 1.0 / temperature;
   for (int64_t row_i = blockIdx.x; row_i < n_rows; row_i += gridDim.x) {
     const char* row = logits + row_i * row_stride_bytes;
@@ -547,7 +556,8 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_bwd_kernel(
 
     const float glp = (MODE != kBwdEnt) ? g_logprob[row_i] : 0.0f;
     const float gh = (MODE != kBwdLp) ? g_entropy[row_i] : 0.0f;
-    if (glp == 0.0f && gh == 0.0f) {
+    const bool skipped = row_mask != nullptr && row_mask[row_i] == 0;  // forward gave constants
+    if (skipped || (glp == 0.0f && gh == 0.0f)) {
       zero_row<DT>(out_row, g);
       continue;
     }
@@ -579,7 +589,7 @@ static int grid_for_rows(int64_t n_rows) {
 template <int DT>
 static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
                       const int64_t* labels, double temperature, float* logprob, float* entropy,
-                      float* row_stats, hipStream_t stream) {
+                      float* row_stats, const uint8_t* row_mask, hipStream_t stream) {
   using E = Elt<DT>;
   const bool want_lp = logprob != nullptr;
   const bool want_ent = entropy != nullptr;
@@ -592,7 +602,7 @@ static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
 #define ORLHF_FWD(M)                                                                          \
   hipLaunchKernelGGL((logprob_entropy_fwd_kernel<DT, M>), grid, block, 0, stream, p, n_rows,  \
                      vocab, stride_bytes, labels, temperature, logprob, entropy, row_stats,   \
-                     scalar_only)
+                     row_mask, scalar_only)
   switch (mode) {
     case kLpOnly: ORLHF_FWD(kLpOnly); break;
     case kEntOnly: ORLHF_FWD(kEntOnly); break;
@@ -608,7 +618,7 @@ template <int DT>
 static int launch_bwd(const void* logits, void* grad, int64_t n_rows, int64_t vocab,
                       int64_t row_stride, int64_t grad_row_stride, const int64_t* labels,
                       double temperature, const float* g_logprob, const float* g_entropy,
-                      const float* row_stats, hipStream_t stream) {
+                      const float* row_stats, const uint8_t* row_mask, hipStream_t stream) {
   using E = Elt<DT>;
   const bool has_lp = g_logprob != nullptr;
   const bool has_ent = g_entropy != nullptr;
@@ -626,7 +636,7 @@ static int launch_bwd(const void* logits, void* grad, int64_t n_rows, int64_t vo
 #define ORLHF_BWD(M)                                                                          \
   hipLaunchKernelGGL((logprob_entropy_bwd_kernel<DT, M>), grid, block, 0, stream, p, gp,      \
                      n_rows, vocab, stride_bytes, gstride_bytes, labels, temperature,         \
-                     g_logprob, g_entropy, row_stats, scalar_only)
+                     g_logprob, g_entropy, row_stats, row_mask, scalar_only)
   switch (mode) {
     case kBwdLp: ORLHF_BWD(kBwdLp); break;
     case kBwdEnt: ORLHF_BWD(kBwdEnt); break;
@@ -645,7 +655,8 @@ using namespace orlhf;
 extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows,
                                          int64_t vocab, int64_t row_stride, const int64_t* labels,
                                          double temperature, float* logprob, float* entropy,
-                                         float* row_stats, int flags, orlhf_stream_t stream) {
+                                         float* row_stats, const uint8_t* row_mask, int flags,
+                                         orlhf_stream_t stream) {
   ORLHF_CHECK_ARG(n_rows >= 0 && vocab > 0, "logprob_entropy_fwd: n_rows=%lld vocab=%lld",
                   (long long)n_rows, (long long)vocab);
   ORLHF_CHECK_ARG(row_stride >= vocab, "logprob_entropy_fwd: row_stride %lld < vocab %lld",
@@ -665,15 +676,15 @@ extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t 
     case ORLHF_F32:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 3u) == 0, "logprob_entropy_fwd: logits not 4-byte aligned");
       return launch_fwd<ORLHF_F32>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                   entropy, row_stats, s);
+                                   entropy, row_stats, row_mask, s);
     case ORLHF_BF16:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 1u) == 0, "logprob_entropy_fwd: logits not 2-byte aligned");
       return launch_fwd<ORLHF_BF16>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                    entropy, row_stats, s);
+                                    entropy, row_stats, row_mask, s);
     case ORLHF_F16:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 1u) == 0, "logprob_entropy_fwd: logits not 2-byte aligned");
       return launch_fwd<ORLHF_F16>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                   entropy, row_stats, s);
+                                   entropy, row_stats, row_mask, s);
     default:
       return fail(ORLHF_ERR_INVALID_ARG, "logprob_entropy_fwd: unknown dtype %d", dtype);
   }
@@ -684,7 +695,7 @@ extern "C" int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, 
                                          int64_t grad_row_stride, const int64_t* labels,
                                          double temperature, const float* g_logprob,
                                          const float* g_entropy, const float* row_stats,
-                                         orlhf_stream_t stream) {
+                                         const uint8_t* row_mask, orlhf_stream_t stream) {
   ORLHF_CHECK_ARG(n_rows >= 0 && vocab > 0, "logprob_entropy_bwd: n_rows=%lld vocab=%lld",
                   (long long)n_rows, (long long)vocab);
   ORLHF_CHECK_ARG(row_stride >= vocab && grad_row_stride >= vocab,
@@ -707,13 +718,13 @@ extern "C" int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, 
   switch (dtype) {
     case ORLHF_F32:
       return launch_bwd<ORLHF_F32>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride,
-                                   labels, temperature, g_logprob, g_entropy, row_stats, s);
+                                   labels, temperature, g_logprob, g_entropy, row_stats, row_mask, s);
     case ORLHF_BF16:
       return launch_bwd<ORLHF_BF16>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride,
-                                    labels, temperature, g_logprob, g_entropy, row_stats, s);
+                                    labels, temperature, g_logprob, g_entropy, row_stats, row_mask, s);
     case ORLHF_F16:
       return launch_bwd<ORLHF_F16>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride,
-                                   labels, temperature, g_logprob, g_entropy, row_stats, s);
+                                   labels, temperature, g_logprob, g_entropy, row_stats, row_mask, s);
     default:
       return fail(ORLHF_ERR_INVALID_ARG, "logprob_entropy_bwd: unknown dtype %d", dtype);
   }

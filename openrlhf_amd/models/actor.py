@@ -1,0 +1,94 @@
+"""The numerics tail of ``Actor.forward`` as one fused call.
+
+Mirrors what openrlhf/models/actor.py:265-296 does after the model has produced logits:
+(fp32 up-cast,) entropy on the unscaled logits, log-prob of the next token on logits/T, re-pad
+of packed outputs with the unpadding indices (openrlhf/models/ring_attn_utils.py:129-140,181),
+drop of the last column, slice of the last A columns, multiplication by the action mask.
+
+Differences by construction: bf16 logits are consumed directly (no [N, V] fp32 copy), log-prob
+and entropy come from ONE pass over the logits, and with ``skip_masked=True`` (default) positions
+whose log-prob the reference multiplies by zero are not read at all, forward or backward; their
+entropy is returned as 0 (the trainer only ever aggregates entropy under the same mask,
+openrlhf/trainer/ray/ppo_actor.py:345-350).
+"""
+from typing import Optional, Tuple, Union
+
+import torch
+
+from .utils import logprobs_and_entropy_from_logits
+
+
+def unpad_indices(attention_mask: torch.Tensor) -> torch.Tensor:
+    """Flat positions of the attended tokens in row-major order: the ``indices`` flash-attn's
+    unpad_input returns (openrlhf/models/ring_attn_utils.py:130)."""
+    return torch.nonzero(attention_mask.reshape(-1), as_tuple=False).squeeze(-1)
+
+
+def actor_forward_tail(
+    logits: torch.Tensor,
+    sequences: torch.Tensor,
+    action_mask: Optional[torch.Tensor] = None,
+    attention_mask: Optional[torch.Tensor] = None,
+    temperature: float = 1.0,
+    packed_indices: Optional[torch.Tensor] = None,
+    return_entropy: bool = False,
+    inplace_backward: bool = False,
+    skip_masked: bool = True,
+) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
+    """Action log-probs ``[B, A]`` (or all ``[B, T-1]`` log-probs when ``action_mask`` is None)
+    from the model's logits, plus ``entropy[:, :-1]`` when ``return_entropy``.
+
+    logits: ``[B, T, V]`` (padded batch) or ``[1, Ttot, V]`` / ``[Ttot, V]`` with
+    ``packed_indices`` = the flat positions of the packed tokens in the ``[B, T]`` grid
+    (``unpad_indices(attention_mask)``). sequences: ``[B, T]`` token ids; labels are the sequences
+    rolled left by one per padded row, as in the reference.
+    """
+    batch, seqlen = sequences.shape
+    rolled = torch.roll(sequences, shifts=-1, dims=1)
+
+    # which (b, t) positions are needed: the last A of the first T-1 columns, under the action mask
+    need = torch.zeros(batch, seqlen, dtype=torch.bool, device=sequences.device)
+    if action_mask is not None:
+        width = action_mask.shape[1]
+        need[:, seqlen - 1 - width : seqlen - 1] = action_mask != 0
+    else:
+        need[:, : seqlen - 1] = True if attention_mask is None else attention_mask[:, : seqlen - 1] != 0
+    if not skip_masked:
+        need = None
+
+    if packed_indices is None:
+        labels = rolled
+        row_mask = need
+        lp, ent = logprobs_and_entropy_from_logits(
+            logits, labels, temperature, inplace_backward=inplace_backward, row_mask=row_mask
+        ) if return_entropy else (_lp_only(logits, labels, temperature, inplace_backward, row_mask), None)
+    else:
+        flat_logits = logits.reshape(-1, logits.shape[-1])
+        labels = rolled.reshape(-1)[packed_indices]
+        row_mask = None if need is None else need.reshape(-1)[packed_indices]
+        if return_entropy:
+            lp_p, ent_p = logprobs_and_entropy_from_logits(
+                flat_logits, labels, temperature, inplace_backward=inplace_backward, row_mask=row_mask
+            )
+        else:
+            lp_p, ent_p = _lp_only(flat_logits, labels, temperature, inplace_backward, row_mask), None
+
+        def repad(flat):
+            full = flat.new_zeros(batch * seqlen)
+            return full.index_copy(0, packed_indices, flat).view(batch, seqlen)
+
+        lp = repad(lp_p)
+        ent = None if ent_p is None else repad(ent_p)
+
+    lp = lp[:, :-1]
+    if action_mask is not None:
+        lp = lp[:, -action_mask.shape[1] :] * action_mask.float()
+    if return_entropy:
+        return lp, ent[:, :-1]
+    return lp
+
+
+def _lp_only(logits, labels, temperature, inplace_backward, row_mask):
+    from .utils import _LogprobEntropy
+
+    return _LogprobEntropy.apply(logits, labels, temperature, True, False, inplace_backward, row_mask)[0]

@@ -44,8 +44,8 @@ class _LogprobEntropy(torch.autograd.Function):
     """logits -> (log-prob of label, entropy), one vocabulary pass forward, one backward."""
 
     @staticmethod
-    def forward(ctx, logits, labels, temperature, want_logprob, want_entropy, inplace_backward):
-        dev = require_gpu(logits, labels if want_logprob else None)
+    def forward(ctx, logits, labels, temperature, want_logprob, want_entropy, inplace_backward, row_mask=None):
+        dev = require_gpu(logits, labels if want_logprob else None, row_mask)
         code = _lib.dtype_code(logits)
         batch_shape = logits.shape[:-1]
         # a detached alias: shares storage and the version counter with `logits`, but is not a
@@ -61,6 +61,12 @@ class _LogprobEntropy(torch.autograd.Function):
             lab = lab.contiguous()
         else:
             lab = None
+        if row_mask is not None:
+            if row_mask.shape != batch_shape:
+                raise ValueError(f"row_mask shape {tuple(row_mask.shape)} != logits batch shape {tuple(batch_shape)}")
+            rmask = (row_mask != 0).reshape(-1).to(torch.uint8).contiguous()
+        else:
+            rmask = None
         needs_grad = ctx.needs_input_grad[0]
         opts = dict(device=dev, dtype=torch.float32)
         logprob = torch.empty(n_rows, **opts) if want_logprob else None
@@ -69,7 +75,7 @@ class _LogprobEntropy(torch.autograd.Function):
         with torch.cuda.device(dev):
             call(
                 "orlhf_logprob_entropy_fwd", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
-                float(temperature), ptr(logprob), ptr(entropy), ptr(stats), 0, stream_of(dev),
+                float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), 0, stream_of(dev),
             )
         ctx.temperature = float(temperature)
         ctx.inplace = bool(inplace_backward)
@@ -80,16 +86,16 @@ class _LogprobEntropy(torch.autograd.Function):
         ctx.logits_shape = logits.shape
         ctx.set_materialize_grads(False)
         if needs_grad:
-            ctx.save_for_backward(rows, lab, stats)
+            ctx.save_for_backward(rows, lab, stats, rmask)
         out_lp = logprob.view(batch_shape) if want_logprob else None
         out_ent = entropy.view(batch_shape) if want_entropy else None
         return out_lp, out_ent
 
     @staticmethod
     def backward(ctx, g_logprob, g_entropy):
-        rows, lab, stats = ctx.saved_tensors
+        rows, lab, stats, rmask = ctx.saved_tensors
         if g_logprob is None and g_entropy is None:
-            return None, None, None, None, None, None
+            return None, None, None, None, None, None, None
         dev = rows.device
         n_rows, vocab = rows.shape
         code = _lib.dtype_code(rows)
@@ -104,7 +110,7 @@ class _LogprobEntropy(torch.autograd.Function):
             call(
                 "orlhf_logprob_entropy_bwd", ptr(rows), ptr(grad_rows), code, n_rows, vocab,
                 ctx.row_stride, grad_stride, ptr(lab), ctx.temperature, ptr(glp), ptr(gent),
-                ptr(stats), stream_of(dev),
+                ptr(stats), ptr(rmask), stream_of(dev),
             )
         if grad_rows is rows:
             # the logits storage now holds the gradient: bump the shared version counter so that
@@ -112,7 +118,7 @@ class _LogprobEntropy(torch.autograd.Function):
             # as logits
             torch.autograd.graph.increment_version(rows)
         grad = grad_rows if grad_rows.shape == ctx.logits_shape else grad_rows.view(ctx.logits_shape)
-        return grad, None, None, None, None, None
+        return grad, None, None, None, None, None, None
 
 
 def logprobs_and_entropy_from_logits(
@@ -120,6 +126,7 @@ def logprobs_and_entropy_from_logits(
     labels: torch.Tensor,
     temperature: float = 1.0,
     inplace_backward: bool = False,
+    row_mask: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """(log_probs_from_logits(logits, labels, temperature), compute_entropy(logits)) from one
     pass over the logits: the log-prob uses logits / temperature, the entropy the unscaled
@@ -127,8 +134,10 @@ def logprobs_and_entropy_from_logits(
 
     ``inplace_backward=True`` writes d(loss)/d(logits) over the logits storage in backward
     instead of allocating a second [N, V] tensor; the logits are unusable afterwards.
+    ``row_mask`` (same shape as ``labels``): positions with 0 are skipped, their outputs are 0
+    and their logits get zero gradient without being read (prompt and padding positions).
     """
-    return _LogprobEntropy.apply(logits, labels, temperature, True, True, inplace_backward)
+    return _LogprobEntropy.apply(logits, labels, temperature, True, True, inplace_backward, row_mask)
 
 
 def log_probs_from_logits(

@@ -41,18 +41,18 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     def err():
         return lib.orlhf_last_error().decode()
 
-    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 0, 0, None, 1.0, None, None, None, 0, None) == -1
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 0, 0, None, 1.0, None, None, None, None, 0, None) == -1
     assert "vocab" in err()
-    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 4, None, 1.0, None, None, None, 0, None) == -1
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 4, None, 1.0, None, None, None, None, 0, None) == -1
     assert "row_stride" in err()
-    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 8, None, 1.0, None, None, None, 0, None) == -1
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 8, None, 1.0, None, None, None, None, 0, None) == -1
     assert "both NULL" in err()
-    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 8, None, 0.0, 8, None, None, 0, None) == -1
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 4, 8, 8, None, 0.0, 8, None, None, None, 0, None) == -1
     assert "temperature" in err()
-    assert lib.orlhf_logprob_entropy_fwd(8, 9, 4, 8, 8, 8, 1.0, 8, None, None, 0, None) == -1
+    assert lib.orlhf_logprob_entropy_fwd(8, 9, 4, 8, 8, 8, 1.0, 8, None, None, None, 0, None) == -1
     assert "dtype" in err()
-    assert lib.orlhf_logprob_entropy_fwd(None, 0, 0, 8, 8, None, 1.0, 8, None, None, 0, None) == 0  # empty: no launch
-    assert lib.orlhf_logprob_entropy_bwd(None, None, 1, 2, 8, 8, 8, None, 1.0, None, None, None, None) == -1
+    assert lib.orlhf_logprob_entropy_fwd(None, 0, 0, 8, 8, None, 1.0, 8, None, None, None, 0, None) == 0  # empty: no launch
+    assert lib.orlhf_logprob_entropy_bwd(None, None, 1, 2, 8, 8, 8, None, 1.0, None, None, None, None, None) == -1
     assert lib.orlhf_approx_kl_fwd(None, None, 0, 5, 7, None, None) == -1 and "estimator" in err()
     assert lib.orlhf_approx_kl_fwd(None, None, 0, 0, 0, None, None) == 0
     assert lib.orlhf_masked_aggregate_fwd(None, None, 9, 1, 1, None, 0, None, None, None, None, None) == -1
