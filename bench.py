@@ -3,17 +3,25 @@ logits at V = 151936 (BASELINE config 2), one GPU.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
-One step = one forward and one backward of ``logprobs_and_entropy_from_logits`` over the whole
-packed batch (16 sequences, lengths uniform in [512, 3072], ~28.7 K tokens, 8.7 GB of logits),
-called through the public Python API, i.e. through the C ABI into the HIP kernels. The backward
-overwrites the logits with their gradient, so every step gets logits nobody has touched: a ring
-of buffers is refilled from a pristine copy between timed segments (the refill is outside the
-timed segments; each segment is bracketed by torch.cuda.synchronize()).
+One step = log-prob + entropy forward AND backward over the whole packed batch (16 sequences,
+lengths uniform in [512, 3072], ~30 K tokens, ~9 GB of logits) with the upstream gradients of
+the config given, called through the public Python API, i.e. through the C ABI into the HIP
+kernels. The gradient overwrites the logits, so every step gets logits nobody has touched: a
+ring of buffers is refilled from a pristine copy between timed segments (the refill is outside
+the timed segments; each segment is bracketed by torch.cuda.synchronize()).
 
-Prints ONE JSON line. `value` = tokens/s over the timed steps with inputs resident in HBM;
-`roofline` prices the dominant kernel (the backward: it moves 2/3 of the bytes) against the
-published 8 TB/s, from HIP-event durations taken on the launch stream inside the timed steps;
-`cpu_baseline` is the CPU oracle (the reference's op sequence on torch CPU) on a row sample.
+Two ways of doing the step are timed back to back on the same data, K steps each:
+  * `fused_one_pass` (reported as `value`): ``fused_logprob_entropy_fwd_bwd``, one kernel that
+    reads every row once, keeps it in the registers of a CU and writes the gradient once;
+  * `autograd_two_kernels`: ``logprobs_and_entropy_from_logits`` forward, then
+    ``torch.autograd.grad`` running the in-place backward kernel (the reference's call pattern).
+Both produce logprob, entropy and d/d(logits); the tests check them against the same oracle.
+
+Prints ONE JSON line. `value` = tokens/s with inputs resident in HBM; `roofline` prices the
+dominant kernel against the published 8 TB/s with the algorithmic bytes of forward+backward
+(3 x V x 2 bytes per token: read for the forward, read and write for the backward), from
+HIP-event durations on the launch stream inside the timed steps; `traffic` is what the kernel
+really moves (rocprofv3 counters); `cpu_baseline` is the CPU oracle on a row sample.
 """
 import argparse
 import json
@@ -120,7 +128,7 @@ def main():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
 
     _ensure_built()
-    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
@@ -130,9 +138,9 @@ def main():
     ring = max(1, min(args.ring, args.steps + args.warmup))
     bufs = [torch.empty_like(pristine) for _ in range(ring)]
 
-    fwd_ms, bwd_ms = [], []
+    fwd_ms, bwd_ms, fused_ms = [], [], []
 
-    def step(buf, timed):
+    def step_two_kernels(buf, timed):
         x = buf.requires_grad_(True)
         if timed:
             e0, e1, e2 = (torch.cuda.Event(enable_timing=True) for _ in range(3))
@@ -149,7 +157,18 @@ def main():
             return e0, e1, e2
         return None
 
-    def run_segment(count, timed):
+    def step_fused(buf, timed):
+        if timed:
+            e0, e1 = (torch.cuda.Event(enable_timing=True) for _ in range(2))
+            e0.record()
+        lp, ent, grad = fused_logprob_entropy_fwd_bwd(buf, labels, g_lp, g_ent, 1.0, inplace=True)
+        assert grad.data_ptr() == buf.data_ptr()
+        if timed:
+            e1.record()
+            return e0, e1
+        return None
+
+    def run_segment(step, count, timed):
         for b in bufs[:count]:
             b.detach_().copy_(pristine)  # fresh logits; outside the timed segment
         torch.cuda.synchronize()
@@ -158,30 +177,44 @@ def main():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         if timed:
-            for e0, e1, e2 in evs:
-                fwd_ms.append(e0.elapsed_time(e1))
-                bwd_ms.append(e1.elapsed_time(e2))
+            for ev in evs:
+                if len(ev) == 3:
+                    fwd_ms.append(ev[0].elapsed_time(ev[1]))
+                    bwd_ms.append(ev[1].elapsed_time(ev[2]))
+                else:
+                    fused_ms.append(ev[0].elapsed_time(ev[1]))
         return dt
 
-    left = args.warmup
-    while left > 0:
-        c = min(left, ring)
-        run_segment(c, False)
-        left -= c
-    total, left = 0.0, args.steps
-    while left > 0:
-        c = min(left, ring)
-        total += run_segment(c, True)
-        left -= c
+    def run(step):
+        left = args.warmup
+        while left > 0:
+            c = min(left, ring)
+            run_segment(step, c, False)
+            left -= c
+        total, left = 0.0, args.steps
+        while left > 0:
+            c = min(left, ring)
+            total += run_segment(step, c, True)
+            left -= c
+        return total
+
+    total_two = run(step_two_kernels)
+    total = run(step_fused)
 
     ms_per_step = total / args.steps * 1e3
     tok_s = n_tok * args.steps / total
     fwd_avg = sum(fwd_ms) / len(fwd_ms)
     bwd_avg = sum(bwd_ms) / len(bwd_ms)
-    fwd_bytes = n_tok * (row_bytes + 8 + 24)       # logits + label + logprob, entropy, 4 row stats
-    bwd_bytes = n_tok * (2 * row_bytes + 8 + 24)   # read logits, write grad + label, 2 grads, 4 stats
+    fused_avg = sum(fused_ms) / len(fused_ms)
+    small = 8 + 24                                  # label + logprob, entropy, 2 upstream grads / 4 row stats
+    fwd_bytes = n_tok * (row_bytes + small)         # read logits
+    bwd_bytes = n_tok * (2 * row_bytes + small)     # read logits, write grad
+    step_bytes = n_tok * (3 * row_bytes + 2 * small)  # forward + backward, algorithmic
+    fused_moved = n_tok * (2 * row_bytes + small)   # what the one-pass kernel has to move
     bwd_gbs = bwd_bytes / (bwd_avg * 1e-3) / 1e9
     fwd_gbs = fwd_bytes / (fwd_avg * 1e-3) / 1e9
+    fused_gbs = step_bytes / (fused_avg * 1e-3) / 1e9
+    traffic = measured_traffic("fused", n_tok)
 
     out = {
         "metric": METRIC,
@@ -198,29 +231,44 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": "BASELINE config 2: 16 sequences, lengths uniform in [512,3072], packed to one row; bf16 "
-                        "logits [T_total,151936] ~N(0,3), 1% of rows with one +15 spike, temperature 1.0; fused "
+                        "logits [T_total,151936] ~N(0,3), 1% of rows with one +15 spike, temperature 1.0; "
                         "logprob+entropy forward and in-place backward, upstream grads ~N(0,1)",
             "total_tokens": n_tok,
             "vocab": VOCAB,
             "logits_gb": n_tok * row_bytes / 1e9,
-            "entry": "openrlhf_amd.models.utils.logprobs_and_entropy_from_logits(inplace_backward=True)",
+            "entry": "openrlhf_amd.models.utils.fused_logprob_entropy_fwd_bwd(inplace=True)",
         },
-        "achieved_hbm_gbs_fwd_bwd": (fwd_bytes + bwd_bytes) * args.steps / total / 1e9,
         "roofline": {
             "bound": "hbm",
-            "kernel": "logprob_entropy_bwd_kernel<bf16, lp+entropy, T=1> (in place)",
-            "achieved": bwd_gbs,
+            "kernel": "logprob_entropy_fused_pipe_kernel<bf16, lp+entropy, T=1> (forward+backward in one pass, in place)",
+            "achieved": fused_gbs,
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
-            "frac": bwd_gbs / HBM_PEAK_GBS,
-            "traffic": measured_traffic("backward", n_tok),
-            "bytes_per_launch": bwd_bytes,
-            "avg_launch_ms": bwd_avg,
-            "other_kernels": {
+            "frac": fused_gbs / HBM_PEAK_GBS,
+            "traffic": traffic,
+            "bytes_per_launch": step_bytes,
+            "avg_launch_ms": fused_avg,
+            "note": "achieved = algorithmic bytes of forward+backward (3*V*2 B per token, read-read-write) / launch "
+                    "time; the kernel keeps each row on chip and really moves 2*V*2 B per token, see moved_*",
+            "moved_bytes_per_launch": fused_moved,
+            "moved_gbs": fused_moved / (fused_avg * 1e-3) / 1e9,
+            "moved_frac_of_peak": fused_moved / (fused_avg * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        },
+        "autograd_two_kernels": {
+            "entry": "logprobs_and_entropy_from_logits(inplace_backward=True) + torch.autograd.grad",
+            "value": n_tok * args.steps / total_two,
+            "unit": "tokens/s",
+            "ms_per_step": total_two / args.steps * 1e3,
+            "achieved_hbm_gbs": (fwd_bytes + bwd_bytes) * args.steps / total_two / 1e9,
+            "kernels": {
+                "logprob_entropy_bwd_kernel<bf16, lp+entropy, T=1> (in place)": {
+                    "achieved": bwd_gbs, "frac": bwd_gbs / HBM_PEAK_GBS, "bytes_per_launch": bwd_bytes,
+                    "avg_launch_ms": bwd_avg, "traffic": measured_traffic("backward", n_tok),
+                },
                 "logprob_entropy_fwd_kernel<bf16, lp+entropy, T=1>": {
                     "achieved": fwd_gbs, "frac": fwd_gbs / HBM_PEAK_GBS, "bytes_per_launch": fwd_bytes,
-                    "avg_launch_ms": fwd_avg,
-                }
+                    "avg_launch_ms": fwd_avg, "traffic": measured_traffic("forward", n_tok),
+                },
             },
         },
     }

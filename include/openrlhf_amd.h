@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 2
+#define ORLHF_ABI_VERSION 3
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -109,6 +109,27 @@ int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, int dtype, 
                               const int64_t* labels, double temperature, const float* g_logprob,
                               const float* g_entropy, const float* row_stats,
                               const uint8_t* row_mask, orlhf_stream_t stream);
+
+/*
+ * Forward and backward in ONE pass for callers that know the upstream weights when the forward
+ * runs, i.e. whose loss is sum_i w_logprob[i]*logprob[i] + w_entropy[i]*entropy[i] (SFT:
+ * w_logprob = -mask/N, openrlhf/models/loss.py:104): computes logprob / entropy exactly as
+ * orlhf_logprob_entropy_fwd and writes d(loss)/d(logits) exactly as orlhf_logprob_entropy_bwd
+ * with g = w, but reads every logits row once (the row stays in the registers / LDS of one CU),
+ * so a token costs 2*V*sizeof(dtype) bytes of HBM traffic instead of 3*V*sizeof(dtype).
+ * Replaces the same reference lines as the two calls above (openrlhf/models/utils.py:129-163,
+ * 182-186 and their autograd). grad_logits may alias logits. w_* / logprob / entropy nullable
+ * (a NULL weight array is all zeros). Returns ORLHF_ERR_UNSUPPORTED when a row does not fit on
+ * chip (vocab > orlhf_logprob_entropy_fwd_bwd_max_vocab(dtype): 155648 for bf16/fp16, 77824 for
+ * fp32) or when logits and grad rows differ in their 16-byte phase; callers then use the two
+ * separate entry points.
+ */
+int64_t orlhf_logprob_entropy_fwd_bwd_max_vocab(int dtype);
+int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logits, int dtype, int64_t n_rows,
+                                  int64_t vocab, int64_t row_stride, int64_t grad_row_stride,
+                                  const int64_t* labels, double temperature, const float* w_logprob,
+                                  const float* w_entropy, float* logprob, float* entropy,
+                                  const uint8_t* row_mask, orlhf_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Per-token kernels: KL, masked aggregation, PPO policy loss, value loss

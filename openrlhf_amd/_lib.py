@@ -21,7 +21,7 @@ POLICY_PPO, POLICY_GSPO = 0, 1
 IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 
 class Norm(Structure):
@@ -51,6 +51,8 @@ SIGNATURES = {
     "orlhf_last_error": (c_char_p, []),
     "orlhf_logprob_entropy_fwd": (c_int, [P, c_int, I64, I64, I64, P, c_double, P, P, P, P, c_int, P]),
     "orlhf_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P]),
+    "orlhf_logprob_entropy_fwd_bwd_max_vocab": (I64, [c_int]),
+    "orlhf_logprob_entropy_fwd_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P, P]),
     "orlhf_approx_kl_fwd": (c_int, [P, P, c_int, I64, c_int, P, P]),
     "orlhf_approx_kl_bwd": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
     "orlhf_token_workspace_bytes": (I64, [I64, I64]),

@@ -31,13 +31,14 @@ _KL_CODES = {"k1": _lib.KL_K1, "k2": _lib.KL_K2, "k3": _lib.KL_K3}
 
 # ------------------------------------------------------------------ vocabulary rows
 def _as_rows(logits: torch.Tensor):
-    """[..., V] -> (2-D tensor sharing storage when the layout allows, row stride in elements)."""
+    """[..., V] -> (2-D tensor, row stride in elements, whether it aliases the input's storage:
+    it does unless the layout forces a contiguous copy)."""
     vocab = logits.shape[-1]
     if logits.is_contiguous():
-        return logits.view(-1, vocab), vocab
+        return logits.view(-1, vocab), vocab, True
     if logits.dim() == 2 and logits.stride(1) == 1 and logits.stride(0) >= vocab:
-        return logits, logits.stride(0)
-    return logits.contiguous().view(-1, vocab), vocab
+        return logits, logits.stride(0), True
+    return logits.contiguous().view(-1, vocab), vocab, False
 
 
 class _LogprobEntropy(torch.autograd.Function):
@@ -50,7 +51,7 @@ class _LogprobEntropy(torch.autograd.Function):
         batch_shape = logits.shape[:-1]
         # a detached alias: shares storage and the version counter with `logits`, but is not a
         # view autograd tracks, so handing it back as the (in-place) gradient is legal
-        rows, row_stride = _as_rows(logits.detach())
+        rows, row_stride, aliases = _as_rows(logits.detach())
         n_rows, vocab = rows.shape
         if want_logprob:
             if labels.shape != batch_shape:
@@ -80,9 +81,7 @@ class _LogprobEntropy(torch.autograd.Function):
         ctx.temperature = float(temperature)
         ctx.inplace = bool(inplace_backward)
         ctx.row_stride = row_stride
-        ctx.shares_storage = rows.data_ptr() == logits.data_ptr() and (
-            logits.is_contiguous() or rows is logits
-        )
+        ctx.shares_storage = aliases
         ctx.logits_shape = logits.shape
         ctx.set_materialize_grads(False)
         if needs_grad:
@@ -317,3 +316,69 @@ def compute_reward(
         call("orlhf_compute_reward", ptr(rf), float(kl_coef), ptr(klf), mptr, mcode, n_rows, n_cols, ptr(cu),
              1 if reward_clip_range else 0, float(lo), float(hi), ptr(out), None, stream_of(dev))
     return out
+
+
+# ------------------------------------------------------------------ one-pass forward + backward
+@torch.no_grad()
+def fused_logprob_entropy_fwd_bwd(
+    logits: torch.Tensor,
+    labels: torch.Tensor,
+    w_logprob: Optional[torch.Tensor] = None,
+    w_entropy: Optional[torch.Tensor] = None,
+    temperature: float = 1.0,
+    inplace: bool = True,
+    row_mask: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Forward and backward of ``logprobs_and_entropy_from_logits`` in one pass over the logits
+    for a loss that is linear in the outputs: ``loss = sum(w_logprob * logprob) + sum(w_entropy *
+    entropy)`` with weights known up front (SFT: ``w_logprob = -mask / n_tokens``). Returns
+    ``(logprob, entropy, d loss / d logits)``; with ``inplace=True`` the gradient overwrites the
+    logits storage. Every row is read once and written once (2 x V x itemsize bytes per token
+    instead of 3 x); rows that do not fit on one CU take the separate forward and backward
+    kernels, with the same results. Not an autograd function: the gradient is returned."""
+    dev = require_gpu(logits, labels, w_logprob, w_entropy, row_mask)
+    code = _lib.dtype_code(logits)
+    batch_shape = logits.shape[:-1]
+    rows, row_stride, shares = _as_rows(logits.detach())
+    n_rows, vocab = rows.shape
+    if labels.shape != batch_shape:
+        raise ValueError(f"labels shape {tuple(labels.shape)} != logits batch shape {tuple(batch_shape)}")
+    lab = labels.reshape(-1).to(torch.int64).contiguous()
+
+    def flat(t, name):
+        if t is None:
+            return None
+        if t.shape != batch_shape:
+            raise ValueError(f"{name} shape {tuple(t.shape)} != logits batch shape {tuple(batch_shape)}")
+        return t.reshape(-1).to(torch.float32).contiguous()
+
+    wlp, went = flat(w_logprob, "w_logprob"), flat(w_entropy, "w_entropy")
+    rmask = None if row_mask is None else (row_mask != 0).reshape(-1).to(torch.uint8).contiguous()
+    opts = dict(device=dev, dtype=torch.float32)
+    logprob, entropy = torch.empty(n_rows, **opts), torch.empty(n_rows, **opts)
+    if inplace and shares:
+        grad_rows, grad_stride = rows, row_stride
+    else:
+        grad_rows, grad_stride = torch.empty((n_rows, vocab), device=dev, dtype=rows.dtype), vocab
+    lib = _lib.load()
+    fits = vocab <= lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(code)
+    same_phase = ((rows.data_ptr() ^ grad_rows.data_ptr()) & 15) == 0 and (
+        ((row_stride - grad_stride) * rows.element_size()) & 15
+    ) == 0
+    with torch.cuda.device(dev):
+        if fits and same_phase:
+            call("orlhf_logprob_entropy_fwd_bwd", ptr(rows), ptr(grad_rows), code, n_rows, vocab, row_stride,
+                 grad_stride, ptr(lab), float(temperature), ptr(wlp), ptr(went), ptr(logprob), ptr(entropy),
+                 ptr(rmask), stream_of(dev))
+        else:
+            stats = torch.empty(n_rows, 4, **opts)
+            zeros = torch.zeros(n_rows, **opts)
+            call("orlhf_logprob_entropy_fwd", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
+                 float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), 0, stream_of(dev))
+            call("orlhf_logprob_entropy_bwd", ptr(rows), ptr(grad_rows), code, n_rows, vocab, row_stride,
+                 grad_stride, ptr(lab), float(temperature), ptr(wlp if wlp is not None else zeros),
+                 ptr(went if went is not None else zeros), ptr(stats), ptr(rmask), stream_of(dev))
+    if grad_rows is rows:
+        torch.autograd.graph.increment_version(rows)
+    grad = grad_rows if grad_rows.shape == logits.shape else grad_rows.view(logits.shape)
+    return logprob.view(batch_shape), entropy.view(batch_shape), grad

@@ -110,14 +110,14 @@ def test_row_view_and_norm_plumbing():
     from openrlhf_amd.models.utils import _as_rows, _rows_of
 
     x = torch.zeros(2, 5, 16)
-    rows, stride = _as_rows(x)
-    assert rows.shape == (10, 16) and stride == 16 and rows.data_ptr() == x.data_ptr()
+    rows, stride, aliases = _as_rows(x)
+    assert rows.shape == (10, 16) and stride == 16 and rows.data_ptr() == x.data_ptr() and aliases
     y = torch.zeros(6, 20)[:, :16]
-    rows, stride = _as_rows(y)
-    assert rows.shape == (6, 16) and stride == 20 and rows.data_ptr() == y.data_ptr()
+    rows, stride, aliases = _as_rows(y)
+    assert rows.shape == (6, 16) and stride == 20 and rows.data_ptr() == y.data_ptr() and aliases
     z = torch.zeros(16, 6).t()
-    rows, stride = _as_rows(z)
-    assert rows.is_contiguous() and stride == 16
+    rows, stride, aliases = _as_rows(z)
+    assert rows.is_contiguous() and stride == 16 and not aliases
     assert _rows_of(torch.zeros(3, 4, 7), None) == (12, 7)
     assert _rows_of(torch.zeros(30), torch.tensor([0, 10, 30])) == (2, 30)
     keep = []

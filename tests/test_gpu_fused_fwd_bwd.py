@@ -1,0 +1,97 @@
+"""The one-pass forward+backward kernel against the fp64 oracle and against the separate
+forward and backward kernels (same tolerances: 1e-5 abs for fp32 logits, 2e-3 abs for bf16/fp16;
+gradients within the rounding of the logits dtype)."""
+import pytest
+import torch
+
+from oracle import token_numerics as otn
+
+pytestmark = pytest.mark.gpu
+
+
+def _case(rows, vocab, dtype, std, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = (torch.randn(rows, vocab, generator=g) * std)
+    r = torch.randperm(rows, generator=g)[: max(1, rows // 10)]
+    x[r, torch.randint(0, vocab, (len(r),), generator=g)] += 15.0
+    x = x.to(dtype)
+    labels = torch.randint(0, vocab, (rows,), generator=g)
+    w_lp, w_ent = torch.randn(rows, generator=g), torch.randn(rows, generator=g)
+    w_lp[0] = 0.0
+    w_ent[0] = 0.0
+    return x, labels, w_lp, w_ent
+
+
+def _analytic_grad64(x, labels, temperature, g_lp, g_ent):
+    x64 = x.double()
+    p_t = torch.softmax(x64 / temperature, -1)
+    p = torch.softmax(x64, -1)
+    onehot = torch.zeros_like(x64).scatter_(1, labels.unsqueeze(1), 1.0)
+    ex = (p * x64).sum(-1, keepdim=True)
+    return g_lp.double()[:, None] * (onehot - p_t) / temperature + g_ent.double()[:, None] * p * (ex - x64)
+
+
+@pytest.mark.parametrize(
+    "rows,vocab,dtype,std,temperature",
+    [
+        (40, 151936, torch.bfloat16, 3.0, 1.0),   # config-2 row: registers only
+        (12, 262144, torch.bfloat16, 4.0, 0.6),   # config-5 row: registers + LDS, two statistic sets
+        (12, 200000, torch.float16, 2.0, 1.0),    # LDS path, fp16
+        (33, 32000, torch.float32, 2.0, 1.0),
+        (33, 50257, torch.bfloat16, 3.0, 0.7),    # scalar tail
+        (17, 100003, torch.float32, 2.0, 1.3),    # fp32 LDS path, odd vocabulary
+        (300, 7, torch.float32, 1.0, 1.0),
+        (64, 4096, torch.bfloat16, 2.0, 1.0),
+        (5, 400000, torch.bfloat16, 2.0, 1.0),    # does not fit on chip: separate kernels
+    ],
+)
+@pytest.mark.parametrize("inplace", [True, False])
+def test_fused_matches_oracle_and_two_kernel_path(cuda, rows, vocab, dtype, std, temperature, inplace):
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
+
+    x, labels, w_lp, w_ent = _case(rows, vocab, dtype, std, seed=rows + vocab)
+    ref_lp = otn.log_probs_from_logits(x.double(), labels, temperature)
+    ref_ent = otn.compute_entropy(x.double())
+    ref_grad = _analytic_grad64(x, labels, temperature, w_lp, w_ent)
+
+    xd = x.to(cuda)
+    lp2, ent2 = logprobs_and_entropy_from_logits(xd, labels.to(cuda), temperature)
+    lp, ent, grad = fused_logprob_entropy_fwd_bwd(xd, labels.to(cuda), w_lp.to(cuda), w_ent.to(cuda), temperature,
+                                                  inplace=inplace)
+    assert (grad.data_ptr() == xd.data_ptr()) == inplace and grad.dtype == dtype and grad.shape == x.shape
+    atol = 1e-5 if dtype == torch.float32 else 2e-3
+    assert (lp.cpu().double() - ref_lp).abs().max().item() <= atol
+    assert (ent.cpu().double() - ref_ent).abs().max().item() <= atol
+    assert (lp - lp2).abs().max().item() <= 2e-5 and (ent - ent2).abs().max().item() <= 2e-5
+    err = (grad.cpu().double() - ref_grad).abs()
+    if dtype == torch.float32:  # 1e-5 relative to the gradient scale (entries reach |w| * |x| ~ 20 here)
+        assert err.max().item() <= 1e-5 * max(1.0, ref_grad.abs().max().item())
+    else:
+        eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        assert (err <= eps * ref_grad.abs() + 1e-6).all(), err.max().item()
+    assert grad[0].abs().max().item() == 0.0
+
+
+def test_fused_misaligned_rows_row_mask_and_optional_weights(cuda):
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd
+
+    rows, vocab, stride = 10, 4099, 4099 + 5
+    g = torch.Generator().manual_seed(3)
+    base = (torch.randn(rows * stride + 3, generator=g) * 2).to(torch.bfloat16)
+    labels = torch.randint(0, vocab, (rows,), generator=g)
+    w_lp = torch.randn(rows, generator=g)
+    mask = torch.ones(rows, dtype=torch.bool)
+    mask[3] = False
+    for off in (0, 1, 3):
+        x = base[off : off + rows * stride].view(rows, stride)[:, :vocab]
+        xd = base.to(cuda)[off : off + rows * stride].view(rows, stride)[:, :vocab]
+        lp, ent, grad = fused_logprob_entropy_fwd_bwd(xd, labels.to(cuda), w_lp.to(cuda), None, 1.0, inplace=True,
+                                                      row_mask=mask.to(cuda))
+        assert grad.data_ptr() == xd.data_ptr()
+        ref_lp = otn.log_probs_from_logits(x.contiguous().double(), labels)
+        ref = _analytic_grad64(x.contiguous(), labels, 1.0, w_lp, torch.zeros(rows))
+        keep = mask
+        assert (lp.cpu().double() - ref_lp)[keep].abs().max().item() <= 2e-3
+        assert lp[3].item() == 0.0 and ent[3].item() == 0.0 and grad[3].abs().max().item() == 0.0
+        err = (grad.cpu().double() - ref)[keep].abs()
+        assert (err <= 2.0 ** -8 * ref[keep].abs() + 1e-6).all()
