@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 3
+#define ORLHF_ABI_VERSION 4
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -130,6 +130,52 @@ int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logits, int dty
                                   const int64_t* labels, double temperature, const float* w_logprob,
                                   const float* w_entropy, float* logprob, float* entropy,
                                   const uint8_t* row_mask, orlhf_stream_t stream);
+
+/*
+ * The loss assembly of the PPO actor step (openrlhf/trainer/ray/ppo_actor.py:305-352) folded into
+ * the one-pass kernel: for every logits row the kernel computes logprob and entropy, evaluates
+ *   loss = sum_i policy_coef[i] * L_ppo(lp_i; old_i, adv_i [, rollout_i])       (loss.py:166-218)
+ *        + kl_coef * sum_i token_coef[i] * KL_est(lp_i - base_i)                (utils.py:78-95)
+ *        - entropy_coef * sum_i token_coef[i] * entropy_i
+ * 's derivative wrt logprob_i and entropy_i on the spot, and writes d(loss)/d(logits), all with
+ * one read and one write of the logits. All arrays are float [n_rows], aligned with the logits
+ * rows. policy_coef / token_coef are the aggregation weights (row_coef of
+ * orlhf_masked_aggregate_fwd times the mask, times any loss scale); rows where both are 0 get a
+ * zero gradient. Token-level importance corrections only (TIS, ICEPOP); GSPO and seq-mask-TIS need
+ * a sequence-level ratio before any token can be differentiated and are not fusable. The loss
+ * VALUES are obtained afterwards from the returned per-token logprob / entropy with
+ * orlhf_policy_loss_fwd, orlhf_approx_kl_fwd and orlhf_masked_aggregate_fwd (17 B/token).
+ */
+typedef struct orlhf_step_terms {
+  const float* old_log_probs;
+  const float* advantages;
+  const float* rollout_log_probs; /* NULL unless is_correction != NONE */
+  const float* base_log_probs;    /* NULL: no KL term */
+  const float* policy_coef;
+  const float* token_coef;
+  float clip_eps_low, clip_eps_high;
+  float dual_clip;                /* <= 0: off */
+  int is_correction;              /* ORLHF_IS_NONE / _TIS / _ICEPOP */
+  float is_low, is_high;
+  int kl_estimator;               /* orlhf_kl_estimator */
+  float kl_coef;
+  float entropy_coef;
+} orlhf_step_terms;
+
+int orlhf_policy_step_fwd_bwd(const void* logits, void* grad_logits, int dtype, int64_t n_rows,
+                              int64_t vocab, int64_t row_stride, int64_t grad_row_stride,
+                              const int64_t* labels, double temperature, const orlhf_step_terms* terms,
+                              float* logprob, float* entropy, const uint8_t* row_mask,
+                              orlhf_stream_t stream);
+
+/*
+ * data[i] *= g[0] / expected, skipped entirely (every workgroup returns at once) when the ratio
+ * is 1: lets an autograd backward hand out a gradient that was produced ahead of time with the
+ * scale `expected` and still be correct if the upstream gradient turns out different, without a
+ * host synchronisation. No reference counterpart.
+ */
+int orlhf_rescale_inplace_if(void* data, int dtype, int64_t n, const float* g, float expected,
+                             orlhf_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Per-token kernels: KL, masked aggregation, PPO policy loss, value loss

@@ -21,7 +21,7 @@ POLICY_PPO, POLICY_GSPO = 0, 1
 IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 
 class Norm(Structure):
@@ -42,6 +42,26 @@ class PolicyParams(Structure):
     ]
 
 
+class StepTerms(Structure):
+    _fields_ = [
+        ("old_log_probs", c_void_p),
+        ("advantages", c_void_p),
+        ("rollout_log_probs", c_void_p),
+        ("base_log_probs", c_void_p),
+        ("policy_coef", c_void_p),
+        ("token_coef", c_void_p),
+        ("clip_eps_low", c_float),
+        ("clip_eps_high", c_float),
+        ("dual_clip", c_float),
+        ("is_correction", c_int),
+        ("is_low", c_float),
+        ("is_high", c_float),
+        ("kl_estimator", c_int),
+        ("kl_coef", c_float),
+        ("entropy_coef", c_float),
+    ]
+
+
 P = c_void_p
 I64 = c_int64
 
@@ -53,6 +73,8 @@ SIGNATURES = {
     "orlhf_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P]),
     "orlhf_logprob_entropy_fwd_bwd_max_vocab": (I64, [c_int]),
     "orlhf_logprob_entropy_fwd_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P, P]),
+    "orlhf_policy_step_fwd_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, POINTER(StepTerms), P, P, P, P]),
+    "orlhf_rescale_inplace_if": (c_int, [P, c_int, I64, P, c_float, P]),
     "orlhf_approx_kl_fwd": (c_int, [P, P, c_int, I64, c_int, P, P]),
     "orlhf_approx_kl_bwd": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
     "orlhf_token_workspace_bytes": (I64, [I64, I64]),

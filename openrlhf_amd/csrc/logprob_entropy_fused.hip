@@ -7,6 +7,7 @@
 // 512-thread workgroup (8 wave64, 2 per SIMD, up to 256 VGPRs each) owns a CU and a row: every
 // lane keeps 38 16-byte chunks of the row in registers (rows up to 38*512 chunks: 155648 bf16 /
 // fp16 or 77824 fp32 elements; longer rows are left to the separate kernels).
+#include "token_terms.h"
 #include "vocab_rows.h"
 
 namespace orlhf {
@@ -40,12 +41,24 @@ __device__ __forceinline__ void launder(u32x4& v) {
 // whole row is on chip the exponent reference is the wave maximum of each lane's first chunk (as
 // in the stand-alone forward); if the sums come out non-finite the exact maximum is taken from
 // the resident registers and the sums are redone, all on chip.
-template <int DT, int MODE, int REG_CHUNKS>
+// Per-token loss terms of a PPO step, evaluated on the freshly computed log-prob of each row
+// (TERMS kernels): the upstream weights are then d(loss)/d(logprob) and d(loss)/d(entropy) of
+//   loss = sum_i policy_coef[i] * L_ppo(lp_i) + kl_coef * sum_i token_coef[i] * KL(lp_i - base_i)
+//          - entropy_coef * sum_i token_coef[i] * H_i.
+struct StepTerms {
+  const float *old_lp, *adv, *rollout, *base, *policy_coef, *token_coef;
+  PolicyTok pol;  // clip / dual-clip / importance-correction parameters (pointers unused)
+  int kl_estimator;
+  float kl_coef, entropy_coef;
+};
+
+template <int DT, int MODE, int REG_CHUNKS, bool TERMS>
 __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel(
     const char* logits, char* grad, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
     int64_t grad_stride_bytes, const int64_t* __restrict__ labels, double temperature,
     const float* __restrict__ w_logprob, const float* __restrict__ w_entropy,
-    float* __restrict__ logprob, float* __restrict__ entropy, const uint8_t* __restrict__ row_mask) {
+    float* __restrict__ logprob, float* __restrict__ entropy, const uint8_t* __restrict__ row_mask,
+    StepTerms terms) {
   using E = Elt<DT>;
   using MT = ModeTraits<MODE>;
   constexpr int EPV = E::kPerVec;
@@ -202,17 +215,36 @@ __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel
         if (!MT::kScaledSet) lse_t = lse_1;
       }
       const int64_t label = (MODE != kEntOnly) ? labels[row_i] : -1;
-      if (MODE != kEntOnly && logprob != nullptr) {
-        float lp;
+      float lp = 0.0f;
+      if (MODE != kEntOnly) {
         if (label >= 0 && label < vocab)
           lp = (float)((double)E::load1(row + label * E::kSize) * inv_t - lse_t);
         else
           lp = (label == -100) ? 0.0f : NAN;
-        logprob[row_i] = lp;
+        if (logprob != nullptr) logprob[row_i] = lp;
       }
       if (MT::kPlainSet && entropy != nullptr) entropy[row_i] = (float)(lse_1 - ex);
-      const float glp = (MODE != kEntOnly && w_logprob != nullptr) ? w_logprob[row_i] : 0.0f;
-      const float gh = (MT::kPlainSet && w_entropy != nullptr) ? w_entropy[row_i] : 0.0f;
+      float glp = 0.0f, gh = 0.0f;
+      if (TERMS) {
+        const float pc = terms.policy_coef[row_i];
+        const float tc = terms.token_coef[row_i];
+        if (pc != 0.0f) {
+          const float old_v = terms.old_lp[row_i];
+          const float w = terms.rollout != nullptr ? terms.pol.token_is_weight_of(old_v, terms.rollout[row_i]) : 1.0f;
+          glp = pc * terms.pol.ppo_grad_of(lp, old_v, terms.adv[row_i], w);
+        }
+        if (tc != 0.0f) {
+          if (terms.base != nullptr) {
+            float kv, kd;
+            kl_value(terms.kl_estimator, lp - terms.base[row_i], kv, kd);
+            glp += terms.kl_coef * tc * kd;
+          }
+          gh = -terms.entropy_coef * tc;
+        }
+      } else {
+        glp = (MODE != kEntOnly && w_logprob != nullptr) ? w_logprob[row_i] : 0.0f;
+        gh = (MT::kPlainSet && w_entropy != nullptr) ? w_entropy[row_i] : 0.0f;
+      }
       lds_bcast[0] = -(float)(lse_t * 1.4426950408889634);
       lds_bcast[1] = -(float)(lse_1 * 1.4426950408889634);
       lds_bcast[2] = -(float)((double)glp * inv_t);
@@ -268,10 +300,10 @@ template <int DT>
 static int launch_fused(const void* logits, void* grad, int64_t n_rows, int64_t vocab, int64_t row_stride,
                         int64_t grad_row_stride, const int64_t* labels, double temperature,
                         const float* w_logprob, const float* w_entropy, float* logprob, float* entropy,
-                        const uint8_t* row_mask, int n_cu, hipStream_t stream) {
+                        const uint8_t* row_mask, const StepTerms* terms, int n_cu, hipStream_t stream) {
   using E = Elt<DT>;
-  const bool want_ent = entropy != nullptr || w_entropy != nullptr;
-  const bool want_lp = logprob != nullptr || w_logprob != nullptr;
+  const bool want_ent = entropy != nullptr || w_entropy != nullptr || (terms != nullptr && terms->entropy_coef != 0.0f);
+  const bool want_lp = logprob != nullptr || w_logprob != nullptr || terms != nullptr;
   const bool t1 = (temperature == 1.0);
   const int mode = !want_ent ? kLpOnly : (!want_lp ? kEntOnly : (t1 ? kBothT1 : kBothT));
   const char* p = (const char*)logits;
@@ -280,9 +312,16 @@ static int launch_fused(const void* logits, void* grad, int64_t n_rows, int64_t 
   // one workgroup per CU (it takes the whole register file), walking rows grid-stride
   const int64_t blocks = n_rows < n_cu ? n_rows : n_cu;
   const dim3 grid((unsigned)blocks), block(kFusedBlock);
-#define ORLHF_FUSED(M)                                                                                        \
-  hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunks>), grid, block, 0, stream, p, gp, \
-                     n_rows, vocab, sb, gsb, labels, temperature, w_logprob, w_entropy, logprob, entropy, row_mask)
+  StepTerms none = {};
+#define ORLHF_FUSED(M)                                                                                             \
+  if (terms != nullptr)                                                                                            \
+    hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunks, true>), grid, block, 0, stream,  \
+                       p, gp, n_rows, vocab, sb, gsb, labels, temperature, w_logprob, w_entropy, logprob, entropy, \
+                       row_mask, *terms);                                                                          \
+  else                                                                                                             \
+    hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunks, false>), grid, block, 0, stream, \
+                       p, gp, n_rows, vocab, sb, gsb, labels, temperature, w_logprob, w_entropy, logprob, entropy, \
+                       row_mask, none)
   switch (mode) {
     case kLpOnly: ORLHF_FUSED(kLpOnly); break;
     case kEntOnly: ORLHF_FUSED(kEntOnly); break;
@@ -304,11 +343,10 @@ extern "C" int64_t orlhf_logprob_entropy_fwd_bwd_max_vocab(int dtype) {
   return (int64_t)kFusedRegChunks * kFusedBlock * per_vec;
 }
 
-extern "C" int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logits, int dtype, int64_t n_rows,
-                                             int64_t vocab, int64_t row_stride, int64_t grad_row_stride,
-                                             const int64_t* labels, double temperature, const float* w_logprob,
-                                             const float* w_entropy, float* logprob, float* entropy,
-                                             const uint8_t* row_mask, orlhf_stream_t stream) {
+static int fused_entry(const void* logits, void* grad_logits, int dtype, int64_t n_rows, int64_t vocab,
+                       int64_t row_stride, int64_t grad_row_stride, const int64_t* labels, double temperature,
+                       const float* w_logprob, const float* w_entropy, float* logprob, float* entropy,
+                       const uint8_t* row_mask, const StepTerms* terms, orlhf_stream_t stream) {
   ORLHF_CHECK_ARG(n_rows >= 0 && vocab > 0, "logprob_entropy_fwd_bwd: n_rows=%lld vocab=%lld", (long long)n_rows,
                   (long long)vocab);
   ORLHF_CHECK_ARG(row_stride >= vocab && grad_row_stride >= vocab,
@@ -317,11 +355,12 @@ extern "C" int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logi
   ORLHF_CHECK_ARG(temperature > 0.0 && temperature == temperature, "logprob_entropy_fwd_bwd: temperature must be > 0");
   ORLHF_CHECK_ARG(dtype == ORLHF_F32 || dtype == ORLHF_BF16 || dtype == ORLHF_F16,
                   "logprob_entropy_fwd_bwd: unknown dtype %d", dtype);
-  ORLHF_CHECK_ARG(w_logprob != nullptr || w_entropy != nullptr || logprob != nullptr || entropy != nullptr,
+  ORLHF_CHECK_ARG(terms != nullptr || w_logprob != nullptr || w_entropy != nullptr || logprob != nullptr ||
+                      entropy != nullptr,
                   "logprob_entropy_fwd_bwd: nothing to compute");
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(logits != nullptr && grad_logits != nullptr, "logprob_entropy_fwd_bwd: NULL logits / grad_logits");
-  ORLHF_CHECK_ARG((logprob == nullptr && w_logprob == nullptr) || labels != nullptr,
+  ORLHF_CHECK_ARG((logprob == nullptr && w_logprob == nullptr && terms == nullptr) || labels != nullptr,
                   "logprob_entropy_fwd_bwd: labels is NULL");
   const int esize = dtype == ORLHF_F32 ? 4 : 2;
   ORLHF_CHECK_ARG((((uintptr_t)logits | (uintptr_t)grad_logits) & (uintptr_t)(esize - 1)) == 0,
@@ -346,12 +385,93 @@ extern "C" int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logi
   switch (dtype) {
     case ORLHF_F32:
       return launch_fused<ORLHF_F32>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride, labels,
-                                     temperature, w_logprob, w_entropy, logprob, entropy, row_mask, n_cu, s);
+                                     temperature, w_logprob, w_entropy, logprob, entropy, row_mask, terms, n_cu, s);
     case ORLHF_BF16:
       return launch_fused<ORLHF_BF16>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride, labels,
-                                      temperature, w_logprob, w_entropy, logprob, entropy, row_mask, n_cu, s);
+                                      temperature, w_logprob, w_entropy, logprob, entropy, row_mask, terms, n_cu, s);
     default:
       return launch_fused<ORLHF_F16>(logits, grad_logits, n_rows, vocab, row_stride, grad_row_stride, labels,
-                                     temperature, w_logprob, w_entropy, logprob, entropy, row_mask, n_cu, s);
+                                     temperature, w_logprob, w_entropy, logprob, entropy, row_mask, terms, n_cu, s);
   }
+}
+
+
+extern "C" int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logits, int dtype, int64_t n_rows,
+                                             int64_t vocab, int64_t row_stride, int64_t grad_row_stride,
+                                             const int64_t* labels, double temperature, const float* w_logprob,
+                                             const float* w_entropy, float* logprob, float* entropy,
+                                             const uint8_t* row_mask, orlhf_stream_t stream) {
+  return fused_entry(logits, grad_logits, dtype, n_rows, vocab, row_stride, grad_row_stride, labels, temperature,
+                     w_logprob, w_entropy, logprob, entropy, row_mask, nullptr, stream);
+}
+
+extern "C" int orlhf_policy_step_fwd_bwd(const void* logits, void* grad_logits, int dtype, int64_t n_rows,
+                                         int64_t vocab, int64_t row_stride, int64_t grad_row_stride,
+                                         const int64_t* labels, double temperature, const orlhf_step_terms* t,
+                                         float* logprob, float* entropy, const uint8_t* row_mask,
+                                         orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(t != nullptr, "policy_step_fwd_bwd: terms is NULL");
+  ORLHF_CHECK_ARG(n_rows == 0 || (t->old_log_probs && t->advantages && t->policy_coef && t->token_coef),
+                  "policy_step_fwd_bwd: old_log_probs / advantages / policy_coef / token_coef must be given");
+  ORLHF_CHECK_ARG(t->is_correction == ORLHF_IS_NONE || t->is_correction == ORLHF_IS_TIS ||
+                      t->is_correction == ORLHF_IS_ICEPOP,
+                  "policy_step_fwd_bwd: only token-level importance corrections (none, tis, icepop) can be fused, got %d",
+                  t->is_correction);
+  ORLHF_CHECK_ARG(t->is_correction == ORLHF_IS_NONE || t->rollout_log_probs != nullptr,
+                  "policy_step_fwd_bwd: importance correction needs rollout_log_probs");
+  ORLHF_CHECK_ARG(t->base_log_probs == nullptr || (t->kl_estimator >= ORLHF_KL_K1 && t->kl_estimator <= ORLHF_KL_K3),
+                  "policy_step_fwd_bwd: unknown kl_estimator %d", t->kl_estimator);
+  ORLHF_CHECK_ARG(!(t->dual_clip > 0.0f) || t->dual_clip > 1.0f, "policy_step_fwd_bwd: dual_clip must be > 1.0, got %g",
+                  (double)t->dual_clip);
+  StepTerms st = {};
+  st.old_lp = t->old_log_probs;
+  st.adv = t->advantages;
+  st.rollout = t->is_correction == ORLHF_IS_NONE ? nullptr : t->rollout_log_probs;
+  st.base = t->base_log_probs;
+  st.policy_coef = t->policy_coef;
+  st.token_coef = t->token_coef;
+  st.pol.lp = st.pol.old = st.pol.adv = st.pol.rollout = st.pol.row_aux = nullptr;
+  st.pol.lo = 1.0f - t->clip_eps_low;
+  st.pol.hi = 1.0f + t->clip_eps_high;
+  st.pol.dual = t->dual_clip;
+  st.pol.gspo = 0;
+  st.pol.is_mode = t->is_correction;
+  st.pol.is_lo = t->is_low;
+  st.pol.is_hi = t->is_high;
+  st.kl_estimator = t->kl_estimator;
+  st.kl_coef = t->kl_coef;
+  st.entropy_coef = t->entropy_coef;
+  return fused_entry(logits, grad_logits, dtype, n_rows, vocab, row_stride, grad_row_stride, labels, temperature,
+                     nullptr, nullptr, logprob, entropy, row_mask, &st, stream);
+}
+
+// ---------------------------------------------------------------- conditional in-place rescale
+namespace orlhf {
+template <int DT>
+__global__ __launch_bounds__(kBlock) void rescale_if_kernel(char* data, int64_t n, const float* __restrict__ g,
+                                                            float expected) {
+  using E = Elt<DT>;
+  const float f = g[0] / expected;
+  if (f == 1.0f) return;  // the usual case: the gradient was produced with the right scale
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    E::store1(data + i * E::kSize, E::load1(data + i * E::kSize) * f);
+}
+}  // namespace orlhf
+
+extern "C" int orlhf_rescale_inplace_if(void* data, int dtype, int64_t n, const float* g, float expected,
+                                        orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n >= 0 && expected != 0.0f && expected == expected, "rescale_inplace_if: n=%lld expected=%g",
+                  (long long)n, (double)expected);
+  if (n == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(data != nullptr && g != nullptr, "rescale_inplace_if: NULL pointer");
+  const dim3 grid(flat_grid(n, 16384)), block(kBlock);
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case ORLHF_F32: hipLaunchKernelGGL(rescale_if_kernel<ORLHF_F32>, grid, block, 0, s, (char*)data, n, g, expected); break;
+    case ORLHF_BF16: hipLaunchKernelGGL(rescale_if_kernel<ORLHF_BF16>, grid, block, 0, s, (char*)data, n, g, expected); break;
+    case ORLHF_F16: hipLaunchKernelGGL(rescale_if_kernel<ORLHF_F16>, grid, block, 0, s, (char*)data, n, g, expected); break;
+    default: return fail(ORLHF_ERR_INVALID_ARG, "rescale_inplace_if: unknown dtype %d", dtype);
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_rescale_inplace_if");
+  return ORLHF_OK;
 }

@@ -1,0 +1,222 @@
+"""The loss assembly of the PPO actor training step on hand-written HIP kernels.
+
+Mirrors openrlhf/trainer/ray/ppo_actor.py:294-352 (ActorPPOTrainer.training_step between the
+model forward and strategy.backward): action log-probs and entropy from the logits
+(openrlhf/models/actor.py:265-296), PolicyLoss, the optional KL loss
+``aggregate_loss(compute_approx_kl(...))`` times the KL coefficient, the optional entropy bonus,
+and their sum.
+
+``actor_loss_step`` composes the separate kernels in the reference's order and is an ordinary
+autograd graph. ``fused_actor_loss_step`` produces the same numbers from ONE pass over the logits:
+the per-token derivative of the whole loss is evaluated inside the vocabulary-row kernel as soon
+as a row's log-prob is known, and d(loss)/d(logits) is written over the logits (2 x V bytes per
+token instead of 3 x; prompt and padding rows are neither read nor computed). It needs the
+aggregation weights before the pass, which only depend on the action mask and on the
+``loss_batch_info`` normalisers (openrlhf/utils/loss_utils.py:15-105).
+
+Not mirrored: the Mixtral auxiliary loss (a scalar the model returns, added by the caller), the
+optimizer step, DeepSpeed. GSPO and seq-mask-TIS need a sequence-level ratio before any token can
+be differentiated; ``fused_actor_loss_step`` refuses them (use ``actor_loss_step``).
+"""
+from typing import Optional
+
+import torch
+
+from ... import _lib
+from ..._lib import call, ptr, require_gpu, stream_of
+from ...models.actor import actor_forward_tail
+from ...models.loss import PolicyLoss, aggregate_loss
+from ...models.utils import _KL_CODES, _as_rows, _f32, _workspace, compute_approx_kl, masked_mean
+
+
+def actor_loss_step(
+    logits, sequences, attention_mask, action_mask, old_action_log_probs, advantages, policy_loss_fn: PolicyLoss,
+    base_action_log_probs=None, kl_estimator="k1", kl_coef=0.0, entropy_coef=None, rollout_log_probs=None,
+    temperature=1.0, packed_indices=None, dp_size=1, batch_num_tokens=None, global_batch_size=None,
+    inplace_backward=False,
+):
+    """Reference-order composition (ppo_actor.py:294-352) on the separate kernels; differentiable."""
+    info = dict(dp_size=dp_size, batch_num_tokens=batch_num_tokens, global_batch_size=global_batch_size)
+    want_entropy = entropy_coef is not None
+    out = actor_forward_tail(logits, sequences, action_mask, attention_mask, temperature=temperature,
+                             packed_indices=packed_indices, return_entropy=want_entropy,
+                             inplace_backward=inplace_backward)
+    action_log_probs, entropy = out if want_entropy else (out, None)
+    actor_loss, clip_ratio, ppo_kl, vllm_kl = policy_loss_fn(
+        action_log_probs, old_action_log_probs, advantages, action_mask=action_mask,
+        rollout_log_probs=rollout_log_probs, **info)
+    result = dict(actor_loss=actor_loss, clip_ratio=clip_ratio, ppo_kl=ppo_kl, vllm_kl=vllm_kl,
+                  action_log_probs=action_log_probs, entropy=entropy, kl_loss=None, entropy_loss=None)
+    loss = actor_loss
+    if base_action_log_probs is not None:
+        kl = compute_approx_kl(action_log_probs, base_action_log_probs, kl_estimator=kl_estimator)
+        result["kl_loss"] = aggregate_loss(kl, action_mask, **info)
+        loss = loss + result["kl_loss"] * kl_coef
+    if want_entropy:
+        result["entropy_loss"] = aggregate_loss(entropy[:, -action_mask.shape[1]:], action_mask, **info)
+        if entropy_coef != 0:
+            loss = loss - result["entropy_loss"] * entropy_coef
+    result["loss"] = loss
+    return result
+
+
+def _aggregation_coef(action_mask, token_level, dp_size, norm_value):
+    """d(aggregate_loss)/d(token loss) for every [B, A] position: row weight times the mask."""
+    dev = action_mask.device
+    b, a = action_mask.shape
+    mkeep, mptr, mcode = _lib.mask_arg(action_mask)
+    keep = []
+    norm = _lib.make_norm(dp_size, norm_value, keep)
+    ws = _workspace(b, a, dev)
+    dummy = torch.zeros(b, a, dtype=torch.float32, device=dev)
+    out = torch.empty(1, dtype=torch.float32, device=dev)
+    row_coef = torch.empty(max(b, 1), dtype=torch.float32, device=dev)
+    with torch.cuda.device(dev):
+        call("orlhf_masked_aggregate_fwd", ptr(dummy), mptr, mcode, b, a, None,
+             _lib.AGG_TOKEN_MEAN if token_level else _lib.AGG_SEQ_MEAN, norm, ptr(ws), ptr(out), ptr(row_coef),
+             stream_of(dev))
+    return row_coef[:b, None] * action_mask.to(torch.float32)
+
+
+class _HandOverGradient(torch.autograd.Function):
+    """Connects a loss value to logits whose gradient has already been written: backward hands
+    that gradient over, rescaled on the device only if the upstream gradient is not the scale
+    it was produced with."""
+
+    @staticmethod
+    def forward(ctx, logits, loss_value, grad_logits, produced_scale):
+        ctx.save_for_backward(grad_logits)
+        ctx.produced_scale = float(produced_scale)
+        return loss_value.clone()
+
+    @staticmethod
+    def backward(ctx, g):
+        (grad,) = ctx.saved_tensors
+        dev = grad.device
+        gf = g.reshape(-1)[:1].to(torch.float32).contiguous()
+        with torch.cuda.device(dev):
+            call("orlhf_rescale_inplace_if", ptr(grad), _lib.dtype_code(grad), grad.numel(), ptr(gf),
+                 ctx.produced_scale, stream_of(dev))
+        return grad, None, None, None
+
+
+def fused_actor_loss_step(
+    logits, sequences, attention_mask, action_mask, old_action_log_probs, advantages, policy_loss_fn: PolicyLoss,
+    base_action_log_probs=None, kl_estimator="k1", kl_coef=0.0, entropy_coef=None, rollout_log_probs=None,
+    temperature=1.0, packed_indices=None, dp_size=1, batch_num_tokens=None, global_batch_size=None,
+    loss_scale=1.0,
+):
+    """Same results as ``actor_loss_step`` followed by ``(loss * loss_scale).backward()`` down to
+    the logits, from one pass over them. Returns the same dict plus ``grad_logits`` (aliasing the
+    logits storage, already holding ``loss_scale * d(loss)/d(logits)``). ``result["loss"]`` is
+    attached to ``logits`` in the autograd graph: ``(result["loss"] * loss_scale).backward()``
+    (what a gradient-accumulating engine does with ``loss_scale = 1 / accumulation_steps``) hands
+    the stored gradient to the layer that produced the logits without another pass.
+
+    logits: contiguous ``[B, T, V]``, or packed ``[Ttot, V]`` / ``[1, Ttot, V]`` with
+    ``packed_indices``. The logits are consumed: their storage holds the gradient afterwards.
+    """
+    if policy_loss_fn.policy_loss_type != "ppo":
+        raise ValueError("fused_actor_loss_step fuses the token-level PPO surrogate only; use actor_loss_step for "
+                         f"policy_loss_type={policy_loss_fn.policy_loss_type!r}")
+    use_is = bool(policy_loss_fn.enable_vllm_is_correction)
+    if use_is and policy_loss_fn.vllm_is_correction_type == "seq-mask-tis":
+        raise ValueError("seq-mask-tis needs a sequence-level ratio first; use actor_loss_step")
+    if use_is and rollout_log_probs is None:
+        raise ValueError("enable_vllm_is_correction needs rollout_log_probs")
+    if base_action_log_probs is not None and kl_estimator not in _KL_CODES:
+        raise ValueError(f"Unknown kl_estimator: {kl_estimator}")
+    dev = require_gpu(logits, sequences, action_mask, old_action_log_probs, advantages)
+    batch, seqlen = sequences.shape
+    width = action_mask.shape[1]
+    lo_col, hi_col = seqlen - 1 - width, seqlen - 1
+    info = dict(dp_size=dp_size, batch_num_tokens=batch_num_tokens, global_batch_size=global_batch_size)
+
+    with torch.no_grad():
+        pol_norm = batch_num_tokens if policy_loss_fn.token_level_loss else global_batch_size
+        policy_coef = _aggregation_coef(action_mask, policy_loss_fn.token_level_loss, dp_size, pol_norm) * loss_scale
+        token_coef = _aggregation_coef(action_mask, True, dp_size, batch_num_tokens) * loss_scale
+
+        def to_rows(t):  # [B, A] -> one value per logits row
+            if t is None:
+                return None
+            full = torch.zeros(batch, seqlen, dtype=torch.float32, device=dev)
+            full[:, lo_col:hi_col] = t.to(torch.float32)
+            flat = full.reshape(-1)
+            return (flat if packed_indices is None else flat[packed_indices]).contiguous()
+
+        old_r, adv_r = to_rows(old_action_log_probs), to_rows(advantages)
+        roll_r = to_rows(rollout_log_probs) if use_is else None
+        base_r = to_rows(base_action_log_probs)
+        pc_r, tc_r = to_rows(policy_coef), to_rows(token_coef)
+        need = torch.zeros(batch, seqlen, dtype=torch.uint8, device=dev)
+        need[:, lo_col:hi_col] = (action_mask != 0).to(torch.uint8)
+        labels = torch.roll(sequences, shifts=-1, dims=1).reshape(-1)
+        if packed_indices is not None:
+            need_r, labels = need.reshape(-1)[packed_indices].contiguous(), labels[packed_indices]
+        else:
+            need_r = need.reshape(-1)
+        labels = labels.to(torch.int64).contiguous()
+
+        rows, row_stride, aliases = _as_rows(logits.detach().reshape(-1, logits.shape[-1]) if logits.dim() == 3
+                                            else logits.detach())
+        if not aliases or rows.data_ptr() != logits.data_ptr():
+            raise ValueError("fused_actor_loss_step needs logits it can overwrite: contiguous [B, T, V] or [Ttot, V]")
+        n_rows, vocab = rows.shape
+        if n_rows != labels.numel():
+            raise ValueError(f"{n_rows} logits rows for {labels.numel()} token positions")
+        code = _lib.dtype_code(rows)
+        if vocab > _lib.load().orlhf_logprob_entropy_fwd_bwd_max_vocab(code):
+            raise ValueError(f"a row of {vocab} {rows.dtype} logits does not fit on one CU; use actor_loss_step")
+
+        terms = _lib.StepTerms()
+        terms.old_log_probs, terms.advantages = ptr(old_r), ptr(adv_r)
+        terms.rollout_log_probs, terms.base_log_probs = ptr(roll_r), ptr(base_r)
+        terms.policy_coef, terms.token_coef = ptr(pc_r), ptr(tc_r)
+        terms.clip_eps_low, terms.clip_eps_high = float(policy_loss_fn.clip_eps_low), float(policy_loss_fn.clip_eps_high)
+        terms.dual_clip = float(policy_loss_fn.dual_clip) if policy_loss_fn.dual_clip is not None else 0.0
+        terms.is_correction = ({"tis": _lib.IS_TIS, "icepop": _lib.IS_ICEPOP}[policy_loss_fn.vllm_is_correction_type]
+                               if use_is else _lib.IS_NONE)
+        if use_is:
+            terms.is_low, terms.is_high = (float(v) for v in policy_loss_fn.vllm_is_truncated_threshold)
+        terms.kl_estimator = _KL_CODES.get(kl_estimator, 0)
+        terms.kl_coef = float(kl_coef) if base_r is not None else 0.0
+        want_entropy = entropy_coef is not None
+        terms.entropy_coef = float(entropy_coef) if want_entropy else 0.0
+
+        lp_r = torch.empty(n_rows, dtype=torch.float32, device=dev)
+        ent_r = torch.empty(n_rows, dtype=torch.float32, device=dev) if want_entropy else None
+        with torch.cuda.device(dev):
+            call("orlhf_policy_step_fwd_bwd", ptr(rows), ptr(rows), code, n_rows, vocab, row_stride, row_stride,
+                 ptr(labels), float(temperature), terms, ptr(lp_r), ptr(ent_r), ptr(need_r), stream_of(dev))
+        torch.autograd.graph.increment_version(rows)
+
+        def from_rows(t):  # one value per logits row -> [B, A]
+            if packed_indices is not None:
+                t = torch.zeros(batch * seqlen, dtype=torch.float32, device=dev).index_copy(0, packed_indices, t)
+            return t.view(batch, seqlen)[:, lo_col:hi_col]
+
+        action_log_probs = from_rows(lp_r) * action_mask.float()
+        entropy = from_rows(ent_r) if want_entropy else None
+
+        # the values, from the per-token outputs (17 B/token kernels)
+        actor_loss, clip_ratio, ppo_kl, vllm_kl = policy_loss_fn(
+            action_log_probs, old_action_log_probs, advantages, action_mask=action_mask,
+            rollout_log_probs=rollout_log_probs, **info)
+        loss = actor_loss
+        kl_loss = entropy_loss = None
+        if base_action_log_probs is not None:
+            kl_loss = aggregate_loss(compute_approx_kl(action_log_probs, base_action_log_probs, kl_estimator),
+                                     action_mask, **info)
+            loss = loss + kl_loss * kl_coef
+        if want_entropy:
+            entropy_loss = aggregate_loss(entropy, action_mask, **info)
+            if entropy_coef != 0:
+                loss = loss - entropy_loss * entropy_coef
+
+    grad_logits = rows if rows.shape == logits.shape else rows.view(logits.shape)
+    if logits.requires_grad:
+        loss = _HandOverGradient.apply(logits, loss, grad_logits, loss_scale)
+    return dict(loss=loss, actor_loss=actor_loss, clip_ratio=clip_ratio, ppo_kl=ppo_kl, vllm_kl=vllm_kl,
+                kl_loss=kl_loss, entropy_loss=entropy_loss, action_log_probs=action_log_probs, entropy=entropy,
+                grad_logits=grad_logits)
