@@ -112,6 +112,57 @@ def measured_traffic(kernel, n_tok):
     return None
 
 
+def bench_ppo_step(args, pristine, bufs, cu, ring, dev):
+    """Extra figure on the same packed logits: the whole PPO actor loss step (log-probs, entropy,
+    clipped surrogate, k3 KL loss, entropy bonus, their derivative down to the logits) through
+    ``fused_actor_loss_step``: the one-pass kernel plus the per-token kernels for the loss values."""
+    from openrlhf_amd.models.actor import unpad_indices
+    from openrlhf_amd.models.loss import PolicyLoss
+    from openrlhf_amd.trainer.ray.ppo_actor import fused_actor_loss_step
+
+    g = torch.Generator(device="cpu").manual_seed(99)
+    lens = (cu[1:] - cu[:-1])
+    b, t = lens.numel(), int(lens.max())
+    attn = (torch.arange(t)[None, :] < lens[:, None]).long().to(dev)
+    seqs = (torch.randint(1, VOCAB, (b, t), generator=g).to(dev)) * attn
+    action_mask = attn[:, 1:].bool()  # every generated position is an action
+    a = t - 1
+    old = (-torch.rand(b, a, generator=g) * 14).to(dev)
+    ref = (-torch.rand(b, a, generator=g) * 14).to(dev)
+    adv = torch.randn(b, a, generator=g).to(dev)
+    idx = unpad_indices(attn)
+    fn = PolicyLoss(0.2, 0.2)
+    n_tok = pristine.shape[0]
+
+    def one(buf):
+        return fused_actor_loss_step(buf, seqs, attn, action_mask, old, adv, fn, base_action_log_probs=ref,
+                                     kl_estimator="k3", kl_coef=0.01, entropy_coef=0.001, packed_indices=idx)
+
+    total, left, first = 0.0, args.steps, True
+    while left > 0:
+        c = min(left, ring)
+        for buf in bufs[:c]:
+            buf.detach_().copy_(pristine)
+        if first:
+            one(bufs[0])
+            bufs[0].detach_().copy_(pristine)
+            first = False
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(c):
+            out = one(bufs[i])
+        torch.cuda.synchronize()
+        total += time.perf_counter() - t0
+        left -= c
+    return {
+        "entry": "openrlhf_amd.trainer.ray.ppo_actor.fused_actor_loss_step (PPO clip 0.2 + 0.01*k3 KL loss + 0.001*entropy)",
+        "value": n_tok * args.steps / total,
+        "unit": "tokens/s",
+        "ms_per_step": total / args.steps * 1e3,
+        "loss": float(out["loss"]),
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -120,6 +171,7 @@ def main():
     ap.add_argument("--ring", type=int, default=6, help="distinct logits buffers per timed segment")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU-baseline sample")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-ppo-step", action="store_true", help="skip the extra fused PPO actor step measurement")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path shards by rows with no collective "
@@ -200,6 +252,7 @@ def main():
 
     total_two = run(step_two_kernels)
     total = run(step_fused)
+    ppo = None if args.no_ppo_step else bench_ppo_step(args, pristine, bufs, cu, ring, dev)
 
     ms_per_step = total / args.steps * 1e3
     tok_s = n_tok * args.steps / total
@@ -272,6 +325,8 @@ def main():
             },
         },
     }
+    if ppo is not None:
+        out["ppo_actor_step_fused"] = ppo
     if not args.no_cpu_baseline:
         rows = min(args.cpu_rows, n_tok)
         cpu_tok_s, cpu_s = cpu_baseline(pristine[:rows], labels[:rows], g_lp[:rows], g_ent[:rows])
