@@ -163,6 +163,82 @@ def bench_ppo_step(args, pristine, bufs, cu, ring, dev):
     }
 
 
+def bench_per_token(args, dev):
+    """--workload per_token: the small kernels at the sizes of BASELINE configs 3 and 4 (per-token
+    fp32 tensors; MBs, not GBs: these launches are latency-bound, the figures are for the record).
+    Prints one JSON line with achieved GB/s per entry point (algorithmic bytes / event time)."""
+    from openrlhf_amd.models.loss import PolicyLoss, ValueLoss
+    from openrlhf_amd.models.utils import compute_approx_kl, compute_reward
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import (
+        get_advantages_and_returns, get_cumulative_returns, whiten_advantages)
+
+    g = torch.Generator(device="cpu").manual_seed(7)
+
+    def timed(fn, n=10):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    res = {}
+
+    def record(name, ms, tokens, bytes_per_token):
+        res[name] = {"ms": ms, "tokens": tokens, "bytes_per_token": bytes_per_token,
+                     "achieved_gbs": tokens * bytes_per_token / (ms * 1e-3) / 1e9,
+                     "frac_of_hbm_peak": tokens * bytes_per_token / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS}
+
+    # config 3: 256 sequences, lognormal(7, 0.8) lengths in [16, 8192], padded [B, A]
+    b = 256
+    lens = torch.clamp(torch.exp(torch.randn(b, generator=g) * 0.8 + 7.0), 16, 8192).long()
+    a = int(lens.max())
+    mask = (torch.arange(a)[None, :] < lens[:, None]).to(dev)
+    values = torch.randn(b, a, generator=g).to(dev)
+    kl = (torch.randn(b, a, generator=g) * 0.05).to(dev)
+    r = (torch.rand(b, generator=g) < 0.5).float().to(dev)
+    padded = b * a
+    rew = compute_reward(r, 0.01, kl, action_mask=mask)
+    record("config3.compute_reward", timed(lambda: compute_reward(r, 0.01, kl, action_mask=mask)), padded, 4 + 1 + 1 + 4)
+    record("config3.gae_scan", timed(lambda: get_advantages_and_returns(values, rew, mask, 1.0, 0.95)), padded, 17)
+    adv, ret = get_advantages_and_returns(values, rew, mask, 1.0, 0.95)
+    record("config3.whiten", timed(lambda: whiten_advantages([adv], [mask])), padded, 14)
+    vnew = (values + 0.1).requires_grad_(True)
+    vl = ValueLoss(0.2)
+
+    def value_step():
+        loss = vl(vnew, values, ret, action_mask=mask)
+        torch.autograd.grad(loss, vnew)
+
+    record("config3.value_loss_fwd_bwd", timed(value_step), padded, 30)
+
+    # config 4: 512 x 8 sequences, lengths uniform in [64, 16384], padded [B, A]
+    b = 4096
+    lens = torch.randint(64, 16385, (b,), generator=g)
+    a = int(lens.max())
+    mask = (torch.arange(a, device=dev)[None, :] < lens.to(dev)[:, None])
+    lp = -torch.rand(b, a, device=dev) * 2
+    old = lp + torch.randn(b, a, device=dev) * 0.05
+    ref = lp + torch.randn(b, a, device=dev) * 0.1
+    adv = torch.randn(b, a, device=dev)
+    padded = b * a
+    record("config4.approx_kl_k3", timed(lambda: compute_approx_kl(lp, ref, "k3")), padded, 12)
+    record("config4.discounted_returns", timed(lambda: get_cumulative_returns(adv, mask, 1.0)), padded, 9)
+    x = lp.clone().requires_grad_(True)
+    pl = PolicyLoss(0.2, 0.2, dual_clip=3.0, token_level_loss=False)
+
+    def policy_step():
+        out = pl(x, old, adv, action_mask=mask)
+        torch.autograd.grad(out[0], x)
+
+    record("config4.policy_loss_fwd_bwd", timed(policy_step), padded, 13 + 17)
+    print(json.dumps({"workload": "per-token kernels at BASELINE config 3 / config 4 sizes (padded [B, A] fp32)",
+                      "n_gpus": 1, "unit": "GB/s", "peak": HBM_PEAK_GBS, "entries": res}), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -170,6 +246,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--ring", type=int, default=6, help="distinct logits buffers per timed segment")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU-baseline sample")
+    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token"],
+                    help="logprob: the headline step (default); per_token: the small kernels of configs 3/4")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ppo-step", action="store_true", help="skip the extra fused PPO actor step measurement")
     args = ap.parse_args()
@@ -184,6 +262,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "per_token":
+        bench_per_token(args, dev)
+        return
     pristine, labels, g_lp, g_ent, cu = make_workload(dev)
     n_tok = pristine.shape[0]
     row_bytes = VOCAB * 2
