@@ -6,7 +6,8 @@
 // carry C entering from later tokens. Maps compose associatively; a wave composes its 64 maps with
 // log2(64) cross-lane steps, the 4 waves of the workgroup chain through LDS, and a row longer than
 // one tile (kBlock * kScanItems tokens) walks its tiles from the end carrying one number. Carries
-// and the in-lane recurrence are fp64, inputs and outputs fp32.
+// and the in-lane recurrence are fp64, inputs and outputs fp32. A tile goes through LDS both ways
+// so that global loads and stores are coalesced while each lane works on consecutive tokens.
 #include "common.h"
 
 namespace orlhf {
@@ -95,6 +96,11 @@ __device__ __forceinline__ Affine compose(const Affine& outer, const Affine& inn
   return r;
 }
 
+// LDS staging index: one pad word per 32 keeps a lane's 8 consecutive tokens (stride-8 access
+// over the wave) off each other's banks.
+__device__ __forceinline__ int scan_slot(int p) { return p + (p >> 5); }
+constexpr int kScanLds = kScanTile + kScanTile / 32 + 2;
+
 template <int MASK_DT, bool GAE>
 __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const float* __restrict__ values,
                                                               const float* __restrict__ rewards,
@@ -103,6 +109,8 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
                                                               float* __restrict__ ret) {
   __shared__ Affine lds_wave[kWavesPerBlock];
   __shared__ double lds_carry;
+  __shared__ float lds_v[kScanLds];  // masked values in, returns out
+  __shared__ float lds_r[kScanLds];  // masked rewards in, advantages out
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
 
@@ -118,25 +126,36 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
     const int64_t n_tiles = (len + kScanTile - 1) / kScanTile;
     double tile_carry = 0.0;  // A at the first token of the previous (later) tile
     for (int64_t tile = n_tiles - 1; tile >= 0; --tile) {
-      const int64_t t0 = tile * kScanTile + (int64_t)threadIdx.x * kScanItems;
-      // masked inputs of this lane's tokens, plus the value of the token after them
+      const int64_t tile0 = tile * kScanTile;
+      // ---- coalesced load of the tile (masked) into LDS; token tile0+kScanTile is the
+      //      "value after the tile" the last lane needs
+#pragma unroll
+      for (int k = 0; k < kScanItems; ++k) {
+        const int p = threadIdx.x + k * kBlock;
+        const int64_t t = tile0 + p;
+        float rv = 0.0f, vv = 0.0f;
+        if (t < len) {
+          const float m = load_mask<MASK_DT>(mask, start + t);
+          rv = m * rewards[start + t];
+          if (GAE) vv = m * values[start + t];
+        }
+        lds_r[scan_slot(p)] = rv;
+        if (GAE) lds_v[scan_slot(p)] = vv;
+      }
+      if (GAE && threadIdx.x == 0) {
+        const int64_t t = tile0 + kScanTile;
+        lds_v[scan_slot(kScanTile)] = t < len ? load_mask<MASK_DT>(mask, start + t) * values[start + t] : 0.0f;
+      }
+      __syncthreads();
+      // ---- this lane's kScanItems consecutive tokens
+      const int p0 = threadIdx.x * kScanItems;
       float v[kScanItems + 1], rw[kScanItems];
 #pragma unroll
       for (int j = 0; j < kScanItems; ++j) {
-        const int64_t t = t0 + j;
-        if (t < len) {
-          const float m = load_mask<MASK_DT>(mask, start + t);
-          rw[j] = m * rewards[start + t];
-          v[j] = GAE ? m * values[start + t] : 0.0f;
-        } else {
-          rw[j] = 0.0f;
-          v[j] = 0.0f;
-        }
+        rw[j] = lds_r[scan_slot(p0 + j)];
+        v[j] = GAE ? lds_v[scan_slot(p0 + j)] : 0.0f;
       }
-      {
-        const int64_t t = t0 + kScanItems;
-        v[kScanItems] = (GAE && t < len) ? load_mask<MASK_DT>(mask, start + t) * values[start + t] : 0.0f;
-      }
+      v[kScanItems] = GAE ? lds_v[scan_slot(p0 + kScanItems)] : 0.0f;
       // in-lane recurrence with zero carry-in
       double local[kScanItems];
       double run = 0.0;
@@ -158,7 +177,7 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
         if (lane + d < kWave) f = compose(f, o);
       }
       if (lane == 0) lds_wave[wave] = f;
-      __syncthreads();
+      __syncthreads();  // also: every lane has read its inputs from LDS
       // carry entering this wave = maps of the later waves applied to the tile carry
       double wave_carry = tile_carry;
       for (int w = kWavesPerBlock - 1; w > wave; --w) wave_carry = lds_wave[w].b + lds_wave[w].a * wave_carry;
@@ -169,20 +188,32 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
       const double carry = (lane == kWave - 1) ? wave_carry : nxt.b + nxt.a * wave_carry;
 #pragma unroll
       for (int j = 0; j < kScanItems; ++j) {
-        const int64_t t = t0 + j;
-        if (t < len) {
-          const double a_t = local[j] + pw[kScanItems - j] * carry;
-          if (GAE) {
-            adv[start + t] = (float)a_t;
-            ret[start + t] = (float)(a_t + (double)v[j]);
-          } else {
-            ret[start + t] = (float)a_t;
-          }
+        const double a_t = local[j] + pw[kScanItems - j] * carry;
+        if (GAE) {
+          lds_r[scan_slot(p0 + j)] = (float)a_t;
+          lds_v[scan_slot(p0 + j)] = (float)(a_t + (double)v[j]);
+        } else {
+          lds_r[scan_slot(p0 + j)] = (float)a_t;
         }
       }
       if (threadIdx.x == 0) lds_carry = local[0] + pw[kScanItems] * carry;
       __syncthreads();
       tile_carry = lds_carry;
+      // ---- coalesced store of the tile
+#pragma unroll
+      for (int k = 0; k < kScanItems; ++k) {
+        const int p = threadIdx.x + k * kBlock;
+        const int64_t t = tile0 + p;
+        if (t < len) {
+          if (GAE) {
+            adv[start + t] = lds_r[scan_slot(p)];
+            ret[start + t] = lds_v[scan_slot(p)];
+          } else {
+            ret[start + t] = lds_r[scan_slot(p)];
+          }
+        }
+      }
+      __syncthreads();  // LDS is refilled by the next tile
     }
   }
 }
