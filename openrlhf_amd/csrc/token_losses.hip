@@ -211,6 +211,25 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
   }
 }
 
+// Stage 1b: fold the chunk partials of every row into one entry per row, one lane per row, so
+// that the single-workgroup finaliser reads n_rows entries instead of n_rows * n_chunks.
+template <int NQ>
+__global__ __launch_bounds__(kBlock) void rows_fold_kernel(int64_t n_rows, int n_chunks,
+                                                           const double* __restrict__ partial,
+                                                           double* __restrict__ row_total) {
+  for (int64_t b = (int64_t)blockIdx.x * kBlock + threadIdx.x; b < n_rows; b += (int64_t)gridDim.x * kBlock) {
+    double rq[NQ];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) rq[i] = 0.0;
+    for (int c = 0; c < n_chunks; ++c) {
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) rq[i] += partial[(b * n_chunks + c) * NQ + i];
+    }
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) row_total[b * NQ + i] = rq[i];
+  }
+}
+
 // Row prepass results for GSPO (kind 0) and seq-mask-TIS (kind 1): row_aux[b] = {value, 1/max(cnt,1)}.
 __global__ __launch_bounds__(kBlock) void row_aux_kernel(int64_t n_rows, int n_chunks,
                                                          const double* __restrict__ partial, int kind,
@@ -364,6 +383,23 @@ static void launch_grad(int mask_dt, Rows rows, const void* mask, const Tok& tok
 }
 
 
+// Folds chunk partials per row (when there is more than one chunk) and runs the finaliser.
+template <int NQ>
+static void launch_final(int64_t n_rows, int n_chunks, double* partial, int mode, const NormArg& norm,
+                         float post_scale, int n_out, float* out, float* row_coef, hipStream_t s) {
+  const double* src = partial;
+  int chunks = n_chunks;
+  if (n_chunks > 1 && n_rows > 0) {
+    double* row_total = partial + n_rows * (int64_t)n_chunks * NQ;
+    hipLaunchKernelGGL(rows_fold_kernel<NQ>, dim3(flat_grid(n_rows, 4096)), dim3(kBlock), 0, s, n_rows, n_chunks,
+                       partial, row_total);
+    src = row_total;
+    chunks = 1;
+  }
+  hipLaunchKernelGGL(rows_final_kernel<NQ>, dim3(1), dim3(kBlock), 0, s, n_rows, chunks, src, mode, norm, post_scale,
+                     n_out, out, row_coef);
+}
+
 static PolicyTok policy_tok(const float* lp, const float* old, const float* adv, const float* rollout,
                             const float* row_aux, const orlhf_policy_params* p) {
   PolicyTok t;
@@ -401,7 +437,8 @@ using namespace orlhf;
 
 extern "C" int64_t orlhf_token_workspace_bytes(int64_t n_rows, int64_t n_cols) {
   if (n_rows < 0 || n_cols < 0) return 0;
-  return (n_rows > 0 ? n_rows : 1) * chunks_of(n_cols) * kMaxQ * (int64_t)sizeof(double) + 256;
+  // chunk partials, then one folded entry per row
+  return (n_rows > 0 ? n_rows : 1) * (chunks_of(n_cols) + 1) * kMaxQ * (int64_t)sizeof(double) + 256;
 }
 
 extern "C" int orlhf_approx_kl_fwd(const void* log_probs, const void* log_probs_base, int dtype, int64_t n,
@@ -458,8 +495,7 @@ extern "C" int orlhf_masked_aggregate_fwd(const float* x, const void* mask, int 
     launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
     ORLHF_CHECK_LAUNCH("orlhf_masked_aggregate_fwd(partial)");
   }
-  hipLaunchKernelGGL(rows_final_kernel<2>, dim3(1), dim3(kBlock), 0, s, n_rows, n_chunks, partial, mode,
-                     norm_arg(norm), 1.0f, 1, out, row_coef);
+  launch_final<2>(n_rows, n_chunks, partial, mode, norm_arg(norm), 1.0f, 1, out, row_coef, s);
   ORLHF_CHECK_LAUNCH("orlhf_masked_aggregate_fwd(final)");
   return ORLHF_OK;
 }
@@ -514,8 +550,7 @@ extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_lo
   }
   const int mode = (params->token_level && !gspo) ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN;
   const int n_out = (use_is && !gspo) ? 4 : 3;
-  hipLaunchKernelGGL(rows_final_kernel<5>, dim3(1), dim3(kBlock), 0, s, n_rows, n_chunks, partial, mode,
-                     norm_arg(&params->norm), 1.0f, n_out, out4, row_coef);
+  launch_final<5>(n_rows, n_chunks, partial, mode, norm_arg(&params->norm), 1.0f, n_out, out4, row_coef, s);
   ORLHF_CHECK_LAUNCH("orlhf_policy_loss_fwd(final)");
   return ORLHF_OK;
 }
@@ -573,8 +608,8 @@ extern "C" int orlhf_value_loss_fwd(const float* values, const float* old_values
     launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
     ORLHF_CHECK_LAUNCH("orlhf_value_loss_fwd(partial)");
   }
-  hipLaunchKernelGGL(rows_final_kernel<2>, dim3(1), dim3(kBlock), 0, s, n_rows, n_chunks, partial,
-                     token_level ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN, norm_arg(norm), 0.5f, 1, out, row_coef);
+  launch_final<2>(n_rows, n_chunks, partial, token_level ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN, norm_arg(norm),
+                  0.5f, 1, out, row_coef, s);
   ORLHF_CHECK_LAUNCH("orlhf_value_loss_fwd(final)");
   return ORLHF_OK;
 }
