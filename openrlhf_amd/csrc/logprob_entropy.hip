@@ -216,7 +216,8 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
     if (g.nvec > 0) {
       const uint32_t v = (uint32_t)tid < g.nvec ? (uint32_t)tid : g.nvec - 1;
       float x[E::kPerVec];
-      E::unpack(load_vec(row + g.head * E::kSize + v * 16u), x);
+      // temporal load on purpose: the streaming pass reads these 4 KiB again and should hit in L2
+      E::unpack(*(const u32x4*)(row + g.head * E::kSize + v * 16u), x);
 #pragma unroll
       for (int j = 0; j < E::kPerVec; ++j) m_ref = fmaxf(m_ref, x[j]);
     } else {

@@ -186,22 +186,36 @@ __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel
     bool ok = true;
     if (MT::kScaledSet) ok = ok && (sumT > 0.0f && sumT < INFINITY);
     if (MT::kPlainSet) ok = ok && (sum1 > 0.0f && sum1 < INFINITY) && (fabsf(sumX) < INFINITY);
+    bool plus_inf_row = false;  // maximum +inf and no NaN: logsumexp is +inf, softmax undefined
     if (!ok) {  // workgroup-uniform, rare: the row is on chip, take its exact maximum
       float m = xs;
+      bool nan_seen = xs != xs;
 #pragma unroll
       for (int c = 0; c < REG_CHUNKS; ++c) {
         float x[EPV];
         launder(buf[c]);
         E::unpack(buf[c], x);
 #pragma unroll
-        for (int j = 0; j < EPV; ++j) m = fmaxf(m, x[j]);
+        for (int j = 0; j < EPV; ++j) {
+          m = fmaxf(m, x[j]);
+          nan_seen = nan_seen || (x[j] != x[j]);
+        }
       }
       m = wave_max(m);
-      if (lane == 0) lds_max[wave] = m;
+      const bool wave_nan = __ballot(nan_seen) != 0ull;
+      if (lane == 0) {
+        lds_max[wave] = m;
+        lds_sum[wave][5] = wave_nan ? 1.0f : 0.0f;
+      }
       __syncthreads();
       m = lds_max[0];
+      float nans = lds_sum[0][5];
 #pragma unroll
-      for (int w = 1; w < kFusedWaves; ++w) m = fmaxf(m, lds_max[w]);
+      for (int w = 1; w < kFusedWaves; ++w) {
+        m = fmaxf(m, lds_max[w]);
+        nans += lds_sum[w][5];
+      }
+      plus_inf_row = (m == INFINITY) && (nans == 0.0f);
       sums(m);
     }
 
@@ -213,6 +227,10 @@ __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel
         lse_1 = (double)ref1 * kLn2d + log((double)sum1);
         ex = (double)sumX / (double)sum1;
         if (!MT::kScaledSet) lse_t = lse_1;
+      }
+      if (plus_inf_row) {  // what torch.logsumexp / softmax give for a +inf logit
+        lse_t = lse_1 = INFINITY;
+        ex = NAN;
       }
       const int64_t label = (MODE != kEntOnly) ? labels[row_i] : -1;
       float lp = 0.0f;

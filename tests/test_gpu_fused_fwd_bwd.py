@@ -95,3 +95,41 @@ def test_fused_misaligned_rows_row_mask_and_optional_weights(cuda):
         assert lp[3].item() == 0.0 and ent[3].item() == 0.0 and grad[3].abs().max().item() == 0.0
         err = (grad.cpu().double() - ref)[keep].abs()
         assert (err <= 2.0 ** -8 * ref[keep].abs() + 1e-6).all()
+
+
+def test_fused_extreme_rows(cuda):
+    """Rows the reference-maximum shortcut cannot handle (late huge spike, very low start, -inf
+    entries) go through the on-chip exact-maximum path of the one-pass kernel and agree with the
+    separate kernels and the oracle; +inf / NaN rows give the same inf / NaN pattern."""
+    import math
+
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
+
+    vocab = 20000
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(6, vocab, generator=g)
+    x[0, vocab - 5] = 500.0
+    x[1, :1000] = -1.0e4
+    x[2, ::3] = float("-inf")
+    x[3, 17] = float("inf")
+    x[4, 9] = float("nan")
+    x[5] = x[5] * 30.0
+    labels = torch.tensor([vocab - 5, 5000, 1, 3, 4, 7])
+    w = torch.randn(6, generator=g)
+    ref_lp = otn.log_probs_from_logits(x.double(), labels)
+    ref_ent = otn.compute_entropy(x.double())
+    xd = x.to(cuda)
+    lp2, ent2 = logprobs_and_entropy_from_logits(xd, labels.to(cuda))
+    lp, ent, grad = fused_logprob_entropy_fwd_bwd(xd, labels.to(cuda), w.to(cuda), None, 1.0, inplace=False)
+    lp, ent = lp.cpu().double(), ent.cpu().double()
+    for i in (0, 1, 5):
+        assert abs(lp[i] - ref_lp[i]) <= 1e-5 * max(1.0, abs(ref_lp[i].item()) * 1e-1)
+        assert abs(ent[i] - ref_ent[i]) <= 1e-4
+        gref = _analytic_grad64(x[i:i + 1], labels[i:i + 1], 1.0, w[i:i + 1], torch.zeros(1))
+        # softmax of fp32 logits of magnitude |x| carries ~1e-7 * |x| of rounding in the exponent
+        tol = 1e-5 * max(1.0, gref.abs().max().item()) + 2e-7 * x[i].abs()[x[i].abs() < 1e30].max().item()
+        assert (grad[i:i + 1].cpu().double() - gref).abs().max().item() <= tol
+    assert abs(lp[2] - ref_lp[2]) <= 1e-5 and math.isnan(ent[2])
+    assert lp[3] == float("-inf") and math.isnan(ent[3])
+    assert math.isnan(lp[4]) and math.isnan(ent[4])
+    assert torch.equal(lp2.cpu().isnan(), lp.isnan()) and torch.equal(ent2.cpu().isnan(), ent.isnan())
