@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 4
+#define ORLHF_ABI_VERSION 5
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -93,6 +93,15 @@ int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows, int
                               int64_t row_stride, const int64_t* labels, double temperature,
                               float* logprob, float* entropy, float* row_stats,
                               const uint8_t* row_mask, int flags, orlhf_stream_t stream);
+
+/*
+ * logits[i,j] <- logits[i,j] / divisor, rounded to `dtype`, in place: the side effect of
+ * logits.div_(temperature) in log_probs_from_logits (openrlhf/models/utils.py:140-141), for
+ * callers that read the scaled logits afterwards. The log-prob entry points never need it (they
+ * fold the division into their loads).
+ */
+int orlhf_divide_rows_inplace(void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                              int64_t row_stride, double divisor, orlhf_stream_t stream);
 
 /*
  * Backward of the above in one streaming pass, written in the logits dtype:
@@ -219,6 +228,14 @@ int orlhf_masked_aggregate_fwd(const float* x, const void* mask, int mask_dtype,
                                int64_t n_cols, const int64_t* cu_seqlens, int mode,
                                const orlhf_norm* norm, void* workspace, float* out,
                                float* row_coef, orlhf_stream_t stream);
+/*
+ * The loss normalisers of one batch (openrlhf/utils/loss_utils.py:33-47,66-74): out2[0] =
+ * sum(mask) (batch_num_tokens before its all-reduce), out2[1] = number of rows whose mask sum is
+ * > 0 (global_batch_size before its all-reduce). fp64 accumulation, fp32 out.
+ */
+int orlhf_mask_counts(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                      const int64_t* cu_seqlens, void* workspace, float* out2, orlhf_stream_t stream);
+
 /* g_x[b,t] = g(b) * row_coef[b] * mask[b,t]; g(b) = g_out[0] (scalar modes) or g_out[b]. */
 int orlhf_masked_aggregate_bwd(const float* g_out, const void* mask, int mask_dtype,
                                int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens, int mode,

@@ -21,7 +21,7 @@ POLICY_PPO, POLICY_GSPO = 0, 1
 IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 
 class Norm(Structure):
@@ -70,6 +70,7 @@ SIGNATURES = {
     "orlhf_version": (c_int, []),
     "orlhf_last_error": (c_char_p, []),
     "orlhf_logprob_entropy_fwd": (c_int, [P, c_int, I64, I64, I64, P, c_double, P, P, P, P, c_int, P]),
+    "orlhf_divide_rows_inplace": (c_int, [P, c_int, I64, I64, I64, c_double, P]),
     "orlhf_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P]),
     "orlhf_logprob_entropy_fwd_bwd_max_vocab": (I64, [c_int]),
     "orlhf_logprob_entropy_fwd_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P, P]),
@@ -79,6 +80,7 @@ SIGNATURES = {
     "orlhf_approx_kl_bwd": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
     "orlhf_token_workspace_bytes": (I64, [I64, I64]),
     "orlhf_masked_aggregate_fwd": (c_int, [P, P, c_int, I64, I64, P, c_int, POINTER(Norm), P, P, P, P]),
+    "orlhf_mask_counts": (c_int, [P, c_int, I64, I64, P, P, P, P]),
     "orlhf_masked_aggregate_bwd": (c_int, [P, P, c_int, I64, I64, P, c_int, P, P, P]),
     "orlhf_policy_loss_fwd": (c_int, [P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P]),
     "orlhf_policy_loss_bwd": (c_int, [P, P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P]),

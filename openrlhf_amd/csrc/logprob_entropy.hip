@@ -471,9 +471,53 @@ static int launch_bwd(const void* logits, void* grad, int64_t n_rows, int64_t vo
   return ORLHF_OK;
 }
 
+// logits <- round_to_dtype(logits / divisor), row by row: the reference's in-place
+// logits.div_(temperature) for callers that rely on that side effect.
+struct DivideFn {
+  float divisor;
+  template <int N>
+  __device__ __forceinline__ void vec(float (&x)[N], uint32_t) const {
+#pragma unroll
+    for (int j = 0; j < N; ++j) x[j] = x[j] / divisor;
+  }
+  __device__ __forceinline__ void one(float& x, uint32_t) const { x = x / divisor; }
+};
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void divide_rows_kernel(char* logits, int64_t n_rows, int64_t vocab,
+                                                             int64_t row_stride_bytes, float divisor) {
+  DivideFn fn{divisor};
+  for (int64_t row_i = blockIdx.x; row_i < n_rows; row_i += gridDim.x) {
+    char* row = logits + row_i * row_stride_bytes;
+    const RowGeom g = row_geom<DT>(row, vocab, false);
+    traverse_row<DT, true>(row, row, g, fn);
+  }
+}
+
 }  // namespace orlhf
 
 using namespace orlhf;
+
+extern "C" int orlhf_divide_rows_inplace(void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                                         int64_t row_stride, double divisor, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_rows >= 0 && vocab > 0 && row_stride >= vocab, "divide_rows_inplace: n_rows=%lld vocab=%lld stride=%lld",
+                  (long long)n_rows, (long long)vocab, (long long)row_stride);
+  ORLHF_CHECK_ARG(vocab < (1ll << 29), "divide_rows_inplace: vocab %lld too large", (long long)vocab);
+  ORLHF_CHECK_ARG(divisor == divisor && divisor != 0.0, "divide_rows_inplace: divisor must be a non-zero number");
+  if (n_rows == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(logits != nullptr, "divide_rows_inplace: logits is NULL");
+  const dim3 grid(grid_for_rows(n_rows)), block(kBlock);
+  hipStream_t s = (hipStream_t)stream;
+  char* p = (char*)logits;
+  switch (dtype) {
+    case ORLHF_F32: hipLaunchKernelGGL(divide_rows_kernel<ORLHF_F32>, grid, block, 0, s, p, n_rows, vocab, row_stride * 4, (float)divisor); break;
+    case ORLHF_BF16: hipLaunchKernelGGL(divide_rows_kernel<ORLHF_BF16>, grid, block, 0, s, p, n_rows, vocab, row_stride * 2, (float)divisor); break;
+    case ORLHF_F16: hipLaunchKernelGGL(divide_rows_kernel<ORLHF_F16>, grid, block, 0, s, p, n_rows, vocab, row_stride * 2, (float)divisor); break;
+    default: return fail(ORLHF_ERR_INVALID_ARG, "divide_rows_inplace: unknown dtype %d", dtype);
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_divide_rows_inplace");
+  return ORLHF_OK;
+}
 
 extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows,
                                          int64_t vocab, int64_t row_stride, const int64_t* labels,

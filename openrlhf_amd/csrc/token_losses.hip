@@ -36,6 +36,16 @@ static inline NormArg norm_arg(const orlhf_norm* n) {
 // Each functor evaluates one token: q[] are the quantities to reduce (already multiplied by the
 // mask weight where the reference multiplies), and grad() is d(token loss)/d(input).
 
+constexpr int kAggCounts = 3;  // internal finaliser mode: out = {sum(mask), #rows with sum(mask) > 0}
+
+struct CountTok {  // loss normalisers: the mask alone
+  static constexpr int kQ = 2;
+  __device__ __forceinline__ void eval(int64_t, int64_t, float m, float* q) const {
+    q[0] = m;
+    q[1] = m;
+  }
+};
+
 struct AggTok {  // aggregate_loss / masked_mean: x*m and m
   static constexpr int kQ = 2;
   const float* x;
@@ -159,7 +169,7 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
     }
 #pragma unroll
     for (int i = 0; i < NQ; ++i) tot[i] += rq[i];
-    if (mode == ORLHF_AGG_SEQ_MEAN) {
+    if (mode == ORLHF_AGG_SEQ_MEAN || mode == kAggCounts) {
       if (rq[1] > 0.0) {
         seq_sum += rq[0] / (rq[1] + 1e-8);
         seq_cnt += 1.0;
@@ -183,6 +193,13 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
   seq_sum = block_sum(seq_sum, lds);
   seq_cnt = block_sum(seq_cnt, lds);
 
+  if (mode == kAggCounts) {
+    if (threadIdx.x == 0) {
+      out[0] = (float)tot[1];
+      out[1] = (float)seq_cnt;
+    }
+    return;
+  }
   const bool given = norm.dev != nullptr || norm.value == norm.value;
   const double denom_given = norm.dev != nullptr ? (double)norm.dev[0] : norm.value;
   double scale;  // d(loss)/d(numerator)
@@ -497,6 +514,24 @@ extern "C" int orlhf_masked_aggregate_fwd(const float* x, const void* mask, int 
   }
   launch_final<2>(n_rows, n_chunks, partial, mode, norm_arg(norm), 1.0f, 1, out, row_coef, s);
   ORLHF_CHECK_LAUNCH("orlhf_masked_aggregate_fwd(final)");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_mask_counts(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                                 const int64_t* cu_seqlens, void* workspace, float* out2, orlhf_stream_t stream) {
+  if (int rc = check_rows("mask_counts", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(out2 != nullptr && workspace != nullptr, "mask_counts: NULL out2 / workspace");
+  hipStream_t s = (hipStream_t)stream;
+  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const int n_chunks = (int)chunks_of(n_cols);
+  double* partial = (double*)workspace;
+  if (n_rows > 0) {
+    launch_partial(mask_dtype, rows, mask, CountTok{}, partial, n_chunks, s);
+    ORLHF_CHECK_LAUNCH("orlhf_mask_counts(partial)");
+  }
+  NormArg none{1.0, (double)NAN, nullptr};
+  launch_final<2>(n_rows, n_chunks, partial, kAggCounts, none, 1.0f, 2, out2, nullptr, s);
+  ORLHF_CHECK_LAUNCH("orlhf_mask_counts(final)");
   return ORLHF_OK;
 }
 

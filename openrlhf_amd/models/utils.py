@@ -140,10 +140,33 @@ def logprobs_and_entropy_from_logits(
 
 
 def log_probs_from_logits(
-    logits: torch.Tensor, labels: torch.Tensor, temperature: float = 1.0, inplace_backward: bool = False
+    logits: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float = 1.0,
+    inplace_backward: bool = False,
+    mutate_logits: bool = False,
 ) -> torch.Tensor:
     """log_softmax(logits / temperature) gathered at ``labels``
-    (openrlhf/models/utils.py:139-163), fp32 result."""
+    (openrlhf/models/utils.py:139-163), fp32 result.
+
+    ``mutate_logits=True`` reproduces the reference's side effect for ``temperature != 1``: the
+    caller's logits are divided by the temperature in place (rounded to their dtype) and the
+    log-prob is taken from the stored quotient, exactly the reference's order of operations.
+    It costs an extra read+write of the logits and is for inference-mode callers that read the
+    scaled logits afterwards; it refuses tensors that require grad."""
+    if mutate_logits and temperature != 1.0:
+        if logits.requires_grad and torch.is_grad_enabled():
+            raise RuntimeError("mutate_logits=True changes the logits in place and is not tracked by autograd; "
+                               "call it under torch.no_grad() or leave mutate_logits=False")
+        dev = require_gpu(logits)
+        rows, row_stride, aliases = _as_rows(logits.detach())
+        if not aliases:
+            raise ValueError("mutate_logits=True needs logits whose rows can be addressed in place")
+        with torch.cuda.device(dev):
+            call("orlhf_divide_rows_inplace", ptr(rows), _lib.dtype_code(rows), rows.shape[0], rows.shape[1],
+                 row_stride, float(temperature), stream_of(dev))
+        torch.autograd.graph.increment_version(rows)
+        temperature = 1.0
     return _LogprobEntropy.apply(logits, labels, temperature, True, False, inplace_backward)[0]
 
 

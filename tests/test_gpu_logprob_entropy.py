@@ -228,3 +228,27 @@ def test_backward_single_outputs_and_reuse_guard(cuda):
     out.backward(retain_graph=True)
     with pytest.raises(RuntimeError):
         out.backward()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_mutate_logits_reproduces_the_reference_side_effect(cuda, dtype):
+    """mutate_logits=True: the logits end up divided by the temperature in place (rounded to
+    their dtype, torch's div_) and the log-prob is that of the stored quotient."""
+    from openrlhf_amd.models.utils import log_probs_from_logits
+
+    x, labels = _logits(21, 5003, dtype, 2.0, seed=77)
+    t = 0.6
+    z = x.clone().div_(t)  # what the reference leaves in the caller's tensor
+    ref = otn.log_probs_from_logits(z.double(), labels, 1.0)
+    xd = x.to(cuda)
+    with torch.no_grad():
+        lp = log_probs_from_logits(xd, labels.to(cuda), t, mutate_logits=True)
+    if dtype == torch.float32:
+        assert (xd.cpu() - z).abs().max().item() <= 2e-7 * z.abs().max().item()
+    else:
+        assert torch.equal(xd.cpu(), z)
+    atol = FP32_ATOL if dtype == torch.float32 else BF16_ATOL
+    assert (lp.cpu().double() - otn.log_probs_from_logits(xd.cpu().double(), labels, 1.0)).abs().max().item() <= atol
+    assert (lp.cpu().double() - ref).abs().max().item() <= atol
+    with pytest.raises(RuntimeError):
+        log_probs_from_logits(x.to(cuda).requires_grad_(True), labels.to(cuda), t, mutate_logits=True)

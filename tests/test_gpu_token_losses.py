@@ -370,3 +370,41 @@ def test_config1_plumbing(cuda):
     _close(klm, klm64, ATOL)
     (out[0] + 0.01 * klm).backward()
     assert (xd.grad.cpu().double() - x64.grad).abs().max().item() <= 1e-7
+
+
+# ------------------------------------------------------------------ loss normalisers
+def test_loss_batch_info_and_grad_accum_window(cuda):
+    """tests/test_loss_aggregation.py:86-94,151-193 of the reference on the HIP path: counts from
+    the mask kernel, fully masked rows excluded, and a gradient-accumulation window that turns
+    per-micro-batch losses into one token mean over the optimizer step."""
+    from openrlhf_amd.models.loss import aggregate_loss
+    from openrlhf_amd.utils.loss_utils import get_loss_batch_info, iter_grad_accum_global_norm, mask_counts
+
+    d = cuda
+    _, _, _, _, mask = _tok(33, 2100, seed=13)
+    mask[7] = 0
+    tokens, samples = mask_counts(mask.to(d).bool())
+    assert tokens.item() == mask.sum().item() and samples.item() == 32.0
+    loss = torch.tensor([[1.0, 3.0], [5.0, 7.0]], device=d)
+    m = torch.tensor([[1.0, 1.0], [0.0, 0.0]], device=d)
+    info = get_loss_batch_info(strategy=object(), loss_mask=m)
+    assert info["global_batch_size"].item() == 1.0 and info["batch_num_tokens"].item() == 2.0 and info["dp_size"] == 1
+    assert torch.allclose(aggregate_loss(loss, m, token_level_loss=False, **info), torch.tensor(2.0, device=d))
+    info = get_loss_batch_info(strategy=object(), loss_mask=m, batch_num_tokens=5.0, global_batch_size=3)
+    assert info["batch_num_tokens"].item() == 5.0 and info["global_batch_size"].item() == 3.0
+
+    mb0, m0 = torch.tensor([[1.0, 2.0, 0.0]], device=d), torch.tensor([[1.0, 1.0, 0.0]], device=d)
+    mb1 = torch.tensor([[3.0, 4.0, 5.0], [6.0, 7.0, 0.0]], device=d)
+    m1 = torch.tensor([[1.0, 1.0, 1.0], [1.0, 1.0, 0.0]], device=d)
+    n_global = m0.sum() + m1.sum()
+    expected = ((mb0 * m0).sum() + (mb1 * m1).sum()) / n_global
+    items = [(mb0, m0), (mb1, m1)]
+    emitted = list(iter_grad_accum_global_norm(items, strategy=object(), accumulated_gradient=2, mask_fn=lambda it: it[1]))
+    assert len(emitted) == 2
+    acc = 0.0
+    for (x, mk), inf in emitted:
+        assert torch.allclose(inf["batch_num_tokens"], n_global / 2)
+        acc = acc + aggregate_loss(x, mk, dp_size=inf["dp_size"], batch_num_tokens=inf["batch_num_tokens"]) / 2
+    assert torch.allclose(acc, expected)
+    per_mb = (aggregate_loss(mb0, m0) + aggregate_loss(mb1, m1)) / 2
+    assert not torch.allclose(per_mb, expected)
