@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 5
+#define ORLHF_ABI_VERSION 6
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -51,6 +51,12 @@ enum orlhf_agg_mode {
 };
 enum orlhf_policy_type { ORLHF_POLICY_PPO = 0, ORLHF_POLICY_GSPO = 1 };
 enum orlhf_is_correction { ORLHF_IS_NONE = 0, ORLHF_IS_TIS = 1, ORLHF_IS_ICEPOP = 2, ORLHF_IS_SEQ_MASK_TIS = 3 };
+enum orlhf_pair_loss {
+  ORLHF_PAIR_DPO_SIGMOID = 0, /* DPOLoss, ipo=False (label smoothing = conservative DPO)   */
+  ORLHF_PAIR_DPO_IPO = 1,     /* DPOLoss, ipo=True                                          */
+  ORLHF_PAIR_LOGSIGMOID = 2,  /* PairWiseLoss: -logsigmoid(chosen - rejected [- margin])    */
+  ORLHF_PAIR_LOGEXP = 3       /* LogExpLoss: log(1 + exp(rejected - chosen))                */
+};
 enum orlhf_group_estimator {
   ORLHF_GROUP_IDENTITY = 0, /* gae, reinforce: rewards unchanged                                 */
   ORLHF_GROUP_RLOO = 1,     /* r - (sum - r)/(n-1)                                               */
@@ -337,6 +343,49 @@ int orlhf_group_normalize(const float* rewards, const int64_t* indices, int64_t 
 int64_t orlhf_whiten_workspace_bytes(int64_t n);
 int orlhf_masked_whiten(const float* x, const void* mask, int mask_dtype, int64_t n, int std_norm,
                         void* workspace, float* out, float* stats, orlhf_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Sequence-level pieces of the preference trainers (the callers next to the hot path).
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * DPOTrainer._get_batch_logps (openrlhf/trainer/dpo_trainer.py:362-382): per-sequence sum and
+ * mean of per-token log-probs [n_rows, n_cols] (n_cols = T-1) under the loss mask
+ *   m[b,t] = attention_mask[b,t+1] != 0  and  t+1 >= prompt_id_lens[b]
+ * built on the fly from attention_mask [n_rows, n_cols+1] (mask dtype as elsewhere; NONE = all
+ * ones) and prompt_id_lens (int64 [n_rows], nullable = no prompt masking); the reference clones
+ * the mask, clears it row by row from Python and shifts it. sums / means / counts (float
+ * [n_rows], each nullable): sum(lp*m), that sum / sum(m) (NaN when no loss token, as torch) and
+ * sum(m) (keep it for the backward).
+ */
+int orlhf_sequence_logps_fwd(const float* per_token_logps, const void* attention_mask, int mask_dtype,
+                             const int64_t* prompt_id_lens, int64_t n_rows, int64_t n_cols,
+                             float* sums, float* means, float* counts, orlhf_stream_t stream);
+/* g_per_token[b,t] = m[b,t] * (g_sums[b] + g_means[b] / counts[b]); g_sums / g_means nullable. */
+int orlhf_sequence_logps_bwd(const float* g_sums, const float* g_means, const void* attention_mask,
+                             int mask_dtype, const int64_t* prompt_id_lens, const float* counts,
+                             int64_t n_rows, int64_t n_cols, float* g_per_token,
+                             orlhf_stream_t stream);
+
+/*
+ * Pairwise losses over n (chosen, rejected) scalars, mean over pairs (NaN for n == 0):
+ * DPOLoss (openrlhf/models/loss.py:300-335), PairWiseLoss (:272-284), LogExpLoss (:287-297).
+ * logit z = (chosen - rejected) - (ref_chosen - ref_rejected); ref_chosen / ref_rejected are
+ * nullable (0): for PairWiseLoss pass the margin as ref_chosen. kind: enum orlhf_pair_loss.
+ *   DPO_SIGMOID: -logsigmoid(beta z)(1 - label_smoothing) - logsigmoid(-beta z) label_smoothing
+ *   DPO_IPO: (z - 1/(2 beta))^2      LOGSIGMOID: -logsigmoid(z)      LOGEXP: log(1 + exp(-z))
+ * chosen_rewards / rejected_rewards (float [n], nullable): beta*(chosen - ref_chosen) and
+ * beta*(rejected - ref_rejected), the detached reward estimates DPOLoss returns.
+ */
+int orlhf_pair_loss_fwd(const float* chosen, const float* rejected, const float* ref_chosen,
+                        const float* ref_rejected, int64_t n, int kind, double beta,
+                        double label_smoothing, float* loss, float* chosen_rewards,
+                        float* rejected_rewards, orlhf_stream_t stream);
+/* g_chosen = g_out[0]/n * dloss/dz, g_rejected = -g_chosen (each nullable). */
+int orlhf_pair_loss_bwd(const float* g_out, const float* chosen, const float* rejected,
+                        const float* ref_chosen, const float* ref_rejected, int64_t n, int kind,
+                        double beta, double label_smoothing, float* g_chosen, float* g_rejected,
+                        orlhf_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -20,8 +20,9 @@ AGG_TOKEN_MEAN, AGG_SEQ_MEAN, AGG_ROW_MEAN = 0, 1, 2
 POLICY_PPO, POLICY_GSPO = 0, 1
 IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
+PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 
 class Norm(Structure):
@@ -92,6 +93,10 @@ SIGNATURES = {
     "orlhf_group_normalize": (c_int, [P, P, I64, I64, c_int, P, P, P, P]),
     "orlhf_whiten_workspace_bytes": (I64, [I64]),
     "orlhf_masked_whiten": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
+    "orlhf_sequence_logps_fwd": (c_int, [P, P, c_int, P, I64, I64, P, P, P, P]),
+    "orlhf_sequence_logps_bwd": (c_int, [P, P, P, c_int, P, P, I64, I64, P, P]),
+    "orlhf_pair_loss_fwd": (c_int, [P, P, P, P, I64, c_int, c_double, c_double, P, P, P, P]),
+    "orlhf_pair_loss_bwd": (c_int, [P, P, P, P, P, I64, c_int, c_double, c_double, P, P, P]),
 }
 
 _lib = None

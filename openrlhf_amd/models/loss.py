@@ -5,6 +5,9 @@ Mirrors (paths relative to the OpenRLHF tree):
   SFTLoss          openrlhf/models/loss.py:87-113
   PolicyLoss       openrlhf/models/loss.py:116-230
   ValueLoss        openrlhf/models/loss.py:233-269
+  PairWiseLoss     openrlhf/models/loss.py:272-284
+  LogExpLoss       openrlhf/models/loss.py:287-297
+  DPOLoss          openrlhf/models/loss.py:300-335
 
 Each loss is one elementwise + reduction launch pair forward and one elementwise launch
 backward instead of the reference's chain of ~20 eager kernels. Per-token inputs are consumed
@@ -251,3 +254,76 @@ class ValueLoss(nn.Module):
             values, old_values if self.clip_eps is not None else None, returns, action_mask, self.clip_eps,
             self.token_level_loss, dp_size, norm_value, cu_seqlens,
         )
+
+
+class _PairLossFn(torch.autograd.Function):
+    """mean over pairs of a pairwise loss of z = (chosen - rejected) - (ref_chosen - ref_rejected)."""
+
+    @staticmethod
+    def forward(ctx, chosen, rejected, ref_chosen, ref_rejected, kind, beta, label_smoothing, want_rewards):
+        dev = require_gpu(chosen, rejected, ref_chosen, ref_rejected)
+        if chosen.shape != rejected.shape:
+            raise ValueError(f"chosen {tuple(chosen.shape)} and rejected {tuple(rejected.shape)} differ in shape")
+        a, b = _f32(chosen).reshape(-1), _f32(rejected).reshape(-1)
+        c = None if ref_chosen is None else _f32(ref_chosen.detach()).expand_as(chosen).reshape(-1).contiguous()
+        d = None if ref_rejected is None else _f32(ref_rejected.detach()).expand_as(chosen).reshape(-1).contiguous()
+        n = a.numel()
+        loss = torch.empty(1, dtype=torch.float32, device=dev)
+        cr = torch.empty(n, dtype=torch.float32, device=dev) if want_rewards else None
+        rr = torch.empty(n, dtype=torch.float32, device=dev) if want_rewards else None
+        with torch.cuda.device(dev):
+            call("orlhf_pair_loss_fwd", ptr(a), ptr(b), ptr(c), ptr(d), n, kind, float(beta), float(label_smoothing),
+                 ptr(loss), ptr(cr), ptr(rr), stream_of(dev))
+        ctx.save_for_backward(a, b, c, d)
+        ctx.cfg = (kind, float(beta), float(label_smoothing), chosen.shape, chosen.dtype, rejected.dtype)
+        if want_rewards:
+            cr, rr = cr.view(chosen.shape), rr.view(chosen.shape)
+            ctx.mark_non_differentiable(cr, rr)
+        return loss.reshape(()), cr, rr
+
+    @staticmethod
+    def backward(ctx, g_loss, _g_cr, _g_rr):
+        a, b, c, d = ctx.saved_tensors
+        kind, beta, smooth, shape, dt_a, dt_b = ctx.cfg
+        dev = a.device
+        g = g_loss.reshape(1).to(torch.float32).contiguous()
+        ga = torch.empty_like(a) if ctx.needs_input_grad[0] else None
+        gb = torch.empty_like(b) if ctx.needs_input_grad[1] else None
+        with torch.cuda.device(dev):
+            call("orlhf_pair_loss_bwd", ptr(g), ptr(a), ptr(b), ptr(c), ptr(d), a.numel(), kind, beta, smooth,
+                 ptr(ga), ptr(gb), stream_of(dev))
+        ga = None if ga is None else ga.view(shape).to(dt_a)
+        gb = None if gb is None else gb.view(shape).to(dt_b)
+        return ga, gb, None, None, None, None, None, None
+
+
+class DPOLoss(nn.Module):
+    """DPO / conservative DPO / IPO preference loss (openrlhf/models/loss.py:300-335): returns
+    ``(loss, chosen_rewards, rejected_rewards)``; the reference log-probs carry no gradient."""
+
+    def __init__(self, beta: float, label_smoothing: float = 0.0, ipo: bool = False) -> None:
+        super().__init__()
+        self.beta = beta
+        self.label_smoothing = label_smoothing
+        self.ipo = ipo
+
+    def forward(self, policy_chosen_logps, policy_rejected_logps, reference_chosen_logps, reference_rejected_logps):
+        kind = _lib.PAIR_DPO_IPO if self.ipo else _lib.PAIR_DPO_SIGMOID
+        return _PairLossFn.apply(policy_chosen_logps, policy_rejected_logps, reference_chosen_logps,
+                                 reference_rejected_logps, kind, self.beta, self.label_smoothing, True)
+
+
+class PairWiseLoss(nn.Module):
+    """Reward-model pairwise loss -logsigmoid(chosen - rejected [- margin]).mean()
+    (openrlhf/models/loss.py:272-284)."""
+
+    def forward(self, chosen_reward, reject_reward, margin=None):
+        return _PairLossFn.apply(chosen_reward, reject_reward, margin, None, _lib.PAIR_LOGSIGMOID, 1.0, 0.0, False)[0]
+
+
+class LogExpLoss(nn.Module):
+    """Reward-model loss log(1 + exp(rejected - chosen)).mean(); the margin is ignored, as in the
+    reference (openrlhf/models/loss.py:287-297)."""
+
+    def forward(self, chosen_reward, reject_reward, margin=None):
+        return _PairLossFn.apply(chosen_reward, reject_reward, None, None, _lib.PAIR_LOGEXP, 1.0, 0.0, False)[0]

@@ -1,4 +1,5 @@
-"""Oracle for openrlhf/models/loss.py (aggregate_loss, PolicyLoss, ValueLoss). Test
+"""Oracle for openrlhf/models/loss.py (aggregate_loss, PolicyLoss, ValueLoss, DPOLoss, PairWiseLoss,
+LogExpLoss) and the DPO trainer's per-sequence log-prob sums. Test
 infrastructure, CPU torch; differentiable, so torch autograd is the gradient oracle."""
 import torch
 
@@ -111,3 +112,42 @@ def loss_batch_info(loss_mask):
     tokens = loss_mask.sum().to(torch.float32)
     samples = (loss_mask.reshape(loss_mask.shape[0], -1).sum(dim=-1) > 0).sum().to(torch.float32)
     return {"dp_size": 1, "batch_num_tokens": tokens, "global_batch_size": samples}
+
+
+def get_batch_logps(per_token_logps, attention_mask, prompt_id_lens):
+    """DPOTrainer._get_batch_logps (openrlhf/trainer/dpo_trainer.py:362-382): clone the attention
+    mask as bool, clear each row's prompt, drop the first column, then masked sum and mean."""
+    loss_masks = attention_mask.clone().bool()
+    for mask, source_len in zip(loss_masks, prompt_id_lens):
+        mask[:source_len] = False
+    loss_masks = loss_masks[:, 1:]
+    sums = (per_token_logps * loss_masks).sum(-1)
+    means = (per_token_logps * loss_masks).sum(-1) / loss_masks.sum(-1)
+    return sums, means
+
+
+def dpo_loss(policy_chosen, policy_rejected, reference_chosen, reference_rejected, beta, label_smoothing=0.0,
+             ipo=False):
+    """DPOLoss.forward (openrlhf/models/loss.py:300-335)."""
+    F = torch.nn.functional
+    logits = (policy_chosen - policy_rejected) - (reference_chosen - reference_rejected)
+    if ipo:
+        losses = (logits - 1 / (2 * beta)) ** 2
+    else:
+        losses = -F.logsigmoid(beta * logits) * (1 - label_smoothing) - F.logsigmoid(-beta * logits) * label_smoothing
+    chosen_rewards = beta * (policy_chosen - reference_chosen).detach()
+    rejected_rewards = beta * (policy_rejected - reference_rejected).detach()
+    return losses.mean(), chosen_rewards, rejected_rewards
+
+
+def pairwise_loss(chosen_reward, reject_reward, margin=None):
+    """PairWiseLoss.forward (openrlhf/models/loss.py:272-284)."""
+    F = torch.nn.functional
+    if margin is not None:
+        return (-F.logsigmoid(chosen_reward - reject_reward - margin)).mean()
+    return (-F.logsigmoid(chosen_reward - reject_reward)).mean()
+
+
+def logexp_loss(chosen_reward, reject_reward, margin=None):
+    """LogExpLoss.forward (openrlhf/models/loss.py:287-297); the margin is unused there too."""
+    return torch.log(1 + torch.exp(reject_reward - chosen_reward)).mean()

@@ -241,6 +241,52 @@ def whiten(adv, mask, no_std_norm):
     return [[(x - mean) * rstd for x in row] for row in adv]
 
 
+def sequence_logps(lp, att, prompt_lens, g_sum, g_mean):
+    """Scalar restatement of per-sequence sums / means over response tokens and their gradient:
+    token t counts when att[b][t+1] != 0 and t+1 >= prompt_lens[b]."""
+    sums, means, grads = [], [], []
+    for b, row in enumerate(lp):
+        m = [1.0 if (att[b][t + 1] != 0 and t + 1 >= prompt_lens[b]) else 0.0 for t in range(len(row))]
+        s, c = sum(x * w for x, w in zip(row, m)), sum(m)
+        sums.append(s)
+        means.append(s / c if c > 0 else None)
+        grads.append([w * (g_sum[b] + (g_mean[b] / c if c > 0 else 0.0)) for w in m] if c > 0 else None)
+    return sums, means, grads
+
+
+def log_sigmoid(x):
+    return -math.log1p(math.exp(-x)) if x >= 0 else x - math.log1p(math.exp(x))
+
+
+def sigmoid(x):
+    return 1.0 / (1.0 + math.exp(-x)) if x >= 0 else math.exp(x) / (1.0 + math.exp(x))
+
+
+def pair_loss(kind, chosen, rejected, ref_c, ref_r, beta, smooth):
+    """mean loss, d(mean loss)/d(chosen_i) (= -d/d(rejected_i)) and the DPO reward estimates."""
+    n = len(chosen)
+    losses, grads = [], []
+    for i in range(n):
+        z = (chosen[i] - rejected[i]) - ((ref_c[i] if ref_c else 0.0) - (ref_r[i] if ref_r else 0.0))
+        if kind == "dpo":
+            losses.append(-log_sigmoid(beta * z) * (1 - smooth) - log_sigmoid(-beta * z) * smooth)
+            grads.append(beta * (-(1 - smooth) * sigmoid(-beta * z) + smooth * sigmoid(beta * z)) / n)
+        elif kind == "ipo":
+            losses.append((z - 1 / (2 * beta)) ** 2)
+            grads.append(2 * (z - 1 / (2 * beta)) / n)
+        elif kind == "pairwise":
+            losses.append(-log_sigmoid(z))
+            grads.append(-sigmoid(-z) / n)
+        else:  # logexp: log(1 + exp(-z))
+            losses.append(-log_sigmoid(z))
+            grads.append(-sigmoid(-z) / n)
+    out = {"loss": sum(losses) / n, "g_chosen": grads}
+    if kind in ("dpo", "ipo"):
+        out["chosen_rewards"] = [beta * (chosen[i] - ref_c[i]) for i in range(n)]
+        out["rejected_rewards"] = [beta * (rejected[i] - ref_r[i]) for i in range(n)]
+    return out
+
+
 def main():
     rng = random.Random(20240607)
     gold = {}
@@ -340,6 +386,40 @@ def main():
         shaped, std = group_normalize(exp_order, perm, n, est)
         gold["group_normalize"]["cases"].append({"estimator": est, "out": shaped, "group_std": std})
     gold["whiten"] = [{"no_std_norm": f, "out": whiten(adv, mask, f)} for f in (False, True)]
+
+    # sequence-level: response sums / means with left padding, right padding, an attention hole and
+    # a sequence whose prompt covers everything; pairwise losses with large and tiny logits
+    att = [[1] * (a + 1) for _ in range(b)]
+    att[0][0] = att[0][1] = 0
+    for t in range(13, a + 1):
+        att[1][t] = 0
+    att[2][9] = 0
+    prompt_lens = [5, 3, 7, a + 1]
+    g_sum = [f32(rng.gauss(0, 1)) for _ in range(b)]
+    g_mean = [f32(rng.gauss(0, 1)) for _ in range(b)]
+    sums, means, grads = sequence_logps(lp, att, prompt_lens, g_sum, g_mean)
+    gold["sequence_logps"] = {"attention_mask": att, "prompt_id_lens": prompt_lens, "g_sums": g_sum, "g_means": g_mean,
+                              "sums": sums, "means": means, "grad": grads}
+    n_pairs = 7
+    chosen = [f32(rng.gauss(-40, 12)) for _ in range(n_pairs)]
+    rejected = [f32(c + rng.gauss(0, 6)) for c in chosen]
+    ref_c = [f32(c + rng.gauss(0, 3)) for c in chosen]
+    ref_r = [f32(r_ + rng.gauss(0, 3)) for r_ in rejected]
+    rejected[0] = f32(chosen[0] - 60.0)
+    rejected[1] = f32(chosen[1] + 60.0)
+    margin = [f32(rng.uniform(0, 2)) for _ in range(n_pairs)]
+    cr = [f32(rng.gauss(0, 2)) for _ in range(n_pairs)]
+    rr = [f32(rng.gauss(0, 2)) for _ in range(n_pairs)]
+    gold["pair_loss"] = {
+        "chosen": chosen, "rejected": rejected, "ref_chosen": ref_c, "ref_rejected": ref_r,
+        "chosen_reward": cr, "reject_reward": rr, "margin": margin,
+        "dpo": [{"beta": be, "label_smoothing": ls, "ipo": ipo,
+                 "out": pair_loss("ipo" if ipo else "dpo", chosen, rejected, ref_c, ref_r, be, ls)}
+                for be, ls, ipo in ((0.1, 0.0, False), (0.5, 0.1, False), (0.1, 0.0, True))],
+        "pairwise": pair_loss("pairwise", cr, rr, None, None, 1.0, 0.0),
+        "pairwise_margin": pair_loss("pairwise", cr, rr, margin, None, 1.0, 0.0),
+        "logexp": pair_loss("logexp", cr, rr, None, None, 1.0, 0.0),
+    }
 
     with open(OUT, "w") as fh:
         json.dump(gold, fh)

@@ -283,3 +283,57 @@ def test_group_normalize_and_whiten_golden():
     close((out[0] * mask).sum() / mask.sum(), 0.0, 1e-12)
     close(((out[0] ** 2) * mask).sum() / mask.sum(), 1.0, 1e-9)
     assert out[0][2].abs().min() > 0  # the fully masked row is whitened too
+
+
+# ------------------------------------------------------------------ sequence level (DPO / RM)
+def test_sequence_logps_golden_and_closed_forms():
+    s = GOLD["sequence_logps"]
+    lp = T(GOLD["tokens"]["log_probs"]).requires_grad_(True)
+    att, lens = torch.tensor(s["attention_mask"]), s["prompt_id_lens"]
+    sums, means = ol.get_batch_logps(lp, att, lens)
+    close(sums.detach(), s["sums"], 1e-12)
+    for b, ref in enumerate(s["means"]):
+        if ref is None:
+            assert torch.isnan(means[b])
+        else:
+            close(means[b].detach(), ref, 1e-12)
+    keep = [b for b, ref in enumerate(s["means"]) if ref is not None]
+    (g,) = torch.autograd.grad((sums * T(s["g_sums"])).sum() + (means[keep] * T(s["g_means"])[keep]).sum(), lp)
+    for b in keep:
+        close(g[b], s["grad"][b], 1e-12)
+    # no prompt, full attention: plain row sums and means of every column
+    full = torch.ones(4, 17, dtype=torch.long)
+    sums, means = ol.get_batch_logps(lp.detach(), full, [0, 0, 0, 0])
+    close(sums, lp.detach().sum(-1), 1e-12)
+    close(means, lp.detach().mean(-1), 1e-12)
+    # the prompt length counts in tokens of the unshifted sequence: prompt p leaves columns p-1..
+    sums, _ = ol.get_batch_logps(lp.detach(), full, [4, 4, 4, 4])
+    close(sums, lp.detach()[:, 3:].sum(-1), 1e-12)
+
+
+def test_pair_losses_golden_and_closed_forms():
+    p = GOLD["pair_loss"]
+    c, r, rc, rr = (T(p[k]) for k in ("chosen", "rejected", "ref_chosen", "ref_rejected"))
+    for case in p["dpo"]:
+        cg = c.clone().requires_grad_(True)
+        rg = r.clone().requires_grad_(True)
+        loss, cr_, rr_ = ol.dpo_loss(cg, rg, rc, rr, case["beta"], case["label_smoothing"], case["ipo"])
+        close(loss.detach(), case["out"]["loss"], 1e-11)
+        close(cr_, case["out"]["chosen_rewards"], 1e-12)
+        close(rr_, case["out"]["rejected_rewards"], 1e-12)
+        gc, gr = torch.autograd.grad(loss, (cg, rg))
+        close(gc, case["out"]["g_chosen"], 1e-11)
+        close(gr, -T(case["out"]["g_chosen"]), 1e-11)
+    a, b, m = T(p["chosen_reward"]), T(p["reject_reward"]), T(p["margin"])
+    close(ol.pairwise_loss(a, b), p["pairwise"]["loss"], 1e-12)
+    close(ol.pairwise_loss(a, b, m), p["pairwise_margin"]["loss"], 1e-12)
+    close(ol.logexp_loss(a, b), p["logexp"]["loss"], 1e-12)
+    # closed forms: equal rewards give ln 2; the two reward-model losses are the same function
+    z = torch.zeros(5, dtype=torch.float64)
+    close(ol.pairwise_loss(z, z), math.log(2.0), 1e-15)
+    close(ol.logexp_loss(a, b), ol.pairwise_loss(a, b), 1e-12)
+    # DPO at the reference policy is ln 2 whatever beta; IPO's minimum sits at z = 1/(2 beta)
+    close(ol.dpo_loss(c, r, c, r, 0.3)[0], math.log(2.0), 1e-15)
+    close(ol.dpo_loss(c + 1 / (2 * 0.25), c, rc, rc, 0.25, ipo=True)[0], 0.0, 1e-12)
+    # label smoothing 0.5 makes the loss even in z
+    close(ol.dpo_loss(c, r, rc, rr, 0.2, 0.5)[0], ol.dpo_loss(r, c, rr, rc, 0.2, 0.5)[0], 1e-12)
