@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 6
+#define ORLHF_ABI_VERSION 7
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -386,6 +386,42 @@ int orlhf_pair_loss_bwd(const float* g_out, const float* chosen, const float* re
                         const float* ref_chosen, const float* ref_rejected, int64_t n, int kind,
                         double beta, double label_smoothing, float* g_chosen, float* g_rejected,
                         orlhf_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Row layouts: padded [n_rows, n_cols] + mask  <->  packed flat tokens + cu_seqlens. Index work
+ * and copies, bit-exact. The per-token entry points above take either layout.
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * Per mask row: first = first non-zero column (n_cols if none), end = one past the last non-zero
+ * column (0 if none), length = end - first (0 if none); each output int64 [n_rows], nullable.
+ * Right-padded rows: length is what remove_padding_in_sequences keeps
+ * (openrlhf/trainer/ppo_utils/experience.py:236-247, attention_mask.flip(0).argmax()); interior
+ * zeros stay inside the extent.
+ */
+int orlhf_row_extents(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                      int64_t* first, int64_t* end, int64_t* length, orlhf_stream_t stream);
+
+/* cu_seqlens[0] = 0, cu_seqlens[i+1] = cu_seqlens[i] + lengths[i] (int64 [n_rows+1]): the
+ * boundaries flash-attn's unpad_input returns (openrlhf/models/ring_attn_utils.py:129-140). */
+int orlhf_cu_seqlens(const int64_t* lengths, int64_t n_rows, int64_t* cu_seqlens,
+                     orlhf_stream_t stream);
+
+/* dst[cu[b] + j] = src[b, first[b] + j] for j < cu[b+1] - cu[b]; first nullable (0). Elements
+ * are elem_bytes (1, 2, 4, 8) wide and copied as bits. */
+int orlhf_pack_rows(const void* src, int elem_bytes, int64_t n_rows, int64_t n_cols,
+                    const int64_t* first, const int64_t* cu_seqlens, void* dst,
+                    orlhf_stream_t stream);
+
+/*
+ * zero_pad_sequences(..., side, value, stack=True) (openrlhf/utils/utils.py:93-106) from the
+ * packed layout: dst [n_rows, n_cols] is filled with fill_bits (low elem_bytes bytes) and row b
+ * receives src[cu[b] .. cu[b+1]) at its right end (left_side = 1: padding on the left) or at
+ * its left end (left_side = 0). Rows longer than n_cols are cut.
+ */
+int orlhf_pad_rows(const void* src, int elem_bytes, const int64_t* cu_seqlens, int64_t n_rows,
+                   int64_t n_cols, int left_side, uint64_t fill_bits, void* dst,
+                   orlhf_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -6,7 +6,7 @@ is not on a GPU, the call raises. Build with ``python -m openrlhf_amd.csrc.build
 import ctypes
 import math
 import os
-from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int64, c_void_p
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int64, c_uint64, c_void_p
 
 import torch
 
@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 
 class Norm(Structure):
@@ -93,6 +93,10 @@ SIGNATURES = {
     "orlhf_group_normalize": (c_int, [P, P, I64, I64, c_int, P, P, P, P]),
     "orlhf_whiten_workspace_bytes": (I64, [I64]),
     "orlhf_masked_whiten": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
+    "orlhf_row_extents": (c_int, [P, c_int, I64, I64, P, P, P, P]),
+    "orlhf_cu_seqlens": (c_int, [P, I64, P, P]),
+    "orlhf_pack_rows": (c_int, [P, c_int, I64, I64, P, P, P, P]),
+    "orlhf_pad_rows": (c_int, [P, c_int, P, I64, I64, c_int, c_uint64, P, P]),
     "orlhf_sequence_logps_fwd": (c_int, [P, P, c_int, P, I64, I64, P, P, P, P]),
     "orlhf_sequence_logps_bwd": (c_int, [P, P, P, c_int, P, P, I64, I64, P, P]),
     "orlhf_pair_loss_fwd": (c_int, [P, P, P, P, I64, c_int, c_double, c_double, P, P, P, P]),

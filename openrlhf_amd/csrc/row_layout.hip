@@ -1,0 +1,184 @@
+// Row layout kernels for gfx950: between the reference's padded [B, A] per-token tensors (plus a
+// mask) and the packed layout (flat tokens + cu_seqlens) that every per-token kernel of this
+// library also accepts. Pure index work and copies: bit-exact, HBM/latency-bound.
+//
+//   row_extents   first / one-past-last non-zero column of every mask row
+//   cu_seqlens    exclusive prefix sum of row lengths (one workgroup, chained 256-wide scans)
+//   pack_rows     dst[cu[b] + j] = src[b, first[b] + j]
+//   pad_rows      dst[b, :] = fill, then the row's tokens on the left or on the right side
+#include "common.h"
+
+namespace orlhf {
+
+template <int MASK_DT>
+__global__ __launch_bounds__(kBlock) void row_extents_kernel(const void* __restrict__ mask, int64_t n_rows,
+                                                             int64_t n_cols, int64_t* __restrict__ first,
+                                                             int64_t* __restrict__ end,
+                                                             int64_t* __restrict__ length) {
+  __shared__ long long lds_lo[kWavesPerBlock], lds_hi[kWavesPerBlock];
+  for (int64_t b = blockIdx.x; b < n_rows; b += gridDim.x) {
+    long long lo = n_cols, hi = 0;  // no non-zero column: first = n_cols, end = 0
+    for (int64_t t = threadIdx.x; t < n_cols; t += kBlock) {
+      if (load_mask<MASK_DT>(mask, b * n_cols + t) != 0.0f) {
+        lo = t < lo ? t : lo;
+        hi = t + 1 > hi ? t + 1 : hi;
+      }
+    }
+#pragma unroll
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+      const long long l2 = __shfl_xor(lo, o, kWave), h2 = __shfl_xor(hi, o, kWave);
+      lo = l2 < lo ? l2 : lo;
+      hi = h2 > hi ? h2 : hi;
+    }
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) lds_lo[wave] = lo, lds_hi[wave] = hi;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        lo = lds_lo[w] < lo ? lds_lo[w] : lo;
+        hi = lds_hi[w] > hi ? lds_hi[w] : hi;
+      }
+      if (first != nullptr) first[b] = lo;
+      if (end != nullptr) end[b] = hi;
+      if (length != nullptr) length[b] = hi > lo ? hi - lo : 0;
+    }
+    __syncthreads();
+  }
+}
+
+// cu[0] = 0, cu[i+1] = cu[i] + lengths[i]. One workgroup walks the rows 256 at a time.
+__global__ __launch_bounds__(kBlock) void cu_seqlens_kernel(const int64_t* __restrict__ lengths, int64_t n_rows,
+                                                            int64_t* __restrict__ cu) {
+  __shared__ long long wave_tot[kWavesPerBlock];
+  __shared__ long long carry_s;
+  if (threadIdx.x == 0) {
+    carry_s = 0;
+    cu[0] = 0;
+  }
+  __syncthreads();
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  for (int64_t base = 0; base < n_rows; base += kBlock) {
+    const int64_t i = base + threadIdx.x;
+    long long v = i < n_rows ? lengths[i] : 0;
+#pragma unroll
+    for (int o = 1; o < kWave; o <<= 1) {  // inclusive scan inside the wave
+      const long long up = __shfl_up(v, o, kWave);
+      if (lane >= o) v += up;
+    }
+    if (lane == kWave - 1) wave_tot[wave] = v;
+    __syncthreads();
+    long long before = carry_s;
+    for (int w = 0; w < wave; ++w) before += wave_tot[w];
+    if (i < n_rows) cu[i + 1] = before + v;
+    __syncthreads();
+    if (threadIdx.x == kBlock - 1) carry_s = before + v;
+    __syncthreads();
+  }
+}
+
+template <typename E>
+__global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__ src, int64_t n_rows, int64_t n_cols,
+                                                           const int64_t* __restrict__ first,
+                                                           const int64_t* __restrict__ cu, E* __restrict__ dst) {
+  const int64_t chunks = (n_cols + kBlock - 1) / kBlock;
+  for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
+    const int64_t b = w / chunks, j = (w % chunks) * kBlock + threadIdx.x;
+    const int64_t start = cu[b], len = cu[b + 1] - start;
+    const int64_t f = first != nullptr ? first[b] : 0;
+    if (j < len && f + j < n_cols) dst[start + j] = src[b * n_cols + f + j];
+  }
+}
+
+template <typename E>
+__global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ src, const int64_t* __restrict__ cu,
+                                                          int64_t n_rows, int64_t n_cols, int left, E fill,
+                                                          E* __restrict__ dst) {
+  const int64_t chunks = (n_cols + kBlock - 1) / kBlock;
+  for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
+    const int64_t b = w / chunks, t = (w % chunks) * kBlock + threadIdx.x;
+    if (t >= n_cols) continue;
+    const int64_t start = cu[b];
+    int64_t len = cu[b + 1] - start;
+    len = len < n_cols ? len : n_cols;  // a longer row is cut at n_cols (checked by the caller when it can)
+    const int64_t j = left ? t - (n_cols - len) : t;
+    dst[b * n_cols + t] = (j >= 0 && j < len) ? src[start + j] : fill;
+  }
+}
+
+static inline unsigned copy_grid(int64_t n_rows, int64_t n_cols) {
+  const int64_t chunks = (n_cols + kBlock - 1) / kBlock;
+  const int64_t g = n_rows * chunks;
+  return (unsigned)(g < 262144 ? (g > 0 ? g : 1) : 262144);
+}
+
+}  // namespace orlhf
+
+using namespace orlhf;
+
+extern "C" int orlhf_row_extents(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols, int64_t* first,
+                                 int64_t* end, int64_t* length, orlhf_stream_t stream) {
+  if (int rc = check_rows("row_extents", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(mask_dtype != ORLHF_MASK_NONE, "row_extents: needs a mask");
+  if (n_rows == 0) return ORLHF_OK;
+  const dim3 grid((unsigned)(n_rows < 65536 ? n_rows : 65536)), block(kBlock);
+  hipStream_t s = (hipStream_t)stream;
+  switch (mask_dtype) {
+    case ORLHF_MASK_U8:
+      hipLaunchKernelGGL(row_extents_kernel<ORLHF_MASK_U8>, grid, block, 0, s, mask, n_rows, n_cols, first, end, length);
+      break;
+    case ORLHF_MASK_F32:
+      hipLaunchKernelGGL(row_extents_kernel<ORLHF_MASK_F32>, grid, block, 0, s, mask, n_rows, n_cols, first, end, length);
+      break;
+    default:
+      hipLaunchKernelGGL(row_extents_kernel<ORLHF_MASK_I64>, grid, block, 0, s, mask, n_rows, n_cols, first, end, length);
+      break;
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_row_extents");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_cu_seqlens(const int64_t* lengths, int64_t n_rows, int64_t* cu_seqlens, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_rows >= 0, "cu_seqlens: n_rows=%lld", (long long)n_rows);
+  ORLHF_CHECK_ARG(cu_seqlens != nullptr && (lengths != nullptr || n_rows == 0), "cu_seqlens: NULL argument");
+  hipLaunchKernelGGL(cu_seqlens_kernel, dim3(1), dim3(kBlock), 0, (hipStream_t)stream, lengths, n_rows, cu_seqlens);
+  ORLHF_CHECK_LAUNCH("orlhf_cu_seqlens");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_pack_rows(const void* src, int elem_bytes, int64_t n_rows, int64_t n_cols, const int64_t* first,
+                               const int64_t* cu_seqlens, void* dst, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_rows >= 0 && n_cols >= 0, "pack_rows: n_rows=%lld n_cols=%lld", (long long)n_rows, (long long)n_cols);
+  if (n_rows * n_cols == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(src != nullptr && dst != nullptr && cu_seqlens != nullptr, "pack_rows: NULL argument");
+  const dim3 grid(copy_grid(n_rows, n_cols)), block(kBlock);
+  hipStream_t s = (hipStream_t)stream;
+  switch (elem_bytes) {
+    case 1: hipLaunchKernelGGL(pack_rows_kernel<uint8_t>, grid, block, 0, s, (const uint8_t*)src, n_rows, n_cols, first, cu_seqlens, (uint8_t*)dst); break;
+    case 2: hipLaunchKernelGGL(pack_rows_kernel<uint16_t>, grid, block, 0, s, (const uint16_t*)src, n_rows, n_cols, first, cu_seqlens, (uint16_t*)dst); break;
+    case 4: hipLaunchKernelGGL(pack_rows_kernel<uint32_t>, grid, block, 0, s, (const uint32_t*)src, n_rows, n_cols, first, cu_seqlens, (uint32_t*)dst); break;
+    case 8: hipLaunchKernelGGL(pack_rows_kernel<uint64_t>, grid, block, 0, s, (const uint64_t*)src, n_rows, n_cols, first, cu_seqlens, (uint64_t*)dst); break;
+    default: return fail(ORLHF_ERR_INVALID_ARG, "pack_rows: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_pack_rows");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_pad_rows(const void* src, int elem_bytes, const int64_t* cu_seqlens, int64_t n_rows,
+                              int64_t n_cols, int left_side, uint64_t fill_bits, void* dst, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_rows >= 0 && n_cols >= 0, "pad_rows: n_rows=%lld n_cols=%lld", (long long)n_rows, (long long)n_cols);
+  if (n_rows * n_cols == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(dst != nullptr && cu_seqlens != nullptr, "pad_rows: NULL argument");
+  const dim3 grid(copy_grid(n_rows, n_cols)), block(kBlock);
+  hipStream_t s = (hipStream_t)stream;
+  const int left = left_side != 0;
+  switch (elem_bytes) {
+    case 1: hipLaunchKernelGGL(pad_rows_kernel<uint8_t>, grid, block, 0, s, (const uint8_t*)src, cu_seqlens, n_rows, n_cols, left, (uint8_t)fill_bits, (uint8_t*)dst); break;
+    case 2: hipLaunchKernelGGL(pad_rows_kernel<uint16_t>, grid, block, 0, s, (const uint16_t*)src, cu_seqlens, n_rows, n_cols, left, (uint16_t)fill_bits, (uint16_t*)dst); break;
+    case 4: hipLaunchKernelGGL(pad_rows_kernel<uint32_t>, grid, block, 0, s, (const uint32_t*)src, cu_seqlens, n_rows, n_cols, left, (uint32_t)fill_bits, (uint32_t*)dst); break;
+    case 8: hipLaunchKernelGGL(pad_rows_kernel<uint64_t>, grid, block, 0, s, (const uint64_t*)src, cu_seqlens, n_rows, n_cols, left, (uint64_t)fill_bits, (uint64_t*)dst); break;
+    default: return fail(ORLHF_ERR_INVALID_ARG, "pad_rows: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_pad_rows");
+  return ORLHF_OK;
+}

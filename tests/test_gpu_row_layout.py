@@ -1,0 +1,181 @@
+"""Row layout kernels (mask extents, cu_seqlens, pack, pad) and the packed Experience fields:
+bit-exact against torch indexing, the layout oracle and the reference's padding helper
+(openrlhf/utils/utils.py:93-106, openrlhf/trainer/ppo_utils/experience.py:199-247), and the
+packed per-token chain against the padded one."""
+import pytest
+import torch
+
+from oracle import advantages as oa
+from oracle import layout as olay
+from oracle import losses as ol
+from oracle import token_numerics as otn
+
+pytestmark = pytest.mark.gpu
+
+
+def _mask(b, a, seed, holes=True):
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(0, a + 1, (b,), generator=g)
+    left = torch.randint(0, 4, (b,), generator=g)
+    cols = torch.arange(a)[None, :]
+    m = (cols >= left[:, None]) & (cols < lens[:, None])
+    if holes and a > 4:
+        m[torch.arange(b), torch.randint(0, a, (b,), generator=g)] = False
+    if b > 2:
+        m[1] = False  # an empty row
+        m[2] = True   # a full row
+    return m
+
+
+@pytest.mark.parametrize("dtype", [torch.bool, torch.uint8, torch.int64, torch.float32, torch.int32])
+@pytest.mark.parametrize("shape", [(1, 1), (7, 300), (64, 2049)])
+def test_row_extents_bit_exact(cuda, dtype, shape):
+    from openrlhf_amd.trainer.ppo_utils.experience import row_extents
+
+    b, a = shape
+    m = _mask(b, a, seed=b + a)
+    first, end, length = (t.cpu() for t in row_extents(m.to(dtype).to(cuda)))
+    for r in range(b):
+        nz = m[r].nonzero().reshape(-1)
+        if nz.numel() == 0:
+            assert (first[r], end[r], length[r]) == (a, 0, 0)
+        else:
+            assert (first[r], end[r], length[r]) == (nz[0], nz[-1] + 1, nz[-1] + 1 - nz[0])
+    # right-padded rows: the length remove_padding_in_sequences keeps
+    right = _mask(b, a, seed=3 * b + a, holes=False)
+    right[:, 0] = True
+    _, end, _ = row_extents(right.to(dtype).to(cuda))
+    assert end.cpu().tolist() == [olay.unpadded_length(row.long()) for row in right]
+
+
+@pytest.mark.parametrize("n", [0, 1, 255, 256, 257, 5000])
+def test_cu_seqlens_bit_exact(cuda, n):
+    from openrlhf_amd.trainer.ppo_utils.experience import cu_seqlens_of
+
+    g = torch.Generator().manual_seed(n)
+    lens = torch.randint(0, 70000, (n,), generator=g)
+    cu = cu_seqlens_of(lens.to(cuda)).cpu()
+    ref = torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)])
+    assert cu.dtype == torch.int64 and torch.equal(cu, ref)
+    # int32 lengths and sums beyond 2^31 stay exact
+    big = torch.full((max(n, 1),), 2 ** 30 + 7, dtype=torch.int32)
+    assert torch.equal(cu_seqlens_of(big.to(cuda)).cpu()[-1], big.long().sum())
+
+
+def test_cu_seqlens_matches_unpad_boundaries(cuda):
+    from openrlhf_amd.trainer.ppo_utils.experience import cu_seqlens_of, row_extents
+
+    att = _mask(9, 77, seed=5, holes=False).long()
+    _, _, length = row_extents(att.to(cuda))
+    assert torch.equal(cu_seqlens_of(length).cpu(), olay.unpad_boundaries(att))
+
+
+@pytest.mark.parametrize("dtype", [torch.bool, torch.bfloat16, torch.float32, torch.int64, torch.float64, torch.int8])
+@pytest.mark.parametrize("side", ["left", "right"])
+def test_pack_and_pad_round_trip(cuda, dtype, side):
+    from openrlhf_amd.trainer.ppo_utils.experience import cu_seqlens_of, pack_padded, pad_packed, row_extents
+
+    b, a = 33, 517
+    m = _mask(b, a, seed=17)
+    g = torch.Generator().manual_seed(1)
+    x = (torch.randn(b, a, generator=g) * 100).to(dtype) if dtype != torch.bool else torch.rand(b, a, generator=g) > 0.5
+    first, end, length = row_extents(m.to(cuda))
+    cu = cu_seqlens_of(length)
+    flat = pack_padded(x.to(cuda), cu, first)
+    ref = torch.cat([x[r, int(first[r]): int(end[r])] if int(length[r]) else x[r, :0] for r in range(b)])
+    assert flat.dtype == x.dtype and torch.equal(flat.cpu(), ref)
+    assert torch.equal(pack_padded(x.to(cuda), cu, first, total=ref.numel()), flat)
+    value = True if dtype == torch.bool else (-3 if dtype != torch.bfloat16 else -3.5)
+    back = pad_packed(flat, cu, a + 5, side, value).cpu()
+    rows = [x[r, int(first[r]): int(end[r])] if int(length[r]) else x[r, :0] for r in range(b)]
+    want = olay.zero_pad_sequences(rows + [x.new_zeros(a + 5)], side, value, stack=True)[:-1]
+    assert back.dtype == x.dtype and torch.equal(back, want)
+    # first = None packs from column 0 (right-padded rows)
+    lens = torch.randint(0, a + 1, (b,), generator=g)
+    cu0 = cu_seqlens_of(lens.to(cuda))
+    flat0 = pack_padded(x.to(cuda), cu0)
+    assert torch.equal(flat0.cpu(), torch.cat([x[r, : int(lens[r])] for r in range(b)]))
+
+
+@pytest.mark.parametrize("side", ["left", "right"])
+@pytest.mark.parametrize("stack", [True, False])
+def test_zero_pad_sequences_vs_reference_semantics(cuda, side, stack):
+    from openrlhf_amd.utils.utils import zero_pad_sequences
+
+    g = torch.Generator().manual_seed(2)
+    one_d = [torch.randn(n, generator=g) for n in (5, 1, 9, 9, 3)]
+    got = zero_pad_sequences([t.to(cuda) for t in one_d], side, 0.25, stack).cpu()
+    assert torch.equal(got, olay.zero_pad_sequences(one_d, side, 0.25, stack))
+    ids = [torch.randint(0, 50000, (n,), generator=g) for n in (4, 12, 7)]
+    got = zero_pad_sequences([t.to(cuda) for t in ids], side, 151643, stack).cpu()
+    want = olay.zero_pad_sequences(ids, side, 151643, stack)
+    assert got.dtype == want.dtype and torch.equal(got, want)
+    if stack:
+        two_d = [torch.randn(3, n, generator=g) for n in (6, 2, 11)]
+    else:
+        two_d = [torch.randn(r, n, generator=g) for r, n in ((2, 6), (1, 2), (4, 11))]  # Experience._merge_item
+    got = zero_pad_sequences([t.to(cuda) for t in two_d], side, 0, stack).cpu()
+    assert torch.equal(got, olay.zero_pad_sequences(two_d, side, 0, stack))
+    masks = [torch.rand(n, generator=g) > 0.3 for n in (3, 8)]
+    got = zero_pad_sequences([t.to(cuda) for t in masks], side, 0, stack).cpu()
+    want = olay.zero_pad_sequences(masks, side, 0, stack)
+    assert got.dtype == torch.bool and torch.equal(got, want)
+    with pytest.raises(AssertionError):
+        zero_pad_sequences([t.to(cuda) for t in one_d], "middle")
+
+
+def test_packed_steps_chain_equals_padded_chain(cuda):
+    """Reward shaping -> GAE -> whitening -> PolicyLoss / ValueLoss on fields packed once equals
+    the same chain on the padded tensors (and the oracle), and the packed outputs re-pad to the
+    padded ones at every action position."""
+    from openrlhf_amd.models.loss import PolicyLoss, ValueLoss
+    from openrlhf_amd.models.utils import compute_approx_kl, compute_reward
+    from openrlhf_amd.trainer.ppo_utils.experience import PackedSteps
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import get_advantages_and_returns
+
+    g = torch.Generator().manual_seed(8)
+    b, a = 24, 700
+    lens = torch.randint(1, a + 1, (b,), generator=g)
+    lens[0] = a
+    mask = torch.arange(a)[None, :] < lens[:, None]
+    lp = -torch.rand(b, a, generator=g) * 3
+    old = lp + torch.randn(b, a, generator=g) * 0.05
+    base = lp + torch.randn(b, a, generator=g) * 0.1
+    values = torch.randn(b, a, generator=g)
+    r = torch.randn(b, generator=g)
+    d = lambda t: t.to(cuda)  # noqa: E731
+
+    # padded chain on the GPU
+    kl_p = compute_approx_kl(d(old), d(base), kl_estimator="k1")
+    rew_p = compute_reward(d(r), 0.05, kl_p, action_mask=d(mask))
+    adv_p, ret_p = get_advantages_and_returns(d(values), rew_p, d(mask), 1.0, 0.95)
+    pl_p = PolicyLoss(0.2, 0.2)(d(lp), d(old), adv_p, action_mask=d(mask))[0]
+    vl_p = ValueLoss(0.2)(d(values) + 0.1, d(values), ret_p, action_mask=d(mask))
+
+    # packed once, packed all the way
+    ps = PackedSteps.from_padded(dict(lp=d(lp), old=d(old), base=d(base), values=d(values), mask=d(mask), none=None),
+                                 d(mask))
+    assert ps.total == int(lens.sum()) and ps.fields["none"] is None
+    cu = ps.cu_seqlens
+    assert torch.equal(cu.cpu(), torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)]))
+    kl_k = compute_approx_kl(ps["old"], ps["base"], kl_estimator="k1")
+    rew_k = compute_reward(d(r), 0.05, kl_k, action_mask=ps["mask"], cu_seqlens=cu)
+    adv_k, ret_k = get_advantages_and_returns(ps["values"], rew_k, ps["mask"], 1.0, 0.95, cu_seqlens=cu)
+    pl_k = PolicyLoss(0.2, 0.2)(ps["lp"], ps["old"], adv_k, action_mask=ps["mask"], cu_seqlens=cu)[0]
+    vl_k = ValueLoss(0.2)(ps["values"] + 0.1, ps["values"], ret_k, action_mask=ps["mask"], cu_seqlens=cu)
+
+    from openrlhf_amd.trainer.ppo_utils.experience import pad_packed
+    m = d(mask)
+    assert torch.equal(pad_packed(rew_k, cu, a) * m, rew_p * m)
+    assert torch.equal(pad_packed(adv_k, cu, a) * m, adv_p * m)
+    assert torch.equal(pad_packed(ret_k, cu, a) * m, ret_p * m)
+    assert abs(pl_k.item() - pl_p.item()) <= 1e-6 and abs(vl_k.item() - vl_p.item()) <= 1e-6
+
+    # and against the oracle's padded chain
+    kl_o = otn.compute_approx_kl(old.double(), base.double(), "k1")
+    rew_o = otn.compute_reward(r.double(), 0.05, kl_o, mask)
+    adv_o, ret_o = oa.get_advantages_and_returns(values.double(), rew_o, mask.double(), 1.0, 0.95)
+    pl_o = ol.policy_loss(lp.double(), old.double(), adv_o, mask.double(), None, clip_eps_low=0.2, clip_eps_high=0.2)[0]
+    scale = max(1.0, adv_o.abs().max().item())
+    assert ((pad_packed(adv_k, cu, a).cpu().double() - adv_o) * mask).abs().max().item() <= 1e-5 * scale
+    assert abs(pl_k.item() - pl_o.item()) <= 1e-5 * max(1.0, abs(pl_o.item()))

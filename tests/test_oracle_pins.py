@@ -337,3 +337,18 @@ def test_pair_losses_golden_and_closed_forms():
     close(ol.dpo_loss(c + 1 / (2 * 0.25), c, rc, rc, 0.25, ipo=True)[0], 0.0, 1e-12)
     # label smoothing 0.5 makes the loss even in z
     close(ol.dpo_loss(c, r, rc, rr, 0.2, 0.5)[0], ol.dpo_loss(r, c, rr, rc, 0.2, 0.5)[0], 1e-12)
+
+
+# ------------------------------------------------------------------ layout helpers
+def test_layout_oracle_known_answers():
+    from oracle import layout as olay
+
+    a, b = torch.tensor([1, 2, 3]), torch.tensor([4])
+    assert olay.zero_pad_sequences([a, b], "left", 0, stack=True).tolist() == [[1, 2, 3], [0, 0, 4]]
+    assert olay.zero_pad_sequences([a, b], "right", 9, stack=True).tolist() == [[1, 2, 3], [4, 9, 9]]
+    assert olay.zero_pad_sequences([a, b], "right", 9).tolist() == [1, 2, 3, 4, 9, 9]
+    m = olay.zero_pad_sequences([torch.ones(2, 2), torch.full((1, 3), 2.0)], "right")
+    assert m.tolist() == [[1, 1, 0], [1, 1, 0], [2, 2, 2]]
+    assert olay.unpadded_length(torch.tensor([0, 1, 1, 0, 1, 0, 0])) == 5
+    assert olay.unpadded_length(torch.tensor([1, 1, 1])) == 3
+    assert olay.unpad_boundaries(torch.tensor([[1, 1, 0], [1, 1, 1], [0, 0, 0]])).tolist() == [0, 2, 5, 5]
