@@ -235,6 +235,31 @@ def bench_per_token(args, dev):
         torch.autograd.grad(out[0], x)
 
     record("config4.policy_loss_fwd_bwd", timed(policy_step), padded, 13 + 17)
+
+    # the same batch packed once (flat tokens + cu_seqlens): padding is neither stored nor read
+    from openrlhf_amd.trainer.dpo_trainer import get_batch_logps
+    from openrlhf_amd.trainer.ppo_utils.experience import PackedSteps, pad_packed
+
+    real = int(lens.sum())
+    fields = dict(lp=lp, old=old, adv=adv, mask=mask)
+    ps = PackedSteps.from_padded(fields, mask, total=real)
+    # pack: mask extents (1 B/padded token) + per field read and write of the real tokens
+    record("config4.pack_4_fields", timed(lambda: PackedSteps.from_padded(fields, mask, total=real)),
+           real, 2 * 13 + padded / real)
+    record("config4.pad_1_field", timed(lambda: pad_packed(ps["adv"], ps.cu_seqlens, a)), padded, 4 + 4 * real / padded)
+    cu = ps.cu_seqlens
+    record("config4.discounted_returns_packed",
+           timed(lambda: get_cumulative_returns(ps["adv"], ps["mask"], 1.0, cu_seqlens=cu, max_seqlen=a)), real, 9)
+    xk = ps["lp"].clone().requires_grad_(True)
+
+    def policy_step_packed():
+        out = pl(xk, ps["old"], ps["adv"], action_mask=ps["mask"], cu_seqlens=cu, max_seqlen=a)
+        torch.autograd.grad(out[0], xk)
+
+    record("config4.policy_loss_fwd_bwd_packed", timed(policy_step_packed), real, 13 + 17)
+    att = torch.cat([mask[:, :1], mask], dim=1)
+    prompt_lens = torch.randint(1, 64, (b,), generator=g).to(dev)
+    record("config4.dpo_sequence_logps", timed(lambda: get_batch_logps(lp, att, prompt_lens)), padded, 5)
     print(json.dumps({"workload": "per-token kernels at BASELINE config 3 / config 4 sizes (padded [B, A] fp32)",
                       "n_gpus": 1, "unit": "GB/s", "peak": HBM_PEAK_GBS, "entries": res}), flush=True)
 

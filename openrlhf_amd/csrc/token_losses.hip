@@ -1,18 +1,23 @@
 // Per-token kernels for gfx950: approximate KL, masked token / sequence aggregation, the PPO
 // (and GSPO) policy surrogate and the clipped value loss, each with its backward.
 //
-// Layout: a [n_rows, n_cols] problem is cut into chunks of kChunk tokens of one row; a workgroup
-// evaluates one chunk elementwise (coalesced 4-byte loads, 4 tokens per lane) and reduces the
-// quantities it needs to one fp64 partial per (row, chunk). A second, single-workgroup kernel
-// folds the partials per row and over rows in a fixed order and writes the scalars plus a
-// per-row aggregation weight that the backward kernels multiply with. No atomics anywhere:
+// Layout: a [n_rows, n_cols] problem is cut into chunks of kChunk = 4096 tokens of one row; a
+// workgroup walks one chunk in four sub-chunks (coalesced 4-byte loads, 4 tokens per lane and
+// step: launching a 256-thread workgroup costs the dispatcher 3-5 ns, as much as streaming
+// 20-30 KB, so a workgroup has to move more than that) and reduces the quantities it needs to
+// one fp64 partial per (row, chunk), all quantities through the cross-lane steps together. A
+// fold kernel sums the chunks of each row, a single-workgroup kernel folds the rows in a fixed
+// order and writes the scalars plus a per-row aggregation weight that the backward kernels
+// multiply with. Chunks past the end of a short packed row return at once. No atomics anywhere:
 // the result is bit-reproducible. All of these are HBM-bound streams of 4-17 bytes per token.
 #include "token_terms.h"
 
 namespace orlhf {
 
-constexpr int kTokPerLane = 4;
-constexpr int kChunk = kBlock * kTokPerLane;  // tokens of one row per workgroup
+constexpr int kTokPerLane = 4;                // loads in flight per lane and array
+constexpr int kSub = 4;                       // sub-chunks a workgroup walks one after the other
+constexpr int kSubChunk = kBlock * kTokPerLane;
+constexpr int kChunk = kSubChunk * kSub;      // tokens of one row per workgroup
 constexpr int kMaxQ = 6;                      // quantities reduced per token
 constexpr int kMaxGridY = 32768;
 
@@ -117,30 +122,52 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
                                                               Tok tok, double* __restrict__ partial,
                                                               int n_chunks) {
   constexpr int NQ = Tok::kQ;
-  __shared__ double lds[kWavesPerBlock];
+  __shared__ double lds[NQ][kWavesPerBlock];
   for (int64_t b = blockIdx.y; b < rows.n_rows; b += gridDim.y) {
     int64_t start, len;
     row_span(rows, b, start, len);
     const int64_t c0 = (int64_t)blockIdx.x * kChunk;
+    double* out = partial + (b * n_chunks + blockIdx.x) * NQ;
+    if (c0 >= len) {  // a chunk past the end of a short (packed) row: nothing to read or reduce
+      if (threadIdx.x < NQ) out[threadIdx.x] = 0.0;
+      continue;
+    }
     double acc[NQ];
 #pragma unroll
     for (int i = 0; i < NQ; ++i) acc[i] = 0.0;
+#pragma unroll 1
+    for (int64_t s0 = c0; s0 < c0 + kChunk && s0 < len; s0 += kSubChunk) {
 #pragma unroll
-    for (int k = 0; k < kTokPerLane; ++k) {
-      const int64_t t = c0 + threadIdx.x + k * kBlock;
-      if (t < len) {
-        const float m = load_mask<MASK_DT>(mask, start + t);
-        float q[NQ];
-        tok.eval(b, start + t, m, q);
+      for (int k = 0; k < kTokPerLane; ++k) {
+        const int64_t t = s0 + threadIdx.x + k * kBlock;
+        if (t < len) {
+          const float m = load_mask<MASK_DT>(mask, start + t);
+          float q[NQ];
+          tok.eval(b, start + t, m, q);
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) acc[i] += (double)q[i];
+          for (int i = 0; i < NQ; ++i) acc[i] += (double)q[i];
+        }
       }
     }
+    // all quantities through the wave shuffles together (independent chains), one barrier
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) {
-      const double r = block_sum(acc[i], lds);
-      if (threadIdx.x == 0) partial[(b * n_chunks + blockIdx.x) * NQ + i] = r;
+    for (int o = kWave / 2; o > 0; o >>= 1) {
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) acc[i] += __shfl_xor(acc[i], o, kWave);
     }
+    const int wave = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) lds[i][wave] = acc[i];
+    }
+    __syncthreads();
+    if (threadIdx.x < NQ) {
+      double r = 0.0;
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) r += lds[threadIdx.x][w];
+      out[threadIdx.x] = r;
+    }
+    __syncthreads();
   }
 }
 
@@ -281,14 +308,18 @@ __global__ __launch_bounds__(kBlock) void rows_grad_kernel(Rows rows, const void
   for (int64_t b = blockIdx.y; b < rows.n_rows; b += gridDim.y) {
     int64_t start, len;
     row_span(rows, b, start, len);
-    const float w = (g_per_row ? g_out[b] : g_out[0]) * row_coef[b];
     const int64_t c0 = (int64_t)blockIdx.x * kChunk;
+    if (c0 >= len) continue;
+    const float w = (g_per_row ? g_out[b] : g_out[0]) * row_coef[b];
+#pragma unroll 1
+    for (int64_t s0 = c0; s0 < c0 + kChunk && s0 < len; s0 += kSubChunk) {
 #pragma unroll
-    for (int k = 0; k < kTokPerLane; ++k) {
-      const int64_t t = c0 + threadIdx.x + k * kBlock;
-      if (t < len) {
-        const float m = load_mask<MASK_DT>(mask, start + t);
-        g[start + t] = w * m * tok.grad(b, start + t, m);
+      for (int k = 0; k < kTokPerLane; ++k) {
+        const int64_t t = s0 + threadIdx.x + k * kBlock;
+        if (t < len) {
+          const float m = load_mask<MASK_DT>(mask, start + t);
+          g[start + t] = w * m * tok.grad(b, start + t, m);
+        }
       }
     }
   }
@@ -309,15 +340,13 @@ __global__ __launch_bounds__(kBlock) void gspo_grad_kernel(Rows rows, const void
   for (int64_t b = blockIdx.y; b < rows.n_rows; b += gridDim.y) {
     int64_t start, len;
     row_span(rows, b, start, len);
+    const int64_t c0 = (int64_t)blockIdx.x * kChunk;
+    if (c0 >= len) continue;
     double rs = 0.0;
     for (int c = 0; c < n_chunks; ++c) rs += partial[b * n_chunks + c];
     const float w = g_out[0] * row_coef[b] * (float)rs * row_aux[b * 2] * row_aux[b * 2 + 1];
-    const int64_t c0 = (int64_t)blockIdx.x * kChunk;
-#pragma unroll
-    for (int k = 0; k < kTokPerLane; ++k) {
-      const int64_t t = c0 + threadIdx.x + k * kBlock;
-      if (t < len) g[start + t] = w * load_mask<MASK_DT>(mask, start + t);
-    }
+    for (int64_t t = c0 + threadIdx.x; t < c0 + kChunk && t < len; t += kBlock)
+      g[start + t] = w * load_mask<MASK_DT>(mask, start + t);
   }
 }
 

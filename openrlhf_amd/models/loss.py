@@ -13,7 +13,9 @@ Each loss is one elementwise + reduction launch pair forward and one elementwise
 backward instead of the reference's chain of ~20 eager kernels. Per-token inputs are consumed
 as fp32. ``batch_num_tokens`` / ``global_batch_size`` may be Python numbers or 0-dim tensors
 (device tensors are read on the device, no host synchronisation). Every loss also accepts the
-packed layout: flat per-token tensors plus ``cu_seqlens`` (int64 [B+1]).
+packed layout: flat per-token tensors plus ``cu_seqlens`` (int64 [B+1]) and ``max_seqlen``, a
+bound on the longest row that sizes the launch (rows longer than it would be cut; when it is
+omitted the longest row is read back from ``cu_seqlens``, one synchronisation).
 """
 from typing import Optional
 
@@ -22,7 +24,7 @@ import torch.nn as nn
 
 from .. import _lib
 from .._lib import call, ptr, require_gpu, stream_of
-from .utils import _Aggregate, _cu_arg, _f32, _rows_of, _workspace, masked_mean  # noqa: F401
+from .utils import _Aggregate, _cu_arg, _f32, _packed, _rows_of, _workspace, masked_mean  # noqa: F401
 
 
 def aggregate_loss(
@@ -33,10 +35,12 @@ def aggregate_loss(
     batch_num_tokens: Optional[float] = None,
     global_batch_size: Optional[float] = None,
     cu_seqlens: Optional[torch.Tensor] = None,
+    max_seqlen: Optional[int] = None,
 ) -> torch.Tensor:
     """token_level_loss=True: sum(loss*mask) / (sum(mask) or batch_num_tokens) [* dp_size when
     the global count is given]; False: mean over non-empty rows of sum(loss*mask)/(count+1e-8),
     or that sum / global_batch_size * dp_size (openrlhf/models/loss.py:11-39)."""
+    cu_seqlens = _packed(cu_seqlens, max_seqlen)
     if token_level_loss:
         return _Aggregate.apply(loss, loss_mask, _lib.AGG_TOKEN_MEAN, dp_size, batch_num_tokens, cu_seqlens)
     return _Aggregate.apply(loss, loss_mask, _lib.AGG_SEQ_MEAN, dp_size, global_batch_size, cu_seqlens)
@@ -158,6 +162,7 @@ class PolicyLoss(nn.Module):
         batch_num_tokens: Optional[float] = None,
         global_batch_size: Optional[float] = None,
         cu_seqlens: Optional[torch.Tensor] = None,
+        max_seqlen: Optional[int] = None,
     ):
         if self.policy_loss_type == "ppo":
             policy_type = _lib.POLICY_PPO
@@ -182,7 +187,7 @@ class PolicyLoss(nn.Module):
         norm_value = batch_num_tokens if (self.token_level_loss and policy_type == _lib.POLICY_PPO) else global_batch_size
         loss, clip_ratio, ppo_kl, vllm_kl = _PolicyLossFn.apply(
             log_probs, old_log_probs, advantages, action_mask, rollout_log_probs if use_is else None, cfg,
-            dp_size, norm_value, cu_seqlens,
+            dp_size, norm_value, _packed(cu_seqlens, max_seqlen),
         )
         if not (use_is and policy_type == _lib.POLICY_PPO):
             vllm_kl = None
@@ -248,11 +253,12 @@ class ValueLoss(nn.Module):
         batch_num_tokens: Optional[float] = None,
         global_batch_size: Optional[float] = None,
         cu_seqlens: Optional[torch.Tensor] = None,
+        max_seqlen: Optional[int] = None,
     ) -> torch.Tensor:
         norm_value = batch_num_tokens if self.token_level_loss else global_batch_size
         return _ValueLossFn.apply(
             values, old_values if self.clip_eps is not None else None, returns, action_mask, self.clip_eps,
-            self.token_level_loss, dp_size, norm_value, cu_seqlens,
+            self.token_level_loss, dp_size, norm_value, _packed(cu_seqlens, max_seqlen),
         )
 
 

@@ -184,11 +184,27 @@ def _f32(t: torch.Tensor) -> torch.Tensor:
     return t.contiguous()
 
 
-def _rows_of(t: torch.Tensor, cu_seqlens: Optional[torch.Tensor]):
-    """(n_rows, n_cols) of a padded [..., A] tensor, or of a packed flat tensor + cu_seqlens."""
+def _packed(cu_seqlens, max_seqlen):
+    """What the mirrors hand down for the packed layout: the boundaries with the caller's bound on
+    the longest row (None: measured from the boundaries when the launch is sized)."""
+    return None if cu_seqlens is None else (cu_seqlens, max_seqlen)
+
+
+def _split_packed(cu_seqlens):
+    return cu_seqlens if isinstance(cu_seqlens, tuple) else (cu_seqlens, None)
+
+
+def _rows_of(t: torch.Tensor, cu_seqlens):
+    """(n_rows, n_cols) of a padded [..., A] tensor, or of a packed flat tensor + cu_seqlens, where
+    n_cols bounds the longest row: it sizes the launch grid and the workspace, so it has to be
+    tight. Without the caller's ``max_seqlen`` it is read back from the boundaries (one
+    synchronisation)."""
     if cu_seqlens is not None:
-        n_rows = cu_seqlens.numel() - 1
-        return n_rows, max(int(t.numel()), 1)
+        cu, bound = _split_packed(cu_seqlens)
+        n_rows = cu.numel() - 1
+        if bound is None:
+            bound = int((cu[1:] - cu[:-1]).max()) if n_rows > 0 else 1
+        return n_rows, max(int(bound), 1)
     if t.dim() == 0:
         return 1, 1
     n_cols = t.shape[-1]
@@ -198,8 +214,8 @@ def _rows_of(t: torch.Tensor, cu_seqlens: Optional[torch.Tensor]):
 def _cu_arg(cu_seqlens, dev):
     if cu_seqlens is None:
         return None
-    cu = cu_seqlens.to(device=dev, dtype=torch.int64).contiguous()
-    return cu
+    cu, _ = _split_packed(cu_seqlens)
+    return cu.to(device=dev, dtype=torch.int64).contiguous()
 
 
 def _workspace(n_rows, n_cols, dev):
@@ -286,7 +302,7 @@ class _Aggregate(torch.autograd.Function):
         ctx.x_shape, ctx.x_dtype = x.shape, x.dtype
         ctx.save_for_backward(mkeep, cu, row_coef)
         if mode == _lib.AGG_ROW_MEAN:
-            return out.view(x.shape[:-1]) if cu_seqlens is None else out
+            return out.view(x.shape[:-1]) if cu is None else out
         return out.view(())
 
     @staticmethod
@@ -323,11 +339,14 @@ def compute_reward(
     action_mask: Optional[torch.Tensor] = None,
     reward_clip_range: Tuple[float, float] = None,
     cu_seqlens: Optional[torch.Tensor] = None,
+    max_seqlen: Optional[int] = None,
 ) -> torch.Tensor:
     """Per-token reward: -max(kl_coef, 0) * kl everywhere plus the (clipped) scalar reward r[b]
     at row b's last unmasked column (openrlhf/models/utils.py:98-126). Forward only."""
     dev = require_gpu(r, kl, action_mask)
     klf, rf = _f32(kl.detach()), _f32(r.detach()).reshape(-1)
+    # one workgroup per row walks the row from its own boundaries: the bound is not used
+    cu_seqlens = _packed(cu_seqlens, max_seqlen if max_seqlen is not None else klf.numel())
     n_rows, n_cols = _rows_of(klf, cu_seqlens)
     if rf.numel() != n_rows:
         raise ValueError(f"r has {rf.numel()} entries for {n_rows} rows")

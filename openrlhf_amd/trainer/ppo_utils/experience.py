@@ -118,6 +118,11 @@ class PackedSteps:
         packed = {k: (None if v is None else pack_padded(v, cu, first, total)) for k, v in fields.items()}
         return cls(cu, first, mask.shape[1], total, packed)
 
+    @property
+    def max_seqlen(self) -> int:
+        """A bound on the longest row, known without reading anything back: the padded width."""
+        return self.n_cols
+
     def to_padded(self, name: str, side: str = "right", value=0) -> torch.Tensor:
         """The named field back as a right- (or left-) padded ``[B, n_cols]`` tensor."""
         return pad_packed(self.fields[name], self.cu_seqlens, self.n_cols, side, value)

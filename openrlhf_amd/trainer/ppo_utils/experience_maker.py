@@ -24,7 +24,7 @@ import torch
 
 from ... import _lib
 from ..._lib import call, ptr, stream_of
-from ...models.utils import _cu_arg, _f32, _rows_of, compute_reward
+from ...models.utils import _cu_arg, _f32, _packed, _rows_of, compute_reward
 
 _GROUP_CODES = {
     "gae": _lib.GROUP_IDENTITY,
@@ -64,6 +64,7 @@ def get_advantages_and_returns(
     gamma: float,
     lambd: float,
     cu_seqlens: Optional[torch.Tensor] = None,
+    max_seqlen: Optional[int] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """GAE (experience_maker.py:332-377): with v = mask*values, r = mask*rewards,
     delta_t = r_t + gamma*v_{t+1} - v_t, A_t = delta_t + gamma*lambd*A_{t+1}; returns = A + v.
@@ -71,7 +72,8 @@ def get_advantages_and_returns(
     dev, home = _device_for(values, rewards, action_mask)
     v, r = _f32(_on_gpu(values, dev)), _f32(_on_gpu(rewards, dev))
     mkeep, mptr, mcode = _lib.mask_arg(_on_gpu(action_mask, dev))
-    n_rows, n_cols = _rows_of(v, cu_seqlens)
+    # the scans walk each row from its own boundaries: the bound on the row length is not used
+    n_rows, n_cols = _rows_of(v, _packed(cu_seqlens, max_seqlen if max_seqlen is not None else v.numel()))
     cu = _cu_arg(cu_seqlens, dev)
     adv, ret = torch.empty_like(v), torch.empty_like(v)
     with torch.cuda.device(dev):
@@ -86,12 +88,13 @@ def get_cumulative_returns(
     action_mask: Optional[torch.Tensor],
     gamma: float,
     cu_seqlens: Optional[torch.Tensor] = None,
+    max_seqlen: Optional[int] = None,
 ) -> torch.Tensor:
     """Discounted reward-to-go G_t = mask_t*r_t + gamma*G_{t+1} (experience_maker.py:379-411)."""
     dev, home = _device_for(rewards, action_mask)
     r = _f32(_on_gpu(rewards, dev))
     mkeep, mptr, mcode = _lib.mask_arg(_on_gpu(action_mask, dev))
-    n_rows, n_cols = _rows_of(r, cu_seqlens)
+    n_rows, n_cols = _rows_of(r, _packed(cu_seqlens, max_seqlen if max_seqlen is not None else r.numel()))
     cu = _cu_arg(cu_seqlens, dev)
     ret = torch.empty_like(r)
     with torch.cuda.device(dev):

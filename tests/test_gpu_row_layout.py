@@ -161,8 +161,9 @@ def test_packed_steps_chain_equals_padded_chain(cuda):
     kl_k = compute_approx_kl(ps["old"], ps["base"], kl_estimator="k1")
     rew_k = compute_reward(d(r), 0.05, kl_k, action_mask=ps["mask"], cu_seqlens=cu)
     adv_k, ret_k = get_advantages_and_returns(ps["values"], rew_k, ps["mask"], 1.0, 0.95, cu_seqlens=cu)
-    pl_k = PolicyLoss(0.2, 0.2)(ps["lp"], ps["old"], adv_k, action_mask=ps["mask"], cu_seqlens=cu)[0]
-    vl_k = ValueLoss(0.2)(ps["values"] + 0.1, ps["values"], ret_k, action_mask=ps["mask"], cu_seqlens=cu)
+    pl_k = PolicyLoss(0.2, 0.2)(ps["lp"], ps["old"], adv_k, action_mask=ps["mask"], cu_seqlens=cu,
+                                max_seqlen=ps.max_seqlen)[0]
+    vl_k = ValueLoss(0.2)(ps["values"] + 0.1, ps["values"], ret_k, action_mask=ps["mask"], cu_seqlens=cu)  # measured bound
 
     from openrlhf_amd.trainer.ppo_utils.experience import pad_packed
     m = d(mask)
