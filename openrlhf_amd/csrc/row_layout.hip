@@ -18,6 +18,7 @@ __global__ __launch_bounds__(kBlock) void row_extents_kernel(const void* __restr
   __shared__ long long lds_lo[kWavesPerBlock], lds_hi[kWavesPerBlock];
   for (int64_t b = blockIdx.x; b < n_rows; b += gridDim.x) {
     long long lo = n_cols, hi = 0;  // no non-zero column: first = n_cols, end = 0
+#pragma unroll 8
     for (int64_t t = threadIdx.x; t < n_cols; t += kBlock) {
       if (load_mask<MASK_DT>(mask, b * n_cols + t) != 0.0f) {
         lo = t < lo ? t : lo;
@@ -77,16 +78,26 @@ __global__ __launch_bounds__(kBlock) void cu_seqlens_kernel(const int64_t* __res
   }
 }
 
+// A workgroup moves kCopyChunk consecutive columns of one row: launching a workgroup costs as
+// much as streaming tens of KB, so one element per thread would be bound by the launch rate.
+constexpr int kCopyChunk = 4096;
+
 template <typename E>
 __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__ src, int64_t n_rows, int64_t n_cols,
                                                            const int64_t* __restrict__ first,
                                                            const int64_t* __restrict__ cu, E* __restrict__ dst) {
-  const int64_t chunks = (n_cols + kBlock - 1) / kBlock;
+  const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
   for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
-    const int64_t b = w / chunks, j = (w % chunks) * kBlock + threadIdx.x;
+    const int64_t b = w / chunks, j0 = (w - b * chunks) * kCopyChunk;
     const int64_t start = cu[b], len = cu[b + 1] - start;
+    if (j0 >= len) continue;
     const int64_t f = first != nullptr ? first[b] : 0;
-    if (j < len && f + j < n_cols) dst[start + j] = src[b * n_cols + f + j];
+    int64_t stop = j0 + kCopyChunk < len ? j0 + kCopyChunk : len;
+    stop = stop < n_cols - f ? stop : n_cols - f;
+    const E* in = src + b * n_cols + f;
+    E* out = dst + start;
+#pragma unroll 4
+    for (int64_t j = j0 + threadIdx.x; j < stop; j += kBlock) out[j] = in[j];
   }
 }
 
@@ -94,20 +105,23 @@ template <typename E>
 __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ src, const int64_t* __restrict__ cu,
                                                           int64_t n_rows, int64_t n_cols, int left, E fill,
                                                           E* __restrict__ dst) {
-  const int64_t chunks = (n_cols + kBlock - 1) / kBlock;
+  const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
   for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
-    const int64_t b = w / chunks, t = (w % chunks) * kBlock + threadIdx.x;
-    if (t >= n_cols) continue;
+    const int64_t b = w / chunks, t0 = (w - b * chunks) * kCopyChunk;
     const int64_t start = cu[b];
     int64_t len = cu[b + 1] - start;
-    len = len < n_cols ? len : n_cols;  // a longer row is cut at n_cols (checked by the caller when it can)
-    const int64_t j = left ? t - (n_cols - len) : t;
-    dst[b * n_cols + t] = (j >= 0 && j < len) ? src[start + j] : fill;
+    len = len < n_cols ? len : n_cols;  // a longer row is cut at n_cols
+    const int64_t shift = left ? n_cols - len : 0;  // column of the row's first token
+    const int64_t stop = t0 + kCopyChunk < n_cols ? t0 + kCopyChunk : n_cols;
+    E* out = dst + b * n_cols;
+#pragma unroll 4
+    for (int64_t t = t0 + threadIdx.x; t < stop; t += kBlock)
+      out[t] = (t >= shift && t < shift + len) ? src[start + (t - shift)] : fill;
   }
 }
 
 static inline unsigned copy_grid(int64_t n_rows, int64_t n_cols) {
-  const int64_t chunks = (n_cols + kBlock - 1) / kBlock;
+  const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
   const int64_t g = n_rows * chunks;
   return (unsigned)(g < 262144 ? (g > 0 ? g : 1) : 262144);
 }

@@ -27,6 +27,7 @@ __global__ __launch_bounds__(kBlock) void sequence_logps_fwd_kernel(const float*
   __shared__ double lds[kWavesPerBlock];
   for (int64_t b = blockIdx.x; b < n_rows; b += gridDim.x) {
     double s = 0.0, c = 0.0;
+#pragma unroll 8
     for (int64_t t = threadIdx.x; t < n_cols; t += kBlock) {
       const float m = dpo_mask<MASK_DT>(att, prompt_lens, b, t, n_cols + 1);
       s += (double)(lp[b * n_cols + t] * m);  // the reference multiplies by the mask (NaN * 0 stays NaN)
@@ -43,6 +44,8 @@ __global__ __launch_bounds__(kBlock) void sequence_logps_fwd_kernel(const float*
   }
 }
 
+constexpr int kSeqChunk = 4096;  // columns of one row per workgroup in the backward
+
 // g[b,t] = m * (g_sum[b] + g_mean[b] / count[b])
 template <int MASK_DT>
 __global__ __launch_bounds__(kBlock) void sequence_logps_bwd_kernel(const float* __restrict__ g_sums,
@@ -52,13 +55,15 @@ __global__ __launch_bounds__(kBlock) void sequence_logps_bwd_kernel(const float*
                                                                     const float* __restrict__ counts,
                                                                     int64_t n_rows, int64_t n_cols,
                                                                     float* __restrict__ g) {
-  const int64_t chunks = (n_cols + kBlock - 1) / kBlock;
+  const int64_t chunks = (n_cols + kSeqChunk - 1) / kSeqChunk;
   for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
-    const int64_t b = w / chunks, t = (w % chunks) * kBlock + threadIdx.x;
-    if (t >= n_cols) continue;
+    const int64_t b = w / chunks, t0 = (w - b * chunks) * kSeqChunk;
     float up = g_sums != nullptr ? g_sums[b] : 0.0f;
     if (g_means != nullptr) up += g_means[b] / counts[b];
-    g[b * n_cols + t] = up * dpo_mask<MASK_DT>(att, prompt_lens, b, t, n_cols + 1);
+    const int64_t stop = t0 + kSeqChunk < n_cols ? t0 + kSeqChunk : n_cols;
+#pragma unroll 4
+    for (int64_t t = t0 + threadIdx.x; t < stop; t += kBlock)
+      g[b * n_cols + t] = up * dpo_mask<MASK_DT>(att, prompt_lens, b, t, n_cols + 1);
   }
 }
 
@@ -191,7 +196,7 @@ extern "C" int orlhf_sequence_logps_bwd(const float* g_sums, const float* g_mean
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(g_per_token != nullptr, "sequence_logps_bwd: g_per_token is NULL");
   ORLHF_CHECK_ARG(g_means == nullptr || counts != nullptr, "sequence_logps_bwd: g_means needs the forward's counts");
-  const int64_t chunks = (n_cols + kBlock - 1) / kBlock;
+  const int64_t chunks = (n_cols + kSeqChunk - 1) / kSeqChunk;
   const dim3 grid((unsigned)(n_rows * chunks < 65536 ? n_rows * chunks : 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_LAUNCH(M)                                                                                      \
