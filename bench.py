@@ -1,5 +1,5 @@
 """Headline benchmark: fused log-prob + entropy forward + in-place backward over packed bf16
-logits at V = 151936 (BASELINE config 2), one GPU.
+logits at V = 151936 (the 16-sequence packed workload of the headline metric), one GPU.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline]
 
@@ -164,7 +164,7 @@ def bench_ppo_step(args, pristine, bufs, cu, ring, dev):
 
 
 def bench_per_token(args, dev):
-    """--workload per_token: the small kernels at the sizes of BASELINE configs 3 and 4 (per-token
+    """--workload per_token: the small kernels at the sizes of the PPO (256 x 8K) and GRPO (4096 x 16K) batches (per-token
     fp32 tensors; MBs, not GBs: these launches are latency-bound, the figures are for the record).
     Prints one JSON line with achieved GB/s per entry point (algorithmic bytes / event time)."""
     from openrlhf_amd.models.loss import PolicyLoss, ValueLoss
@@ -278,7 +278,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (the path shards by rows with no collective "
-                 "on it; see DESIGN.md); run with --gpus 1")
+                 "on it); run with --gpus 1")
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible; the HIP path has no CPU fallback")
 

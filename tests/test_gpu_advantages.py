@@ -220,7 +220,7 @@ def test_whitening(cuda, no_std_norm):
 # ------------------------------------------------------------------ config 3 shape, end to end
 @pytest.mark.parametrize("estimator", ["gae", "reinforce_baseline", "group_norm", "rloo"])
 def test_compute_advantages_and_returns_pipeline(cuda, estimator):
-    """A down-scaled BASELINE config 3 / 4: experiences with CPU tensors as the reference's
+    """A down-scaled PPO / GRPO batch: experiences with CPU tensors as the reference's
     controller holds them; k1 KL penalty 0.01, gamma 1, lambda 0.95; compared with the oracle's
     composition of the same steps (experience_maker.py:237-330)."""
     from openrlhf_amd.trainer.ppo_utils.experience_maker import AdvantageFunctions

@@ -1,4 +1,4 @@
-"""The five BASELINE configurations at their full sizes on one MI355X.
+"""The five benchmark configurations of the headline metric at their full sizes on one MI355X.
 
 Configs 1, 3 and 4 are compared with the CPU oracle in full. Configs 2 and 5 (9.4 GB / 34 GB of
 logits) are compared with the fp64 oracle on a row sample and, over all rows, through properties

@@ -331,7 +331,7 @@ def test_value_loss_matches_oracle(cuda, clip_eps, token_level):
 
 # ------------------------------------------------------------------ config 1 end to end
 def test_config1_plumbing(cuda):
-    """BASELINE config 1: fp32 logits [4, 256, 32000] ~ N(0, 2), labels uniform, action mask with
+    """The CPU-runnable configuration: fp32 logits [4, 256, 32000] ~ N(0, 2), labels uniform, action mask with
     0-64 right-padding zeros per row; log_probs_from_logits -> k3 KL vs ref = lp + N(0, 0.05) ->
     PolicyLoss(eps 0.2, token mean) with old = lp + N(0, 0.02), advantages ~ N(0, 1)."""
     from openrlhf_amd.models.loss import PolicyLoss
