@@ -4,6 +4,7 @@ from typing import List
 import torch
 
 from ..trainer.ppo_utils.experience import pad_packed
+from ..trainer.ppo_utils.experience_maker import _gpu_device
 
 
 def zero_pad_sequences(sequences: List[torch.Tensor], side: str = "left", value: int = 0,
@@ -11,7 +12,9 @@ def zero_pad_sequences(sequences: List[torch.Tensor], side: str = "left", value:
     """Pads tensors that differ in their last dimension to the longest one on ``side`` and stacks
     (new leading dimension) or concatenates them along dimension 0
     (openrlhf/utils/utils.py:93-106). One gather of the inputs plus one kernel instead of one
-    ``F.pad`` per sequence; row lengths come from the shapes, nothing is read back."""
+    ``F.pad`` per sequence; row lengths come from the shapes, nothing is read back. CPU tensors
+    (the reference pads on the controller) are gathered, copied to the current GPU in one piece,
+    padded there and copied back."""
     assert side in ("left", "right")
     if not sequences:
         raise ValueError("max() arg is an empty sequence")
@@ -29,10 +32,11 @@ def zero_pad_sequences(sequences: List[torch.Tensor], side: str = "left", value:
         rows = s.numel() // s.size(-1) if s.size(-1) else (int(torch.tensor(s.shape[:-1]).prod()) if s.dim() > 1 else 1)
         rows_per.append(rows)
         lengths.extend([s.size(-1)] * rows)
-    dev = sequences[0].device
-    flat = torch.cat([s.reshape(-1).to(dtype) for s in sequences])
+    home = sequences[0].device
+    dev = home if home.type == "cuda" else _gpu_device()
+    flat = torch.cat([s.reshape(-1).to(dtype) for s in sequences]).to(dev)
     cu = torch.tensor([0] + lengths, dtype=torch.int64).cumsum(0).to(dev)
-    out = pad_packed(flat, cu, max_len, side, value)
+    out = pad_packed(flat, cu, max_len, side, value).to(home)
     if stack:
         return out.view(len(sequences), *lead, max_len)
     inner = sequences[0].shape[1:-1]

@@ -122,6 +122,9 @@ def test_zero_pad_sequences_vs_reference_semantics(cuda, side, stack):
     assert got.dtype == torch.bool and torch.equal(got, want)
     with pytest.raises(AssertionError):
         zero_pad_sequences([t.to(cuda) for t in one_d], "middle")
+    # CPU tensors (the controller's experiences) come back on the CPU
+    got = zero_pad_sequences(ids, side, 151643, stack)
+    assert got.device.type == "cpu" and torch.equal(got, olay.zero_pad_sequences(ids, side, 151643, stack))
 
 
 def test_packed_steps_chain_equals_padded_chain(cuda):
