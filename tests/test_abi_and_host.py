@@ -130,3 +130,21 @@ def test_row_view_and_norm_plumbing():
     assert _lib.mask_arg(None)[2] == _lib.MASK_NONE
     assert _lib.mask_arg(torch.ones(3, dtype=torch.bool))[2] == _lib.MASK_U8
     assert _lib.mask_arg(torch.ones(3, dtype=torch.int32))[2] == _lib.MASK_F32
+
+
+def test_header_is_plain_c(tmp_path):
+    """The public header compiles as C99 on its own (no C++, no HIP, no torch types), and a C
+    caller can name every entry point."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc")
+    names = _declared()
+    src = tmp_path / "use_header.c"
+    body = "\n".join(f"    (void)&{n};" for n in names)
+    src.write_text(f'#include "openrlhf_amd.h"\nint main(void) {{\n{body}\n    return 0;\n}}\n')
+    res = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only",
+                          "-I", os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
