@@ -78,8 +78,9 @@ __global__ __launch_bounds__(kBlock) void cu_seqlens_kernel(const int64_t* __res
   }
 }
 
-// A workgroup moves kCopyChunk consecutive columns of one row: launching a workgroup costs as
-// much as streaming tens of KB, so one element per thread would be bound by the launch rate.
+// A workgroup moves kCopyChunk consecutive columns of one row. (row, chunk) items are numbered
+// with the row varying fastest: workgroups go to the XCDs round-robin by index, and numbered
+// chunk-fastest the chunks that hold tokens of short rows would pile up on a few XCDs.
 constexpr int kCopyChunk = 4096;
 
 template <typename E>
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__
                                                            const int64_t* __restrict__ cu, E* __restrict__ dst) {
   const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
   for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
-    const int64_t b = w / chunks, j0 = (w - b * chunks) * kCopyChunk;
+    const int64_t chunk = w / n_rows, b = w - chunk * n_rows, j0 = chunk * kCopyChunk;  // rows vary fastest
     const int64_t start = cu[b], len = cu[b + 1] - start;
     if (j0 >= len) continue;
     const int64_t f = first != nullptr ? first[b] : 0;
@@ -107,7 +108,7 @@ __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ 
                                                           E* __restrict__ dst) {
   const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
   for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
-    const int64_t b = w / chunks, t0 = (w - b * chunks) * kCopyChunk;
+    const int64_t chunk = w / n_rows, b = w - chunk * n_rows, t0 = chunk * kCopyChunk;
     const int64_t start = cu[b];
     int64_t len = cu[b + 1] - start;
     len = len < n_cols ? len : n_cols;  // a longer row is cut at n_cols

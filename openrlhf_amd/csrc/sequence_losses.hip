@@ -57,7 +57,7 @@ __global__ __launch_bounds__(kBlock) void sequence_logps_bwd_kernel(const float*
                                                                     float* __restrict__ g) {
   const int64_t chunks = (n_cols + kSeqChunk - 1) / kSeqChunk;
   for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
-    const int64_t b = w / chunks, t0 = (w - b * chunks) * kSeqChunk;
+    const int64_t chunk = w / n_rows, b = w - chunk * n_rows, t0 = chunk * kSeqChunk;
     float up = g_sums != nullptr ? g_sums[b] : 0.0f;
     if (g_means != nullptr) up += g_means[b] / counts[b];
     const int64_t stop = t0 + kSeqChunk < n_cols ? t0 + kSeqChunk : n_cols;
