@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 7
+#define ORLHF_ABI_VERSION 8
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -47,7 +47,8 @@ enum orlhf_kl_estimator { ORLHF_KL_K1 = 0, ORLHF_KL_K2 = 1, ORLHF_KL_K3 = 2 };
 enum orlhf_agg_mode {
   ORLHF_AGG_TOKEN_MEAN = 0, /* sum(x*m) / (sum(m) | batch_num_tokens) * dp_size                  */
   ORLHF_AGG_SEQ_MEAN = 1,   /* mean over non-empty rows of sum(x*m)/(sum(m)+1e-8)               */
-  ORLHF_AGG_ROW_MEAN = 2    /* per-row sum(x*m)/sum(m), output [n_rows] (masked_mean, dim=-1)   */
+  ORLHF_AGG_ROW_MEAN = 2,   /* per-row sum(x*m)/sum(m), output [n_rows] (masked_mean, dim=-1)   */
+  ORLHF_AGG_SEQ_MEAN_TOKEN_SUM = 3 /* mean over non-empty rows of sum(x*m): not in the reference  */
 };
 enum orlhf_policy_type { ORLHF_POLICY_PPO = 0, ORLHF_POLICY_GSPO = 1 };
 enum orlhf_is_correction { ORLHF_IS_NONE = 0, ORLHF_IS_TIS = 1, ORLHF_IS_ICEPOP = 2, ORLHF_IS_SEQ_MASK_TIS = 3 };
@@ -343,6 +344,27 @@ int orlhf_group_normalize(const float* rewards, const int64_t* indices, int64_t 
 int64_t orlhf_whiten_workspace_bytes(int64_t n);
 int orlhf_masked_whiten(const float* x, const void* mask, int mask_dtype, int64_t n, int std_norm,
                         void* workspace, float* out, float* stats, orlhf_stream_t stream);
+
+/*
+ * The KL block of experience making (openrlhf/trainer/ppo_utils/experience_maker.py:202-216) in
+ * one pass: kl = compute_approx_kl(log_probs, log_probs_base, estimator) (float, nullable),
+ * kl_mean[b] = masked_mean(kl, mask, dim=-1), diff_mean[b] = masked_mean(log_probs -
+ * log_probs_base, mask, dim=-1) (float [n_rows], each nullable; an empty row gives NaN as the
+ * reference's 0/0). enabled == 0 is the branch without a reference model: kl and both
+ * differences are zeros and the log-prob pointers are not read. Inputs of `dtype`, fp32 maths.
+ */
+int orlhf_kl_rows(const void* log_probs, const void* log_probs_base, int dtype, const void* mask,
+                  int mask_dtype, int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
+                  int estimator, int enabled, float* kl, float* kl_mean, float* diff_mean,
+                  orlhf_stream_t stream);
+
+/*
+ * masked_normalize (openrlhf/models/utils.py:172-179) over each row: mean = sum(x*m)/max(sum(m),1),
+ * c = (x - mean)*m, var = sum(c^2)/max(sum(m),1), out = c * rsqrt(max(var, eps)). out may alias x.
+ */
+int orlhf_masked_normalize_rows(const float* x, const void* mask, int mask_dtype, int64_t n_rows,
+                                int64_t n_cols, const int64_t* cu_seqlens, float eps, float* out,
+                                orlhf_stream_t stream);
 
 /* ------------------------------------------------------------------------------------------
  * Sequence-level pieces of the preference trainers (the callers next to the hot path).

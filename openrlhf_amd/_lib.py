@@ -16,13 +16,13 @@ LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libo
 F32, BF16, F16 = 0, 1, 2
 MASK_NONE, MASK_U8, MASK_F32, MASK_I64 = 0, 1, 2, 3
 KL_K1, KL_K2, KL_K3 = 0, 1, 2
-AGG_TOKEN_MEAN, AGG_SEQ_MEAN, AGG_ROW_MEAN = 0, 1, 2
+AGG_TOKEN_MEAN, AGG_SEQ_MEAN, AGG_ROW_MEAN, AGG_SEQ_MEAN_TOKEN_SUM = 0, 1, 2, 3
 POLICY_PPO, POLICY_GSPO = 0, 1
 IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 
 class Norm(Structure):
@@ -93,6 +93,8 @@ SIGNATURES = {
     "orlhf_group_normalize": (c_int, [P, P, I64, I64, c_int, P, P, P, P]),
     "orlhf_whiten_workspace_bytes": (I64, [I64]),
     "orlhf_masked_whiten": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
+    "orlhf_kl_rows": (c_int, [P, P, c_int, P, c_int, I64, I64, P, c_int, c_int, P, P, P, P]),
+    "orlhf_masked_normalize_rows": (c_int, [P, P, c_int, I64, I64, P, c_float, P, P]),
     "orlhf_row_extents": (c_int, [P, c_int, I64, I64, P, P, P, P]),
     "orlhf_cu_seqlens": (c_int, [P, I64, P, P]),
     "orlhf_pack_rows": (c_int, [P, c_int, I64, I64, P, P, P, P]),

@@ -44,7 +44,7 @@ static inline NormArg norm_arg(const orlhf_norm* n) {
 // Each functor evaluates one token: q[] are the quantities to reduce (already multiplied by the
 // mask weight where the reference multiplies), and grad() is d(token loss)/d(input).
 
-constexpr int kAggCounts = 3;  // internal finaliser mode: out = {sum(mask), #rows with sum(mask) > 0}
+constexpr int kAggCounts = 100;  // internal finaliser mode: out = {sum(mask), #rows with sum(mask) > 0}
 
 struct CountTok {  // loss normalisers: the mask alone
   static constexpr int kQ = 2;
@@ -201,9 +201,9 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
     }
 #pragma unroll
     for (int i = 0; i < NQ; ++i) tot[i] += rq[i];
-    if (mode == ORLHF_AGG_SEQ_MEAN || mode == kAggCounts) {
+    if (mode == ORLHF_AGG_SEQ_MEAN || mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM || mode == kAggCounts) {
       if (rq[1] > 0.0) {
-        seq_sum += rq[0] / (rq[1] + 1e-8);
+        seq_sum += mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM ? rq[0] : rq[0] / (rq[1] + 1e-8);
         seq_cnt += 1.0;
       } else if (rq[0] != rq[0]) {
         seq_sum += rq[0];  // NaN * 0 stays NaN in the reference
@@ -253,6 +253,8 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
       double c;
       if (mode == ORLHF_AGG_TOKEN_MEAN)
         c = scale;
+      else if (mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM)
+        c = cnt > 0.0 ? scale : 0.0;
       else
         c = cnt > 0.0 ? scale / (cnt + 1e-8) : 0.0;
       row_coef[b] = (float)((double)post_scale * c);
@@ -539,7 +541,7 @@ extern "C" int orlhf_masked_aggregate_fwd(const float* x, const void* mask, int 
                                           const orlhf_norm* norm, void* workspace, float* out,
                                           float* row_coef, orlhf_stream_t stream) {
   if (int rc = check_rows("masked_aggregate_fwd", n_rows, n_cols, mask, mask_dtype)) return rc;
-  ORLHF_CHECK_ARG(mode >= ORLHF_AGG_TOKEN_MEAN && mode <= ORLHF_AGG_ROW_MEAN, "masked_aggregate_fwd: unknown mode %d", mode);
+  ORLHF_CHECK_ARG(mode >= ORLHF_AGG_TOKEN_MEAN && mode <= ORLHF_AGG_SEQ_MEAN_TOKEN_SUM, "masked_aggregate_fwd: unknown mode %d", mode);
   ORLHF_CHECK_ARG(out != nullptr && workspace != nullptr, "masked_aggregate_fwd: NULL out / workspace");
   ORLHF_CHECK_ARG(x != nullptr || n_rows * n_cols == 0, "masked_aggregate_fwd: x is NULL");
   hipStream_t s = (hipStream_t)stream;
@@ -578,7 +580,7 @@ extern "C" int orlhf_masked_aggregate_bwd(const float* g_out, const void* mask, 
                                           int64_t n_cols, const int64_t* cu_seqlens, int mode,
                                           const float* row_coef, float* g_x, orlhf_stream_t stream) {
   if (int rc = check_rows("masked_aggregate_bwd", n_rows, n_cols, mask, mask_dtype)) return rc;
-  ORLHF_CHECK_ARG(mode >= ORLHF_AGG_TOKEN_MEAN && mode <= ORLHF_AGG_ROW_MEAN, "masked_aggregate_bwd: unknown mode %d", mode);
+  ORLHF_CHECK_ARG(mode >= ORLHF_AGG_TOKEN_MEAN && mode <= ORLHF_AGG_SEQ_MEAN_TOKEN_SUM, "masked_aggregate_bwd: unknown mode %d", mode);
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(g_out && row_coef && g_x, "masked_aggregate_bwd: NULL pointer");
   const Rows rows{n_rows, n_cols, cu_seqlens};

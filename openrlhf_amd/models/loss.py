@@ -36,11 +36,19 @@ def aggregate_loss(
     global_batch_size: Optional[float] = None,
     cu_seqlens: Optional[torch.Tensor] = None,
     max_seqlen: Optional[int] = None,
+    seq_token_sum: bool = False,
 ) -> torch.Tensor:
     """token_level_loss=True: sum(loss*mask) / (sum(mask) or batch_num_tokens) [* dp_size when
     the global count is given]; False: mean over non-empty rows of sum(loss*mask)/(count+1e-8),
-    or that sum / global_batch_size * dp_size (openrlhf/models/loss.py:11-39)."""
+    or that sum / global_batch_size * dp_size (openrlhf/models/loss.py:11-39).
+
+    ``seq_token_sum=True`` (not in the reference; with ``token_level_loss=False``) averages the
+    per-sequence token SUMS instead of the per-sequence token means."""
     cu_seqlens = _packed(cu_seqlens, max_seqlen)
+    if seq_token_sum:
+        if token_level_loss:
+            raise ValueError("seq_token_sum is a sequence-level mode: pass token_level_loss=False")
+        return _Aggregate.apply(loss, loss_mask, _lib.AGG_SEQ_MEAN_TOKEN_SUM, dp_size, global_batch_size, cu_seqlens)
     if token_level_loss:
         return _Aggregate.apply(loss, loss_mask, _lib.AGG_TOKEN_MEAN, dp_size, batch_num_tokens, cu_seqlens)
     return _Aggregate.apply(loss, loss_mask, _lib.AGG_SEQ_MEAN, dp_size, global_batch_size, cu_seqlens)

@@ -5,6 +5,7 @@ Mirrors (paths relative to the OpenRLHF tree):
   compute_reward           openrlhf/models/utils.py:98-126
   log_probs_from_logits    openrlhf/models/utils.py:139-163
   masked_mean              openrlhf/models/utils.py:166-169
+  masked_normalize         openrlhf/models/utils.py:172-179
   compute_entropy          openrlhf/models/utils.py:182-186
 plus ``logprobs_and_entropy_from_logits``, the one-pass form of what Actor.forward does with
 two calls (openrlhf/models/actor.py:269-285).
@@ -358,6 +359,28 @@ def compute_reward(
         call("orlhf_compute_reward", ptr(rf), float(kl_coef), ptr(klf), mptr, mcode, n_rows, n_cols, ptr(cu),
              1 if reward_clip_range else 0, float(lo), float(hi), ptr(out), None, stream_of(dev))
     return out
+
+
+@torch.no_grad()
+def masked_normalize(tensor: torch.Tensor, mask: torch.Tensor, dim: int = 1, eps: float = 1e-8) -> torch.Tensor:
+    """Per-row masked whitening (openrlhf/models/utils.py:172-179): mean and biased variance over
+    the unmasked entries along ``dim`` (count clamped to >= 1), result zero at masked entries.
+    Forward only: nothing in the reference calls it, it is kept for API completeness."""
+    dev = require_gpu(tensor, mask)
+    nd = tensor.dim()
+    d = dim if dim >= 0 else dim + nd
+    x = _f32(tensor.movedim(d, -1)) if d != nd - 1 else _f32(tensor)
+    m = mask.expand_as(tensor)
+    m = m.movedim(d, -1) if d != nd - 1 else m
+    mkeep, mptr, mcode = _lib.mask_arg(m)
+    n_cols = x.shape[-1]
+    n_rows = x.numel() // n_cols if n_cols else 0
+    out = torch.empty_like(x)
+    with torch.cuda.device(dev):
+        call("orlhf_masked_normalize_rows", ptr(x), mptr, mcode, n_rows, n_cols, None, float(eps), ptr(out),
+             stream_of(dev))
+    out = out.movedim(-1, d) if d != nd - 1 else out
+    return out.to(tensor.dtype)
 
 
 # ------------------------------------------------------------------ one-pass forward + backward

@@ -24,7 +24,7 @@ import torch
 
 from ... import _lib
 from ..._lib import call, ptr, stream_of
-from ...models.utils import _cu_arg, _f32, _packed, _rows_of, compute_reward
+from ...models.utils import _KL_CODES, _cu_arg, _f32, _packed, _rows_of, compute_reward
 
 _GROUP_CODES = {
     "gae": _lib.GROUP_IDENTITY,
@@ -54,6 +54,49 @@ def _device_for(*tensors) -> Tuple[torch.device, torch.device]:
     home = next(t.device for t in tensors if t is not None)
     gpu = next((t.device for t in tensors if t is not None and t.is_cuda), None)
     return (gpu if gpu is not None else _gpu_device()), home
+
+
+@torch.no_grad()
+def experience_kl(
+    action_log_probs: torch.Tensor,
+    base_action_log_probs: Optional[torch.Tensor],
+    action_mask: Optional[torch.Tensor],
+    kl_estimator: str = "k1",
+    cu_seqlens: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """The KL block of ``make_experience`` (experience_maker.py:202-216) in one pass over the
+    log-probs: ``(kl, kl_mean, logprobs_diff_mean)`` with ``kl = compute_approx_kl(lp, base)``,
+    ``kl_mean = masked_mean(kl, mask, dim=-1)`` and the masked row mean of ``lp - base``.
+    ``base_action_log_probs=None`` is the branch without a reference model (or with the KL taken
+    as a loss): zeros, and means of zeros."""
+    if kl_estimator not in _KL_CODES:
+        raise ValueError(f"Unknown kl_estimator: {kl_estimator}")
+    dev, home = _device_for(action_log_probs, base_action_log_probs, action_mask)
+    lp = _on_gpu(action_log_probs, dev)
+    enabled = base_action_log_probs is not None
+    if enabled:
+        base = _on_gpu(base_action_log_probs, dev)
+        if lp.dtype == base.dtype and lp.dtype in _lib._DTYPES:
+            lp, base = lp.contiguous(), base.contiguous()
+        else:
+            lp, base = _f32(lp), _f32(base)
+        if base.shape != lp.shape:
+            raise ValueError(f"log-prob shapes differ: {tuple(lp.shape)} vs {tuple(base.shape)}")
+    else:
+        lp, base = lp.contiguous(), None
+    mkeep, mptr, mcode = _lib.mask_arg(_on_gpu(action_mask, dev))
+    n_rows, n_cols = _rows_of(lp, _packed(cu_seqlens, lp.numel()))
+    cu = _cu_arg(cu_seqlens, dev)
+    kl = torch.empty(lp.shape, dtype=torch.float32, device=dev)
+    kl_mean = torch.empty(n_rows, dtype=torch.float32, device=dev)
+    diff_mean = torch.empty(n_rows, dtype=torch.float32, device=dev)
+    code = _lib.dtype_code(lp) if enabled else _lib.F32
+    with torch.cuda.device(dev):
+        call("orlhf_kl_rows", ptr(lp) if enabled else None, ptr(base), code, mptr, mcode, n_rows, n_cols, ptr(cu),
+             _KL_CODES[kl_estimator], 1 if enabled else 0, ptr(kl), ptr(kl_mean), ptr(diff_mean), stream_of(dev))
+    if not enabled:  # the reference keeps the log-prob dtype for its zeros
+        kl = kl.to(action_log_probs.dtype)
+    return kl.to(home), kl_mean.to(home), diff_mean.to(home)
 
 
 @torch.no_grad()

@@ -6,6 +6,17 @@ import torch
 from .token_numerics import masked_mean
 
 
+def aggregate_seq_token_sum(loss, loss_mask, dp_size=1, global_batch_size=None):
+    """Sequence mean of token SUMS. Not in the reference (openrlhf/models/loss.py:29-39 divides
+    every sequence by its token count): the same lines with that division removed."""
+    cnt = loss_mask.sum(dim=-1)
+    seq = (loss * loss_mask).sum(dim=-1)
+    seq_mask = (cnt > 0).to(loss.dtype)
+    if global_batch_size is None:
+        return masked_mean(seq, seq_mask)
+    return (seq * seq_mask).sum() / global_batch_size * dp_size
+
+
 def aggregate_loss(loss, loss_mask, token_level_loss=True, dp_size=1, batch_num_tokens=None, global_batch_size=None):
     """Token-mean or mean of per-sequence token-means (openrlhf/models/loss.py:11-39)."""
     if token_level_loss:

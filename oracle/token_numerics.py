@@ -98,3 +98,25 @@ def actor_forward_tail(logits, sequences, attention_mask, action_mask, temperatu
     ent, lp = ent[:, :-1], lp[:, :-1]
     width = action_mask.shape[1]
     return lp[:, -width:] * action_mask.float(), ent
+
+
+def masked_normalize(tensor: torch.Tensor, mask: torch.Tensor, dim: int = 1, eps: float = 1e-8) -> torch.Tensor:
+    """openrlhf/models/utils.py:172-179: masked per-row whitening with the count clamped to >= 1
+    and the biased variance clamped to >= eps."""
+    mask_sum = mask.sum(dim=dim, keepdim=True).clamp(min=1)
+    mean = (tensor * mask).sum(dim=dim, keepdim=True) / mask_sum
+    mean_centered = (tensor - mean) * mask
+    var = (mean_centered**2).sum(dim=dim, keepdim=True) / mask_sum
+    return mean_centered * var.clamp(min=eps).rsqrt()
+
+
+def experience_kl(action_log_probs, base_action_log_probs, action_mask, kl_estimator="k1"):
+    """The KL block of make_experience (openrlhf/trainer/ppo_utils/experience_maker.py:202-216):
+    per-token KL estimate and the per-sequence masked means the trainer logs."""
+    if base_action_log_probs is not None:
+        kl = compute_approx_kl(action_log_probs, base_action_log_probs, kl_estimator=kl_estimator)
+        diff = action_log_probs.float() - base_action_log_probs.float()
+    else:
+        kl = torch.zeros_like(action_log_probs)
+        diff = torch.zeros_like(action_log_probs)
+    return kl, masked_mean(kl, action_mask, dim=-1), masked_mean(diff, action_mask, dim=-1)

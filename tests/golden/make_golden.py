@@ -287,6 +287,28 @@ def pair_loss(kind, chosen, rejected, ref_c, ref_r, beta, smooth):
     return out
 
 
+def masked_normalize(x, mask, eps):
+    out = []
+    for row, rm in zip(x, mask):
+        cnt = max(sum(rm), 1.0)
+        mean = sum(v * m for v, m in zip(row, rm)) / cnt
+        cen = [(v - mean) * m for v, m in zip(row, rm)]
+        var = sum(c * c for c in cen) / cnt
+        r = 1.0 / math.sqrt(max(var, eps))
+        out.append([c * r for c in cen])
+    return out
+
+
+def kl_rows(lp, base, mask, est):
+    kl = approx_kl(lp, base, est)
+    means, diffs = [], []
+    for b, rm in enumerate(mask):
+        c = sum(rm)
+        means.append(sum(k * m for k, m in zip(kl[b], rm)) / c if c > 0 else None)
+        diffs.append(sum((f32(p) - f32(q)) * m for p, q, m in zip(lp[b], base[b], rm)) / c if c > 0 else None)
+    return means, diffs
+
+
 def main():
     rng = random.Random(20240607)
     gold = {}
@@ -420,6 +442,13 @@ def main():
         "pairwise_margin": pair_loss("pairwise", cr, rr, margin, None, 1.0, 0.0),
         "logexp": pair_loss("logexp", cr, rr, None, None, 1.0, 0.0),
     }
+
+    gold["masked_normalize"] = {"eps": 1e-8, "out": masked_normalize(adv, mask, 1e-8)}
+    gold["kl_rows"] = {est: dict(zip(("kl_mean", "diff_mean"), kl_rows(lp, base, mask, est))) for est in ("k1", "k3")}
+    seq_sums = [sum(x * m for x, m in zip(ra, rm)) for ra, rm in zip(adv, mask)]
+    nonempty = [s_ for s_, rm in zip(seq_sums, mask) if sum(rm) > 0]
+    gold["aggregate"]["seq_token_sum"] = sum(nonempty) / len(nonempty)
+    gold["aggregate"]["seq_token_sum_global"] = sum(nonempty) / 5.0 * 2
 
     with open(OUT, "w") as fh:
         json.dump(gold, fh)

@@ -352,3 +352,32 @@ def test_layout_oracle_known_answers():
     assert olay.unpadded_length(torch.tensor([0, 1, 1, 0, 1, 0, 0])) == 5
     assert olay.unpadded_length(torch.tensor([1, 1, 1])) == 3
     assert olay.unpad_boundaries(torch.tensor([[1, 1, 0], [1, 1, 1], [0, 0, 0]])).tolist() == [0, 2, 5, 5]
+
+
+def test_masked_normalize_kl_rows_and_token_sum_golden():
+    tok = GOLD["tokens"]
+    adv, mask = T(tok["advantages"]), T(tok["mask"])
+    out = otn.masked_normalize(adv, mask, dim=1, eps=GOLD["masked_normalize"]["eps"])
+    close(out, GOLD["masked_normalize"]["out"], 1e-10)
+    full = torch.ones_like(mask)
+    z = otn.masked_normalize(adv, full)
+    close(z.mean(dim=1), torch.zeros(4), 1e-12)
+    close((z ** 2).mean(dim=1), torch.ones(4), 1e-9)  # biased variance 1 over the row
+    assert (otn.masked_normalize(adv, mask)[mask == 0] == 0).all()
+    lp, base = T(tok["log_probs"]), T(tok["base_log_probs"])
+    for est, ref in GOLD["kl_rows"].items():
+        kl, kl_mean, diff_mean = otn.experience_kl(lp, base, mask, est)
+        close(kl, GOLD["approx_kl"][est], 1e-10)
+        for b in range(4):
+            if ref["kl_mean"][b] is None:
+                assert torch.isnan(kl_mean[b]) and torch.isnan(diff_mean[b])
+            else:
+                close(kl_mean[b], ref["kl_mean"][b], 1e-10)
+                close(diff_mean[b], ref["diff_mean"][b], 1e-7)  # the reference forms lp.float() - base.float()
+    kl, kl_mean, _ = otn.experience_kl(lp, None, full, "k1")
+    assert (kl == 0).all() and (kl_mean == 0).all()
+    agg = GOLD["aggregate"]
+    close(ol.aggregate_seq_token_sum(adv, mask), agg["seq_token_sum"], 1e-12)
+    close(ol.aggregate_seq_token_sum(adv, mask, dp_size=2, global_batch_size=5.0), agg["seq_token_sum_global"], 1e-12)
+    # every sequence of the same length L: token-sum mode = L * the reference's seq-mean mode
+    close(ol.aggregate_seq_token_sum(adv, full), 16 * ol.aggregate_loss(adv, full, token_level_loss=False), 1e-9)
