@@ -73,7 +73,7 @@ def make_workload(dev, seed=1234):
     return logits, labels, g_lp, g_ent, cu
 
 
-def cpu_baseline(logits_rows, labels, g_lp, g_ent, repeats=3):
+def cpu_baseline(logits_rows, labels, g_lp, g_ent, repeats=5):
     """The CPU oracle on a row sample: bf16 -> fp32 up-cast, entropy, gather - chunked logsumexp,
     autograd backward (the reference's op sequence, openrlhf/models/actor.py:267-285)."""
     from oracle import token_numerics as otn
@@ -91,7 +91,17 @@ def cpu_baseline(logits_rows, labels, g_lp, g_ent, repeats=3):
         del x, ent, lp
     times = sorted(times[1:])  # first run is warm-up
     med = times[len(times) // 2]
-    return x_bf16.shape[0] / med, med
+    return x_bf16.shape[0] / med, med, repeats
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown CPU"
 
 
 def measured_traffic(kernel, n_tok):
@@ -435,15 +445,16 @@ def main():
         out["ppo_actor_step_fused"] = ppo
     if not args.no_cpu_baseline:
         rows = min(args.cpu_rows, n_tok)
-        cpu_tok_s, cpu_s = cpu_baseline(pristine[:rows], labels[:rows], g_lp[:rows], g_ent[:rows])
+        cpu_tok_s, cpu_s, cpu_runs = cpu_baseline(pristine[:rows], labels[:rows], g_lp[:rows], g_ent[:rows])
         out["cpu_baseline"] = {
             "value": cpu_tok_s,
             "unit": "tokens/s",
             "cores": torch.get_num_threads(),
             "kind": "port",
             "sample": f"first {rows} rows of the same workload at full V (bf16->fp32 up-cast, entropy, gather - "
-                      f"chunked logsumexp, autograd backward) on torch CPU, median of 3 runs of {cpu_s:.2f} s; "
-                      f"os.cpu_count()={os.cpu_count()}",
+                      f"chunked logsumexp, autograd backward) on torch CPU, median of {cpu_runs} runs of "
+                      f"{cpu_s:.2f} s after one warm-up run; {cpu_model()}, os.cpu_count()={os.cpu_count()}, "
+                      f"torch.get_num_threads()={torch.get_num_threads()}",
         }
     print(json.dumps(out), flush=True)
 

@@ -146,6 +146,7 @@ def log_probs_from_logits(
     temperature: float = 1.0,
     inplace_backward: bool = False,
     mutate_logits: bool = False,
+    out_dtype: Optional[torch.dtype] = None,
 ) -> torch.Tensor:
     """log_softmax(logits / temperature) gathered at ``labels``
     (openrlhf/models/utils.py:139-163), fp32 result.
@@ -154,7 +155,10 @@ def log_probs_from_logits(
     caller's logits are divided by the temperature in place (rounded to their dtype) and the
     log-prob is taken from the stored quotient, exactly the reference's order of operations.
     It costs an extra read+write of the logits and is for inference-mode callers that read the
-    scaled logits afterwards; it refuses tensors that require grad."""
+    scaled logits afterwards; it refuses tensors that require grad.
+
+    ``out_dtype`` casts the fp32 result (``out_dtype=logits.dtype`` gives the dtype the
+    reference's bf16 / fp16 branch returns, computed in fp32 and rounded once)."""
     if mutate_logits and temperature != 1.0:
         if logits.requires_grad and torch.is_grad_enabled():
             raise RuntimeError("mutate_logits=True changes the logits in place and is not tracked by autograd; "
@@ -168,7 +172,8 @@ def log_probs_from_logits(
                  row_stride, float(temperature), stream_of(dev))
         torch.autograd.graph.increment_version(rows)
         temperature = 1.0
-    return _LogprobEntropy.apply(logits, labels, temperature, True, False, inplace_backward)[0]
+    out = _LogprobEntropy.apply(logits, labels, temperature, True, False, inplace_backward)[0]
+    return out if out_dtype is None or out_dtype == out.dtype else out.to(out_dtype)
 
 
 def compute_entropy(logits: torch.Tensor, inplace_backward: bool = False) -> torch.Tensor:

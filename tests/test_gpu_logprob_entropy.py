@@ -252,3 +252,15 @@ def test_mutate_logits_reproduces_the_reference_side_effect(cuda, dtype):
     assert (lp.cpu().double() - ref).abs().max().item() <= atol
     with pytest.raises(RuntimeError):
         log_probs_from_logits(x.to(cuda).requires_grad_(True), labels.to(cuda), t, mutate_logits=True)
+
+
+def test_out_dtype_matches_the_reference_branch_dtype(cuda):
+    """out_dtype=logits.dtype: what the reference's bf16 branch returns, within one bf16 rounding
+    of the fp32 result (the reference rounds inside log_softmax as well, so it is not bit-equal)."""
+    from openrlhf_amd.models.utils import log_probs_from_logits
+
+    x, labels = _logits(9, 4001, torch.bfloat16, 2.0, seed=5)
+    lp32 = log_probs_from_logits(x.to(cuda), labels.to(cuda))
+    lp16 = log_probs_from_logits(x.to(cuda), labels.to(cuda), out_dtype=torch.bfloat16)
+    assert lp32.dtype == torch.float32 and lp16.dtype == torch.bfloat16
+    assert torch.equal(lp16, lp32.to(torch.bfloat16))
