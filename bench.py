@@ -225,6 +225,32 @@ def bench_per_token(args, dev):
 
     record("config3.value_loss_fwd_bwd", timed(value_step), padded, 30)
 
+    # the whole launch-bound chain of the step (reward shaping, GAE, whitening, both losses'
+    # forward), eagerly and as one captured HIP graph replayed
+    from openrlhf_amd.models.loss import PolicyLoss as _PL
+    pol3 = _PL(0.2, 0.2)
+    old3 = -torch.rand(b, a, device=dev)
+    lp3 = old3 + torch.randn(b, a, device=dev) * 0.02
+
+    def chain():
+        rew_ = compute_reward(r, 0.01, kl, action_mask=mask)
+        adv_, ret_ = get_advantages_and_returns(values, rew_, mask, 1.0, 0.95)
+        (adv_w,) = whiten_advantages([adv_], [mask])
+        return pol3(lp3, old3, adv_w, action_mask=mask)[0], vl(values + 0.1, values, ret_, action_mask=mask)
+
+    chain_bytes = 10 + 17 + 14 + 13 + 13
+    record("config3.chain_eager", timed(chain), padded, chain_bytes)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        chain()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph), torch.no_grad():
+        chain()
+    record("config3.chain_graph_replay", timed(graph.replay), padded, chain_bytes)
+
     # config 4: 512 x 8 sequences, lengths uniform in [64, 16384], padded [B, A]
     b = 4096
     lens = torch.randint(64, 16385, (b,), generator=g)

@@ -2,6 +2,7 @@
 
 Mirrors (paths relative to the OpenRLHF tree):
   aggregate_loss   openrlhf/models/loss.py:11-39
+  GPTLMLoss        openrlhf/models/loss.py:42-84
   SFTLoss          openrlhf/models/loss.py:87-113
   PolicyLoss       openrlhf/models/loss.py:116-230
   ValueLoss        openrlhf/models/loss.py:233-269
@@ -52,6 +53,31 @@ def aggregate_loss(
     if token_level_loss:
         return _Aggregate.apply(loss, loss_mask, _lib.AGG_TOKEN_MEAN, dp_size, batch_num_tokens, cu_seqlens)
     return _Aggregate.apply(loss, loss_mask, _lib.AGG_SEQ_MEAN, dp_size, global_batch_size, cu_seqlens)
+
+
+class GPTLMLoss(nn.Module):
+    """Next-token cross entropy with ``ignore_index = -100`` averaged over the kept positions
+    (openrlhf/models/loss.py:42-84, the path without ring attention): position t is scored against
+    ``labels[..., t+1]``. The logits are read in place (no shifted contiguous copy), ignored
+    positions are neither read nor differentiated; all labels ignored gives NaN, as
+    ``nn.CrossEntropyLoss`` does."""
+
+    def __init__(self, ring_attn_group=None):
+        super().__init__()
+        if ring_attn_group is not None:
+            raise NotImplementedError("GPTLMLoss over a ring-attention group needs collectives; one GPU is built")
+        self.IGNORE_INDEX = -100
+
+    def forward(self, logits: torch.Tensor, labels: torch.Tensor, inplace_backward: bool = False) -> torch.Tensor:
+        from .utils import _LogprobEntropy
+
+        if labels.shape != logits.shape[:-1]:
+            raise ValueError(f"labels {tuple(labels.shape)} do not match logits {tuple(logits.shape)}")
+        nxt = torch.roll(labels, shifts=-1, dims=-1).clone()
+        nxt[..., -1] = self.IGNORE_INDEX
+        keep = nxt != self.IGNORE_INDEX
+        lp = _LogprobEntropy.apply(logits, nxt, 1.0, True, False, inplace_backward, keep)[0]
+        return _Aggregate.apply(-lp, keep, _lib.AGG_TOKEN_MEAN, 1, None, None)
 
 
 class SFTLoss(nn.Module):

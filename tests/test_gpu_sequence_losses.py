@@ -280,3 +280,31 @@ def test_sft_loss_step_fused_and_unfused_vs_oracle(cuda, dtype, token_level, glo
         _close(lp_f, (lp_ref * (shifted != 0)).detach(), tol)
         (loss_f * scale).backward()
         _close(xf.grad.float(), ref_g * scale, gtol * scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gpt_lm_loss_vs_torch_cross_entropy(cuda, dtype):
+    """GPTLMLoss against the library routine the reference calls (nn.CrossEntropyLoss with
+    ignore_index=-100 on the shifted logits / labels), value and gradient."""
+    from openrlhf_amd.models.loss import GPTLMLoss
+
+    g = torch.Generator().manual_seed(21)
+    b, t, vocab = 3, 29, 4099
+    logits = (torch.randn(b, t, vocab, generator=g) * 2).to(dtype)
+    labels = torch.randint(0, vocab, (b, t), generator=g)
+    labels[:, :6] = -100
+    labels[1, 15:19] = -100
+    labels[2, 1:] = -100  # a sample whose every shifted label is ignored
+    x64 = logits.double().requires_grad_(True)
+    ref = torch.nn.CrossEntropyLoss(ignore_index=-100)(x64[..., :-1, :].reshape(-1, vocab), labels[..., 1:].reshape(-1))
+    (ref_g,) = torch.autograd.grad(ref, x64)
+    xd = logits.to(cuda).requires_grad_(True)
+    loss = GPTLMLoss()(xd, labels.to(cuda))
+    _close(loss, ref.detach(), 1e-5 if dtype == torch.float32 else 2e-3)
+    (gd,) = torch.autograd.grad(loss, xd)
+    _close(gd.float(), ref_g, (2e-5 if dtype == torch.float32 else 2.0 ** -8) * ref_g.abs().max().item())
+    assert (gd.cpu()[:, -1] == 0).all() and (gd.cpu()[2] == 0).all()
+    everything_ignored = torch.full((b, t), -100)
+    assert torch.isnan(GPTLMLoss()(logits.to(cuda), everything_ignored.to(cuda)))
+    with pytest.raises(NotImplementedError):
+        GPTLMLoss(ring_attn_group=object())
