@@ -142,15 +142,29 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
     for (int i = 0; i < NQ; ++i) acc[i] = 0.0;
 #pragma unroll 1
     for (int64_t s0 = c0; s0 < c0 + kChunk && s0 < len; s0 += kSubChunk) {
+      if (s0 + kSubChunk <= len) {  // whole sub-chunk in the row: no per-token branch between the loads
+        float q[kTokPerLane][NQ];
 #pragma unroll
-      for (int k = 0; k < kTokPerLane; ++k) {
-        const int64_t t = s0 + threadIdx.x + k * kBlock;
-        if (t < len) {
-          const float m = load_mask<MASK_DT>(mask, start + t);
-          float q[NQ];
-          tok.eval(b, start + t, m, q);
+        for (int k = 0; k < kTokPerLane; ++k) {
+          const int64_t i = start + s0 + threadIdx.x + k * kBlock;
+          tok.eval(b, i, load_mask<MASK_DT>(mask, i), q[k]);
+        }
 #pragma unroll
-          for (int i = 0; i < NQ; ++i) acc[i] += (double)q[i];
+        for (int k = 0; k < kTokPerLane; ++k) {
+#pragma unroll
+          for (int i = 0; i < NQ; ++i) acc[i] += (double)q[k][i];
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < kTokPerLane; ++k) {
+          const int64_t t = s0 + threadIdx.x + k * kBlock;
+          if (t < len) {
+            const float m = load_mask<MASK_DT>(mask, start + t);
+            float q[NQ];
+            tok.eval(b, start + t, m, q);
+#pragma unroll
+            for (int i = 0; i < NQ; ++i) acc[i] += (double)q[i];
+          }
         }
       }
     }
@@ -322,12 +336,24 @@ __global__ __launch_bounds__(kBlock) void rows_grad_kernel(Rows rows, const void
     const float w = (g_per_row ? g_out[b] : g_out[0]) * row_coef[b];
 #pragma unroll 1
     for (int64_t s0 = c0; s0 < c0 + kChunk && s0 < len; s0 += kSubChunk) {
+      if (s0 + kSubChunk <= len) {
+        float out[kTokPerLane];
 #pragma unroll
-      for (int k = 0; k < kTokPerLane; ++k) {
-        const int64_t t = s0 + threadIdx.x + k * kBlock;
-        if (t < len) {
-          const float m = load_mask<MASK_DT>(mask, start + t);
-          g[start + t] = w * m * tok.grad(b, start + t, m);
+        for (int k = 0; k < kTokPerLane; ++k) {
+          const int64_t i = start + s0 + threadIdx.x + k * kBlock;
+          const float m = load_mask<MASK_DT>(mask, i);
+          out[k] = w * m * tok.grad(b, i, m);
+        }
+#pragma unroll
+        for (int k = 0; k < kTokPerLane; ++k) g[start + s0 + threadIdx.x + k * kBlock] = out[k];
+      } else {
+#pragma unroll
+        for (int k = 0; k < kTokPerLane; ++k) {
+          const int64_t t = s0 + threadIdx.x + k * kBlock;
+          if (t < len) {
+            const float m = load_mask<MASK_DT>(mask, start + t);
+            g[start + t] = w * m * tok.grad(b, start + t, m);
+          }
         }
       }
     }
