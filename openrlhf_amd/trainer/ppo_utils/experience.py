@@ -129,3 +129,224 @@ class PackedSteps:
 
     def __getitem__(self, name: str) -> torch.Tensor:
         return self.fields[name]
+
+
+# ---------------------------------------------------------------------------------------------
+# The Experience container (openrlhf/trainer/ppo_utils/experience.py:29-283) with the reference's
+# field names and batch helpers. Per-step fields are [B, T] / [B, A] tensors padded on the right,
+# per-episode fields are [B]; everything else is per-sample metadata. Padding and un-padding go
+# through the row kernels above; `packed()` hands the per-step fields to the per-token kernels in
+# the packed layout.
+# ---------------------------------------------------------------------------------------------
+import itertools
+from dataclasses import fields as _dc_fields
+from typing import Any, List
+
+STEP_FIELDS = ("sequences", "attention_mask", "action_mask", "action_log_probs", "base_action_log_probs",
+               "rollout_log_probs", "values", "returns", "advantages", "kl")
+EPISODE_FIELDS = ("rewards", "scores", "response_length", "truncated", "total_length")
+
+
+def _map_tensors(value, fn):
+    """fn applied to every tensor inside a tensor / list / dict value; anything else is returned as is."""
+    if isinstance(value, torch.Tensor):
+        return fn(value)
+    if isinstance(value, list):
+        return [_map_tensors(v, fn) for v in value]
+    if isinstance(value, dict):
+        return {k: _map_tensors(v, fn) for k, v in value.items()}
+    return value
+
+
+def _pad_rows(tensors: List[torch.Tensor], value, stack: bool) -> torch.Tensor:
+    from ...utils.utils import zero_pad_sequences
+
+    return zero_pad_sequences(tensors, side="right", value=value, stack=stack)
+
+
+@dataclass
+class Experience:
+    """One batch of rollout data (openrlhf/trainer/ppo_utils/experience.py:29-69)."""
+
+    sequences: Optional[torch.Tensor] = None            # (B, T) prompt + response token ids
+    attention_mask: Optional[torch.Tensor] = None       # (B, T)
+    action_mask: Optional[torch.Tensor] = None          # (B, A)
+    action_log_probs: Optional[torch.Tensor] = None     # (B, A) current policy
+    base_action_log_probs: Optional[torch.Tensor] = None  # (B, A) reference policy
+    rollout_log_probs: Optional[torch.Tensor] = None    # (B, A) rollout engine
+    values: Optional[torch.Tensor] = None               # (B, A)
+    returns: Optional[torch.Tensor] = None              # (B, A)
+    advantages: Optional[torch.Tensor] = None           # (B, A)
+    kl: Optional[torch.Tensor] = None                   # (B, A)
+    rewards: Optional[torch.Tensor] = None              # (B,)
+    scores: Optional[torch.Tensor] = None               # (B,)
+    response_length: Optional[torch.Tensor] = None      # (B,)
+    truncated: Optional[torch.Tensor] = None            # (B,)
+    total_length: Optional[torch.Tensor] = None         # (B,)
+    index: Optional[List[int]] = None
+    prompts: list = field(default_factory=list)
+    labels: list = field(default_factory=list)
+    images: list = field(default_factory=list)
+    mm_train_inputs: list = field(default_factory=list)
+    info: dict = field(default_factory=dict)
+
+    @classmethod
+    def is_step_tensor_field(cls, name: str) -> bool:
+        return name in STEP_FIELDS
+
+    @classmethod
+    def is_episode_tensor_field(cls, name: str) -> bool:
+        return name in EPISODE_FIELDS
+
+    @torch.no_grad()
+    def to_device(self, device) -> "Experience":
+        for f in _dc_fields(self):
+            setattr(self, f.name, _map_tensors(getattr(self, f.name), lambda t: t.to(device)))
+        return self
+
+    def pin_memory(self) -> "Experience":
+        for f in _dc_fields(self):
+            setattr(self, f.name, _map_tensors(getattr(self, f.name), lambda t: t.pin_memory()))
+        return self
+
+    @staticmethod
+    def _merge_item(items: List, pad_value: int = 0) -> Any:
+        """Tensors of differing width are right-padded and concatenated along the batch; lists are
+        chained; dicts are merged key by key (experience.py:103-129)."""
+        head = items[0]
+        if isinstance(head, torch.Tensor):
+            return _pad_rows(items, pad_value, stack=False)
+        if isinstance(head, list):
+            return list(itertools.chain.from_iterable(items))
+        if isinstance(head, dict):
+            keys = []
+            for d in items:
+                keys.extend(k for k in d if k not in keys)
+            return {k: Experience._merge_item([d[k] for d in items if k in d], pad_value) for k in keys}
+        if head is None:
+            return None
+        raise ValueError(f"Unsupported type: {type(head)}")
+
+    @staticmethod
+    def concat_experiences(experiences_list: List["Experience"], pad_token_id) -> "Experience":
+        """All batches as one; token ids are padded with ``pad_token_id``, everything else with 0
+        (experience.py:131-158)."""
+        if not experiences_list:
+            return Experience()
+        merged = {}
+        for f in _dc_fields(Experience):
+            pad = pad_token_id if f.name == "sequences" else 0
+            merged[f.name] = Experience._merge_item([getattr(e, f.name) for e in experiences_list], pad)
+        return Experience(**merged)
+
+    def packed(self, names=None, total: Optional[int] = None) -> PackedSteps:
+        """The ``[B, A]`` per-step fields (``names``: default every one that is set) packed over the
+        extent of the action mask, for the per-token kernels' ``cu_seqlens`` form."""
+        width = self.action_mask.shape[1]
+        if names is None:
+            names = [n for n in STEP_FIELDS if getattr(self, n) is not None and getattr(self, n).shape[1:] == (width,)]
+        return PackedSteps.from_padded({n: getattr(self, n) for n in names}, self.action_mask, total=total)
+
+
+def split_experience_batch(experience: Experience) -> List[Experience]:
+    """One single-sample Experience per row of the batch (experience.py:164-196)."""
+    batch_size = len(experience.sequences)
+    experience.index = None
+
+    def row_of(name, value, i):
+        if value is None:
+            return None
+        if isinstance(value, torch.Tensor):
+            if len(value) != batch_size:
+                raise ValueError(f"Size of {name} ({len(value)}) does not match batch_size ({batch_size})")
+            return value[i]
+        if isinstance(value, dict):
+            out = {}
+            for k, v in value.items():
+                if not isinstance(v, (torch.Tensor, list)):
+                    raise TypeError(f"Unsupported type for {name}[{k}]: {type(v)}")
+                if len(v) != batch_size:
+                    raise ValueError(f"Size of {name}[{k}] ({len(v)}) does not match batch_size ({batch_size})")
+                out[k] = v[i]
+            return out
+        if isinstance(value, list):
+            return [value[i]] if len(value) == batch_size else value
+        return value
+
+    return [Experience(**{f.name: row_of(f.name, getattr(experience, f.name), i) for f in _dc_fields(Experience)})
+            for i in range(batch_size)]
+
+
+def make_experience_batch(items: List[Experience], packing_samples=False) -> Experience:
+    """Single-sample Experiences back into one batch: per-step tensors are right-padded with 0 and
+    stacked, per-episode tensors stacked, numeric info entries become tensors, lists are chained
+    (experience.py:199-233)."""
+    if not items:
+        raise ValueError("Empty items list")
+    batch = {}
+    for f in _dc_fields(Experience):
+        values = [getattr(it, f.name) for it in items]
+        head = values[0]
+        if head is None:
+            batch[f.name] = None
+        elif isinstance(head, torch.Tensor):
+            if Experience.is_step_tensor_field(f.name):
+                batch[f.name] = _pad_rows(values, 0, stack=True)
+            elif Experience.is_episode_tensor_field(f.name) or head.dim() == 0:
+                batch[f.name] = torch.stack(values)
+            else:
+                raise ValueError(f"Unsupported tensor field batching rule for {f.name}")
+        elif isinstance(head, dict):
+            out = {}
+            for key in head:
+                vals = [v[key] for v in values]
+                kind = type(vals[0])
+                if not all(isinstance(v, kind) for v in vals):
+                    raise TypeError(f"Inconsistent types in {f.name}[{key}]")
+                out[key] = torch.tensor(vals) if all(isinstance(v, (int, float)) for v in vals) else vals
+            batch[f.name] = out
+        elif isinstance(head, list):
+            batch[f.name] = list(itertools.chain.from_iterable(values))
+    return Experience(**batch)
+
+
+def remove_padding_in_sequences(items: List[Experience]) -> List[Experience]:
+    """Per-step fields of single-sample Experiences cut after the last attended position: what
+    ``attention_mask.flip(0).argmax()`` trailing zeros remove (experience.py:236-247). The cut
+    lengths of all samples come from one extent kernel over the stacked masks when they share a
+    width, else sample by sample."""
+    if not items:
+        return items
+    masks = [it.attention_mask for it in items]
+    if all(m.is_cuda for m in masks) and len({m.numel() for m in masks}) == 1:
+        _, end, _ = row_extents(torch.stack(masks))
+        keep = end.tolist()
+    else:
+        keep = [m.numel() - int(m.flip(0).argmax()) for m in masks]
+    for it, mask, n in zip(items, masks, keep):
+        pad = mask.numel() - (n if n > 0 else mask.numel())  # an all-zero mask keeps everything (argmax 0)
+        if pad == 0:
+            continue
+        for name in STEP_FIELDS:
+            value = getattr(it, name)
+            if isinstance(value, torch.Tensor):
+                setattr(it, name, value[:-pad])
+    return items
+
+
+def balance_experiences(experiences, args):
+    """Spreads long and short sequences evenly over the data-parallel ranks by pairing chunks of
+    the length-sorted samples from both ends (experience.py:250-283)."""
+    samples = [s for exp in experiences for s in split_experience_batch(exp)]
+    samples.sort(key=lambda s: s.total_length, reverse=True)
+    width = args.actor.num_nodes * args.actor.num_gpus_per_node // args.ds.ring_attn_size // args.ds.tensor_parallel_size
+    chunks = [samples[i: i + width] for i in range(0, len(samples), width)]
+    half = len(chunks) // 2
+    front, back = chunks[:half], [c[::-1] for c in chunks[half:]]
+    order = []
+    for i in range(half):
+        order += [front[i], back[-(i + 1)]]
+    if len(back) > len(front):
+        order.append(back[0])
+    columns = itertools.zip_longest(*order)
+    return [make_experience_batch([s for s in col if s is not None]) for col in columns]
