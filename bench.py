@@ -173,6 +173,49 @@ def bench_ppo_step(args, pristine, bufs, cu, ring, dev):
     }
 
 
+def bench_kernels(args, dev):
+    """--workload kernels: the three vocabulary-row kernels launched back to back on ONE resident
+    buffer of --rows x 151936 bf16 logits (forward, in-place backward, one-pass forward+backward,
+    5 launches each), for counter collection with rocprofv3 --pmc. Prints one JSON line of event
+    times; the in-place launches overwrite the buffer, which does not matter for counters."""
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
+
+    n = args.rows
+    x = torch.empty(n, VOCAB, device=dev, dtype=torch.bfloat16)
+    for lo in range(0, n, 2048):
+        x[lo:lo + 2048] = (torch.randn(min(2048, n - lo), VOCAB, device=dev) * 3).to(torch.bfloat16)
+    labels = torch.randint(0, VOCAB, (n,), device=dev)
+    g_lp, g_ent = torch.randn(n, device=dev), torch.randn(n, device=dev)
+
+    def forward():
+        with torch.no_grad():
+            logprobs_and_entropy_from_logits(x, labels)
+
+    def backward():
+        xg = x.requires_grad_(True)
+        lp, ent = logprobs_and_entropy_from_logits(xg, labels, inplace_backward=True)
+        torch.autograd.backward([lp, ent], [g_lp, g_ent])
+        xg.grad = None
+        x.requires_grad_(False)
+
+    def one_pass():
+        fused_logprob_entropy_fwd_bwd(x, labels, g_lp, g_ent, inplace=True)
+
+    out = {}
+    for name, fn in (("forward", forward), ("forward_then_backward", backward), ("one_pass", one_pass)):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(4):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = e0.elapsed_time(e1) / 4
+    print(json.dumps({"workload": f"vocabulary-row kernels on {n} x {VOCAB} bf16 logits", "n_gpus": 1, "unit": "ms",
+                      "entries": out}), flush=True)
+
+
 def bench_per_token(args, dev):
     """--workload per_token: the small kernels at the sizes of the PPO (256 x 8K) and GRPO (4096 x 16K) batches (per-token
     fp32 tensors; MBs, not GBs: these launches are latency-bound, the figures are for the record).
@@ -307,8 +350,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--ring", type=int, default=6, help="distinct logits buffers per timed segment")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU-baseline sample")
-    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token"],
+    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token", "kernels"],
                     help="logprob: the headline step (default); per_token: the small kernels of configs 3/4")
+    ap.add_argument("--rows", type=int, default=8192, help="rows of logits for --workload kernels")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ppo-step", action="store_true", help="skip the extra fused PPO actor step measurement")
     args = ap.parse_args()
@@ -323,6 +367,9 @@ def main():
 
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "kernels":
+        bench_kernels(args, dev)
+        return
     if args.workload == "per_token":
         bench_per_token(args, dev)
         return
