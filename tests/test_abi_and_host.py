@@ -148,3 +148,47 @@ def test_header_is_plain_c(tmp_path):
     res = subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only",
                           "-I", os.path.join(ROOT, "include"), str(src)], capture_output=True, text=True)
     assert res.returncode == 0, res.stderr
+
+
+def test_later_entry_points_reject_bad_arguments_without_a_gpu(lib):
+    """The sequence-level, layout, row-statistics and one-pass entries validate before they launch."""
+    from openrlhf_amd import _lib
+
+    def err():
+        return lib.orlhf_last_error().decode()
+
+    assert lib.orlhf_sequence_logps_fwd(None, None, 7, None, 2, 4, None, None, None, None) == -1 and "mask dtype" in err()
+    assert lib.orlhf_sequence_logps_fwd(None, None, 1, None, 2, 4, None, None, None, None) == -1  # mask NULL for dtype u8
+    assert lib.orlhf_sequence_logps_fwd(None, None, 0, None, 0, 4, None, None, None, None) == 0
+    assert lib.orlhf_sequence_logps_bwd(None, 8, None, 0, None, None, 2, 4, 8, None) == -1 and "counts" in err()
+    assert lib.orlhf_pair_loss_fwd(8, 8, None, None, 3, 9, 0.1, 0.0, 8, None, None, None) == -1 and "kind" in err()
+    assert lib.orlhf_pair_loss_fwd(None, 8, None, None, 3, 0, 0.1, 0.0, 8, None, None, None) == -1
+    assert lib.orlhf_pair_loss_fwd(8, 8, None, None, 3, 0, float("nan"), 0.0, 8, None, None, None) == -1 and "NaN" in err()
+    assert lib.orlhf_pair_loss_fwd(8, 8, None, None, -1, 0, 0.1, 0.0, 8, None, None, None) == -1
+    assert lib.orlhf_pair_loss_bwd(None, 8, 8, None, None, 0, 0, 0.1, 0.0, None, None, None) == 0  # nothing to do
+    assert lib.orlhf_row_extents(8, 0, 2, 4, None, None, None, None) == -1 and "needs a mask" in err()
+    assert lib.orlhf_row_extents(None, 1, 2, 4, None, None, None, None) == -1
+    assert lib.orlhf_cu_seqlens(None, 3, None, None) == -1 and "NULL" in err()
+    assert lib.orlhf_cu_seqlens(None, -1, 8, None) == -1
+    assert lib.orlhf_pack_rows(8, 3, 2, 4, None, 8, 8, None) == -1 and "element size" in err()
+    assert lib.orlhf_pack_rows(8, 4, 2, 4, None, None, 8, None) == -1
+    assert lib.orlhf_pack_rows(None, 4, 0, 4, None, None, None, None) == 0
+    assert lib.orlhf_pad_rows(8, 16, 8, 2, 4, 0, 0, 8, None) == -1 and "element size" in err()
+    assert lib.orlhf_pad_rows(8, 4, None, 2, 4, 0, 0, 8, None) == -1
+    assert lib.orlhf_kl_rows(8, 8, 0, None, 0, 2, 4, None, 5, 1, None, None, None, None) == -1 and "estimator" in err()
+    assert lib.orlhf_kl_rows(None, None, 0, None, 0, 2, 4, None, 0, 1, None, None, None, None) == -1
+    assert lib.orlhf_kl_rows(8, 8, 7, None, 0, 2, 4, None, 0, 1, None, None, None, None) == -1 and "dtype" in err()
+    assert lib.orlhf_masked_normalize_rows(None, None, 0, 2, 4, None, 1e-8, None, None) == -1
+    assert lib.orlhf_masked_normalize_rows(None, None, 0, 0, 4, None, 1e-8, None, None) == 0
+    assert lib.orlhf_divide_rows_inplace(8, 1, 2, 8, 8, 0.0, None) == -1 and "divisor" in err()
+    assert lib.orlhf_divide_rows_inplace(None, 1, 2, 8, 8, 0.5, None) == -1
+    assert lib.orlhf_mask_counts(None, 1, 2, 4, None, None, None, None) == -1
+    assert lib.orlhf_masked_aggregate_fwd(None, None, 0, 1, 1, None, 4, None, None, None, None, None) == -1 and "mode" in err()
+    # the one-pass kernel keeps a row on one CU: longer rows are refused with a pointer to the two kernels
+    assert lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(_lib.BF16) == 155648
+    assert lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(_lib.F32) == 77824
+    assert lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(9) == 0
+    assert lib.orlhf_logprob_entropy_fwd_bwd(8, 8, 1, 2, 262144, 262144, 262144, 8, 1.0, 8, None, 8, None, None, None) == -3
+    assert "separate forward and backward" in err()
+    assert lib.orlhf_logprob_entropy_fwd_bwd(16, 32 + 2, 1, 2, 1024, 1024, 1024, 8, 1.0, 8, None, 8, None, None, None) == -3
+    assert "16-byte phases" in err()
