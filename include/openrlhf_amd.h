@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 8
+#define ORLHF_ABI_VERSION 9
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -131,14 +131,16 @@ int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, int dtype, 
  * runs, i.e. whose loss is sum_i w_logprob[i]*logprob[i] + w_entropy[i]*entropy[i] (SFT:
  * w_logprob = -mask/N, openrlhf/models/loss.py:104): computes logprob / entropy exactly as
  * orlhf_logprob_entropy_fwd and writes d(loss)/d(logits) exactly as orlhf_logprob_entropy_bwd
- * with g = w, but reads every logits row once (the row stays in the registers / LDS of one CU),
- * so a token costs 2*V*sizeof(dtype) bytes of HBM traffic instead of 3*V*sizeof(dtype).
+ * with g = w, but reads every logits row once (the row stays in the registers of one CU), so a
+ * token costs 2*V*sizeof(dtype) bytes of HBM traffic instead of 3*V*sizeof(dtype). Rows longer
+ * than the registers hold (155648 bf16/fp16 or 77824 fp32 elements) keep their first 131072 /
+ * 65536 elements there and stream the rest twice (2.5*V at V = 262144).
  * Replaces the same reference lines as the two calls above (openrlhf/models/utils.py:129-163,
  * 182-186 and their autograd). grad_logits may alias logits. w_* / logprob / entropy nullable
- * (a NULL weight array is all zeros). Returns ORLHF_ERR_UNSUPPORTED when a row does not fit on
- * chip (vocab > orlhf_logprob_entropy_fwd_bwd_max_vocab(dtype): 155648 for bf16/fp16, 77824 for
- * fp32) or when logits and grad rows differ in their 16-byte phase; callers then use the two
- * separate entry points.
+ * (a NULL weight array is all zeros). Returns ORLHF_ERR_UNSUPPORTED when a row is too long for
+ * that to pay (vocab > orlhf_logprob_entropy_fwd_bwd_max_vocab(dtype): 524288 for bf16/fp16,
+ * 262144 for fp32) or when logits and grad rows differ in their 16-byte phase; callers then use
+ * the two separate entry points.
  */
 int64_t orlhf_logprob_entropy_fwd_bwd_max_vocab(int dtype);
 int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logits, int dtype, int64_t n_rows,

@@ -6,7 +6,10 @@
 // A row of 151936 bf16 logits is 297 KiB; the vector register file of one CU is 512 KiB. One
 // 512-thread workgroup (8 wave64, 2 per SIMD, up to 256 VGPRs each) owns a CU and a row: every
 // lane keeps 38 16-byte chunks of the row in registers (rows up to 38*512 chunks: 155648 bf16 /
-// fp16 or 77824 fp32 elements; longer rows are left to the separate kernels).
+// fp16 or 77824 fp32 elements). A longer row keeps its first 32*512 chunks in registers and
+// streams the rest twice (once for the sums, once for the gradient, the second time from the
+// caches when they still hold it): 2.5 x V bytes per token at V = 262144 instead of 3 x; rows
+// beyond four times the resident part are left to the separate kernels.
 #include "token_terms.h"
 #include "vocab_rows.h"
 
@@ -16,6 +19,15 @@ constexpr int kFusedBlock = 512;
 constexpr int kFusedWaves = kFusedBlock / kWave;
 constexpr int kAccF = 2;               // independent accumulators per lane
 constexpr int kFusedRegChunks = 38;    // 16-byte chunks of the row each lane keeps in registers
+constexpr int kFusedRegChunksLong = 32;  // the same for rows that do not fit: the rest is streamed twice
+constexpr int kTailInFlight = 6;         // streamed 16-byte chunks in flight per lane (two batches of 3)
+constexpr int kFusedMaxTailFactor = 4;   // longest row = 4 x the resident part; beyond, streaming three
+                                         // quarters of the row twice is no better than the two kernels
+
+constexpr int kTailHalf = kTailInFlight / 2;            // chunks per batch; two batches alternate
+constexpr uint32_t kTailStep = (uint32_t)kTailHalf * 512u;  // vectors one batch covers (512 = workgroup size)
+
+__device__ __forceinline__ u32x4 load_vec_cached(const char* p) { return *(const u32x4*)p; }
 
 // value that contributes exp() == 0 and 0 * x == -0 (not NaN) for lanes past the row end
 template <int DT>
@@ -25,6 +37,17 @@ __device__ __forceinline__ u32x4 neutral_vec() {
   return u32x4{0xfbfffbffu, 0xfbfffbffu, 0xfbfffbffu, 0xfbfffbffu};  // fp16 -65504
 }
 constexpr float kNeutral = -3.0e38f;
+
+// One batch of streamed chunks: vector v0 + u*512 + tid for u < kTailHalf, neutral past the row end.
+template <int DT>
+__device__ __forceinline__ void tail_load(u32x4 (&t)[kTailHalf], const char* body, uint32_t v0, uint32_t nvec,
+                                          uint32_t tid) {
+#pragma unroll
+  for (int u = 0; u < kTailHalf; ++u) {
+    const uint32_t v = v0 + (uint32_t)u * 512u + tid;
+    t[u] = v < nvec ? load_vec_cached(body + v * 16u) : neutral_vec<DT>();
+  }
+}
 
 // Makes the compiler forget what it knows about a resident chunk, so that every pass unpacks the
 // 16-byte chunk again instead of keeping 8 fp32 values per chunk alive across passes (which
@@ -52,7 +75,7 @@ struct StepTerms {
   float kl_coef, entropy_coef;
 };
 
-template <int DT, int MODE, int REG_CHUNKS, bool TERMS>
+template <int DT, int MODE, int REG_CHUNKS, bool TERMS, bool TAIL>
 __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel(
     const char* logits, char* grad, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
     int64_t grad_stride_bytes, const int64_t* __restrict__ labels, double temperature,
@@ -62,6 +85,7 @@ __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel
   using E = Elt<DT>;
   using MT = ModeTraits<MODE>;
   constexpr int EPV = E::kPerVec;
+  constexpr uint32_t kRegVecs = (uint32_t)REG_CHUNKS * kFusedBlock;  // vectors of a row held in registers
   __shared__ float lds_max[kFusedWaves];
   __shared__ float lds_sum[kFusedWaves][8];
   __shared__ float lds_bcast[8];
@@ -143,6 +167,30 @@ __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel
 #pragma unroll
         for (int j = 0; j < EPV; ++j) accumulate(x[j], j % kAccF);
       }
+      if (TAIL) {  // the part of a long row that does not fit in registers is streamed (and stays cached)
+        const char* tbody = row + g.head * E::kSize;
+        auto consume = [&](const u32x4 (&t)[kTailHalf]) {
+#pragma unroll
+          for (int u = 0; u < kTailHalf; ++u) {
+            float x[EPV];
+            E::unpack(t[u], x);
+#pragma unroll
+            for (int j = 0; j < EPV; ++j) accumulate(x[j], j % kAccF);
+          }
+        };
+        u32x4 t0[kTailHalf], t1[kTailHalf];
+        uint32_t v0 = kRegVecs;
+        tail_load<DT>(t0, tbody, v0, g.nvec, tid);
+        while (v0 < g.nvec) {  // two batches alternate: one is in flight while the other is consumed
+          tail_load<DT>(t1, tbody, v0 + kTailStep, g.nvec, tid);
+          consume(t0);
+          v0 += kTailStep;
+          if (v0 >= g.nvec) break;
+          tail_load<DT>(t0, tbody, v0 + kTailStep, g.nvec, tid);
+          consume(t1);
+          v0 += kTailStep;
+        }
+      }
       const float wst = wave_sum(sT[0] + sT[1]);
       const float ws1 = wave_sum(s1[0] + s1[1]);
       const float wt1 = wave_sum(t1[0] + t1[1]);
@@ -199,6 +247,18 @@ __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel
         for (int j = 0; j < EPV; ++j) {
           m = fmaxf(m, x[j]);
           nan_seen = nan_seen || (x[j] != x[j]);
+        }
+      }
+      if (TAIL) {
+        const char* tbody = row + g.head * E::kSize;
+        for (uint32_t v = kRegVecs + tid; v < g.nvec; v += kFusedBlock) {
+          float x[EPV];
+          E::unpack(load_vec_cached(tbody + v * 16u), x);
+#pragma unroll
+          for (int j = 0; j < EPV; ++j) {
+            m = fmaxf(m, x[j]);
+            nan_seen = nan_seen || (x[j] != x[j]);
+          }
         }
       }
       m = wave_max(m);
@@ -300,6 +360,33 @@ __global__ __launch_bounds__(kFusedBlock) void logprob_entropy_fused_pipe_kernel
       }
       buf[c] = v < gn.nvec ? load_vec(nbody + (uint32_t)c * (kFusedBlock * 16u) + tid16) : neutral_vec<DT>();
     }
+    if (TAIL) {  // the streamed part again (from the caches when they still hold it), then its gradient
+      const char* tbody = row + g.head * E::kSize;
+      auto emit = [&](const u32x4 (&t)[kTailHalf], uint32_t base) {
+#pragma unroll
+        for (int u = 0; u < kTailHalf; ++u) {
+          const uint32_t v = base + (uint32_t)u * kFusedBlock + tid;
+          if (v < g.nvec) {
+            float x[EPV];
+            E::unpack(t[u], x);
+            fn.vec(x, v);
+            store_vec(obody + v * 16u, E::pack(x));
+          }
+        }
+      };
+      u32x4 t0[kTailHalf], t1[kTailHalf];
+      uint32_t v0 = kRegVecs;
+      tail_load<DT>(t0, tbody, v0, g.nvec, tid);
+      while (v0 < g.nvec) {
+        tail_load<DT>(t1, tbody, v0 + kTailStep, g.nvec, tid);
+        emit(t0, v0);
+        v0 += kTailStep;
+        if (v0 >= g.nvec) break;
+        tail_load<DT>(t0, tbody, v0 + kTailStep, g.nvec, tid);
+        emit(t1, v0);
+        v0 += kTailStep;
+      }
+    }
     if (tid < nscalar) {
       fn.one(xs, scalar_e);
       E::store1(out_row + scalar_e * E::kSize, xs);
@@ -331,15 +418,19 @@ static int launch_fused(const void* logits, void* grad, int64_t n_rows, int64_t 
   const int64_t blocks = n_rows < n_cu ? n_rows : n_cu;
   const dim3 grid((unsigned)blocks), block(kFusedBlock);
   StepTerms none = {};
+  const bool long_rows = vocab > (int64_t)kFusedRegChunks * kFusedBlock * E::kPerVec;
+#define ORLHF_FUSED_ARGS                                                                                        \
+  grid, block, 0, stream, p, gp, n_rows, vocab, sb, gsb, labels, temperature, w_logprob, w_entropy, logprob, entropy, \
+      row_mask
 #define ORLHF_FUSED(M)                                                                                             \
-  if (terms != nullptr)                                                                                            \
-    hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunks, true>), grid, block, 0, stream,  \
-                       p, gp, n_rows, vocab, sb, gsb, labels, temperature, w_logprob, w_entropy, logprob, entropy, \
-                       row_mask, *terms);                                                                          \
+  if (long_rows && terms != nullptr)                                                                               \
+    hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunksLong, true, true>), ORLHF_FUSED_ARGS, *terms); \
+  else if (long_rows)                                                                                              \
+    hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunksLong, false, true>), ORLHF_FUSED_ARGS, none); \
+  else if (terms != nullptr)                                                                                       \
+    hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunks, true, false>), ORLHF_FUSED_ARGS, *terms); \
   else                                                                                                             \
-    hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunks, false>), grid, block, 0, stream, \
-                       p, gp, n_rows, vocab, sb, gsb, labels, temperature, w_logprob, w_entropy, logprob, entropy, \
-                       row_mask, none)
+    hipLaunchKernelGGL((logprob_entropy_fused_pipe_kernel<DT, M, kFusedRegChunks, false, false>), ORLHF_FUSED_ARGS, none)
   switch (mode) {
     case kLpOnly: ORLHF_FUSED(kLpOnly); break;
     case kEntOnly: ORLHF_FUSED(kEntOnly); break;
@@ -347,6 +438,7 @@ static int launch_fused(const void* logits, void* grad, int64_t n_rows, int64_t 
     default: ORLHF_FUSED(kBothT); break;
   }
 #undef ORLHF_FUSED
+#undef ORLHF_FUSED_ARGS
   ORLHF_CHECK_LAUNCH("orlhf_logprob_entropy_fwd_bwd");
   return ORLHF_OK;
 }
@@ -358,7 +450,7 @@ using namespace orlhf;
 extern "C" int64_t orlhf_logprob_entropy_fwd_bwd_max_vocab(int dtype) {
   const int64_t per_vec = dtype == ORLHF_F32 ? 4 : 8;
   if (dtype != ORLHF_F32 && dtype != ORLHF_BF16 && dtype != ORLHF_F16) return 0;
-  return (int64_t)kFusedRegChunks * kFusedBlock * per_vec;
+  return (int64_t)kFusedMaxTailFactor * kFusedRegChunksLong * kFusedBlock * per_vec;
 }
 
 static int fused_entry(const void* logits, void* grad_logits, int dtype, int64_t n_rows, int64_t vocab,
@@ -385,8 +477,8 @@ static int fused_entry(const void* logits, void* grad_logits, int dtype, int64_t
                   "logprob_entropy_fwd_bwd: pointers not aligned to the element size");
   if (vocab > orlhf_logprob_entropy_fwd_bwd_max_vocab(dtype))
     return fail(ORLHF_ERR_UNSUPPORTED,
-                "logprob_entropy_fwd_bwd: a row of %lld elements does not fit on one CU (max %lld); use the "
-                "separate forward and backward",
+                "logprob_entropy_fwd_bwd: a row of %lld elements is too long for the one-pass kernel (max %lld); "
+                "use the separate forward and backward",
                 (long long)vocab, (long long)orlhf_logprob_entropy_fwd_bwd_max_vocab(dtype));
   const bool same_phase = (((uintptr_t)logits ^ (uintptr_t)grad_logits) & 15u) == 0 &&
                           (((row_stride - grad_row_stride) * esize) & 15) == 0;

@@ -167,7 +167,7 @@ def fused_actor_loss_step(
             raise ValueError(f"{n_rows} logits rows for {labels.numel()} token positions")
         code = _lib.dtype_code(rows)
         if vocab > _lib.load().orlhf_logprob_entropy_fwd_bwd_max_vocab(code):
-            raise ValueError(f"a row of {vocab} {rows.dtype} logits does not fit on one CU; use actor_loss_step")
+            raise ValueError(f"a row of {vocab} {rows.dtype} logits is too long for the one-pass kernel; use actor_loss_step")
 
         terms = _lib.StepTerms()
         terms.old_log_probs, terms.advantages = ptr(old_r), ptr(adv_r)

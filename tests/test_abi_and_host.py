@@ -184,11 +184,12 @@ def test_later_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.orlhf_divide_rows_inplace(None, 1, 2, 8, 8, 0.5, None) == -1
     assert lib.orlhf_mask_counts(None, 1, 2, 4, None, None, None, None) == -1
     assert lib.orlhf_masked_aggregate_fwd(None, None, 0, 1, 1, None, 4, None, None, None, None, None) == -1 and "mode" in err()
-    # the one-pass kernel keeps a row on one CU: longer rows are refused with a pointer to the two kernels
-    assert lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(_lib.BF16) == 155648
-    assert lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(_lib.F32) == 77824
+    # the one-pass kernel keeps (most of) a row on one CU: rows beyond four times the resident part
+    # are refused with a pointer to the two kernels
+    assert lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(_lib.BF16) == 524288
+    assert lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(_lib.F32) == 262144
     assert lib.orlhf_logprob_entropy_fwd_bwd_max_vocab(9) == 0
-    assert lib.orlhf_logprob_entropy_fwd_bwd(8, 8, 1, 2, 262144, 262144, 262144, 8, 1.0, 8, None, 8, None, None, None) == -3
+    assert lib.orlhf_logprob_entropy_fwd_bwd(8, 8, 1, 2, 600000, 600000, 600000, 8, 1.0, 8, None, 8, None, None, None) == -3
     assert "separate forward and backward" in err()
     assert lib.orlhf_logprob_entropy_fwd_bwd(16, 32 + 2, 1, 2, 1024, 1024, 1024, 8, 1.0, 8, None, 8, None, None, None) == -3
     assert "16-byte phases" in err()

@@ -149,3 +149,26 @@ def test_fused_step_rescales_when_upstream_differs(cuda):
     with pytest.raises(ValueError):
         fused_actor_loss_step(logits.to(d), seqs.to(d), attn.to(d), amask.to(d), old.to(d), adv.to(d),
                               PolicyLoss(policy_loss_type="gspo"))
+
+
+def test_fused_step_on_a_vocabulary_longer_than_the_registers(cuda):
+    """V = 262144 (half of every row streamed): the one-pass step against the composed one."""
+    from openrlhf_amd.models.loss import PolicyLoss
+    from openrlhf_amd.trainer.ray.ppo_actor import actor_loss_step, fused_actor_loss_step
+
+    logits, seqs, attn, amask, old, adv, base, roll = _batch(13, b=3, t=16, vocab=262144, a=11)
+    logits = logits.to(torch.bfloat16)
+    d = cuda
+    kw = dict(base_action_log_probs=base.to(d), kl_estimator="k3", kl_coef=0.05, entropy_coef=0.01, temperature=0.6)
+    fn = PolicyLoss(0.2, 0.28, dual_clip=3.0)
+    tensors = (seqs.to(d), attn.to(d), amask.to(d), old.to(d), adv.to(d), fn)
+    xa = logits.to(d).requires_grad_(True)
+    ref = actor_loss_step(xa, *tensors, **kw)
+    ref["loss"].backward()
+    xb = logits.to(d).requires_grad_(True)
+    out = fused_actor_loss_step(xb, *tensors, **kw)
+    out["loss"].backward()
+    for key in ("loss", "actor_loss", "kl_loss", "entropy_loss", "clip_ratio", "ppo_kl"):
+        assert abs(out[key].item() - ref[key].item()) <= 2e-5 * max(1.0, abs(ref[key].item())), key
+    ga, gb = xa.grad.float(), xb.grad.float()
+    assert (ga - gb).abs().max().item() <= 2.0 ** -7 * ga.abs().max().item()

@@ -35,14 +35,16 @@ def _analytic_grad64(x, labels, temperature, g_lp, g_ent):
     "rows,vocab,dtype,std,temperature",
     [
         (40, 151936, torch.bfloat16, 3.0, 1.0),   # config-2 row: registers only
-        (12, 262144, torch.bfloat16, 4.0, 0.6),   # config-5 row: registers + LDS, two statistic sets
-        (12, 200000, torch.float16, 2.0, 1.0),    # LDS path, fp16
+        (12, 262144, torch.bfloat16, 4.0, 0.6),   # config-5 row: half in registers, half streamed twice; two statistic sets
+        (12, 200000, torch.float16, 2.0, 1.0),    # streamed tail, fp16
+        (9, 155649, torch.bfloat16, 3.0, 1.0),    # one element more than the registers hold
         (33, 32000, torch.float32, 2.0, 1.0),
         (33, 50257, torch.bfloat16, 3.0, 0.7),    # scalar tail
-        (17, 100003, torch.float32, 2.0, 1.3),    # fp32 LDS path, odd vocabulary
+        (17, 100003, torch.float32, 2.0, 1.3),    # fp32 streamed tail, odd vocabulary
         (300, 7, torch.float32, 1.0, 1.0),
         (64, 4096, torch.bfloat16, 2.0, 1.0),
-        (5, 400000, torch.bfloat16, 2.0, 1.0),    # does not fit on chip: separate kernels
+        (5, 400000, torch.bfloat16, 2.0, 1.0),    # two thirds of the row streamed
+        (3, 600000, torch.bfloat16, 2.0, 1.0),    # beyond the one-pass limit: separate kernels
     ],
 )
 @pytest.mark.parametrize("inplace", [True, False])
@@ -95,6 +97,42 @@ def test_fused_misaligned_rows_row_mask_and_optional_weights(cuda):
         assert lp[3].item() == 0.0 and ent[3].item() == 0.0 and grad[3].abs().max().item() == 0.0
         err = (grad.cpu().double() - ref)[keep].abs()
         assert (err <= 2.0 ** -8 * ref[keep].abs() + 1e-6).all()
+
+
+def test_fused_extreme_values_in_the_streamed_tail(cuda):
+    """Long rows whose awkward entries sit in the streamed part: a late spike and a very low start
+    force the exact-maximum pass over registers AND tail; -inf / +inf / NaN entries in the tail give
+    the separate kernels' results."""
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
+
+    vocab = 200003
+    g = torch.Generator().manual_seed(19)
+    x = (torch.randn(6, vocab, generator=g) * 2).to(torch.bfloat16)
+    x[0, vocab - 5] = 400.0
+    x[1, :150000] = -3.0e4
+    x[2, 160000::3] = float("-inf")
+    x[3, vocab - 9] = float("inf")
+    x[4, vocab - 2] = float("nan")
+    labels = torch.tensor([vocab - 5, 190000, 160001, 3, 4, 7])
+    w1, w2 = torch.randn(6, generator=g), torch.randn(6, generator=g)
+    a = x.to(cuda).requires_grad_(True)
+    lp2, ent2 = logprobs_and_entropy_from_logits(a, labels.to(cuda), 0.8)
+    (g2,) = torch.autograd.grad((lp2 * w1.to(cuda)).sum() + (ent2 * w2.to(cuda)).sum(), a)
+    lp, ent, grad = fused_logprob_entropy_fwd_bwd(x.to(cuda), labels.to(cuda), w1.to(cuda), w2.to(cuda), 0.8, inplace=True)
+
+    def same(p, q, tol):
+        p, q = p.float().cpu(), q.float().cpu()
+        assert torch.equal(torch.isnan(p), torch.isnan(q))
+        fin = torch.isfinite(p) & torch.isfinite(q)
+        assert torch.equal(p[~fin & ~torch.isnan(p)], q[~fin & ~torch.isnan(q)])  # same infinities
+        if fin.any():
+            assert (p[fin] - q[fin]).abs().max().item() <= tol * max(1.0, q[fin].abs().max().item())
+
+    same(lp, lp2, 2e-5)
+    same(ent, ent2, 2e-5)
+    same(grad, g2, 2.0 ** -7)
+    ref_lp = otn.log_probs_from_logits(x[:3].double(), labels[:3], 0.8)
+    assert (lp[:3].cpu().double() - ref_lp).abs().max().item() <= 2e-3 * max(1.0, ref_lp.abs().max().item() * 1e-2)
 
 
 def test_fused_extreme_rows(cuda):
