@@ -20,7 +20,7 @@ Deliberate differences from the reference, all on the value-preserving side:
   * ``compute_reward`` takes tensors only (the reference's list-of-tensors form of ``kl`` is not
     used by any caller).
 """
-from typing import Optional, Tuple, Union
+from typing import Optional, Tuple
 
 import torch
 

@@ -5,7 +5,7 @@ Mirrors openrlhf/trainer/dpo_trainer.py:306-382 (``concatenated_forward`` after 
 ``_get_batch_logps`` (attention mask with the prompt cleared, shifted by one) is built inside the
 kernel from the attention mask and the prompt lengths: no clone, no per-row Python loop.
 """
-from typing import Optional, Sequence, Union
+from typing import Sequence, Union
 
 import torch
 

@@ -18,15 +18,13 @@ Not mirrored: the Mixtral auxiliary loss (a scalar the model returns, added by t
 optimizer step, DeepSpeed. GSPO and seq-mask-TIS need a sequence-level ratio before any token can
 be differentiated; ``fused_actor_loss_step`` refuses them (use ``actor_loss_step``).
 """
-from typing import Optional
-
 import torch
 
 from ... import _lib
 from ..._lib import call, ptr, require_gpu, stream_of
 from ...models.actor import actor_forward_tail
 from ...models.loss import PolicyLoss, aggregate_loss
-from ...models.utils import _KL_CODES, _as_rows, _f32, _workspace, compute_approx_kl, masked_mean
+from ...models.utils import _KL_CODES, _as_rows, _workspace, compute_approx_kl
 
 
 def actor_loss_step(
