@@ -530,12 +530,12 @@ extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t 
                   (long long)row_stride, (long long)vocab);
   ORLHF_CHECK_ARG(vocab < (1ll << 29), "logprob_entropy_fwd: vocab %lld too large (row must stay below 2 GiB)",
                   (long long)vocab);
-  ORLHF_CHECK_ARG(logprob != nullptr || entropy != nullptr,
-                  "logprob_entropy_fwd: logprob and entropy are both NULL");
   ORLHF_CHECK_ARG(temperature > 0.0 && temperature == temperature,
                   "logprob_entropy_fwd: temperature must be > 0");
   ORLHF_CHECK_ARG(flags == 0, "logprob_entropy_fwd: unknown flags 0x%x", flags);
-  if (n_rows == 0) return ORLHF_OK;
+  if (n_rows == 0) return ORLHF_OK;  // nothing to launch; empty outputs may well be NULL
+  ORLHF_CHECK_ARG(logprob != nullptr || entropy != nullptr,
+                  "logprob_entropy_fwd: logprob and entropy are both NULL");
   ORLHF_CHECK_ARG(logits != nullptr, "logprob_entropy_fwd: logits is NULL");
   ORLHF_CHECK_ARG(logprob == nullptr || labels != nullptr, "logprob_entropy_fwd: labels is NULL");
   hipStream_t s = (hipStream_t)stream;
@@ -570,11 +570,11 @@ extern "C" int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, 
                   (long long)grad_row_stride, (long long)vocab);
   ORLHF_CHECK_ARG(vocab < (1ll << 29), "logprob_entropy_bwd: vocab %lld too large (row must stay below 2 GiB)",
                   (long long)vocab);
-  ORLHF_CHECK_ARG(g_logprob != nullptr || g_entropy != nullptr,
-                  "logprob_entropy_bwd: g_logprob and g_entropy are both NULL");
   ORLHF_CHECK_ARG(temperature > 0.0 && temperature == temperature,
                   "logprob_entropy_bwd: temperature must be > 0");
-  if (n_rows == 0) return ORLHF_OK;
+  if (n_rows == 0) return ORLHF_OK;  // nothing to launch; empty arrays may well be NULL
+  ORLHF_CHECK_ARG(g_logprob != nullptr || g_entropy != nullptr,
+                  "logprob_entropy_bwd: g_logprob and g_entropy are both NULL");
   ORLHF_CHECK_ARG(logits != nullptr && grad_logits != nullptr && row_stats != nullptr,
                   "logprob_entropy_bwd: NULL logits / grad_logits / row_stats");
   ORLHF_CHECK_ARG(g_logprob == nullptr || labels != nullptr, "logprob_entropy_bwd: labels is NULL");

@@ -465,10 +465,10 @@ static int fused_entry(const void* logits, void* grad_logits, int dtype, int64_t
   ORLHF_CHECK_ARG(temperature > 0.0 && temperature == temperature, "logprob_entropy_fwd_bwd: temperature must be > 0");
   ORLHF_CHECK_ARG(dtype == ORLHF_F32 || dtype == ORLHF_BF16 || dtype == ORLHF_F16,
                   "logprob_entropy_fwd_bwd: unknown dtype %d", dtype);
+  if (n_rows == 0) return ORLHF_OK;  // nothing to launch; empty arrays may well be NULL
   ORLHF_CHECK_ARG(terms != nullptr || w_logprob != nullptr || w_entropy != nullptr || logprob != nullptr ||
                       entropy != nullptr,
                   "logprob_entropy_fwd_bwd: nothing to compute");
-  if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(logits != nullptr && grad_logits != nullptr, "logprob_entropy_fwd_bwd: NULL logits / grad_logits");
   ORLHF_CHECK_ARG((logprob == nullptr && w_logprob == nullptr && terms == nullptr) || labels != nullptr,
                   "logprob_entropy_fwd_bwd: labels is NULL");

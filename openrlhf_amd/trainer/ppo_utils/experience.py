@@ -67,6 +67,8 @@ def pack_padded(x: torch.Tensor, cu_seqlens: torch.Tensor, first: Optional[torch
     src = x.contiguous()
     total = int(cu_seqlens[-1]) if total is None else int(total)
     out = torch.empty(total, dtype=x.dtype, device=dev)
+    if total == 0:  # every row is empty: nothing to copy (and no destination to hand over)
+        return out
     cu = cu_seqlens.to(torch.int64).contiguous()
     f = None if first is None else first.to(torch.int64).contiguous()
     with torch.cuda.device(dev):
