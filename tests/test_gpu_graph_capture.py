@@ -131,3 +131,25 @@ def test_logprob_entropy_kernels_replay(cuda, dtype):
             assert torch.equal(got, want)
         for got, want in zip(out_one, eager_one):
             assert torch.equal(got, want)
+
+
+def test_launches_follow_the_current_stream(cuda):
+    """Work queued on a side stream is ordered with the producer of its inputs on that stream
+    (the entry points take the caller's stream, not the default one)."""
+    from openrlhf_amd.models.loss import PolicyLoss
+    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+
+    side = torch.cuda.Stream()
+    n, v = 512, 32000
+    labels = torch.randint(0, v, (n,), device=cuda)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        big = torch.randn(n, v, device=cuda)          # produced on the side stream ...
+        for _ in range(20):
+            big = big * 1.0001 + 0.0001               # ... by a chain of kernels that takes a while
+        lp, ent = logprobs_and_entropy_from_logits(big, labels)   # consumed on the same stream, no sync between
+        loss = PolicyLoss()(lp, lp.detach() + 0.01, ent, action_mask=None)[0]
+    side.synchronize()
+    ref = torch.log_softmax(big.double(), -1).gather(1, labels[:, None]).squeeze(1)
+    assert (lp.double() - ref).abs().max().item() <= 1e-5
+    assert torch.isfinite(loss)
