@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
                                                             NormArg norm, float post_scale, int n_out,
                                                             float* __restrict__ out,
                                                             float* __restrict__ row_coef) {
-  __shared__ double lds[kWavesPerBlock];
+  __shared__ double lds[NQ + 2][kWavesPerBlock];
   double tot[NQ];
 #pragma unroll
   for (int i = 0; i < NQ; ++i) tot[i] = 0.0;
@@ -234,10 +234,34 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
     }
     return;
   }
+  // every sum through the cross-lane steps together, one LDS exchange for all of them
 #pragma unroll
-  for (int i = 0; i < NQ; ++i) tot[i] = block_sum(tot[i], lds);
-  seq_sum = block_sum(seq_sum, lds);
-  seq_cnt = block_sum(seq_cnt, lds);
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) tot[i] += __shfl_xor(tot[i], o, kWave);
+    seq_sum += __shfl_xor(seq_sum, o, kWave);
+    seq_cnt += __shfl_xor(seq_cnt, o, kWave);
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    const int wave = threadIdx.x / kWave;
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) lds[i][wave] = tot[i];
+    lds[NQ][wave] = seq_sum;
+    lds[NQ + 1][wave] = seq_cnt;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int i = 0; i < NQ; ++i) {
+    tot[i] = 0.0;
+#pragma unroll
+    for (int w = 0; w < kWavesPerBlock; ++w) tot[i] += lds[i][w];
+  }
+  seq_sum = seq_cnt = 0.0;
+#pragma unroll
+  for (int w = 0; w < kWavesPerBlock; ++w) {
+    seq_sum += lds[NQ][w];
+    seq_cnt += lds[NQ + 1][w];
+  }
 
   if (mode == kAggCounts) {
     if (threadIdx.x == 0) {
