@@ -180,26 +180,26 @@ def bench_kernels(args, dev):
     times; the in-place launches overwrite the buffer, which does not matter for counters."""
     from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
 
-    n = args.rows
-    x = torch.empty(n, VOCAB, device=dev, dtype=torch.bfloat16)
-    for lo in range(0, n, 2048):
-        x[lo:lo + 2048] = (torch.randn(min(2048, n - lo), VOCAB, device=dev) * 3).to(torch.bfloat16)
-    labels = torch.randint(0, VOCAB, (n,), device=dev)
+    n, vocab, temperature = args.rows, args.vocab, args.temperature
+    x = torch.empty(n, vocab, device=dev, dtype=torch.bfloat16)
+    for lo in range(0, n, 1024):
+        x[lo:lo + 1024] = (torch.randn(min(1024, n - lo), vocab, device=dev) * 3).to(torch.bfloat16)
+    labels = torch.randint(0, vocab, (n,), device=dev)
     g_lp, g_ent = torch.randn(n, device=dev), torch.randn(n, device=dev)
 
     def forward():
         with torch.no_grad():
-            logprobs_and_entropy_from_logits(x, labels)
+            logprobs_and_entropy_from_logits(x, labels, temperature)
 
     def backward():
         xg = x.requires_grad_(True)
-        lp, ent = logprobs_and_entropy_from_logits(xg, labels, inplace_backward=True)
+        lp, ent = logprobs_and_entropy_from_logits(xg, labels, temperature, inplace_backward=True)
         torch.autograd.backward([lp, ent], [g_lp, g_ent])
         xg.grad = None
         x.requires_grad_(False)
 
     def one_pass():
-        fused_logprob_entropy_fwd_bwd(x, labels, g_lp, g_ent, inplace=True)
+        fused_logprob_entropy_fwd_bwd(x, labels, g_lp, g_ent, temperature=temperature, inplace=True)
 
     out = {}
     for name, fn in (("forward", forward), ("forward_then_backward", backward), ("one_pass", one_pass)):
@@ -212,7 +212,8 @@ def bench_kernels(args, dev):
         e1.record()
         torch.cuda.synchronize()
         out[name] = e0.elapsed_time(e1) / 4
-    print(json.dumps({"workload": f"vocabulary-row kernels on {n} x {VOCAB} bf16 logits", "n_gpus": 1, "unit": "ms",
+    print(json.dumps({"workload": f"vocabulary-row kernels on {n} x {vocab} bf16 logits, temperature {temperature}",
+                      "n_gpus": 1, "unit": "ms",
                       "entries": out}), flush=True)
 
 
@@ -353,6 +354,8 @@ def main():
     ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token", "kernels"],
                     help="logprob: the headline step (default); per_token: the small kernels of configs 3/4")
     ap.add_argument("--rows", type=int, default=8192, help="rows of logits for --workload kernels")
+    ap.add_argument("--vocab", type=int, default=VOCAB, help="vocabulary for --workload kernels")
+    ap.add_argument("--temperature", type=float, default=1.0, help="temperature for --workload kernels")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-ppo-step", action="store_true", help="skip the extra fused PPO actor step measurement")
     args = ap.parse_args()
