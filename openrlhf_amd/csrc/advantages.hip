@@ -332,12 +332,11 @@ template <bool GAE>
 static void launch_scan(int mask_dtype, Rows rows, const float* values, const float* rewards, const void* mask,
                         double gamma, double coef, float* adv, float* ret, hipStream_t s) {
   const dim3 grid((unsigned)(rows.n_rows < 65536 ? rows.n_rows : 65536)), block(kBlock);
-  switch (mask_dtype) {
-    case ORLHF_MASK_NONE: hipLaunchKernelGGL((reverse_scan_kernel<ORLHF_MASK_NONE, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, ret); break;
-    case ORLHF_MASK_U8: hipLaunchKernelGGL((reverse_scan_kernel<ORLHF_MASK_U8, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, ret); break;
-    case ORLHF_MASK_F32: hipLaunchKernelGGL((reverse_scan_kernel<ORLHF_MASK_F32, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, ret); break;
-    default: hipLaunchKernelGGL((reverse_scan_kernel<ORLHF_MASK_I64, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, ret); break;
-  }
+#define ORLHF_LAUNCH(M)                                                                                          \
+  hipLaunchKernelGGL((reverse_scan_kernel<M, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, \
+                     ret)
+  ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
+#undef ORLHF_LAUNCH
 }
 
 }  // namespace orlhf
@@ -355,12 +354,11 @@ extern "C" int orlhf_compute_reward(const float* r, float kl_coef, const float* 
   const Rows rows{n_rows, n_cols, cu_seqlens};
   const float neg_coef = -(kl_coef > 0.0f ? kl_coef : 0.0f);
   const dim3 grid((unsigned)(n_rows < 65536 ? n_rows : 65536)), block(kBlock);
-  switch (mask_dtype) {
-    case ORLHF_MASK_NONE: hipLaunchKernelGGL(compute_reward_kernel<ORLHF_MASK_NONE>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, clip_high, reward, eos_index); break;
-    case ORLHF_MASK_U8: hipLaunchKernelGGL(compute_reward_kernel<ORLHF_MASK_U8>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, clip_high, reward, eos_index); break;
-    case ORLHF_MASK_F32: hipLaunchKernelGGL(compute_reward_kernel<ORLHF_MASK_F32>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, clip_high, reward, eos_index); break;
-    default: hipLaunchKernelGGL(compute_reward_kernel<ORLHF_MASK_I64>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, clip_high, reward, eos_index); break;
-  }
+#define ORLHF_LAUNCH(M)                                                                                         \
+  hipLaunchKernelGGL(compute_reward_kernel<M>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, \
+                     clip_high, reward, eos_index)
+  ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
+#undef ORLHF_LAUNCH
   ORLHF_CHECK_LAUNCH("orlhf_compute_reward");
   return ORLHF_OK;
 }
@@ -427,12 +425,9 @@ extern "C" int orlhf_masked_whiten(const float* x, const void* mask, int mask_dt
   float* mean_rstd = (float*)(partial + (int64_t)kWhitenBlocks * 3);
   const int nb = flat_grid(n, kWhitenBlocks);
   const dim3 grid(nb), block(kBlock);
-  switch (mask_dtype) {
-    case ORLHF_MASK_NONE: hipLaunchKernelGGL(whiten_partial_kernel<ORLHF_MASK_NONE>, grid, block, 0, s, x, mask, n, partial); break;
-    case ORLHF_MASK_U8: hipLaunchKernelGGL(whiten_partial_kernel<ORLHF_MASK_U8>, grid, block, 0, s, x, mask, n, partial); break;
-    case ORLHF_MASK_F32: hipLaunchKernelGGL(whiten_partial_kernel<ORLHF_MASK_F32>, grid, block, 0, s, x, mask, n, partial); break;
-    default: hipLaunchKernelGGL(whiten_partial_kernel<ORLHF_MASK_I64>, grid, block, 0, s, x, mask, n, partial); break;
-  }
+#define ORLHF_LAUNCH(M) hipLaunchKernelGGL(whiten_partial_kernel<M>, grid, block, 0, s, x, mask, n, partial)
+  ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
+#undef ORLHF_LAUNCH
   ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(partial)");
   hipLaunchKernelGGL(whiten_final_kernel, dim3(1), block, 0, s, partial, nb, std_norm, mean_rstd, stats);
   ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(final)");

@@ -102,6 +102,16 @@ __device__ __forceinline__ float load_mask(const void* mask, int64_t i) {
 
 inline bool valid_mask_dtype(int m) { return m >= ORLHF_MASK_NONE && m <= ORLHF_MASK_I64; }
 
+// Expands LAUNCH(M) with M = the compile-time mask dtype matching `mask_dt` (validated before by
+// check_rows); LAUNCH is a function-like macro the caller defines around its kernel launch.
+#define ORLHF_FOR_MASK_DTYPE(mask_dt, LAUNCH)              \
+  switch (mask_dt) {                                       \
+    case ORLHF_MASK_NONE: LAUNCH(ORLHF_MASK_NONE); break;  \
+    case ORLHF_MASK_U8: LAUNCH(ORLHF_MASK_U8); break;      \
+    case ORLHF_MASK_F32: LAUNCH(ORLHF_MASK_F32); break;    \
+    default: LAUNCH(ORLHF_MASK_I64); break;                \
+  }
+
 // ---------------------------------------------------------------- per-token row layouts
 // padded: contiguous [n_rows, n_cols]; packed: row b = tokens cu[b] .. cu[b+1]-1 of a flat array.
 struct Rows {

@@ -103,14 +103,6 @@ __global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const flo
 
 using namespace orlhf;
 
-#define ORLHF_MASK_SWITCH(LAUNCH)                      \
-  switch (mask_dtype) {                                \
-    case ORLHF_MASK_NONE: LAUNCH(ORLHF_MASK_NONE); break; \
-    case ORLHF_MASK_U8: LAUNCH(ORLHF_MASK_U8); break;     \
-    case ORLHF_MASK_F32: LAUNCH(ORLHF_MASK_F32); break;   \
-    default: LAUNCH(ORLHF_MASK_I64); break;               \
-  }
-
 extern "C" int orlhf_kl_rows(const void* log_probs, const void* log_probs_base, int dtype, const void* mask,
                              int mask_dtype, int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
                              int estimator, int enabled, float* kl, float* kl_mean, float* diff_mean,
@@ -136,7 +128,7 @@ extern "C" int orlhf_kl_rows(const void* log_probs, const void* log_probs_base, 
       hipLaunchKernelGGL((kl_rows_kernel<ORLHF_F16, M>), grid, block, 0, s, log_probs, log_probs_base, mask, rows,   \
                          estimator, enabled, kl, kl_mean, diff_mean);                                                \
   } while (0)
-  ORLHF_MASK_SWITCH(ORLHF_KL)
+  ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_KL)
 #undef ORLHF_KL
   ORLHF_CHECK_LAUNCH("orlhf_kl_rows");
   return ORLHF_OK;
@@ -153,7 +145,7 @@ extern "C" int orlhf_masked_normalize_rows(const float* x, const void* mask, int
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_NORM(M) \
   hipLaunchKernelGGL(masked_normalize_rows_kernel<M>, grid, block, 0, s, x, mask, rows, eps, out)
-  ORLHF_MASK_SWITCH(ORLHF_NORM)
+  ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_NORM)
 #undef ORLHF_NORM
   ORLHF_CHECK_LAUNCH("orlhf_masked_normalize_rows");
   return ORLHF_OK;

@@ -178,12 +178,7 @@ extern "C" int orlhf_sequence_logps_fwd(const float* per_token_logps, const void
 #define ORLHF_LAUNCH(M)                                                                                        \
   hipLaunchKernelGGL(sequence_logps_fwd_kernel<M>, grid, block, 0, s, per_token_logps, attention_mask, prompt_id_lens, \
                      n_rows, n_cols, sums, means, counts)
-  switch (mask_dtype) {
-    case ORLHF_MASK_NONE: ORLHF_LAUNCH(ORLHF_MASK_NONE); break;
-    case ORLHF_MASK_U8: ORLHF_LAUNCH(ORLHF_MASK_U8); break;
-    case ORLHF_MASK_F32: ORLHF_LAUNCH(ORLHF_MASK_F32); break;
-    default: ORLHF_LAUNCH(ORLHF_MASK_I64); break;
-  }
+  ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
 #undef ORLHF_LAUNCH
   ORLHF_CHECK_LAUNCH("orlhf_sequence_logps_fwd");
   return ORLHF_OK;
@@ -202,12 +197,7 @@ extern "C" int orlhf_sequence_logps_bwd(const float* g_sums, const float* g_mean
 #define ORLHF_LAUNCH(M)                                                                                      \
   hipLaunchKernelGGL(sequence_logps_bwd_kernel<M>, grid, block, 0, s, g_sums, g_means, attention_mask, prompt_id_lens, \
                      counts, n_rows, n_cols, g_per_token)
-  switch (mask_dtype) {
-    case ORLHF_MASK_NONE: ORLHF_LAUNCH(ORLHF_MASK_NONE); break;
-    case ORLHF_MASK_U8: ORLHF_LAUNCH(ORLHF_MASK_U8); break;
-    case ORLHF_MASK_F32: ORLHF_LAUNCH(ORLHF_MASK_F32); break;
-    default: ORLHF_LAUNCH(ORLHF_MASK_I64); break;
-  }
+  ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
 #undef ORLHF_LAUNCH
   ORLHF_CHECK_LAUNCH("orlhf_sequence_logps_bwd");
   return ORLHF_OK;

@@ -454,40 +454,21 @@ template <typename Tok>
 static void launch_partial(int mask_dt, Rows rows, const void* mask, const Tok& tok, double* partial,
                            int n_chunks, hipStream_t s) {
   const dim3 grid = row_grid(rows.n_rows, rows.n_cols), block(kBlock);
-  switch (mask_dt) {
-    case ORLHF_MASK_NONE:
-      hipLaunchKernelGGL((rows_partial_kernel<ORLHF_MASK_NONE, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks);
-      break;
-    case ORLHF_MASK_U8:
-      hipLaunchKernelGGL((rows_partial_kernel<ORLHF_MASK_U8, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks);
-      break;
-    case ORLHF_MASK_F32:
-      hipLaunchKernelGGL((rows_partial_kernel<ORLHF_MASK_F32, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks);
-      break;
-    default:
-      hipLaunchKernelGGL((rows_partial_kernel<ORLHF_MASK_I64, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks);
-      break;
-  }
+#define ORLHF_LAUNCH(M) \
+  hipLaunchKernelGGL((rows_partial_kernel<M, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks)
+  ORLHF_FOR_MASK_DTYPE(mask_dt, ORLHF_LAUNCH)
+#undef ORLHF_LAUNCH
 }
 
 template <typename Tok>
 static void launch_grad(int mask_dt, Rows rows, const void* mask, const Tok& tok, const float* g_out,
                         int g_per_row, const float* row_coef, float* g, hipStream_t s) {
   const dim3 grid = row_grid(rows.n_rows, rows.n_cols), block(kBlock);
-  switch (mask_dt) {
-    case ORLHF_MASK_NONE:
-      hipLaunchKernelGGL((rows_grad_kernel<ORLHF_MASK_NONE, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g, (int)chunks_of(rows.n_cols));
-      break;
-    case ORLHF_MASK_U8:
-      hipLaunchKernelGGL((rows_grad_kernel<ORLHF_MASK_U8, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g, (int)chunks_of(rows.n_cols));
-      break;
-    case ORLHF_MASK_F32:
-      hipLaunchKernelGGL((rows_grad_kernel<ORLHF_MASK_F32, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g, (int)chunks_of(rows.n_cols));
-      break;
-    default:
-      hipLaunchKernelGGL((rows_grad_kernel<ORLHF_MASK_I64, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g, (int)chunks_of(rows.n_cols));
-      break;
-  }
+#define ORLHF_LAUNCH(M)                                                                                    \
+  hipLaunchKernelGGL((rows_grad_kernel<M, Tok>), grid, block, 0, s, rows, mask, tok, g_out, g_per_row, row_coef, g, \
+                     (int)chunks_of(rows.n_cols))
+  ORLHF_FOR_MASK_DTYPE(mask_dt, ORLHF_LAUNCH)
+#undef ORLHF_LAUNCH
 }
 
 
@@ -707,12 +688,11 @@ extern "C" int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs,
   launch_partial(mask_dtype, rows, mask, gt, partial, n_chunks, s);
   ORLHF_CHECK_LAUNCH("orlhf_policy_loss_bwd(gspo partial)");
   const dim3 grid = row_grid(n_rows, n_cols), block(kBlock);
-  switch (mask_dtype) {
-    case ORLHF_MASK_NONE: hipLaunchKernelGGL(gspo_grad_kernel<ORLHF_MASK_NONE>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, g_log_probs); break;
-    case ORLHF_MASK_U8: hipLaunchKernelGGL(gspo_grad_kernel<ORLHF_MASK_U8>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, g_log_probs); break;
-    case ORLHF_MASK_F32: hipLaunchKernelGGL(gspo_grad_kernel<ORLHF_MASK_F32>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, g_log_probs); break;
-    default: hipLaunchKernelGGL(gspo_grad_kernel<ORLHF_MASK_I64>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, g_log_probs); break;
-  }
+#define ORLHF_LAUNCH(M)                                                                                       \
+  hipLaunchKernelGGL(gspo_grad_kernel<M>, grid, block, 0, s, rows, mask, partial, n_chunks, g_out, row_coef, row_aux, \
+                     g_log_probs)
+  ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
+#undef ORLHF_LAUNCH
   ORLHF_CHECK_LAUNCH("orlhf_policy_loss_bwd(gspo grad)");
   return ORLHF_OK;
 }
