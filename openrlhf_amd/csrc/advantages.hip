@@ -31,7 +31,10 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
                                                                 int64_t* __restrict__ eos_index) {
   __shared__ int64_t lds_val[kWavesPerBlock];
   __shared__ int64_t lds_idx[kWavesPerBlock];
-  for (int64_t b = blockIdx.x; b < rows.n_rows; b += gridDim.x) {
+  const int slot_b = slot_bits(rows.n_rows);
+  for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
+    const int64_t b = row_of_slot(slot, slot, slot_b);
+    if (b >= rows.n_rows) continue;
     int64_t start, len;
     row_span(rows, b, start, len);
     if (len <= 0) {
@@ -119,7 +122,10 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
 #pragma unroll
   for (int k = 1; k <= kScanItems; ++k) pw[k] = pw[k - 1] * coef;
 
-  for (int64_t b = blockIdx.x; b < rows.n_rows; b += gridDim.x) {
+  const int slot_b = slot_bits(rows.n_rows);
+  for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
+    const int64_t b = row_of_slot(slot, slot, slot_b);
+    if (b >= rows.n_rows) continue;
     int64_t start, len;
     row_span(rows, b, start, len);
     if (len <= 0) continue;
@@ -331,7 +337,7 @@ __global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* __res
 template <bool GAE>
 static void launch_scan(int mask_dtype, Rows rows, const float* values, const float* rewards, const void* mask,
                         double gamma, double coef, float* adv, float* ret, hipStream_t s) {
-  const dim3 grid((unsigned)(rows.n_rows < 65536 ? rows.n_rows : 65536)), block(kBlock);
+  const dim3 grid(slot_grid(row_slots(rows.n_rows), 65536)), block(kBlock);
 #define ORLHF_LAUNCH(M)                                                                                          \
   hipLaunchKernelGGL((reverse_scan_kernel<M, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, \
                      ret)
@@ -353,7 +359,7 @@ extern "C" int orlhf_compute_reward(const float* r, float kl_coef, const float* 
   hipStream_t s = (hipStream_t)stream;
   const Rows rows{n_rows, n_cols, cu_seqlens};
   const float neg_coef = -(kl_coef > 0.0f ? kl_coef : 0.0f);
-  const dim3 grid((unsigned)(n_rows < 65536 ? n_rows : 65536)), block(kBlock);
+  const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
 #define ORLHF_LAUNCH(M)                                                                                         \
   hipLaunchKernelGGL(compute_reward_kernel<M>, grid, block, 0, s, rows, r, neg_coef, kl, mask, has_clip, clip_low, \
                      clip_high, reward, eos_index)

@@ -129,6 +129,44 @@ __device__ __forceinline__ void row_span(const Rows& r, int64_t b, int64_t& star
   }
 }
 
+// ---------------------------------------------------------------- rows -> workgroups
+// Workgroups are handed out in index order and, as measured, statically: round-robin over the
+// eight XCDs and again over the shader engines inside one. With row b on workgroup b, row lengths
+// that repeat with a short period (long and short rows interleaved by a length balancer, say) put
+// all long rows on a fraction of the chip: with a quarter of the rows long, the per-token loss
+// pass ran as slowly as if it had 2.9 times the tokens. Workgroup slot s therefore works on row
+// row_of_slot(s): rows are permuted inside aligned blocks of 2^bits rows by a small bijective
+// mix, XORed with a hash of the block's number so that no compute unit keeps meeting the same
+// residue. Slot counts are rounded up to whole blocks; slots past n_rows are skipped. Blocks are
+// 1/8 to 1/16 of the rows (8 to 256 rows), which bounds the skipped slots to about 12%.
+__host__ __device__ inline int slot_bits(int64_t n_rows) {
+  const int fl = n_rows > 0 ? 63 - __builtin_clzll((unsigned long long)n_rows) : 0;
+  const int bits = fl - 3;
+  return bits < 3 ? 3 : (bits > 8 ? 8 : bits);
+}
+__host__ __device__ inline int64_t row_slots(int64_t n_rows) {
+  const int64_t blk = (int64_t)1 << slot_bits(n_rows);
+  return (n_rows + blk - 1) & ~(blk - 1);
+}
+// `slot` counts inside one pass over the rows; `item` is the workgroup's global work index (equal
+// to `slot` when a kernel makes a single pass) and only salts the hash.
+__host__ __device__ __forceinline__ int64_t row_of_slot(int64_t slot, int64_t item, int bits) {
+  const uint32_t mask = (1u << bits) - 1u;
+  uint32_t x = (uint32_t)slot & mask;
+  x = (x * 0x9Du) & mask;
+  x ^= x >> ((bits + 1) >> 1);
+  x = (x * 0x35u) & mask;
+  uint32_t h = (uint32_t)(item >> bits) * 0x9E3779B1u;
+  h ^= h >> 15;
+  x ^= (h >> 7) & mask;
+  return (slot & ~(int64_t)mask) | (int64_t)x;
+}
+
+// Grid for a kernel that walks `slots` work items with a grid-size stride.
+inline unsigned slot_grid(int64_t slots, int64_t cap) {
+  return (unsigned)(slots < cap ? (slots > 0 ? slots : 1) : cap);
+}
+
 inline int check_rows(const char* what, int64_t n_rows, int64_t n_cols, const void* mask, int mask_dtype) {
   if (n_rows < 0 || n_cols < 0)
     return fail(ORLHF_ERR_INVALID_ARG, "%s: n_rows=%lld n_cols=%lld", what, (long long)n_rows, (long long)n_cols);

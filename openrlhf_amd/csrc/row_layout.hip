@@ -16,7 +16,10 @@ __global__ __launch_bounds__(kBlock) void row_extents_kernel(const void* __restr
                                                              int64_t* __restrict__ end,
                                                              int64_t* __restrict__ length) {
   __shared__ long long lds_lo[kWavesPerBlock], lds_hi[kWavesPerBlock];
-  for (int64_t b = blockIdx.x; b < n_rows; b += gridDim.x) {
+  const int slot_b = slot_bits(n_rows);
+  for (int64_t slot = blockIdx.x; slot < row_slots(n_rows); slot += gridDim.x) {
+    const int64_t b = row_of_slot(slot, slot, slot_b);
+    if (b >= n_rows) continue;
     long long lo = n_cols, hi = 0;  // no non-zero column: first = n_cols, end = 0
 #pragma unroll 8
     for (int64_t t = threadIdx.x; t < n_cols; t += kBlock) {
@@ -88,8 +91,11 @@ __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__
                                                            const int64_t* __restrict__ first,
                                                            const int64_t* __restrict__ cu, E* __restrict__ dst) {
   const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
-  for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
-    const int64_t chunk = w / n_rows, b = w - chunk * n_rows, j0 = chunk * kCopyChunk;  // rows vary fastest
+  const int64_t slots = row_slots(n_rows);
+  const int slot_b = slot_bits(n_rows);
+  for (int64_t w = blockIdx.x; w < slots * chunks; w += gridDim.x) {
+    const int64_t chunk = w / slots, b = row_of_slot(w - chunk * slots, w, slot_b), j0 = chunk * kCopyChunk;
+    if (b >= n_rows) continue;
     const int64_t start = cu[b], len = cu[b + 1] - start;
     if (j0 >= len) continue;
     const int64_t f = first != nullptr ? first[b] : 0;
@@ -123,8 +129,7 @@ __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ 
 
 static inline unsigned copy_grid(int64_t n_rows, int64_t n_cols) {
   const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
-  const int64_t g = n_rows * chunks;
-  return (unsigned)(g < 262144 ? (g > 0 ? g : 1) : 262144);
+  return slot_grid(row_slots(n_rows) * chunks, 262144);
 }
 
 }  // namespace orlhf
@@ -136,7 +141,7 @@ extern "C" int orlhf_row_extents(const void* mask, int mask_dtype, int64_t n_row
   if (int rc = check_rows("row_extents", n_rows, n_cols, mask, mask_dtype)) return rc;
   ORLHF_CHECK_ARG(mask_dtype != ORLHF_MASK_NONE, "row_extents: needs a mask");
   if (n_rows == 0) return ORLHF_OK;
-  const dim3 grid((unsigned)(n_rows < 65536 ? n_rows : 65536)), block(kBlock);
+  const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
   switch (mask_dtype) {
     case ORLHF_MASK_U8:

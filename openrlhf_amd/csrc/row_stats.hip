@@ -38,7 +38,10 @@ __global__ __launch_bounds__(kBlock) void kl_rows_kernel(const void* __restrict_
                                                          float* __restrict__ kl_mean,
                                                          float* __restrict__ diff_mean) {
   __shared__ double lds[3][kWavesPerBlock];
-  for (int64_t b = blockIdx.x; b < rows.n_rows; b += gridDim.x) {
+  const int slot_b = slot_bits(rows.n_rows);
+  for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
+    const int64_t b = row_of_slot(slot, slot, slot_b);
+    if (b >= rows.n_rows) continue;
     int64_t start, len;
     row_span(rows, b, start, len);
     double sk = 0.0, sd = 0.0, sm = 0.0;
@@ -71,7 +74,10 @@ __global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const flo
                                                                        const void* __restrict__ mask, Rows rows,
                                                                        float eps, float* __restrict__ out) {
   __shared__ double lds[3][kWavesPerBlock];
-  for (int64_t b = blockIdx.x; b < rows.n_rows; b += gridDim.x) {
+  const int slot_b = slot_bits(rows.n_rows);
+  for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
+    const int64_t b = row_of_slot(slot, slot, slot_b);
+    if (b >= rows.n_rows) continue;
     int64_t start, len;
     row_span(rows, b, start, len);
     double s = 0.0, c = 0.0, z = 0.0;
@@ -114,7 +120,7 @@ extern "C" int orlhf_kl_rows(const void* log_probs, const void* log_probs_base, 
   ORLHF_CHECK_ARG(!enabled || n_cols == 0 || (log_probs != nullptr && log_probs_base != nullptr),
                   "kl_rows: log_probs / log_probs_base is NULL");
   const Rows rows{n_rows, n_cols, cu_seqlens};
-  const dim3 grid((unsigned)(n_rows < 65536 ? n_rows : 65536)), block(kBlock);
+  const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_KL(M)                                                                                                  \
   do {                                                                                                               \
@@ -141,7 +147,7 @@ extern "C" int orlhf_masked_normalize_rows(const float* x, const void* mask, int
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(x != nullptr && out != nullptr, "masked_normalize_rows: NULL argument");
   const Rows rows{n_rows, n_cols, cu_seqlens};
-  const dim3 grid((unsigned)(n_rows < 65536 ? n_rows : 65536)), block(kBlock);
+  const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_NORM(M) \
   hipLaunchKernelGGL(masked_normalize_rows_kernel<M>, grid, block, 0, s, x, mask, rows, eps, out)

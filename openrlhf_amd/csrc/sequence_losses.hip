@@ -25,7 +25,10 @@ __global__ __launch_bounds__(kBlock) void sequence_logps_fwd_kernel(const float*
                                                                     float* __restrict__ means,
                                                                     float* __restrict__ counts) {
   __shared__ double lds[kWavesPerBlock];
-  for (int64_t b = blockIdx.x; b < n_rows; b += gridDim.x) {
+  const int slot_b = slot_bits(n_rows);
+  for (int64_t slot = blockIdx.x; slot < row_slots(n_rows); slot += gridDim.x) {
+    const int64_t b = row_of_slot(slot, slot, slot_b);
+    if (b >= n_rows) continue;
     double s = 0.0, c = 0.0;
 #pragma unroll 8
     for (int64_t t = threadIdx.x; t < n_cols; t += kBlock) {
@@ -173,7 +176,7 @@ extern "C" int orlhf_sequence_logps_fwd(const float* per_token_logps, const void
   if (int rc = check_rows("sequence_logps_fwd", n_rows, n_cols, attention_mask, mask_dtype)) return rc;
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(per_token_logps != nullptr || n_cols == 0, "sequence_logps_fwd: per_token_logps is NULL");
-  const dim3 grid((unsigned)(n_rows < 65536 ? n_rows : 65536)), block(kBlock);
+  const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_LAUNCH(M)                                                                                        \
   hipLaunchKernelGGL(sequence_logps_fwd_kernel<M>, grid, block, 0, s, per_token_logps, attention_mask, prompt_id_lens, \

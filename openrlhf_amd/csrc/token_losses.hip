@@ -21,7 +21,8 @@ constexpr int kMaxQ = 6;                      // quantities reduced per token
 // Work items are (row, chunk) pairs numbered with the ROW varying fastest. Workgroups go to the
 // eight XCDs round-robin by their index: numbered chunk-fastest, the chunks that hold tokens in a
 // batch of short packed rows (chunk 0 and 1 of every row, say) would all land on the same two or
-// four XCDs and the rest of the chip would only see the empty tail chunks.
+// four XCDs and the rest of the chip would only see the empty tail chunks. Within a chunk index
+// the rows go through row_of_slot(), so that row lengths with a short period spread as well.
 constexpr int64_t kMaxItemsGrid = 1 << 22;
 
 
@@ -126,9 +127,11 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
                                                               int n_chunks) {
   constexpr int NQ = Tok::kQ;
   __shared__ double lds[NQ][kWavesPerBlock];
-  const int64_t items = rows.n_rows * n_chunks;
+  const int64_t slots = row_slots(rows.n_rows), items = slots * n_chunks;
+  const int slot_b = slot_bits(rows.n_rows);
   for (int64_t item = blockIdx.x; item < items; item += gridDim.x) {
-    const int64_t chunk = item / rows.n_rows, b = item - chunk * rows.n_rows;  // rows vary fastest
+    const int64_t chunk = item / slots, b = row_of_slot(item - chunk * slots, item, slot_b);  // rows vary fastest
+    if (b >= rows.n_rows) continue;
     int64_t start, len;
     row_span(rows, b, start, len);
     const int64_t c0 = chunk * kChunk;
@@ -350,9 +353,11 @@ __global__ __launch_bounds__(kBlock) void rows_grad_kernel(Rows rows, const void
                                                            const float* __restrict__ g_out, int g_per_row,
                                                            const float* __restrict__ row_coef,
                                                            float* __restrict__ g, int n_chunks) {
-  const int64_t items = rows.n_rows * n_chunks;
+  const int64_t slots = row_slots(rows.n_rows), items = slots * n_chunks;
+  const int slot_b = slot_bits(rows.n_rows);
   for (int64_t item = blockIdx.x; item < items; item += gridDim.x) {
-    const int64_t chunk = item / rows.n_rows, b = item - chunk * rows.n_rows;
+    const int64_t chunk = item / slots, b = row_of_slot(item - chunk * slots, item, slot_b);  // rows vary fastest
+    if (b >= rows.n_rows) continue;
     int64_t start, len;
     row_span(rows, b, start, len);
     const int64_t c0 = chunk * kChunk;
@@ -396,9 +401,11 @@ __global__ __launch_bounds__(kBlock) void gspo_grad_kernel(Rows rows, const void
                                                            const float* __restrict__ row_coef,
                                                            const float* __restrict__ row_aux,
                                                            float* __restrict__ g) {
-  const int64_t items = rows.n_rows * n_chunks;
+  const int64_t slots = row_slots(rows.n_rows), items = slots * n_chunks;
+  const int slot_b = slot_bits(rows.n_rows);
   for (int64_t item = blockIdx.x; item < items; item += gridDim.x) {
-    const int64_t chunk = item / rows.n_rows, b = item - chunk * rows.n_rows;
+    const int64_t chunk = item / slots, b = row_of_slot(item - chunk * slots, item, slot_b);  // rows vary fastest
+    if (b >= rows.n_rows) continue;
     int64_t start, len;
     row_span(rows, b, start, len);
     const int64_t c0 = chunk * kChunk;
@@ -446,8 +453,7 @@ __global__ __launch_bounds__(kBlock) void approx_kl_bwd_kernel(const void* __res
 
 // ---------------------------------------------------------------- host helpers
 static inline dim3 row_grid(int64_t n_rows, int64_t n_cols) {
-  const int64_t items = n_rows * chunks_of(n_cols);
-  return dim3((unsigned)(items < kMaxItemsGrid ? (items > 0 ? items : 1) : kMaxItemsGrid));
+  return dim3(slot_grid(row_slots(n_rows) * chunks_of(n_cols), kMaxItemsGrid));
 }
 
 template <typename Tok>
