@@ -40,9 +40,19 @@ struct PolicyTok {
     clipped = s2 < s1 ? 1.0f : 0.0f;
   }
 
-  __device__ __forceinline__ float is_weight(int64_t b, int64_t i) const {
+  // Inputs of one token, in the order the kernels hand them to eval() / grad(); a null pointer
+  // marks an input this configuration does not read.
+  static constexpr int kIn = 4;
+  __device__ __forceinline__ const float* in(int j) const {
+    if (j == 0) return lp;
+    if (j == 1) return old;
+    if (j == 2) return adv;
+    return (is_mode != ORLHF_IS_NONE && !gspo) ? rollout : nullptr;
+  }
+
+  __device__ __forceinline__ float is_weight(int64_t b, float old_v, float roll_v) const {
     if (is_mode == ORLHF_IS_NONE || gspo) return 1.0f;
-    const float w = expf(old[i] - rollout[i]);
+    const float w = expf(old_v - roll_v);
     if (is_mode == ORLHF_IS_TIS) return fminf(fmaxf(w, is_lo), is_hi);
     if (is_mode == ORLHF_IS_ICEPOP) return (w >= is_lo && w <= is_hi) ? w : 0.0f;
     return row_aux[b * 2] * w;  // seq-mask-tis: row keep flag times the unclamped token weight
@@ -55,8 +65,9 @@ struct PolicyTok {
     dr = (raw >= -20.0f && raw <= 20.0f) ? ratio : 0.0f;
   }
 
-  __device__ __forceinline__ void eval(int64_t b, int64_t i, float m, float* q) const {
-    const float raw = lp[i] - old[i];
+  // v = {lp, old, adv, rollout} of the token
+  __device__ __forceinline__ void eval(int64_t b, const float* v, float m, float* q) const {
+    const float raw = v[0] - v[1];
     float ratio, dr;
     if (gspo) {
       ratio = row_aux[b * 2] * m;
@@ -64,13 +75,13 @@ struct PolicyTok {
       ppo_ratio(raw, ratio, dr);
     }
     float loss, dratio, clipped;
-    surrogate(ratio, adv[i], loss, dratio, clipped);
-    loss *= is_weight(b, i);
+    surrogate(ratio, v[2], loss, dratio, clipped);
+    loss *= is_weight(b, v[1], v[3]);
     q[0] = loss * m;
     q[1] = m;
     q[2] = clipped * m;
     q[3] = -raw * m;
-    q[4] = (is_mode != ORLHF_IS_NONE && !gspo) ? (rollout[i] - old[i]) * m : 0.0f;
+    q[4] = (is_mode != ORLHF_IS_NONE && !gspo) ? (v[3] - v[1]) * m : 0.0f;
   }
 
   // d(token loss)/d(lp) of a PPO token from its scalars (no memory access): used where the
@@ -89,9 +100,9 @@ struct PolicyTok {
     return (w >= is_lo && w <= is_hi) ? w : 0.0f;  // ICEPOP
   }
 
-  // PPO: d(token loss)/d(lp[i]).  GSPO: d(token loss)/d(ratio) * m (summed per row by the caller).
-  __device__ __forceinline__ float grad(int64_t b, int64_t i, float m) const {
-    const float raw = lp[i] - old[i];
+  // PPO: d(token loss)/d(lp).  GSPO: d(token loss)/d(ratio) * m (summed per row by the caller).
+  __device__ __forceinline__ float grad(int64_t b, const float* v, float m) const {
+    const float raw = v[0] - v[1];
     float ratio, dr;
     if (gspo) {
       ratio = row_aux[b * 2] * m;
@@ -100,8 +111,8 @@ struct PolicyTok {
       ppo_ratio(raw, ratio, dr);
     }
     float loss, dratio, clipped;
-    surrogate(ratio, adv[i], loss, dratio, clipped);
-    return is_weight(b, i) * dratio * dr;
+    surrogate(ratio, v[2], loss, dratio, clipped);
+    return is_weight(b, v[1], v[3]) * dratio * dr;
   }
 };
 

@@ -87,3 +87,52 @@ def test_logits_in_other_forms(cuda):
     xt = x.view(-1, v).t().contiguous().t()
     assert not xt.is_contiguous()
     assert torch.equal(log_probs_from_logits(xt, labels.view(-1), 0.8), lp.view(-1))
+
+
+def _at_offset(t, off):
+    """The same values in storage that starts `off` elements past an allocation boundary."""
+    buf = torch.empty(t.numel() + off, dtype=t.dtype, device=t.device)
+    view = buf[off:off + t.numel()].view(t.shape)
+    view.copy_(t)
+    return view
+
+
+@pytest.mark.parametrize("off", [1, 2, 3])
+def test_per_token_arrays_off_the_16_byte_boundary(cuda, off):
+    """Arrays on 16-byte boundaries take four-token vector loads, others the element-wise walk:
+    same losses and gradients (the sums differ in their order only)."""
+    from openrlhf_amd.models.loss import PolicyLoss, ValueLoss, aggregate_loss
+    from openrlhf_amd.trainer.ppo_utils.experience import PackedSteps
+
+    g = torch.Generator().manual_seed(20 + off)
+    b, a = 6, 5003
+    lp = (-torch.rand(b, a, generator=g) * 2).to(cuda)
+    old = lp + (torch.randn(b, a, generator=g) * 0.1).to(cuda)
+    adv = torch.randn(b, a, generator=g).to(cuda)
+    lens = torch.tensor([5003, 4097, 1023, 1, 2050, 3333])
+    mask = (torch.arange(a)[None, :] < lens[:, None]).to(cuda)
+    pol, val = PolicyLoss(0.2, 0.28, dual_clip=3.0), ValueLoss(0.2)
+
+    def run(lp_, old_, adv_, mask_, **kw):
+        x = lp_.detach().requires_grad_()
+        loss = pol(x, old_, adv_, action_mask=mask_, **kw)
+        v = val(x, old_, adv_, action_mask=mask_, **kw)
+        agg = aggregate_loss(x * adv_, mask_, **{k: w for k, w in kw.items()})
+        (loss[0] + v + agg).backward()
+        return torch.stack([loss[0], loss[1], loss[2], v, agg]).detach(), x.grad
+
+    for m in (mask, mask.float(), mask.long()):
+        ref, gref = run(lp, old, adv, m)
+        out, gout = run(_at_offset(lp, off), _at_offset(old, off), _at_offset(adv, off), _at_offset(m, off))
+        assert torch.allclose(out, ref, rtol=1e-6, atol=1e-7)
+        assert torch.allclose(gout, gref, rtol=1e-5, atol=1e-9)
+    # packed rows: starts fall on every residue; shifting the storage shifts them all
+    ps = PackedSteps.from_padded(dict(lp=lp, old=old, adv=adv, mask=mask), mask)
+    kw = dict(cu_seqlens=ps.cu_seqlens, max_seqlen=a)
+    ref, gref = run(lp, old, adv, mask)
+    for o in (0, off):
+        out, gout = run(_at_offset(ps["lp"], o), _at_offset(ps["old"], o), _at_offset(ps["adv"], o),
+                        _at_offset(ps["mask"], o), **kw)
+        assert torch.allclose(out, ref, rtol=1e-6, atol=1e-7)
+        packed_ref = PackedSteps.from_padded(dict(g=gref), mask)["g"]
+        assert torch.allclose(gout, packed_ref, rtol=1e-5, atol=1e-9)
