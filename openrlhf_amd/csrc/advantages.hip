@@ -99,21 +99,68 @@ __device__ __forceinline__ Affine compose(const Affine& outer, const Affine& inn
   return r;
 }
 
-// LDS staging index: one pad word per 32 keeps the lanes' strided accesses (each lane reads its
-// kScanItems consecutive tokens) off each other's banks.
-__device__ __forceinline__ int scan_slot(int p) { return p + (p >> 5); }
-constexpr int kScanLds = kScanTile + kScanTile / 32 + 2;
+// One tile of a row in registers: this lane's kScanItems consecutive tokens, masked, plus the
+// value that follows them (the next lane's first; the next tile's first for the last lane).
+struct ScanTile {
+  float r[kScanItems];
+  float v[kScanItems + 1];
+};
 
+// `whole`: the tile lies inside the row and every array allows 16-byte loads. Must be called by
+// all lanes of the workgroup (it exchanges the following value across lanes).
+template <int MASK_DT, bool GAE>
+__device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t tile0, bool whole,
+                                                   const float* __restrict__ values,
+                                                   const float* __restrict__ rewards,
+                                                   const void* __restrict__ mask) {
+  static_assert(kScanItems == 4, "a lane's tokens are one 16-byte load");
+  ScanTile t;
+  const int64_t p0 = tile0 + (int64_t)threadIdx.x * kScanItems;
+  if (whole) {
+    float m[kScanItems];
+    load_mask4<MASK_DT>(mask, rw.base + p0, m);
+    const f32x4 r4 = *(const f32x4*)(rewards + rw.base + p0);
+    f32x4 v4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (GAE) v4 = *(const f32x4*)(values + rw.base + p0);
+#pragma unroll
+    for (int j = 0; j < kScanItems; ++j) {
+      t.r[j] = m[j] * r4[j];
+      t.v[j] = m[j] * v4[j];
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < kScanItems; ++j) {
+      const int64_t p = p0 + j;
+      t.r[j] = 0.0f;
+      t.v[j] = 0.0f;
+      if (p >= rw.lead && p < rw.len) {
+        const float m = load_mask<MASK_DT>(mask, rw.base + p);
+        t.r[j] = m * rewards[rw.base + p];
+        if (GAE) t.v[j] = m * values[rw.base + p];
+      }
+    }
+  }
+  t.v[kScanItems] = 0.0f;
+  if (GAE) {
+    const float from_next_lane = __shfl_down(t.v[0], 1, kWave);
+    const int64_t p = p0 + kScanItems;  // first token of the next wave (or tile) for the last lane
+    float after = 0.0f;
+    if ((threadIdx.x & (kWave - 1)) == kWave - 1 && p < rw.len)
+      after = load_mask<MASK_DT>(mask, rw.base + p) * values[rw.base + p];
+    t.v[kScanItems] = (threadIdx.x & (kWave - 1)) == kWave - 1 ? after : from_next_lane;
+  }
+  return t;
+}
+
+// One workgroup per row, walking it backwards in tiles of kScanTile tokens; the tile before the
+// current one is loaded (straight into registers, no staging) while the current one is scanned.
 template <int MASK_DT, bool GAE>
 __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const float* __restrict__ values,
                                                               const float* __restrict__ rewards,
                                                               const void* __restrict__ mask, double gamma,
                                                               double coef, float* __restrict__ adv,
                                                               float* __restrict__ ret) {
-  __shared__ Affine lds_wave[kWavesPerBlock];
-  __shared__ double lds_carry;
-  __shared__ float lds_v[kScanLds];  // masked values in, returns out
-  __shared__ float lds_r[kScanLds];  // masked rewards in, advantages out
+  __shared__ Affine lds_wave[2][kWavesPerBlock];  // alternating: one barrier per tile is enough
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
 
@@ -123,51 +170,29 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
   for (int k = 1; k <= kScanItems; ++k) pw[k] = pw[k - 1] * coef;
 
   const int slot_b = slot_bits(rows.n_rows);
+  int buf = 0;
   for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
     const int64_t b = row_of_slot(slot, slot, slot_b);
     if (b >= rows.n_rows) continue;
-    int64_t start, len;
-    row_span(rows, b, start, len);
-    if (len <= 0) continue;
-    const int64_t n_tiles = (len + kScanTile - 1) / kScanTile;
+    const RowWalk rw = row_walk(rows, b);
+    if (rw.len <= 0) continue;
+    const int64_t n_tiles = (rw.len + kScanTile - 1) / kScanTile;
     double tile_carry = 0.0;  // A at the first token of the previous (later) tile
+    auto whole = [&](int64_t tile) {
+      return rows.vec && tile * kScanTile >= rw.lead && (tile + 1) * kScanTile <= rw.len;
+    };
+    ScanTile cur = load_scan_tile<MASK_DT, GAE>(rw, (n_tiles - 1) * kScanTile, whole(n_tiles - 1), values, rewards, mask);
     for (int64_t tile = n_tiles - 1; tile >= 0; --tile) {
       const int64_t tile0 = tile * kScanTile;
-      // ---- coalesced load of the tile (masked) into LDS; token tile0+kScanTile is the
-      //      "value after the tile" the last lane needs
-#pragma unroll
-      for (int k = 0; k < kScanItems; ++k) {
-        const int p = threadIdx.x + k * kBlock;
-        const int64_t t = tile0 + p;
-        float rv = 0.0f, vv = 0.0f;
-        if (t < len) {
-          const float m = load_mask<MASK_DT>(mask, start + t);
-          rv = m * rewards[start + t];
-          if (GAE) vv = m * values[start + t];
-        }
-        lds_r[scan_slot(p)] = rv;
-        if (GAE) lds_v[scan_slot(p)] = vv;
-      }
-      if (GAE && threadIdx.x == 0) {
-        const int64_t t = tile0 + kScanTile;
-        lds_v[scan_slot(kScanTile)] = t < len ? load_mask<MASK_DT>(mask, start + t) * values[start + t] : 0.0f;
-      }
-      __syncthreads();
-      // ---- this lane's kScanItems consecutive tokens
-      const int p0 = threadIdx.x * kScanItems;
-      float v[kScanItems + 1], rw[kScanItems];
-#pragma unroll
-      for (int j = 0; j < kScanItems; ++j) {
-        rw[j] = lds_r[scan_slot(p0 + j)];
-        v[j] = GAE ? lds_v[scan_slot(p0 + j)] : 0.0f;
-      }
-      v[kScanItems] = GAE ? lds_v[scan_slot(p0 + kScanItems)] : 0.0f;
+      ScanTile nxt = cur;
+      if (tile > 0) nxt = load_scan_tile<MASK_DT, GAE>(rw, tile0 - kScanTile, whole(tile - 1), values, rewards, mask);
       // in-lane recurrence with zero carry-in
       double local[kScanItems];
       double run = 0.0;
 #pragma unroll
       for (int j = kScanItems - 1; j >= 0; --j) {
-        const double delta = GAE ? ((double)rw[j] + gamma * (double)v[j + 1]) - (double)v[j] : (double)rw[j];
+        const double delta =
+            GAE ? ((double)cur.r[j] + gamma * (double)cur.v[j + 1]) - (double)cur.v[j] : (double)cur.r[j];
         run = delta + coef * run;
         local[j] = run;
       }
@@ -182,44 +207,53 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
         o.b = __shfl_down(f.b, d, kWave);
         if (lane + d < kWave) f = compose(f, o);
       }
-      if (lane == 0) lds_wave[wave] = f;
-      __syncthreads();  // also: every lane has read its inputs from LDS
-      // carry entering this wave = maps of the later waves applied to the tile carry
-      double wave_carry = tile_carry;
-      for (int w = kWavesPerBlock - 1; w > wave; --w) wave_carry = lds_wave[w].b + lds_wave[w].a * wave_carry;
+      if (lane == 0) lds_wave[buf][wave] = f;
+      __syncthreads();
+      // carry entering this wave = maps of the later waves applied to the tile carry; applying
+      // the earlier waves' maps as well gives A at the tile's first token, the next tile's carry
+      double wave_carry = tile_carry, c = tile_carry;
+#pragma unroll
+      for (int w = kWavesPerBlock - 1; w >= 0; --w) {
+        c = lds_wave[buf][w].b + lds_wave[buf][w].a * c;
+        if (w == wave + 1) wave_carry = c;
+      }
+      tile_carry = c;
+      buf ^= 1;
       // carry entering this lane = A at the first token of lane+1
-      Affine nxt;
-      nxt.a = __shfl_down(f.a, 1, kWave);
-      nxt.b = __shfl_down(f.b, 1, kWave);
-      const double carry = (lane == kWave - 1) ? wave_carry : nxt.b + nxt.a * wave_carry;
+      Affine after;
+      after.a = __shfl_down(f.a, 1, kWave);
+      after.b = __shfl_down(f.b, 1, kWave);
+      const double carry = (lane == kWave - 1) ? wave_carry : after.b + after.a * wave_carry;
+      const int64_t p0 = tile0 + (int64_t)threadIdx.x * kScanItems;
+      f32x4 out_a, out_r;
 #pragma unroll
       for (int j = 0; j < kScanItems; ++j) {
         const double a_t = local[j] + pw[kScanItems - j] * carry;
-        if (GAE) {
-          lds_r[scan_slot(p0 + j)] = (float)a_t;
-          lds_v[scan_slot(p0 + j)] = (float)(a_t + (double)v[j]);
-        } else {
-          lds_r[scan_slot(p0 + j)] = (float)a_t;
-        }
+        out_a[j] = (float)a_t;
+        out_r[j] = (float)(a_t + (double)cur.v[j]);
       }
-      if (threadIdx.x == 0) lds_carry = local[0] + pw[kScanItems] * carry;
-      __syncthreads();
-      tile_carry = lds_carry;
-      // ---- coalesced store of the tile
+      if (whole(tile)) {
+        if (GAE) {
+          *(f32x4*)(adv + rw.base + p0) = out_a;
+          *(f32x4*)(ret + rw.base + p0) = out_r;
+        } else {
+          *(f32x4*)(ret + rw.base + p0) = out_a;
+        }
+      } else {
 #pragma unroll
-      for (int k = 0; k < kScanItems; ++k) {
-        const int p = threadIdx.x + k * kBlock;
-        const int64_t t = tile0 + p;
-        if (t < len) {
-          if (GAE) {
-            adv[start + t] = lds_r[scan_slot(p)];
-            ret[start + t] = lds_v[scan_slot(p)];
-          } else {
-            ret[start + t] = lds_r[scan_slot(p)];
+        for (int j = 0; j < kScanItems; ++j) {
+          const int64_t p = p0 + j;
+          if (p >= rw.lead && p < rw.len) {
+            if (GAE) {
+              adv[rw.base + p] = out_a[j];
+              ret[rw.base + p] = out_r[j];
+            } else {
+              ret[rw.base + p] = out_a[j];
+            }
           }
         }
       }
-      __syncthreads();  // LDS is refilled by the next tile
+      cur = nxt;
     }
   }
 }
@@ -375,7 +409,8 @@ extern "C" int orlhf_gae_scan(const float* values, const float* rewards, const v
   if (int rc = check_rows("gae_scan", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(values && rewards && advantages && returns, "gae_scan: NULL pointer");
-  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const Rows rows{n_rows, n_cols, cu_seqlens,
+                  vector_loads_ok(mask, mask_dtype, {values, rewards, advantages, returns}) ? 1 : 0};
   launch_scan<true>(mask_dtype, rows, values, rewards, mask, (double)gamma, (double)gamma * (double)lambd,
                     advantages, returns, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_gae_scan");
@@ -388,7 +423,7 @@ extern "C" int orlhf_discounted_returns(const float* rewards, const void* mask, 
   if (int rc = check_rows("discounted_returns", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(rewards && returns, "discounted_returns: NULL pointer");
-  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {rewards, returns}) ? 1 : 0};
   launch_scan<false>(mask_dtype, rows, nullptr, rewards, mask, (double)gamma, (double)gamma, nullptr, returns,
                      (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_discounted_returns");

@@ -1,6 +1,8 @@
 // Shared device/host helpers for the gfx950 (CDNA4, wave64) token-numerics kernels.
 #pragma once
 #include <hip/hip_runtime.h>
+
+#include <initializer_list>
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -129,6 +131,59 @@ __device__ __forceinline__ void row_span(const Rows& r, int64_t b, int64_t& star
     start = b * r.n_cols;
     len = r.n_cols;
   }
+}
+
+// ---------------------------------------------------------------- four tokens per lane
+// Kernels whose lanes work on four consecutive tokens load them with one 16-byte instruction per
+// fp32 array (and one load of the four mask elements) when Rows::vec says every array allows it.
+inline bool aligned_to(const void* p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
+
+// True when `mask` and every non-null fp32 array in `arrays` are aligned for those loads;
+// otherwise every token takes the element-wise path.
+inline bool vector_loads_ok(const void* mask, int mask_dt, std::initializer_list<const void*> arrays) {
+  bool ok = mask_dt == ORLHF_MASK_NONE || aligned_to(mask, mask_dt == ORLHF_MASK_U8 ? 4 : 16);
+  for (const void* a : arrays) ok = ok && aligned_to(a, 16);
+  return ok;
+}
+
+template <int MASK_DT>
+__device__ __forceinline__ void load_mask4(const void* mask, int64_t i0, float* m) {
+  if (MASK_DT == ORLHF_MASK_NONE) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m[k] = 1.0f;
+  } else if (MASK_DT == ORLHF_MASK_U8) {
+    const uint32_t w = *(const uint32_t*)((const uint8_t*)mask + i0);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m[k] = (float)((w >> (8 * k)) & 0xffu);
+  } else if (MASK_DT == ORLHF_MASK_F32) {
+    const f32x4 x = *(const f32x4*)((const float*)mask + i0);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) m[k] = x[k];
+  } else {
+    typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
+    const i64x2 lo = *(const i64x2*)((const int64_t*)mask + i0), hi = *(const i64x2*)((const int64_t*)mask + i0 + 2);
+    m[0] = (float)lo[0];
+    m[1] = (float)lo[1];
+    m[2] = (float)hi[0];
+    m[3] = (float)hi[1];
+  }
+}
+
+// A row as the chunked kernels walk it: when vector loads are on, the walk starts at the last
+// 16-byte boundary at or before the row's first token (`lead` tokens early, 0..3), so that every
+// whole step of the walk is aligned; tokens before `lead` are not the row's and are skipped.
+struct RowWalk {
+  int64_t base, len;  // flat index of the walk's first position; positions in the walk
+  int lead;
+};
+__device__ __forceinline__ RowWalk row_walk(const Rows& rows, int64_t b) {
+  int64_t start, len;
+  row_span(rows, b, start, len);
+  RowWalk w;
+  w.lead = (rows.vec && len > 0) ? (int)(start & 3) : 0;
+  w.base = start - w.lead;
+  w.len = len > 0 ? len + w.lead : 0;
+  return w;
 }
 
 // ---------------------------------------------------------------- rows -> workgroups

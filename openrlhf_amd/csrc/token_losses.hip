@@ -13,8 +13,6 @@
 // aggregation weight that the backward kernels multiply with. Chunks past the end of a short
 // packed row return at once. No atomics anywhere: the result is bit-reproducible. All of these
 // are HBM-bound streams of 4-17 bytes per token.
-#include <initializer_list>
-
 #include "token_terms.h"
 
 namespace orlhf {
@@ -38,14 +36,9 @@ static inline int64_t chunks_of(const Rows& r) {
   return r.n_cols > 0 ? (r.n_cols + lead + r.chunk - 1) / r.chunk : 1;
 }
 
-static inline bool aligned_to(const void* p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
-
-// Rows of a chunked launch over `arrays` (fp32, null entries ignored) and `mask`: vector loads are
-// on when all of them are aligned for it; otherwise every token takes the element-wise path.
 static Rows make_rows(int64_t n_rows, int64_t n_cols, const int64_t* cu, const void* mask, int mask_dt,
                       std::initializer_list<const void*> arrays) {
-  bool vec = mask_dt == ORLHF_MASK_NONE || aligned_to(mask, mask_dt == ORLHF_MASK_U8 ? 4 : 16);
-  for (const void* a : arrays) vec = vec && aligned_to(a, 16);
+  const bool vec = vector_loads_ok(mask, mask_dt, arrays);
   // 8 steps per work item measured fastest on large batches (16 the same, 4: +8%, 2: +35%);
   // smaller problems get shorter chunks so that a thousand workgroups still exist.
   int steps = 8;
@@ -181,46 +174,6 @@ __device__ __forceinline__ void load_inputs4(const Tok& tok, int64_t i0, float (
 #pragma unroll
     for (int k = 0; k < 4; ++k) v[k][j] = x[k];
   }
-}
-
-template <int MASK_DT>
-__device__ __forceinline__ void load_mask4(const void* mask, int64_t i0, float* m) {
-  if (MASK_DT == ORLHF_MASK_NONE) {
-#pragma unroll
-    for (int k = 0; k < 4; ++k) m[k] = 1.0f;
-  } else if (MASK_DT == ORLHF_MASK_U8) {
-    const uint32_t w = *(const uint32_t*)((const uint8_t*)mask + i0);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) m[k] = (float)((w >> (8 * k)) & 0xffu);
-  } else if (MASK_DT == ORLHF_MASK_F32) {
-    const f32x4 x = *(const f32x4*)((const float*)mask + i0);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) m[k] = x[k];
-  } else {
-    typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
-    const i64x2 lo = *(const i64x2*)((const int64_t*)mask + i0), hi = *(const i64x2*)((const int64_t*)mask + i0 + 2);
-    m[0] = (float)lo[0];
-    m[1] = (float)lo[1];
-    m[2] = (float)hi[0];
-    m[3] = (float)hi[1];
-  }
-}
-
-// A row as the chunked kernels walk it: when vector loads are on, the walk starts at the last
-// 16-byte boundary at or before the row's first token (`lead` tokens early, 0..3), so that every
-// whole step of the walk is aligned; tokens before `lead` are not the row's and are skipped.
-struct RowWalk {
-  int64_t base, len;  // flat index of the walk's first position; positions in the walk
-  int lead;
-};
-__device__ __forceinline__ RowWalk row_walk(const Rows& rows, int64_t b) {
-  int64_t start, len;
-  row_span(rows, b, start, len);
-  RowWalk w;
-  w.lead = (rows.vec && len > 0) ? (int)(start & 3) : 0;
-  w.base = start - w.lead;
-  w.len = len > 0 ? len + w.lead : 0;
-  return w;
 }
 
 // ---------------------------------------------------------------- stage 1: chunk partials
