@@ -23,6 +23,20 @@ __device__ __forceinline__ int64_t mask_as_int(const void* mask, int64_t i) {
 }
 
 template <int MASK_DT>
+__device__ __forceinline__ void mask_as_int4(const void* mask, int64_t i0, int64_t* v) {
+  if (MASK_DT == ORLHF_MASK_I64) {
+    typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
+    const i64x2 lo = *(const i64x2*)((const int64_t*)mask + i0), hi = *(const i64x2*)((const int64_t*)mask + i0 + 2);
+    v[0] = lo[0], v[1] = lo[1], v[2] = hi[0], v[3] = hi[1];
+  } else {  // bytes are exact as floats; a float mask truncates like .long()
+    float m[4];
+    load_mask4<MASK_DT>(mask, i0, m);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = (int64_t)m[k];
+  }
+}
+
+template <int MASK_DT>
 __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const float* __restrict__ r,
                                                                 float neg_coef, const float* __restrict__ kl,
                                                                 const void* __restrict__ mask, int has_clip,
@@ -41,15 +55,24 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
       if (threadIdx.x == 0 && eos_index != nullptr) eos_index[b] = -1;
       continue;
     }
+    const RowWalk rw = row_walk(rows, b);
     // last position where (int64)mask is maximal == argmax over the flipped row
     int64_t best_v = INT64_MIN, best_i = -1;
-    for (int64_t t = threadIdx.x; t < len; t += kBlock) {
-      const int64_t v = mask_as_int<MASK_DT>(mask, start + t);
+    auto see = [&](int64_t v, int64_t t) {
       if (v > best_v || (v == best_v && t > best_i)) {
         best_v = v;
         best_i = t;
       }
-    }
+    };
+    for_row_tokens(
+        rows, rw,
+        [&](int64_t i0) {
+          int64_t v[4];
+          mask_as_int4<MASK_DT>(mask, i0, v);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) see(v[k], i0 + k - start);
+        },
+        [&](int64_t i) { see(mask_as_int<MASK_DT>(mask, i), i - start); });
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) {
       const int64_t ov = __shfl_xor(best_v, o, kWave);
@@ -76,10 +99,16 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
     __syncthreads();
     float rb = r[b];
     if (has_clip) rb = (rb != rb) ? rb : fminf(fmaxf(rb, clip_lo), clip_hi);
-    for (int64_t t = threadIdx.x; t < len; t += kBlock) {
-      const float last = (t == best_i) ? rb : 0.0f;
-      reward[start + t] = last + neg_coef * kl[start + t];
-    }
+    for_row_tokens(
+        rows, rw,
+        [&](int64_t i0) {
+          const f32x4 k4 = *(const f32x4*)(kl + i0);
+          f32x4 o;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) o[k] = ((i0 + k - start == best_i) ? rb : 0.0f) + neg_coef * k4[k];
+          *(f32x4*)(reward + i0) = o;
+        },
+        [&](int64_t i) { reward[i] = ((i - start == best_i) ? rb : 0.0f) + neg_coef * kl[i]; });
     if (threadIdx.x == 0 && eos_index != nullptr) eos_index[b] = best_i;
   }
 }
@@ -391,7 +420,7 @@ extern "C" int orlhf_compute_reward(const float* r, float kl_coef, const float* 
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(r && reward && (kl || n_cols == 0), "compute_reward: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
-  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {kl, reward}) ? 1 : 0};
   const float neg_coef = -(kl_coef > 0.0f ? kl_coef : 0.0f);
   const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
 #define ORLHF_LAUNCH(M)                                                                                         \

@@ -186,6 +186,32 @@ __device__ __forceinline__ RowWalk row_walk(const Rows& rows, int64_t b) {
   return w;
 }
 
+// Walks one row with the whole workgroup: four(i0) for each lane's four consecutive tokens
+// (flat index i0, aligned for a 16-byte load) on every step that lies inside the row when vector
+// loads are on, one(i) per token (stride kBlock) on the steps at the row's ends or on all steps
+// otherwise. Every token of the row is visited exactly once.
+template <typename F4, typename F1>
+__device__ __forceinline__ void for_row_tokens(const Rows& rows, const RowWalk& rw, F4&& four, F1&& one) {
+  constexpr int kStep = kBlock * 4;
+  int64_t s0 = 0;
+  auto edge = [&](int64_t s) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int64_t t = s + threadIdx.x + k * kBlock;
+      if (t >= rw.lead && t < rw.len) one(rw.base + t);
+    }
+  };
+  if (rows.vec) {
+    if (rw.lead > 0 && s0 < rw.len) {
+      edge(s0);
+      s0 += kStep;
+    }
+#pragma unroll 2
+    for (; s0 + kStep <= rw.len; s0 += kStep) four(rw.base + s0 + (int64_t)threadIdx.x * 4);
+  }
+  for (; s0 < rw.len; s0 += kStep) edge(s0);
+}
+
 // ---------------------------------------------------------------- rows -> workgroups
 // Workgroups are handed out in index order and, as measured, statically: round-robin over the
 // eight XCDs and again over the shader engines inside one. With row b on workgroup b, row lengths

@@ -13,6 +13,24 @@ __device__ __forceinline__ float load_lp(const void* p, int64_t i) {
   return (float)((const _Float16*)p)[i];
 }
 
+// four consecutive elements from index i0 (a multiple of four from a 16-byte aligned base)
+template <int DT>
+__device__ __forceinline__ void load_lp4(const void* p, int64_t i0, float* v) {
+  if (DT == ORLHF_F32) {
+    const f32x4 x = *(const f32x4*)((const float*)p + i0);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = x[k];
+  } else {
+    const u32x2 w = *(const u32x2*)((const uint16_t*)p + i0);
+    if (DT == ORLHF_BF16) {
+      v[0] = bf16_lo(w[0]), v[1] = bf16_hi(w[0]), v[2] = bf16_lo(w[1]), v[3] = bf16_hi(w[1]);
+    } else {
+      const f16x2 a = __builtin_bit_cast(f16x2, w[0]), b = __builtin_bit_cast(f16x2, w[1]);
+      v[0] = (float)a[0], v[1] = (float)a[1], v[2] = (float)b[0], v[3] = (float)b[1];
+    }
+  }
+}
+
 __device__ __forceinline__ void block_sum3(double& a, double& b, double& c, double (*lds)[kWavesPerBlock]) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) {
@@ -42,23 +60,43 @@ __global__ __launch_bounds__(kBlock) void kl_rows_kernel(const void* __restrict_
   for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
     const int64_t b = row_of_slot(slot, slot, slot_b);
     if (b >= rows.n_rows) continue;
-    int64_t start, len;
-    row_span(rows, b, start, len);
+    const RowWalk rw = row_walk(rows, b);
     double sk = 0.0, sd = 0.0, sm = 0.0;
-#pragma unroll 4
-    for (int64_t t = threadIdx.x; t < len; t += kBlock) {
-      const int64_t i = start + t;
-      const float m = load_mask<MASK_DT>(mask, i);
-      float v = 0.0f, d = 0.0f, dv;
+    auto token = [&](float x, float y, float m, float& v) {
+      float d = 0.0f, dv;
+      v = 0.0f;
       if (enabled) {
-        d = load_lp<DT>(lp, i) - load_lp<DT>(base, i);
+        d = x - y;
         kl_value(est, d, v, dv);
       }
-      if (kl != nullptr) kl[i] = v;
       sk += (double)(v * m);
       sd += (double)(d * m);
       sm += (double)m;
-    }
+    };
+    for_row_tokens(
+        rows, rw,
+        [&](int64_t i0) {
+          float x[4] = {0.0f, 0.0f, 0.0f, 0.0f}, y[4] = {0.0f, 0.0f, 0.0f, 0.0f}, m[4];
+          if (enabled) {
+            load_lp4<DT>(lp, i0, x);
+            load_lp4<DT>(base, i0, y);
+          }
+          load_mask4<MASK_DT>(mask, i0, m);
+          f32x4 v;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            float vk;
+            token(x[k], y[k], m[k], vk);
+            v[k] = vk;
+          }
+          if (kl != nullptr) *(f32x4*)(kl + i0) = v;
+        },
+        [&](int64_t i) {
+          float v;
+          token(enabled ? load_lp<DT>(lp, i) : 0.0f, enabled ? load_lp<DT>(base, i) : 0.0f,
+                load_mask<MASK_DT>(mask, i), v);
+          if (kl != nullptr) kl[i] = v;
+        });
     block_sum3(sk, sd, sm, lds);
     if (threadIdx.x == 0) {
       if (kl_mean != nullptr) kl_mean[b] = (float)(sk / sm);  // no epsilon: an empty row is NaN, as masked_mean
@@ -78,30 +116,60 @@ __global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const flo
   for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
     const int64_t b = row_of_slot(slot, slot, slot_b);
     if (b >= rows.n_rows) continue;
-    int64_t start, len;
-    row_span(rows, b, start, len);
+    const RowWalk rw = row_walk(rows, b);
     double s = 0.0, c = 0.0, z = 0.0;
-#pragma unroll 4
-    for (int64_t t = threadIdx.x; t < len; t += kBlock) {
-      const float m = load_mask<MASK_DT>(mask, start + t);
-      s += (double)(x[start + t] * m);
-      c += (double)m;
-    }
+    for_row_tokens(
+        rows, rw,
+        [&](int64_t i0) {
+          const f32x4 v = *(const f32x4*)(x + i0);
+          float m[4];
+          load_mask4<MASK_DT>(mask, i0, m);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            s += (double)(v[k] * m[k]);
+            c += (double)m[k];
+          }
+        },
+        [&](int64_t i) {
+          const float m = load_mask<MASK_DT>(mask, i);
+          s += (double)(x[i] * m);
+          c += (double)m;
+        });
     block_sum3(s, c, z, lds);
     const double cnt = c < 1.0 ? 1.0 : c;
     const float mean = (float)(s / cnt);
     double v = 0.0, z1 = 0.0, z2 = 0.0;
-#pragma unroll 4
-    for (int64_t t = threadIdx.x; t < len; t += kBlock) {
-      const float e = (x[start + t] - mean) * load_mask<MASK_DT>(mask, start + t);
-      v += (double)(e * e);
-    }
+    for_row_tokens(
+        rows, rw,
+        [&](int64_t i0) {
+          const f32x4 xv = *(const f32x4*)(x + i0);
+          float m[4];
+          load_mask4<MASK_DT>(mask, i0, m);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            const float e = (xv[k] - mean) * m[k];
+            v += (double)(e * e);
+          }
+        },
+        [&](int64_t i) {
+          const float e = (x[i] - mean) * load_mask<MASK_DT>(mask, i);
+          v += (double)(e * e);
+        });
     block_sum3(v, z1, z2, lds);
     const float var = (float)(v / cnt);
     const float r = 1.0f / sqrtf(var != var ? var : fmaxf(var, eps));
-#pragma unroll 4
-    for (int64_t t = threadIdx.x; t < len; t += kBlock)
-      out[start + t] = (x[start + t] - mean) * load_mask<MASK_DT>(mask, start + t) * r;
+    for_row_tokens(
+        rows, rw,
+        [&](int64_t i0) {
+          const f32x4 xv = *(const f32x4*)(x + i0);
+          float m[4];
+          load_mask4<MASK_DT>(mask, i0, m);
+          f32x4 o;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) o[k] = (xv[k] - mean) * m[k] * r;
+          *(f32x4*)(out + i0) = o;
+        },
+        [&](int64_t i) { out[i] = (x[i] - mean) * load_mask<MASK_DT>(mask, i) * r; });
   }
 }
 
@@ -119,7 +187,7 @@ extern "C" int orlhf_kl_rows(const void* log_probs, const void* log_probs_base, 
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(!enabled || n_cols == 0 || (log_probs != nullptr && log_probs_base != nullptr),
                   "kl_rows: log_probs / log_probs_base is NULL");
-  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {log_probs, log_probs_base, kl}) ? 1 : 0};
   const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_KL(M)                                                                                                  \
@@ -146,7 +214,7 @@ extern "C" int orlhf_masked_normalize_rows(const float* x, const void* mask, int
   if (int rc = check_rows("masked_normalize_rows", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(x != nullptr && out != nullptr, "masked_normalize_rows: NULL argument");
-  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {x, out}) ? 1 : 0};
   const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_NORM(M) \
