@@ -307,6 +307,11 @@ def bench_per_token(args, dev):
     padded = b * a
     record("config4.approx_kl_k3", timed(lambda: compute_approx_kl(lp, ref, "k3")), padded, 12)
     record("config4.discounted_returns", timed(lambda: get_cumulative_returns(adv, mask, 1.0)), padded, 9)
+    record("config4.gae_scan", timed(lambda: get_advantages_and_returns(old, adv, mask, 1.0, 0.95)), padded, 17)
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import experience_kl
+    record("config4.kl_block_k3", timed(lambda: experience_kl(lp, ref, mask, "k3")), padded, 13)
+    r_seq = torch.randn(b, device=dev)
+    record("config4.compute_reward", timed(lambda: compute_reward(r_seq, 0.01, adv, mask)), padded, 4 + 1 + 1 + 4)
     x = lp.clone().requires_grad_(True)
     pl = PolicyLoss(0.2, 0.2, dual_clip=3.0, token_level_loss=False)
 
@@ -330,6 +335,8 @@ def bench_per_token(args, dev):
     cu = ps.cu_seqlens
     record("config4.discounted_returns_packed",
            timed(lambda: get_cumulative_returns(ps["adv"], ps["mask"], 1.0, cu_seqlens=cu, max_seqlen=a)), real, 9)
+    record("config4.gae_scan_packed",
+           timed(lambda: get_advantages_and_returns(ps["old"], ps["adv"], ps["mask"], 1.0, 0.95, cu_seqlens=cu)), real, 17)
     xk = ps["lp"].clone().requires_grad_(True)
 
     def policy_step_packed():
