@@ -312,6 +312,10 @@ def bench_per_token(args, dev):
     record("config4.kl_block_k3", timed(lambda: experience_kl(lp, ref, mask, "k3")), padded, 13)
     r_seq = torch.randn(b, device=dev)
     record("config4.compute_reward", timed(lambda: compute_reward(r_seq, 0.01, adv, mask)), padded, 4 + 1 + 1 + 4)
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import reward_advantages_and_returns
+    # reward + GAE without the per-token reward in memory: kl, values, mask in; advantages, returns out
+    record("config4.reward_gae_one_pass",
+           timed(lambda: reward_advantages_and_returns(r_seq, 0.01, adv, old, mask, 1.0, 0.95)), padded, 17)
     x = lp.clone().requires_grad_(True)
     pl = PolicyLoss(0.2, 0.2, dual_clip=3.0, token_level_loss=False)
 

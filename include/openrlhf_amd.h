@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 9
+#define ORLHF_ABI_VERSION 10
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -326,6 +326,22 @@ int orlhf_gae_scan(const float* values, const float* rewards, const void* mask, 
 int orlhf_discounted_returns(const float* rewards, const void* mask, int mask_dtype,
                              int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
                              float gamma, float* returns, orlhf_stream_t stream);
+
+/*
+ * The per-experience body of compute_advantages_and_returns (experience_maker.py:276-312) in one
+ * pass: compute_reward (openrlhf/models/utils.py:98-126) followed by get_advantages_and_returns
+ * (values and advantages given) or get_cumulative_returns (both NULL), without the per-token
+ * reward ever being stored. Per row: the last maximal mask position is found, then the reverse
+ * scan makes each token reward -max(kl_coef, 0)*kl[t] (+ the clipped r[b] at that position) as
+ * it loads kl. reward_sum[b] (nullable) = the row's token rewards summed over every column,
+ * which is the reference's info["return"] (experience_maker.py:311). Results equal
+ * orlhf_compute_reward followed by orlhf_gae_scan / orlhf_discounted_returns bit for bit.
+ */
+int orlhf_reward_scan(const float* r, float kl_coef, const float* kl, const float* values,
+                      const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                      const int64_t* cu_seqlens, int has_clip, float clip_low, float clip_high,
+                      float gamma, float lambd, float* advantages, float* returns,
+                      float* reward_sum, orlhf_stream_t stream);
 
 /*
  * Group baseline / normalisation of scalar rewards (experience_maker.py:246-272).

@@ -36,6 +36,61 @@ __device__ __forceinline__ void mask_as_int4(const void* mask, int64_t i0, int64
   }
 }
 
+// Index (from the row's first token) of the last position where (int64)mask is maximal: the
+// arg-max over the flipped row that the reference takes. Called by the whole workgroup.
+template <int MASK_DT>
+__device__ __forceinline__ int64_t last_max_of_mask(const Rows& rows, const RowWalk& rw, int64_t start,
+                                                    const void* __restrict__ mask, int64_t* lds_val,
+                                                    int64_t* lds_idx) {
+  int64_t best_v = INT64_MIN, best_i = -1;
+  auto see = [&](int64_t v, int64_t t) {
+    if (v > best_v || (v == best_v && t > best_i)) {
+      best_v = v;
+      best_i = t;
+    }
+  };
+  for_row_tokens(
+      rows, rw,
+      [&](int64_t i0) {
+        int64_t v[4];
+        mask_as_int4<MASK_DT>(mask, i0, v);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) see(v[k], i0 + k - start);
+      },
+      [&](int64_t i) { see(mask_as_int<MASK_DT>(mask, i), i - start); });
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    const int64_t ov = __shfl_xor(best_v, o, kWave);
+    const int64_t oi = __shfl_xor(best_i, o, kWave);
+    if (ov > best_v || (ov == best_v && oi > best_i)) {
+      best_v = ov;
+      best_i = oi;
+    }
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    lds_val[threadIdx.x / kWave] = best_v;
+    lds_idx[threadIdx.x / kWave] = best_i;
+  }
+  __syncthreads();
+  best_v = lds_val[0];
+  best_i = lds_idx[0];
+#pragma unroll
+  for (int w = 1; w < kWavesPerBlock; ++w) {
+    if (lds_val[w] > best_v || (lds_val[w] == best_v && lds_idx[w] > best_i)) {
+      best_v = lds_val[w];
+      best_i = lds_idx[w];
+    }
+  }
+  __syncthreads();
+  return best_i;
+}
+
+// The sequence reward as the reference places it: clipped when a range is given (NaN passes).
+__device__ __forceinline__ float clipped_reward(float rb, int has_clip, float clip_lo, float clip_hi) {
+  if (has_clip) rb = (rb != rb) ? rb : fminf(fmaxf(rb, clip_lo), clip_hi);
+  return rb;
+}
+
 template <int MASK_DT>
 __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const float* __restrict__ r,
                                                                 float neg_coef, const float* __restrict__ kl,
@@ -56,49 +111,8 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
       continue;
     }
     const RowWalk rw = row_walk(rows, b);
-    // last position where (int64)mask is maximal == argmax over the flipped row
-    int64_t best_v = INT64_MIN, best_i = -1;
-    auto see = [&](int64_t v, int64_t t) {
-      if (v > best_v || (v == best_v && t > best_i)) {
-        best_v = v;
-        best_i = t;
-      }
-    };
-    for_row_tokens(
-        rows, rw,
-        [&](int64_t i0) {
-          int64_t v[4];
-          mask_as_int4<MASK_DT>(mask, i0, v);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) see(v[k], i0 + k - start);
-        },
-        [&](int64_t i) { see(mask_as_int<MASK_DT>(mask, i), i - start); });
-#pragma unroll
-    for (int o = kWave / 2; o > 0; o >>= 1) {
-      const int64_t ov = __shfl_xor(best_v, o, kWave);
-      const int64_t oi = __shfl_xor(best_i, o, kWave);
-      if (ov > best_v || (ov == best_v && oi > best_i)) {
-        best_v = ov;
-        best_i = oi;
-      }
-    }
-    if ((threadIdx.x & (kWave - 1)) == 0) {
-      lds_val[threadIdx.x / kWave] = best_v;
-      lds_idx[threadIdx.x / kWave] = best_i;
-    }
-    __syncthreads();
-    best_v = lds_val[0];
-    best_i = lds_idx[0];
-#pragma unroll
-    for (int w = 1; w < kWavesPerBlock; ++w) {
-      if (lds_val[w] > best_v || (lds_val[w] == best_v && lds_idx[w] > best_i)) {
-        best_v = lds_val[w];
-        best_i = lds_idx[w];
-      }
-    }
-    __syncthreads();
-    float rb = r[b];
-    if (has_clip) rb = (rb != rb) ? rb : fminf(fmaxf(rb, clip_lo), clip_hi);
+    const int64_t best_i = last_max_of_mask<MASK_DT>(rows, rw, start, mask, lds_val, lds_idx);
+    const float rb = clipped_reward(r[b], has_clip, clip_lo, clip_hi);
     for_row_tokens(
         rows, rw,
         [&](int64_t i0) {
@@ -135,16 +149,31 @@ struct ScanTile {
   float v[kScanItems + 1];
 };
 
+// Per-token rewards made on the fly from the KL estimate (REWARD mode of the scan): the token
+// reward is neg_coef * kl plus the sequence reward at position `eos` of the walk, as
+// compute_reward_kernel writes it; `sum` collects the row's token rewards.
+struct RowReward {
+  float seq, neg_coef;
+  int64_t eos;  // position in the walk (RowWalk::lead + index in the row)
+  double sum;
+};
+
 // `whole`: the tile lies inside the row and every array allows 16-byte loads. Must be called by
 // all lanes of the workgroup (it exchanges the following value across lanes).
-template <int MASK_DT, bool GAE>
+template <int MASK_DT, bool GAE, bool REWARD>
 __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t tile0, bool whole,
                                                    const float* __restrict__ values,
                                                    const float* __restrict__ rewards,
-                                                   const void* __restrict__ mask) {
+                                                   const void* __restrict__ mask, RowReward& rr) {
   static_assert(kScanItems == 4, "a lane's tokens are one 16-byte load");
   ScanTile t;
   const int64_t p0 = tile0 + (int64_t)threadIdx.x * kScanItems;
+  auto reward_of = [&](float raw, int64_t p) {
+    if (!REWARD) return raw;
+    const float tok = ((p == rr.eos) ? rr.seq : 0.0f) + rr.neg_coef * raw;
+    rr.sum += (double)tok;
+    return tok;
+  };
   if (whole) {
     float m[kScanItems];
     load_mask4<MASK_DT>(mask, rw.base + p0, m);
@@ -153,7 +182,7 @@ __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t ti
     if (GAE) v4 = *(const f32x4*)(values + rw.base + p0);
 #pragma unroll
     for (int j = 0; j < kScanItems; ++j) {
-      t.r[j] = m[j] * r4[j];
+      t.r[j] = m[j] * reward_of(r4[j], p0 + j);
       t.v[j] = m[j] * v4[j];
     }
   } else {
@@ -164,7 +193,7 @@ __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t ti
       t.v[j] = 0.0f;
       if (p >= rw.lead && p < rw.len) {
         const float m = load_mask<MASK_DT>(mask, rw.base + p);
-        t.r[j] = m * rewards[rw.base + p];
+        t.r[j] = m * reward_of(rewards[rw.base + p], p);
         if (GAE) t.v[j] = m * values[rw.base + p];
       }
     }
@@ -183,13 +212,27 @@ __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t ti
 
 // One workgroup per row, walking it backwards in tiles of kScanTile tokens; the tile before the
 // current one is loaded (straight into registers, no staging) while the current one is scanned.
-template <int MASK_DT, bool GAE>
+// REWARD: `rewards` holds the per-token KL estimate and the token rewards are made from it and
+// the sequence rewards `seq` on the fly (compute_reward fused in); reward_sum[b] receives the sum
+// of row b's token rewards.
+struct SeqReward {
+  const float* seq;  // [n_rows]
+  float neg_coef;
+  int has_clip;
+  float clip_lo, clip_hi;
+  float* reward_sum;  // [n_rows], nullable
+};
+
+template <int MASK_DT, bool GAE, bool REWARD>
 __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const float* __restrict__ values,
                                                               const float* __restrict__ rewards,
                                                               const void* __restrict__ mask, double gamma,
-                                                              double coef, float* __restrict__ adv,
+                                                              double coef, SeqReward sr, float* __restrict__ adv,
                                                               float* __restrict__ ret) {
   __shared__ Affine lds_wave[2][kWavesPerBlock];  // alternating: one barrier per tile is enough
+  __shared__ int64_t lds_val[kWavesPerBlock];
+  __shared__ int64_t lds_idx[kWavesPerBlock];
+  __shared__ double lds_sum[kWavesPerBlock];
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
 
@@ -204,17 +247,30 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
     const int64_t b = row_of_slot(slot, slot, slot_b);
     if (b >= rows.n_rows) continue;
     const RowWalk rw = row_walk(rows, b);
-    if (rw.len <= 0) continue;
+    if (rw.len <= 0) {
+      if (REWARD && threadIdx.x == 0 && sr.reward_sum != nullptr) sr.reward_sum[b] = 0.0f;
+      continue;
+    }
+    RowReward rr{0.0f, 0.0f, -1, 0.0};
+    if (REWARD) {
+      rr.seq = clipped_reward(sr.seq[b], sr.has_clip, sr.clip_lo, sr.clip_hi);
+      rr.neg_coef = sr.neg_coef;
+      rr.eos = MASK_DT == ORLHF_MASK_NONE  // without a mask the last column is the last maximum
+                   ? rw.len - 1
+                   : rw.lead + last_max_of_mask<MASK_DT>(rows, rw, rw.base + rw.lead, mask, lds_val, lds_idx);
+    }
     const int64_t n_tiles = (rw.len + kScanTile - 1) / kScanTile;
     double tile_carry = 0.0;  // A at the first token of the previous (later) tile
     auto whole = [&](int64_t tile) {
       return rows.vec && tile * kScanTile >= rw.lead && (tile + 1) * kScanTile <= rw.len;
     };
-    ScanTile cur = load_scan_tile<MASK_DT, GAE>(rw, (n_tiles - 1) * kScanTile, whole(n_tiles - 1), values, rewards, mask);
+    ScanTile cur =
+        load_scan_tile<MASK_DT, GAE, REWARD>(rw, (n_tiles - 1) * kScanTile, whole(n_tiles - 1), values, rewards, mask, rr);
     for (int64_t tile = n_tiles - 1; tile >= 0; --tile) {
       const int64_t tile0 = tile * kScanTile;
       ScanTile nxt = cur;
-      if (tile > 0) nxt = load_scan_tile<MASK_DT, GAE>(rw, tile0 - kScanTile, whole(tile - 1), values, rewards, mask);
+      if (tile > 0)
+        nxt = load_scan_tile<MASK_DT, GAE, REWARD>(rw, tile0 - kScanTile, whole(tile - 1), values, rewards, mask, rr);
       // in-lane recurrence with zero carry-in
       double local[kScanItems];
       double run = 0.0;
@@ -283,6 +339,10 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
         }
       }
       cur = nxt;
+    }
+    if (REWARD && sr.reward_sum != nullptr) {  // uniform: reward_sum is a kernel argument
+      const double total = block_sum(rr.sum, lds_sum);
+      if (threadIdx.x == 0) sr.reward_sum[b] = (float)total;
     }
   }
 }
@@ -397,13 +457,13 @@ __global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* __res
 
 
 
-template <bool GAE>
+template <bool GAE, bool REWARD>
 static void launch_scan(int mask_dtype, Rows rows, const float* values, const float* rewards, const void* mask,
-                        double gamma, double coef, float* adv, float* ret, hipStream_t s) {
+                        double gamma, double coef, const SeqReward& sr, float* adv, float* ret, hipStream_t s) {
   const dim3 grid(slot_grid(row_slots(rows.n_rows), 65536)), block(kBlock);
-#define ORLHF_LAUNCH(M)                                                                                          \
-  hipLaunchKernelGGL((reverse_scan_kernel<M, GAE>), grid, block, 0, s, rows, values, rewards, mask, gamma, coef, adv, \
-                     ret)
+#define ORLHF_LAUNCH(M)                                                                                        \
+  hipLaunchKernelGGL((reverse_scan_kernel<M, GAE, REWARD>), grid, block, 0, s, rows, values, rewards, mask, gamma, \
+                     coef, sr, adv, ret)
   ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
 #undef ORLHF_LAUNCH
 }
@@ -440,8 +500,8 @@ extern "C" int orlhf_gae_scan(const float* values, const float* rewards, const v
   ORLHF_CHECK_ARG(values && rewards && advantages && returns, "gae_scan: NULL pointer");
   const Rows rows{n_rows, n_cols, cu_seqlens,
                   vector_loads_ok(mask, mask_dtype, {values, rewards, advantages, returns}) ? 1 : 0};
-  launch_scan<true>(mask_dtype, rows, values, rewards, mask, (double)gamma, (double)gamma * (double)lambd,
-                    advantages, returns, (hipStream_t)stream);
+  launch_scan<true, false>(mask_dtype, rows, values, rewards, mask, (double)gamma, (double)gamma * (double)lambd,
+                           SeqReward{}, advantages, returns, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_gae_scan");
   return ORLHF_OK;
 }
@@ -453,9 +513,32 @@ extern "C" int orlhf_discounted_returns(const float* rewards, const void* mask, 
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(rewards && returns, "discounted_returns: NULL pointer");
   const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {rewards, returns}) ? 1 : 0};
-  launch_scan<false>(mask_dtype, rows, nullptr, rewards, mask, (double)gamma, (double)gamma, nullptr, returns,
-                     (hipStream_t)stream);
+  launch_scan<false, false>(mask_dtype, rows, nullptr, rewards, mask, (double)gamma, (double)gamma, SeqReward{},
+                            nullptr, returns, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_discounted_returns");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_reward_scan(const float* r, float kl_coef, const float* kl, const float* values,
+                                 const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                                 const int64_t* cu_seqlens, int has_clip, float clip_low, float clip_high,
+                                 float gamma, float lambd, float* advantages, float* returns, float* reward_sum,
+                                 orlhf_stream_t stream) {
+  if (int rc = check_rows("reward_scan", n_rows, n_cols, mask, mask_dtype)) return rc;
+  if (n_rows == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(r != nullptr && returns != nullptr && (kl != nullptr || n_cols == 0), "reward_scan: NULL pointer");
+  ORLHF_CHECK_ARG((values == nullptr) == (advantages == nullptr),
+                  "reward_scan: values and advantages go together (GAE) or are both NULL (discounted returns)");
+  const Rows rows{n_rows, n_cols, cu_seqlens,
+                  vector_loads_ok(mask, mask_dtype, {kl, values, advantages, returns}) ? 1 : 0};
+  const SeqReward sr{r, -(kl_coef > 0.0f ? kl_coef : 0.0f), has_clip, clip_low, clip_high, reward_sum};
+  if (values != nullptr)
+    launch_scan<true, true>(mask_dtype, rows, values, kl, mask, (double)gamma, (double)gamma * (double)lambd, sr,
+                            advantages, returns, (hipStream_t)stream);
+  else
+    launch_scan<false, true>(mask_dtype, rows, nullptr, kl, mask, (double)gamma, (double)gamma, sr, nullptr, returns,
+                             (hipStream_t)stream);
+  ORLHF_CHECK_LAUNCH("orlhf_reward_scan");
   return ORLHF_OK;
 }
 

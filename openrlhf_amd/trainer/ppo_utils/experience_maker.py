@@ -24,7 +24,7 @@ import torch
 
 from ... import _lib
 from ..._lib import call, ptr, stream_of
-from ...models.utils import _KL_CODES, _cu_arg, _f32, _packed, _rows_of, compute_reward
+from ...models.utils import _KL_CODES, _cu_arg, _f32, _packed, _rows_of
 
 _GROUP_CODES = {
     "gae": _lib.GROUP_IDENTITY,
@@ -147,6 +147,46 @@ def get_cumulative_returns(
 
 
 @torch.no_grad()
+def reward_advantages_and_returns(
+    r: torch.Tensor,
+    kl_coef: float,
+    kl: torch.Tensor,
+    values: Optional[torch.Tensor],
+    action_mask: Optional[torch.Tensor],
+    gamma: float,
+    lambd: float = 1.0,
+    reward_clip_range: Optional[Tuple[float, float]] = None,
+    cu_seqlens: Optional[torch.Tensor] = None,
+) -> Tuple[Optional[torch.Tensor], torch.Tensor, torch.Tensor]:
+    """``compute_reward`` followed by GAE (``values`` given) or by the discounted returns
+    (``values=None``) in one pass that never stores the per-token reward: the per-experience body
+    of compute_advantages_and_returns (experience_maker.py:276-312). Returns ``(advantages,
+    returns, reward_sum)``; ``advantages`` is None without values (the reference clones the
+    returns there) and ``reward_sum[b]`` is the per-token reward summed over every column, the
+    reference's ``info["return"]``. Same numbers as the two separate calls."""
+    dev, home = _device_for(r, kl, values, action_mask)
+    klf = _f32(_on_gpu(kl, dev))
+    rf = _f32(_on_gpu(r, dev)).reshape(-1)
+    v = None if values is None else _f32(_on_gpu(values, dev))
+    if v is not None and v.shape != klf.shape:
+        raise ValueError(f"values {tuple(v.shape)} do not match kl {tuple(klf.shape)}")
+    mkeep, mptr, mcode = _lib.mask_arg(_on_gpu(action_mask, dev))
+    n_rows, n_cols = _rows_of(klf, _packed(cu_seqlens, klf.numel()))
+    if rf.numel() != n_rows:
+        raise ValueError(f"r has {rf.numel()} entries for {n_rows} rows")
+    cu = _cu_arg(cu_seqlens, dev)
+    adv = None if v is None else torch.empty_like(klf)
+    ret = torch.empty_like(klf)
+    total = torch.empty(n_rows, dtype=torch.float32, device=dev)
+    lo, hi = (reward_clip_range[0], reward_clip_range[1]) if reward_clip_range else (0.0, 0.0)
+    with torch.cuda.device(dev):
+        call("orlhf_reward_scan", ptr(rf), float(kl_coef), ptr(klf), ptr(v), mptr, mcode, n_rows, n_cols, ptr(cu),
+             1 if reward_clip_range else 0, float(lo), float(hi), float(gamma), float(lambd), ptr(adv), ptr(ret),
+             ptr(total), stream_of(dev))
+    return (None if adv is None else adv.to(home)), ret.to(home), total.to(home)
+
+
+@torch.no_grad()
 def group_normalize_rewards(
     rewards: torch.Tensor,
     indices: Optional[torch.Tensor],
@@ -229,23 +269,24 @@ def compute_advantages_and_returns(
         for e, s in zip(experiences, group_std.split(exp_len)):
             e.info["group_reward_std"] = s
 
+    if advantage_estimator != "gae" and advantage_estimator not in _RETURN_ESTIMATORS:
+        raise Exception(f"Unkown advantage_estimator {advantage_estimator}")
+    dev = _gpu_device()
     for e, reward in zip(experiences, shaped.split(exp_len)):
-        token_reward = compute_reward(
-            _on_gpu(reward, _gpu_device()), kl_coef, _on_gpu(e.kl, _gpu_device()),
-            action_mask=_on_gpu(e.action_mask, _gpu_device()), reward_clip_range=reward_clip_range,
-        )
         home = e.kl.device
         if advantage_estimator == "gae":
-            adv, ret = get_advantages_and_returns(e.values.to(token_reward.device), token_reward,
-                                                  e.action_mask.to(token_reward.device), gamma, lambd)
-            e.advantages, e.returns = adv.to(home), ret.to(home)
-        elif advantage_estimator in _RETURN_ESTIMATORS:
-            g = gamma if advantage_estimator == "reinforce" else 1.0  # the reference forces gamma = 1 here
-            e.returns = get_cumulative_returns(token_reward, e.action_mask.to(token_reward.device), g).to(home)
-            e.advantages = e.returns.clone()
+            values, g, lam = _on_gpu(e.values, dev), gamma, lambd
         else:
-            raise Exception(f"Unkown advantage_estimator {advantage_estimator}")
-        e.info["return"] = token_reward.sum(dim=-1).to(home)
+            values, lam = None, 1.0
+            g = gamma if advantage_estimator == "reinforce" else 1.0  # the reference forces gamma = 1 here
+        # per-token reward, scan and the row sums of the reward in one pass over kl
+        adv, ret, total = reward_advantages_and_returns(
+            _on_gpu(reward, dev), kl_coef, _on_gpu(e.kl, dev), values, _on_gpu(e.action_mask, dev), g, lam,
+            reward_clip_range=reward_clip_range,
+        )
+        e.returns = ret.to(home)
+        e.advantages = e.returns.clone() if adv is None else adv.to(home)
+        e.info["return"] = total.to(home)
         e.kl = None
 
     if advantage_estimator in ("gae", "reinforce", "reinforce_baseline"):

@@ -276,3 +276,84 @@ def test_compute_advantages_and_returns_pipeline(cuda, estimator):
         _rel_close(e.info["return"], i_, 1e-5)
     std_all = torch.cat([e.info["group_reward_std"] for e in out])
     assert (std_all.double() - gstd).abs().max().item() <= 1e-6
+
+
+# ------------------------------------------------------------------ reward + scan in one pass
+@pytest.mark.parametrize("mask_dtype", [torch.bool, torch.int64, torch.float32])
+@pytest.mark.parametrize("gae", [True, False])
+def test_reward_scan_equals_the_two_calls_and_the_oracle(cuda, mask_dtype, gae):
+    """compute_reward + GAE / discounted returns without the per-token reward in memory: the
+    same bits as the two separate kernels, padded and packed, and the oracle's composition
+    (openrlhf/models/utils.py:98-126, experience_maker.py:332-411) within the GAE tolerance."""
+    from openrlhf_amd.models.utils import compute_reward
+    from openrlhf_amd.trainer.ppo_utils.experience import PackedSteps
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import (
+        get_advantages_and_returns, get_cumulative_returns, reward_advantages_and_returns)
+
+    g = torch.Generator().manual_seed(91)
+    b, a = 9, 3001
+    mask = _mask(b, a, 5)
+    mask[3] = 0            # a row without any action token: the reward lands on its last column
+    mask[4, -1] = 1
+    kl = torch.randn(b, a, generator=g) * 0.1
+    values = torch.randn(b, a, generator=g) if gae else None
+    r = torch.randn(b, generator=g) * 3
+    clip = (-2.0, 2.0)
+    gamma, lambd = 0.99, 0.95
+    dm = mask.to(mask_dtype).to(cuda)
+    dkl, dr = kl.to(cuda), r.to(cuda)
+    dv = None if values is None else values.to(cuda)
+
+    adv, ret, total = reward_advantages_and_returns(dr, 0.05, dkl, dv, dm, gamma, lambd, reward_clip_range=clip)
+    rew = compute_reward(dr, 0.05, dkl, dm, reward_clip_range=clip)
+    if gae:
+        adv2, ret2 = get_advantages_and_returns(dv, rew, dm, gamma, lambd)
+        assert torch.equal(adv, adv2)
+    else:
+        ret2 = get_cumulative_returns(rew, dm, gamma)
+        assert adv is None
+    assert torch.equal(ret, ret2)
+    _rel_close(total, rew.double().sum(-1).cpu(), 1e-6)
+
+    o_rew = otn.compute_reward(r.double(), 0.05, kl.double(), mask, clip)
+    if gae:
+        o_adv, o_ret = oa.get_advantages_and_returns(values.double(), o_rew, mask, gamma, lambd)
+        _rel_close(adv, o_adv)
+    else:
+        o_ret = oa.get_cumulative_returns(o_rew, mask, gamma)
+    _rel_close(ret, o_ret)
+    _rel_close(total, o_rew.sum(-1), 1e-5)
+
+    # packed rows (a row of length zero among them), starts on every residue
+    keep = torch.ones(b, a, dtype=torch.bool)
+    lens = torch.tensor([3001, 17, 1024, 0, 2050, 1, 1027, 4, 999])
+    keep = torch.arange(a)[None, :] < lens[:, None]
+    fields = dict(kl=dkl, mask=dm)
+    if gae:
+        fields["v"] = dv
+    ps = PackedSteps.from_padded(fields, keep.to(cuda))
+    p_adv, p_ret, p_total = reward_advantages_and_returns(dr, 0.05, ps["kl"], ps["v"] if gae else None, ps["mask"],
+                                                          gamma, lambd, reward_clip_range=clip, cu_seqlens=ps.cu_seqlens)
+    p_rew = compute_reward(dr, 0.05, ps["kl"], ps["mask"], reward_clip_range=clip, cu_seqlens=ps.cu_seqlens, max_seqlen=a)
+    if gae:
+        q_adv, q_ret = get_advantages_and_returns(ps["v"], p_rew, ps["mask"], gamma, lambd, cu_seqlens=ps.cu_seqlens)
+        assert torch.equal(p_adv, q_adv)
+    else:
+        q_ret = get_cumulative_returns(p_rew, ps["mask"], gamma, cu_seqlens=ps.cu_seqlens)
+    assert torch.equal(p_ret, q_ret)
+    cu = ps.cu_seqlens.cpu()
+    for i in range(b):
+        seg = p_rew[cu[i]:cu[i + 1]].double().sum().item()
+        assert abs(p_total[i].item() - seg) <= 1e-6 * max(1.0, abs(seg))
+
+
+def test_reward_scan_argument_errors(cuda):
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import reward_advantages_and_returns
+
+    kl = torch.zeros(2, 8, device=cuda)
+    with pytest.raises(ValueError):
+        reward_advantages_and_returns(torch.zeros(3, device=cuda), 0.0, kl, None, None, 1.0)
+    with pytest.raises(ValueError):
+        reward_advantages_and_returns(torch.zeros(2, device=cuda), 0.0, kl, torch.zeros(2, 7, device=cuda), None, 1.0, 1.0)
+    adv, ret, total = reward_advantages_and_returns(torch.ones(2, device=cuda), 0.0, kl, None, None, 1.0)
+    assert adv is None and torch.equal(ret, torch.ones(2, 8, device=cuda)) and torch.equal(total, torch.ones(2, device=cuda))
