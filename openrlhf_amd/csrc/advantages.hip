@@ -49,15 +49,40 @@ __device__ __forceinline__ int64_t last_max_of_mask(const Rows& rows, const RowW
       best_i = t;
     }
   };
-  for_row_tokens(
-      rows, rw,
-      [&](int64_t i0) {
-        int64_t v[4];
-        mask_as_int4<MASK_DT>(mask, i0, v);
+  if (MASK_DT == ORLHF_MASK_U8) {
+    // byte masks: 16 tokens per lane and load between the row's first and last 16-byte boundary
+    // (a quarter of the steps of the four-token walk; this pass is latency-bound)
+    const uint8_t* bytes = (const uint8_t*)mask + start;
+    const int64_t len = rw.len - rw.lead;
+    int64_t head = (int64_t)((16 - ((uintptr_t)bytes & 15)) & 15);
+    head = head < len ? head : len;
+    const int64_t groups = (len - head) / 16;
+    int best_byte = -1;  // a lane meets its tokens in rising order: >= keeps the last maximum
+    for (int64_t t = threadIdx.x; t < head; t += kBlock)
+      if ((int)bytes[t] >= best_byte) best_byte = bytes[t], best_i = t;
+#pragma unroll 2
+    for (int64_t g = threadIdx.x; g < groups; g += kBlock) {
+      const u32x4 w = *(const u32x4*)(bytes + head + g * 16);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) see(v[k], i0 + k - start);
-      },
-      [&](int64_t i) { see(mask_as_int<MASK_DT>(mask, i), i - start); });
+      for (int k = 0; k < 16; ++k) {
+        const int v = (int)((w[k / 4] >> (8 * (k % 4))) & 0xffu);
+        if (v >= best_byte) best_byte = v, best_i = head + g * 16 + k;
+      }
+    }
+    for (int64_t t = head + groups * 16 + threadIdx.x; t < len; t += kBlock)
+      if ((int)bytes[t] >= best_byte) best_byte = bytes[t], best_i = t;
+    best_v = best_byte;  // -1 for a lane that saw nothing: below every byte
+  } else {
+    for_row_tokens(
+        rows, rw,
+        [&](int64_t i0) {
+          int64_t v[4];
+          mask_as_int4<MASK_DT>(mask, i0, v);
+#pragma unroll
+          for (int k = 0; k < 4; ++k) see(v[k], i0 + k - start);
+        },
+        [&](int64_t i) { see(mask_as_int<MASK_DT>(mask, i), i - start); });
+  }
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) {
     const int64_t ov = __shfl_xor(best_v, o, kWave);
