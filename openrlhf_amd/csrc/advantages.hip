@@ -420,19 +420,30 @@ __global__ __launch_bounds__(kBlock) void group_normalize_kernel(const float* __
 // ---------------------------------------------------------------- global masked whitening
 constexpr int kWhitenBlocks = 1024;
 
+// vec: x and mask allow 16-byte loads of four consecutive elements
 template <int MASK_DT>
 __global__ __launch_bounds__(kBlock) void whiten_partial_kernel(const float* __restrict__ x,
-                                                                const void* __restrict__ mask, int64_t n,
+                                                                const void* __restrict__ mask, int64_t n, int vec,
                                                                 double* __restrict__ partial) {
   __shared__ double lds[kWavesPerBlock];
   double sx = 0.0, sxx = 0.0, sm = 0.0;
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
-    const double m = (double)load_mask<MASK_DT>(mask, i);
-    const double v = (double)x[i];
+  auto add = [&](float xv, float mv) {
+    const double m = (double)mv, v = (double)xv;
     sx += v * m;
     sxx += v * v * m;
     sm += m;
+  };
+  const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
+  const int64_t groups = vec ? n / 4 : 0;
+#pragma unroll 4
+  for (int64_t g = first; g < groups; g += stride) {
+    const f32x4 v = *(const f32x4*)(x + g * 4);
+    float m[4];
+    load_mask4<MASK_DT>(mask, g * 4, m);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) add(v[k], m[k]);
   }
+  for (int64_t i = groups * 4 + first; i < n; i += stride) add(x[i], load_mask<MASK_DT>(mask, i));
   sx = block_sum(sx, lds);
   sxx = block_sum(sxx, lds);
   sm = block_sum(sm, lds);
@@ -472,15 +483,22 @@ __global__ __launch_bounds__(kBlock) void whiten_final_kernel(const double* __re
   }
 }
 
-__global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* __restrict__ x, int64_t n,
+__global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* __restrict__ x, int64_t n, int vec,
                                                               const float* __restrict__ mean_rstd,
                                                               float* __restrict__ out) {
   const float mean = mean_rstd[0], rstd = mean_rstd[1];
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
-    out[i] = (x[i] - mean) * rstd;
+  const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
+  const int64_t groups = vec ? n / 4 : 0;
+#pragma unroll 2
+  for (int64_t g = first; g < groups; g += stride) {
+    const f32x4 v = *(const f32x4*)(x + g * 4);
+    f32x4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) o[k] = (v[k] - mean) * rstd;
+    *(f32x4*)(out + g * 4) = o;
+  }
+  for (int64_t i = groups * 4 + first; i < n; i += stride) out[i] = (x[i] - mean) * rstd;
 }
-
-
 
 template <bool GAE, bool REWARD>
 static void launch_scan(int mask_dtype, Rows rows, const float* values, const float* rewards, const void* mask,
@@ -603,13 +621,15 @@ extern "C" int orlhf_masked_whiten(const float* x, const void* mask, int mask_dt
   float* mean_rstd = (float*)(partial + (int64_t)kWhitenBlocks * 3);
   const int nb = flat_grid(n, kWhitenBlocks);
   const dim3 grid(nb), block(kBlock);
-#define ORLHF_LAUNCH(M) hipLaunchKernelGGL(whiten_partial_kernel<M>, grid, block, 0, s, x, mask, n, partial)
+  const int vec = vector_loads_ok(mask, mask_dtype, {x}) ? 1 : 0;
+#define ORLHF_LAUNCH(M) hipLaunchKernelGGL(whiten_partial_kernel<M>, grid, block, 0, s, x, mask, n, vec, partial)
   ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
 #undef ORLHF_LAUNCH
   ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(partial)");
   hipLaunchKernelGGL(whiten_final_kernel, dim3(1), block, 0, s, partial, nb, std_norm, mean_rstd, stats);
   ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(final)");
-  hipLaunchKernelGGL(whiten_apply_kernel, dim3(flat_grid(n, 65536)), block, 0, s, x, n, mean_rstd, out);
+  hipLaunchKernelGGL(whiten_apply_kernel, dim3(flat_grid((n + 3) / 4, 65536)), block, 0, s, x, n,
+                     (aligned_to(x, 16) && aligned_to(out, 16)) ? 1 : 0, mean_rstd, out);
   ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(apply)");
   return ORLHF_OK;
 }

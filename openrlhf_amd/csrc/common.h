@@ -186,6 +186,32 @@ __device__ __forceinline__ RowWalk row_walk(const Rows& rows, int64_t b) {
   return w;
 }
 
+// A log-prob element of dtype DT (ORLHF_F32 / ORLHF_BF16 / ORLHF_F16) as fp32.
+template <int DT>
+__device__ __forceinline__ float load_lp(const void* p, int64_t i) {
+  if (DT == ORLHF_F32) return ((const float*)p)[i];
+  if (DT == ORLHF_BF16) return as_float((uint32_t)((const uint16_t*)p)[i] << 16);
+  return (float)((const _Float16*)p)[i];
+}
+
+// four consecutive elements from index i0 (a multiple of four from a 16-byte aligned base)
+template <int DT>
+__device__ __forceinline__ void load_lp4(const void* p, int64_t i0, float* v) {
+  if (DT == ORLHF_F32) {
+    const f32x4 x = *(const f32x4*)((const float*)p + i0);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = x[k];
+  } else {
+    const u32x2 w = *(const u32x2*)((const uint16_t*)p + i0);
+    if (DT == ORLHF_BF16) {
+      v[0] = bf16_lo(w[0]), v[1] = bf16_hi(w[0]), v[2] = bf16_lo(w[1]), v[3] = bf16_hi(w[1]);
+    } else {
+      const f16x2 a = __builtin_bit_cast(f16x2, w[0]), b = __builtin_bit_cast(f16x2, w[1]);
+      v[0] = (float)a[0], v[1] = (float)a[1], v[2] = (float)b[0], v[3] = (float)b[1];
+    }
+  }
+}
+
 // Walks one row with the whole workgroup: four(i0) for each lane's four consecutive tokens
 // (flat index i0, aligned for a 16-byte load) on every step that lies inside the row when vector
 // loads are on, one(i) per token (stride kBlock) on the steps at the row's ends or on all steps

@@ -6,31 +6,6 @@
 
 namespace orlhf {
 
-template <int DT>
-__device__ __forceinline__ float load_lp(const void* p, int64_t i) {
-  if (DT == ORLHF_F32) return ((const float*)p)[i];
-  if (DT == ORLHF_BF16) return as_float((uint32_t)((const uint16_t*)p)[i] << 16);
-  return (float)((const _Float16*)p)[i];
-}
-
-// four consecutive elements from index i0 (a multiple of four from a 16-byte aligned base)
-template <int DT>
-__device__ __forceinline__ void load_lp4(const void* p, int64_t i0, float* v) {
-  if (DT == ORLHF_F32) {
-    const f32x4 x = *(const f32x4*)((const float*)p + i0);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) v[k] = x[k];
-  } else {
-    const u32x2 w = *(const u32x2*)((const uint16_t*)p + i0);
-    if (DT == ORLHF_BF16) {
-      v[0] = bf16_lo(w[0]), v[1] = bf16_hi(w[0]), v[2] = bf16_lo(w[1]), v[3] = bf16_hi(w[1]);
-    } else {
-      const f16x2 a = __builtin_bit_cast(f16x2, w[0]), b = __builtin_bit_cast(f16x2, w[1]);
-      v[0] = (float)a[0], v[1] = (float)a[1], v[2] = (float)b[0], v[3] = (float)b[1];
-    }
-  }
-}
-
 __device__ __forceinline__ void block_sum3(double& a, double& b, double& c, double (*lds)[kWavesPerBlock]) {
 #pragma unroll
   for (int o = kWave / 2; o > 0; o >>= 1) {

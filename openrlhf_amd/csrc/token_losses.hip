@@ -477,20 +477,30 @@ __global__ __launch_bounds__(kBlock) void gspo_grad_kernel(Rows rows, const void
 }
 
 // ---------------------------------------------------------------- approximate KL (flat)
-template <int DT>
-__device__ __forceinline__ float load_as_float(const void* p, int64_t i) {
-  if (DT == ORLHF_F32) return ((const float*)p)[i];
-  if (DT == ORLHF_BF16) return __builtin_bit_cast(float, (uint32_t)((const uint16_t*)p)[i] << 16);
-  return (float)((const _Float16*)p)[i];
-}
-
+// vec: every array allows 16-byte (fp32) / 8-byte (half) loads of four consecutive elements
 template <int DT>
 __global__ __launch_bounds__(kBlock) void approx_kl_fwd_kernel(const void* __restrict__ lp,
                                                                const void* __restrict__ base, int64_t n, int est,
-                                                               float* __restrict__ out) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+                                                               int vec, float* __restrict__ out) {
+  const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
+  const int64_t groups = vec ? n / 4 : 0;
+#pragma unroll 2
+  for (int64_t g = first; g < groups; g += stride) {
+    float x[4], y[4];
+    load_lp4<DT>(lp, g * 4, x);
+    load_lp4<DT>(base, g * 4, y);
+    f32x4 o;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float v, dv;
+      kl_value(est, x[k] - y[k], v, dv);
+      o[k] = v;
+    }
+    *(f32x4*)(out + g * 4) = o;
+  }
+  for (int64_t i = groups * 4 + first; i < n; i += stride) {
     float v, dv;
-    kl_value(est, load_as_float<DT>(lp, i) - load_as_float<DT>(base, i), v, dv);
+    kl_value(est, load_lp<DT>(lp, i) - load_lp<DT>(base, i), v, dv);
     out[i] = v;
   }
 }
@@ -498,11 +508,30 @@ __global__ __launch_bounds__(kBlock) void approx_kl_fwd_kernel(const void* __res
 template <int DT>
 __global__ __launch_bounds__(kBlock) void approx_kl_bwd_kernel(const void* __restrict__ lp,
                                                                const void* __restrict__ base, int64_t n, int est,
-                                                               const float* __restrict__ g_out,
+                                                               int vec, const float* __restrict__ g_out,
                                                                float* __restrict__ g_lp, float* __restrict__ g_base) {
-  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+  const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
+  const int64_t groups = vec ? n / 4 : 0;
+#pragma unroll 2
+  for (int64_t g = first; g < groups; g += stride) {
+    float x[4], y[4];
+    load_lp4<DT>(lp, g * 4, x);
+    load_lp4<DT>(base, g * 4, y);
+    const f32x4 up = *(const f32x4*)(g_out + g * 4);
+    f32x4 o, neg;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      float v, dv;
+      kl_value(est, x[k] - y[k], v, dv);
+      o[k] = up[k] * dv;
+      neg[k] = -o[k];
+    }
+    if (g_lp != nullptr) *(f32x4*)(g_lp + g * 4) = o;
+    if (g_base != nullptr) *(f32x4*)(g_base + g * 4) = neg;
+  }
+  for (int64_t i = groups * 4 + first; i < n; i += stride) {
     float v, dv;
-    kl_value(est, load_as_float<DT>(lp, i) - load_as_float<DT>(base, i), v, dv);
+    kl_value(est, load_lp<DT>(lp, i) - load_lp<DT>(base, i), v, dv);
     const float g = g_out[i] * dv;
     if (g_lp != nullptr) g_lp[i] = g;
     if (g_base != nullptr) g_base[i] = -g;
@@ -602,11 +631,12 @@ extern "C" int orlhf_approx_kl_fwd(const void* log_probs, const void* log_probs_
   if (n == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(log_probs && log_probs_base && out, "approx_kl_fwd: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(flat_grid(n)), block(kBlock);
+  const dim3 grid(flat_grid((n + 3) / 4)), block(kBlock);
+  const int vec = vector_loads_ok(nullptr, ORLHF_MASK_NONE, {log_probs, log_probs_base, out}) ? 1 : 0;
   switch (dtype) {
-    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
-    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
-    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
+    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, out); break;
+    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, out); break;
+    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, out); break;
     default: return fail(ORLHF_ERR_INVALID_ARG, "approx_kl_fwd: unknown dtype %d", dtype);
   }
   ORLHF_CHECK_LAUNCH("orlhf_approx_kl_fwd");
@@ -621,11 +651,12 @@ extern "C" int orlhf_approx_kl_bwd(const void* log_probs, const void* log_probs_
   if (n == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(log_probs && log_probs_base && g_out && (g_lp || g_base), "approx_kl_bwd: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
-  const dim3 grid(flat_grid(n)), block(kBlock);
+  const dim3 grid(flat_grid((n + 3) / 4)), block(kBlock);
+  const int vec = vector_loads_ok(nullptr, ORLHF_MASK_NONE, {log_probs, log_probs_base, g_out, g_lp, g_base}) ? 1 : 0;
   switch (dtype) {
-    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
-    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
-    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
+    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, g_out, g_lp, g_base); break;
+    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, g_out, g_lp, g_base); break;
+    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, g_out, g_lp, g_base); break;
     default: return fail(ORLHF_ERR_INVALID_ARG, "approx_kl_bwd: unknown dtype %d", dtype);
   }
   ORLHF_CHECK_LAUNCH("orlhf_approx_kl_bwd");

@@ -228,8 +228,12 @@ def whiten_advantages(
     biased variance over the unmasked tokens of every block, rstd = rsqrt(max(var, 1e-8)) (1 when
     no_std_norm); (adv - mean) * rstd is applied to every column, masked or not."""
     dev, home = _device_for(*advantages)
-    flat = torch.cat([_on_gpu(a, dev).flatten() for a in advantages]).float()
-    mask = torch.cat([_on_gpu(m, dev).flatten() for m in action_masks])
+    if len(advantages) == 1:  # one block: no gathering copy
+        flat = _f32(_on_gpu(advantages[0], dev)).reshape(-1)
+        mask = _on_gpu(action_masks[0], dev).expand_as(advantages[0]).reshape(-1)
+    else:
+        flat = torch.cat([_on_gpu(a, dev).flatten() for a in advantages]).float()
+        mask = torch.cat([_on_gpu(m, dev).flatten() for m in action_masks])
     mkeep, mptr, mcode = _lib.mask_arg(mask)
     n = flat.numel()
     ws = torch.empty(_lib.load().orlhf_whiten_workspace_bytes(n), dtype=torch.uint8, device=dev)

@@ -136,3 +136,32 @@ def test_per_token_arrays_off_the_16_byte_boundary(cuda, off):
         assert torch.allclose(out, ref, rtol=1e-6, atol=1e-7)
         packed_ref = PackedSteps.from_padded(dict(g=gref), mask)["g"]
         assert torch.allclose(gout, packed_ref, rtol=1e-5, atol=1e-9)
+
+
+@pytest.mark.parametrize("off", [1, 3])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_flat_kernels_off_the_16_byte_boundary(cuda, off, dtype):
+    """The flat kernels (approximate KL forward / backward, global whitening) on storage that
+    does not start on a 16-byte boundary and with a length that is not a multiple of four: the
+    element-wise path gives the same bits as the vector path on aligned storage."""
+    from openrlhf_amd.models.utils import compute_approx_kl
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import whiten_advantages
+
+    g = torch.Generator().manual_seed(40 + off)
+    n = 7 * 1031 + 2
+    lp = (-torch.rand(n, generator=g) * 2).to(dtype).to(cuda)
+    base = (lp.float() + torch.randn(n, generator=g).to(cuda) * 0.3).to(dtype)
+    up = torch.randn(n, generator=g).to(cuda)
+    for est in ("k1", "k2", "k3"):
+        x = lp.clone().requires_grad_()
+        ref = compute_approx_kl(x, base, est)
+        ref.backward(up)
+        y = _at_offset(lp, off).requires_grad_()
+        out = compute_approx_kl(y, _at_offset(base, off), est)
+        out.backward(_at_offset(up, off))
+        assert torch.equal(out, ref) and torch.equal(y.grad, x.grad)
+    adv = lp.float().view(7, -1)[:, :1031].contiguous()
+    mask = (torch.rand(7, 1031, generator=g) > 0.4).to(cuda)
+    ref = whiten_advantages([adv], [mask])[0]
+    out = whiten_advantages([_at_offset(adv, off)], [_at_offset(mask, off)])[0]
+    assert torch.allclose(out, ref, rtol=1e-6, atol=1e-7)
