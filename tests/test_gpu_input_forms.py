@@ -160,7 +160,7 @@ def test_flat_kernels_off_the_16_byte_boundary(cuda, off, dtype):
         out = compute_approx_kl(y, _at_offset(base, off), est)
         out.backward(_at_offset(up, off))
         assert torch.equal(out, ref) and torch.equal(y.grad, x.grad)
-    adv = lp.float().view(7, -1)[:, :1031].contiguous()
+    adv = lp.float()[:7 * 1031].view(7, 1031).contiguous()
     mask = (torch.rand(7, 1031, generator=g) > 0.4).to(cuda)
     ref = whiten_advantages([adv], [mask])[0]
     out = whiten_advantages([_at_offset(adv, off)], [_at_offset(mask, off)])[0]
