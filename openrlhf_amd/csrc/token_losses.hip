@@ -253,9 +253,11 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
 // Quantity 0 is the loss numerator, quantity 1 the mask weight; quantities 2.. are numerators of
 // plain masked means. out[0] = post_scale * aggregate(q0); out[k-1] = sum(qk)/sum(q1), k >= 2.
 // row_coef[b] = post_scale * d(aggregate)/d(row b's masked token sum).
+constexpr int kFinalRows = 8;  // rows per lane whose loads the finaliser issues together
+
 template <int NQ>
-__global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int n_chunks,
-                                                            const double* __restrict__ partial, int mode,
+__global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows,
+                                                            const double* __restrict__ row_total, int mode,
                                                             NormArg norm, float post_scale, int n_out,
                                                             float* __restrict__ out,
                                                             float* __restrict__ row_coef) {
@@ -264,27 +266,35 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
 #pragma unroll
   for (int i = 0; i < NQ; ++i) tot[i] = 0.0;
   double seq_sum = 0.0, seq_cnt = 0.0;
-  for (int64_t b = threadIdx.x; b < n_rows; b += kBlock) {
-    double rq[NQ];
+  // One workgroup walks all rows: the loads of kFinalRows rows per lane are issued together, or
+  // the walk is a chain of load latencies (18 us for 4096 rows with one row at a time).
+  for (int64_t b0 = threadIdx.x; b0 < n_rows; b0 += (int64_t)kFinalRows * kBlock) {
+    double batch[kFinalRows][NQ];
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) rq[i] = 0.0;
-    for (int c = 0; c < n_chunks; ++c) {
+    for (int u = 0; u < kFinalRows; ++u) {
+      const int64_t b = b0 + (int64_t)u * kBlock;
 #pragma unroll
-      for (int i = 0; i < NQ; ++i) rq[i] += partial[(b * n_chunks + c) * NQ + i];
+      for (int i = 0; i < NQ; ++i) batch[u][i] = b < n_rows ? row_total[b * NQ + i] : 0.0;
     }
 #pragma unroll
-    for (int i = 0; i < NQ; ++i) tot[i] += rq[i];
-    if (mode == ORLHF_AGG_SEQ_MEAN || mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM || mode == kAggCounts) {
-      if (rq[1] > 0.0) {
-        seq_sum += mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM ? rq[0] : rq[0] / (rq[1] + 1e-8);
-        seq_cnt += 1.0;
-      } else if (rq[0] != rq[0]) {
-        seq_sum += rq[0];  // NaN * 0 stays NaN in the reference
+    for (int u = 0; u < kFinalRows; ++u) {
+      const int64_t b = b0 + (int64_t)u * kBlock;
+      if (b >= n_rows) break;
+      const double* rq = batch[u];
+#pragma unroll
+      for (int i = 0; i < NQ; ++i) tot[i] += rq[i];
+      if (mode == ORLHF_AGG_SEQ_MEAN || mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM || mode == kAggCounts) {
+        if (rq[1] > 0.0) {
+          seq_sum += mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM ? rq[0] : rq[0] / (rq[1] + 1e-8);
+          seq_cnt += 1.0;
+        } else if (rq[0] != rq[0]) {
+          seq_sum += rq[0];  // NaN * 0 stays NaN in the reference
+        }
+      } else if (mode == ORLHF_AGG_ROW_MEAN) {
+        out[b] = (float)(rq[0] / rq[1]);
       }
-    } else if (mode == ORLHF_AGG_ROW_MEAN) {
-      out[b] = (float)(rq[0] / rq[1]);
+      if (row_coef != nullptr) row_coef[b] = (float)rq[1];  // finished below
     }
-    if (row_coef != nullptr) row_coef[b] = (float)rq[1];  // finished below
   }
   if (mode == ORLHF_AGG_ROW_MEAN) {
     if (row_coef != nullptr) {
@@ -345,16 +355,27 @@ __global__ __launch_bounds__(kBlock) void rows_final_kernel(int64_t n_rows, int 
     for (int i = 2; i < NQ && i - 1 < n_out; ++i) out[i - 1] = (float)(tot[i] / tot[1]);
   }
   if (row_coef != nullptr) {
-    for (int64_t b = threadIdx.x; b < n_rows; b += kBlock) {
-      const double cnt = (double)row_coef[b];
-      double c;
-      if (mode == ORLHF_AGG_TOKEN_MEAN)
-        c = scale;
-      else if (mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM)
-        c = cnt > 0.0 ? scale : 0.0;
-      else
-        c = cnt > 0.0 ? scale / (cnt + 1e-8) : 0.0;
-      row_coef[b] = (float)((double)post_scale * c);
+    for (int64_t b0 = threadIdx.x; b0 < n_rows; b0 += (int64_t)kFinalRows * kBlock) {
+      float cnt_f[kFinalRows];
+#pragma unroll
+      for (int u = 0; u < kFinalRows; ++u) {
+        const int64_t b = b0 + (int64_t)u * kBlock;
+        cnt_f[u] = b < n_rows ? row_coef[b] : 0.0f;
+      }
+#pragma unroll
+      for (int u = 0; u < kFinalRows; ++u) {
+        const int64_t b = b0 + (int64_t)u * kBlock;
+        if (b >= n_rows) break;
+        const double cnt = (double)cnt_f[u];
+        double c;
+        if (mode == ORLHF_AGG_TOKEN_MEAN)
+          c = scale;
+        else if (mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM)
+          c = cnt > 0.0 ? scale : 0.0;
+        else
+          c = cnt > 0.0 ? scale / (cnt + 1e-8) : 0.0;
+        row_coef[b] = (float)((double)post_scale * c);
+      }
     }
   }
 }
@@ -569,17 +590,15 @@ static void launch_grad(int mask_dt, Rows rows, const void* mask, const Tok& tok
 template <int NQ>
 static void launch_final(int64_t n_rows, int n_chunks, double* partial, int mode, const NormArg& norm,
                          float post_scale, int n_out, float* out, float* row_coef, hipStream_t s) {
-  const double* src = partial;
-  int chunks = n_chunks;
+  const double* src = partial;  // one chunk per row: the partials are the row totals
   if (n_chunks > 1 && n_rows > 0) {
     double* row_total = partial + n_rows * (int64_t)n_chunks * NQ;
     hipLaunchKernelGGL(rows_fold_kernel<NQ>, dim3(flat_grid(n_rows, 4096)), dim3(kBlock), 0, s, n_rows, n_chunks,
                        partial, row_total);
     src = row_total;
-    chunks = 1;
   }
-  hipLaunchKernelGGL(rows_final_kernel<NQ>, dim3(1), dim3(kBlock), 0, s, n_rows, chunks, src, mode, norm, post_scale,
-                     n_out, out, row_coef);
+  hipLaunchKernelGGL(rows_final_kernel<NQ>, dim3(1), dim3(kBlock), 0, s, n_rows, src, mode, norm, post_scale, n_out,
+                     out, row_coef);
 }
 
 static PolicyTok policy_tok(const float* lp, const float* old, const float* adv, const float* rollout,
