@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 10
+#define ORLHF_ABI_VERSION 11
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -362,6 +362,18 @@ int orlhf_group_normalize(const float* rewards, const int64_t* indices, int64_t 
 int64_t orlhf_whiten_workspace_bytes(int64_t n);
 int orlhf_masked_whiten(const float* x, const void* mask, int mask_dtype, int64_t n, int std_norm,
                         void* workspace, float* out, float* stats, orlhf_stream_t stream);
+
+/*
+ * The same whitening over a list of blocks (one per experience, as the reference holds them in
+ * experience_maker.py:314-328) without gathering them into one array first: xs / masks / outs
+ * are HOST arrays of n_blocks device pointers, ns the element counts; all masks share
+ * mask_dtype. Statistics are taken over all blocks together. outs[i] may alias xs[i].
+ * workspace: orlhf_whiten_multi_workspace_bytes(ns, n_blocks).
+ */
+int64_t orlhf_whiten_multi_workspace_bytes(const int64_t* ns, int n_blocks);
+int orlhf_masked_whiten_multi(const float* const* xs, const void* const* masks, int mask_dtype,
+                              const int64_t* ns, int n_blocks, int std_norm, void* workspace,
+                              float* const* outs, float* stats, orlhf_stream_t stream);
 
 /*
  * The KL block of experience making (openrlhf/trainer/ppo_utils/experience_maker.py:202-216) in

@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 
 class Norm(Structure):
@@ -95,6 +95,8 @@ SIGNATURES = {
     "orlhf_group_normalize": (c_int, [P, P, I64, I64, c_int, P, P, P, P]),
     "orlhf_whiten_workspace_bytes": (I64, [I64]),
     "orlhf_masked_whiten": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
+    "orlhf_whiten_multi_workspace_bytes": (I64, [P, c_int]),
+    "orlhf_masked_whiten_multi": (c_int, [P, P, c_int, P, c_int, c_int, P, P, P, P]),
     "orlhf_kl_rows": (c_int, [P, P, c_int, P, c_int, I64, I64, P, c_int, c_int, P, P, P, P]),
     "orlhf_masked_normalize_rows": (c_int, [P, P, c_int, I64, I64, P, c_float, P, P]),
     "orlhf_row_extents": (c_int, [P, c_int, I64, I64, P, P, P, P]),

@@ -460,10 +460,21 @@ __global__ __launch_bounds__(kBlock) void whiten_final_kernel(const double* __re
                                                               float* __restrict__ stats_out) {
   __shared__ double lds[kWavesPerBlock];
   double sx = 0.0, sxx = 0.0, sm = 0.0;
-  for (int i = threadIdx.x; i < n_partial; i += kBlock) {
-    sx += partial[i * 3 + 0];
-    sxx += partial[i * 3 + 1];
-    sm += partial[i * 3 + 2];
+  constexpr int kBatch = 8;  // entries per lane loaded together: one workgroup, latency-bound
+  for (int i0 = threadIdx.x; i0 < n_partial; i0 += kBatch * kBlock) {
+    double v[kBatch][3];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int i = i0 + u * kBlock;
+#pragma unroll
+      for (int q = 0; q < 3; ++q) v[u][q] = i < n_partial ? partial[(int64_t)i * 3 + q] : 0.0;
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      sx += v[u][0];
+      sxx += v[u][1];
+      sm += v[u][2];
+    }
   }
   sx = block_sum(sx, lds);
   sxx = block_sum(sxx, lds);
@@ -499,6 +510,104 @@ __global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* __res
   }
   for (int64_t i = groups * 4 + first; i < n; i += stride) out[i] = (x[i] - mean) * rstd;
 }
+
+// ---- whitening over a list of blocks (one per experience) without gathering them first.
+// A launch carries up to kSegs blocks in its arguments; a workgroup finds its block from the
+// table of first workgroup indices and works on kWhitenSpan consecutive elements of it.
+constexpr int kSegs = 16;
+constexpr int kWhitenSpan = kBlock * 4 * 8;
+
+struct WhitenSegs {
+  const float* x[kSegs];
+  const void* mask[kSegs];  // statistics pass
+  float* out[kSegs];        // apply pass
+  int64_t n[kSegs];
+  int first_wg[kSegs + 1];
+  int n_segs;
+};
+
+// Calls four(i0) / one(i) over the span of this workgroup inside its block; vec: per block.
+template <typename F4, typename F1>
+__device__ __forceinline__ void for_span(int64_t lo, int64_t hi, bool vec, F4&& four, F1&& one) {
+#pragma unroll 2
+  for (int64_t s0 = lo; s0 < hi; s0 += kBlock * 4) {
+    if (vec && s0 + kBlock * 4 <= hi) {
+      four(s0 + (int64_t)threadIdx.x * 4);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int64_t i = s0 + threadIdx.x + k * kBlock;
+        if (i < hi) one(i);
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ int segment_of(const WhitenSegs& segs, int wg) {
+  int s = 0;
+  while (s + 1 < segs.n_segs && wg >= segs.first_wg[s + 1]) ++s;
+  return s;
+}
+
+template <int MASK_DT>
+__global__ __launch_bounds__(kBlock) void whiten_partial_multi_kernel(WhitenSegs segs, double* __restrict__ partial) {
+  __shared__ double lds[kWavesPerBlock];
+  const int s = segment_of(segs, blockIdx.x);
+  const float* x = segs.x[s];
+  const void* mask = segs.mask[s];
+  const int64_t lo = (int64_t)(blockIdx.x - segs.first_wg[s]) * kWhitenSpan;
+  const int64_t hi = lo + kWhitenSpan < segs.n[s] ? lo + kWhitenSpan : segs.n[s];
+  const bool vec = (((uintptr_t)x & 15) == 0) &&
+                   (MASK_DT == ORLHF_MASK_NONE || ((uintptr_t)mask & (MASK_DT == ORLHF_MASK_U8 ? 3 : 15)) == 0);
+  double sx = 0.0, sxx = 0.0, sm = 0.0;
+  auto add = [&](float xv, float mv) {
+    const double m = (double)mv, v = (double)xv;
+    sx += v * m;
+    sxx += v * v * m;
+    sm += m;
+  };
+  for_span(
+      lo, hi, vec,
+      [&](int64_t i0) {
+        const f32x4 v = *(const f32x4*)(x + i0);
+        float m[4];
+        load_mask4<MASK_DT>(mask, i0, m);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) add(v[k], m[k]);
+      },
+      [&](int64_t i) { add(x[i], load_mask<MASK_DT>(mask, i)); });
+  sx = block_sum(sx, lds);
+  sxx = block_sum(sxx, lds);
+  sm = block_sum(sm, lds);
+  if (threadIdx.x == 0) {
+    partial[blockIdx.x * 3 + 0] = sx;
+    partial[blockIdx.x * 3 + 1] = sxx;
+    partial[blockIdx.x * 3 + 2] = sm;
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void whiten_apply_multi_kernel(WhitenSegs segs,
+                                                                    const float* __restrict__ mean_rstd) {
+  const int s = segment_of(segs, blockIdx.x);
+  const float* x = segs.x[s];
+  float* out = segs.out[s];
+  const int64_t lo = (int64_t)(blockIdx.x - segs.first_wg[s]) * kWhitenSpan;
+  const int64_t hi = lo + kWhitenSpan < segs.n[s] ? lo + kWhitenSpan : segs.n[s];
+  const bool vec = ((((uintptr_t)x) | ((uintptr_t)out)) & 15) == 0;
+  const float mean = mean_rstd[0], rstd = mean_rstd[1];
+  for_span(
+      lo, hi, vec,
+      [&](int64_t i0) {
+        const f32x4 v = *(const f32x4*)(x + i0);
+        f32x4 o;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) o[k] = (v[k] - mean) * rstd;
+        *(f32x4*)(out + i0) = o;
+      },
+      [&](int64_t i) { out[i] = (x[i] - mean) * rstd; });
+}
+
+static inline int64_t span_wgs(int64_t n) { return (n + kWhitenSpan - 1) / kWhitenSpan; }
 
 template <bool GAE, bool REWARD>
 static void launch_scan(int mask_dtype, Rows rows, const float* values, const float* rewards, const void* mask,
@@ -607,6 +716,74 @@ extern "C" int orlhf_group_normalize(const float* rewards, const int64_t* indice
 
 extern "C" int64_t orlhf_whiten_workspace_bytes(int64_t) {
   return (int64_t)kWhitenBlocks * 3 * (int64_t)sizeof(double) + 64;
+}
+
+extern "C" int64_t orlhf_whiten_multi_workspace_bytes(const int64_t* ns, int n_blocks) {
+  int64_t wgs = 0;
+  for (int i = 0; ns != nullptr && i < n_blocks; ++i) wgs += ns[i] > 0 ? span_wgs(ns[i]) : 0;
+  return (wgs > 0 ? wgs : 1) * 3 * (int64_t)sizeof(double) + 64;
+}
+
+extern "C" int orlhf_masked_whiten_multi(const float* const* xs, const void* const* masks, int mask_dtype,
+                                         const int64_t* ns, int n_blocks, int std_norm, void* workspace,
+                                         float* const* outs, float* stats, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_blocks >= 0, "masked_whiten_multi: n_blocks=%d", n_blocks);
+  ORLHF_CHECK_ARG(valid_mask_dtype(mask_dtype), "masked_whiten_multi: unknown mask dtype %d", mask_dtype);
+  if (n_blocks == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(xs && ns && outs && workspace, "masked_whiten_multi: NULL pointer");
+  ORLHF_CHECK_ARG(mask_dtype == ORLHF_MASK_NONE || masks != nullptr, "masked_whiten_multi: masks is NULL");
+  int64_t total_wgs = 0;
+  for (int i = 0; i < n_blocks; ++i) {
+    ORLHF_CHECK_ARG(ns[i] >= 0, "masked_whiten_multi: ns[%d]=%lld", i, (long long)ns[i]);
+    if (ns[i] == 0) continue;
+    ORLHF_CHECK_ARG(xs[i] && outs[i], "masked_whiten_multi: block %d has a NULL pointer", i);
+    ORLHF_CHECK_ARG(mask_dtype == ORLHF_MASK_NONE || masks[i] != nullptr, "masked_whiten_multi: mask %d is NULL", i);
+    total_wgs += span_wgs(ns[i]);
+  }
+  if (total_wgs == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(total_wgs < (int64_t)1 << 30, "masked_whiten_multi: too many elements");
+  hipStream_t s = (hipStream_t)stream;
+  double* partial = (double*)workspace;
+  float* mean_rstd = (float*)(partial + total_wgs * 3);
+  const dim3 block(kBlock);
+  // pass 0: statistics of every block into consecutive partial entries; pass 1: apply
+  for (int pass = 0; pass < 2; ++pass) {
+    int64_t done_wgs = 0;
+    int i = 0;
+    while (i < n_blocks) {
+      WhitenSegs segs;
+      segs.n_segs = 0;
+      int wgs = 0;
+      for (; i < n_blocks && segs.n_segs < kSegs; ++i) {
+        if (ns[i] == 0) continue;
+        const int k = segs.n_segs++;
+        segs.x[k] = xs[i];
+        segs.mask[k] = mask_dtype == ORLHF_MASK_NONE ? nullptr : masks[i];
+        segs.out[k] = outs[i];
+        segs.n[k] = ns[i];
+        segs.first_wg[k] = wgs;
+        wgs += (int)span_wgs(ns[i]);
+      }
+      if (segs.n_segs == 0) break;
+      segs.first_wg[segs.n_segs] = wgs;
+      if (pass == 0) {
+        double* dst = partial + done_wgs * 3;
+#define ORLHF_LAUNCH(M) hipLaunchKernelGGL(whiten_partial_multi_kernel<M>, dim3(wgs), block, 0, s, segs, dst)
+        ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
+#undef ORLHF_LAUNCH
+        ORLHF_CHECK_LAUNCH("orlhf_masked_whiten_multi(partial)");
+      } else {
+        hipLaunchKernelGGL(whiten_apply_multi_kernel, dim3(wgs), block, 0, s, segs, mean_rstd);
+        ORLHF_CHECK_LAUNCH("orlhf_masked_whiten_multi(apply)");
+      }
+      done_wgs += wgs;
+    }
+    if (pass == 0) {
+      hipLaunchKernelGGL(whiten_final_kernel, dim3(1), block, 0, s, partial, (int)total_wgs, std_norm, mean_rstd, stats);
+      ORLHF_CHECK_LAUNCH("orlhf_masked_whiten_multi(final)");
+    }
+  }
+  return ORLHF_OK;
 }
 
 extern "C" int orlhf_masked_whiten(const float* x, const void* mask, int mask_dtype, int64_t n, int std_norm,

@@ -17,6 +17,7 @@ Only the numerics are mirrored. Length penalties (apply_length_penalties) and th
 half of RemoteExperienceMaker are outside this package; ``compute_advantages_and_returns`` takes a
 ``length_penalty_fn`` hook for the former.
 """
+import ctypes
 import itertools
 from typing import List, Optional, Tuple
 
@@ -34,6 +35,9 @@ _GROUP_CODES = {
     "dr_grpo": _lib.GROUP_BASELINE,
     "group_norm": _lib.GROUP_NORM,
 }
+# whiten_advantages: lists longer than this are gathered into one array first (measured: 512 blocks
+# of 131 072 tokens 5.6 ms block by block against 0.8 ms gathered; 8 blocks 0.18 ms against 0.34 ms)
+_WHITEN_GATHER_ABOVE = 32
 _RETURN_ESTIMATORS = ("reinforce", "rloo", "reinforce_baseline", "group_norm", "dr_grpo")
 
 
@@ -228,21 +232,31 @@ def whiten_advantages(
     biased variance over the unmasked tokens of every block, rstd = rsqrt(max(var, 1e-8)) (1 when
     no_std_norm); (adv - mean) * rstd is applied to every column, masked or not."""
     dev, home = _device_for(*advantages)
-    if len(advantages) == 1:  # one block: no gathering copy
-        flat = _f32(_on_gpu(advantages[0], dev)).reshape(-1)
-        mask = _on_gpu(action_masks[0], dev).expand_as(advantages[0]).reshape(-1)
-    else:
-        flat = torch.cat([_on_gpu(a, dev).flatten() for a in advantages]).float()
-        mask = torch.cat([_on_gpu(m, dev).flatten() for m in action_masks])
-    mkeep, mptr, mcode = _lib.mask_arg(mask)
-    n = flat.numel()
-    ws = torch.empty(_lib.load().orlhf_whiten_workspace_bytes(n), dtype=torch.uint8, device=dev)
-    out = torch.empty_like(flat)
+    if len(advantages) > _WHITEN_GATHER_ABOVE:
+        # many small blocks: per-block host work would outweigh the copy that gathering costs
+        flat = torch.cat([_on_gpu(a, dev).reshape(-1) for a in advantages]).float()
+        mask = torch.cat([_on_gpu(m if m.shape == a.shape else m.expand_as(a), dev).reshape(-1)
+                          for m, a in zip(action_masks, advantages)])
+        pieces = whiten_advantages([flat], [mask], no_std_norm)[0].split([a.numel() for a in advantages])
+        out = [p.view(a.shape) for p, a in zip(pieces, advantages)]
+        return out if home == dev else [o.to(home) for o in out]
+    xs = [_f32(_on_gpu(a, dev)) for a in advantages]
+    masks = [_lib.mask_arg(_on_gpu(m, dev).expand_as(a)) for m, a in zip(action_masks, advantages)]
+    codes = {code for _, _, code in masks}
+    if len(codes) != 1:  # mixed mask dtypes: whiten with float masks
+        masks = [_lib.mask_arg(_on_gpu(m, dev).expand_as(a).float()) for m, a in zip(action_masks, advantages)]
+    mcode = masks[0][2]
+    k = len(xs)
+    ns = (ctypes.c_int64 * k)(*[x.numel() for x in xs])
+    outs = [torch.empty_like(x) for x in xs]
+    ws = torch.empty(_lib.load().orlhf_whiten_multi_workspace_bytes(ns, k), dtype=torch.uint8, device=dev)
+    x_ptrs = (ctypes.c_void_p * k)(*[x.data_ptr() for x in xs])
+    m_ptrs = (ctypes.c_void_p * k)(*[mp for _, mp, _ in masks])
+    o_ptrs = (ctypes.c_void_p * k)(*[o.data_ptr() for o in outs])
     with torch.cuda.device(dev):
-        call("orlhf_masked_whiten", ptr(flat), mptr, mcode, n, 0 if no_std_norm else 1, ptr(ws), ptr(out), None,
-             stream_of(dev))
-    pieces = out.split([a.numel() for a in advantages])
-    return [p.view(a.shape).to(home) for p, a in zip(pieces, advantages)]
+        call("orlhf_masked_whiten_multi", x_ptrs, m_ptrs, mcode, ns, k, 0 if no_std_norm else 1, ptr(ws), o_ptrs,
+             None, stream_of(dev))
+    return [o.view(a.shape).to(home) for o, a in zip(outs, advantages)]
 
 
 @torch.no_grad()

@@ -217,6 +217,48 @@ def test_whitening(cuda, no_std_norm):
     assert out[0].cpu()[masks[0] == 0].abs().min().item() > 0.0
 
 
+def test_whitening_over_many_blocks(cuda):
+    """More blocks than one launch carries, empty blocks among them, blocks longer than one
+    workgroup's span, odd storage offsets and mask dtypes that differ between blocks: the
+    statistics are taken over all of them together (experience_maker.py:314-328)."""
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import whiten_advantages
+
+    g = torch.Generator().manual_seed(12)
+    shapes = [(3, 41), (0, 7), (2, 9001), (1, 1)] * 9 + [(5, 8192)]
+    advs = [torch.randn(s, generator=g) * 2 - 0.7 for s in shapes]
+    masks = [(torch.rand(s, generator=g) > 0.3) for s in shapes]
+    ref, mean, rstd = oa.whiten_advantages([a.double() for a in advs], [m.double() for m in masks])
+
+    def on_gpu(t, i):  # every third block off the 16-byte boundary
+        t = t.to(cuda)
+        if i % 3 == 0 or t.numel() == 0:
+            return t
+        buf = torch.empty(t.numel() + 1, dtype=t.dtype, device=cuda)
+        view = buf[1:].view(t.shape)
+        view.copy_(t)
+        return view
+
+    out = whiten_advantages([on_gpu(a, i) for i, a in enumerate(advs)], [on_gpu(m, i) for i, m in enumerate(masks)])
+    for o, r, s_ in zip(out, ref, shapes):
+        assert tuple(o.shape) == s_
+        if o.numel():
+            _rel_close(o, r)
+    # 30 blocks go block by block in two launches, the 37 above are gathered first
+    k = 30
+    ref30, _, _ = oa.whiten_advantages([a.double() for a in advs[:k]], [m.double() for m in masks[:k]])
+    out30 = whiten_advantages([on_gpu(a, i) for i, a in enumerate(advs[:k])],
+                              [on_gpu(m, i) for i, m in enumerate(masks[:k])])
+    for o, r in zip(out30, ref30):
+        if o.numel():
+            _rel_close(o, r)
+    advs, masks, ref = advs[:k], masks[:k], ref30
+    mixed = whiten_advantages([a.to(cuda) for a in advs],
+                              [m.to(cuda).long() if i % 2 else m.to(cuda) for i, m in enumerate(masks)])
+    for o, r in zip(mixed, ref):
+        if o.numel():
+            _rel_close(o, r)
+
+
 # ------------------------------------------------------------------ config 3 shape, end to end
 @pytest.mark.parametrize("estimator", ["gae", "reinforce_baseline", "group_norm", "rloo"])
 def test_compute_advantages_and_returns_pipeline(cuda, estimator):
