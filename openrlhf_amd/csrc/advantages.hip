@@ -494,9 +494,9 @@ __global__ __launch_bounds__(kBlock) void whiten_final_kernel(const double* __re
   }
 }
 
-__global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* __restrict__ x, int64_t n, int vec,
-                                                              const float* __restrict__ mean_rstd,
-                                                              float* __restrict__ out) {
+// out may be x itself (each lane reads its elements before it writes them): no __restrict__ on them
+__global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* x, int64_t n, int vec,
+                                                              const float* __restrict__ mean_rstd, float* out) {
   const float mean = mean_rstd[0], rstd = mean_rstd[1];
   const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
   const int64_t groups = vec ? n / 4 : 0;

@@ -83,9 +83,9 @@ __global__ __launch_bounds__(kBlock) void kl_rows_kernel(const void* __restrict_
 // out = (x - mean) * m * rsqrt(max(var, eps)), mean = sum(x*m)/max(sum(m), 1),
 // var = sum(((x - mean)*m)^2)/max(sum(m), 1)
 template <int MASK_DT>
-__global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const float* __restrict__ x,
+__global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const float* x,  // out may be x
                                                                        const void* __restrict__ mask, Rows rows,
-                                                                       float eps, float* __restrict__ out) {
+                                                                       float eps, float* out) {
   __shared__ double lds[3][kWavesPerBlock];
   const int slot_b = slot_bits(rows.n_rows);
   for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
