@@ -25,8 +25,7 @@ __device__ __forceinline__ int64_t mask_as_int(const void* mask, int64_t i) {
 template <int MASK_DT>
 __device__ __forceinline__ void mask_as_int4(const void* mask, int64_t i0, int64_t* v) {
   if (MASK_DT == ORLHF_MASK_I64) {
-    typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
-    const i64x2 lo = *(const i64x2*)((const int64_t*)mask + i0), hi = *(const i64x2*)((const int64_t*)mask + i0 + 2);
+    const i64x2e lo = *(const i64x2e*)((const int64_t*)mask + i0), hi = *(const i64x2e*)((const int64_t*)mask + i0 + 2);
     v[0] = lo[0], v[1] = lo[1], v[2] = hi[0], v[3] = hi[1];
   } else {  // bytes are exact as floats; a float mask truncates like .long()
     float m[4];
@@ -74,7 +73,7 @@ __device__ __forceinline__ int64_t last_max_of_mask(const Rows& rows, const RowW
     best_v = best_byte;  // -1 for a lane that saw nothing: below every byte
   } else {
     for_row_tokens(
-        rows, rw,
+        rw,
         [&](int64_t i0) {
           int64_t v[4];
           mask_as_int4<MASK_DT>(mask, i0, v);
@@ -139,13 +138,13 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
     const int64_t best_i = last_max_of_mask<MASK_DT>(rows, rw, start, mask, lds_val, lds_idx);
     const float rb = clipped_reward(r[b], has_clip, clip_lo, clip_hi);
     for_row_tokens(
-        rows, rw,
+        rw,
         [&](int64_t i0) {
-          const f32x4 k4 = *(const f32x4*)(kl + i0);
+          const f32x4 k4 = *(const f32x4e*)(kl + i0);
           f32x4 o;
 #pragma unroll
           for (int k = 0; k < 4; ++k) o[k] = ((i0 + k - start == best_i) ? rb : 0.0f) + neg_coef * k4[k];
-          *(f32x4*)(reward + i0) = o;
+          *(f32x4e*)(reward + i0) = o;
         },
         [&](int64_t i) { reward[i] = ((i - start == best_i) ? rb : 0.0f) + neg_coef * kl[i]; });
     if (threadIdx.x == 0 && eos_index != nullptr) eos_index[b] = best_i;
@@ -183,7 +182,7 @@ struct RowReward {
   double sum;
 };
 
-// `whole`: the tile lies inside the row and every array allows 16-byte loads. Must be called by
+// `whole`: the tile lies inside the row. Must be called by
 // all lanes of the workgroup (it exchanges the following value across lanes).
 template <int MASK_DT, bool GAE, bool REWARD>
 __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t tile0, bool whole,
@@ -202,9 +201,9 @@ __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t ti
   if (whole) {
     float m[kScanItems];
     load_mask4<MASK_DT>(mask, rw.base + p0, m);
-    const f32x4 r4 = *(const f32x4*)(rewards + rw.base + p0);
+    const f32x4 r4 = *(const f32x4e*)(rewards + rw.base + p0);
     f32x4 v4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (GAE) v4 = *(const f32x4*)(values + rw.base + p0);
+    if (GAE) v4 = *(const f32x4e*)(values + rw.base + p0);
 #pragma unroll
     for (int j = 0; j < kScanItems; ++j) {
       t.r[j] = m[j] * reward_of(r4[j], p0 + j);
@@ -287,7 +286,7 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
     const int64_t n_tiles = (rw.len + kScanTile - 1) / kScanTile;
     double tile_carry = 0.0;  // A at the first token of the previous (later) tile
     auto whole = [&](int64_t tile) {
-      return rows.vec && tile * kScanTile >= rw.lead && (tile + 1) * kScanTile <= rw.len;
+      return tile * kScanTile >= rw.lead && (tile + 1) * kScanTile <= rw.len;
     };
     ScanTile cur =
         load_scan_tile<MASK_DT, GAE, REWARD>(rw, (n_tiles - 1) * kScanTile, whole(n_tiles - 1), values, rewards, mask, rr);
@@ -344,10 +343,10 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
       }
       if (whole(tile)) {
         if (GAE) {
-          *(f32x4*)(adv + rw.base + p0) = out_a;
-          *(f32x4*)(ret + rw.base + p0) = out_r;
+          *(f32x4e*)(adv + rw.base + p0) = out_a;
+          *(f32x4e*)(ret + rw.base + p0) = out_r;
         } else {
-          *(f32x4*)(ret + rw.base + p0) = out_a;
+          *(f32x4e*)(ret + rw.base + p0) = out_a;
         }
       } else {
 #pragma unroll
@@ -420,10 +419,9 @@ __global__ __launch_bounds__(kBlock) void group_normalize_kernel(const float* __
 // ---------------------------------------------------------------- global masked whitening
 constexpr int kWhitenBlocks = 1024;
 
-// vec: x and mask allow 16-byte loads of four consecutive elements
 template <int MASK_DT>
 __global__ __launch_bounds__(kBlock) void whiten_partial_kernel(const float* __restrict__ x,
-                                                                const void* __restrict__ mask, int64_t n, int vec,
+                                                                const void* __restrict__ mask, int64_t n,
                                                                 double* __restrict__ partial) {
   __shared__ double lds[kWavesPerBlock];
   double sx = 0.0, sxx = 0.0, sm = 0.0;
@@ -434,10 +432,10 @@ __global__ __launch_bounds__(kBlock) void whiten_partial_kernel(const float* __r
     sm += m;
   };
   const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
-  const int64_t groups = vec ? n / 4 : 0;
+  const int64_t groups = n / 4;
 #pragma unroll 4
   for (int64_t g = first; g < groups; g += stride) {
-    const f32x4 v = *(const f32x4*)(x + g * 4);
+    const f32x4 v = *(const f32x4e*)(x + g * 4);
     float m[4];
     load_mask4<MASK_DT>(mask, g * 4, m);
 #pragma unroll
@@ -495,18 +493,18 @@ __global__ __launch_bounds__(kBlock) void whiten_final_kernel(const double* __re
 }
 
 // out may be x itself (each lane reads its elements before it writes them): no __restrict__ on them
-__global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* x, int64_t n, int vec,
+__global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* x, int64_t n,
                                                               const float* __restrict__ mean_rstd, float* out) {
   const float mean = mean_rstd[0], rstd = mean_rstd[1];
   const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
-  const int64_t groups = vec ? n / 4 : 0;
+  const int64_t groups = n / 4;
 #pragma unroll 2
   for (int64_t g = first; g < groups; g += stride) {
-    const f32x4 v = *(const f32x4*)(x + g * 4);
+    const f32x4 v = *(const f32x4e*)(x + g * 4);
     f32x4 o;
 #pragma unroll
     for (int k = 0; k < 4; ++k) o[k] = (v[k] - mean) * rstd;
-    *(f32x4*)(out + g * 4) = o;
+    *(f32x4e*)(out + g * 4) = o;
   }
   for (int64_t i = groups * 4 + first; i < n; i += stride) out[i] = (x[i] - mean) * rstd;
 }
@@ -526,12 +524,12 @@ struct WhitenSegs {
   int n_segs;
 };
 
-// Calls four(i0) / one(i) over the span of this workgroup inside its block; vec: per block.
+// Calls four(i0) / one(i) over the span of this workgroup inside its block.
 template <typename F4, typename F1>
-__device__ __forceinline__ void for_span(int64_t lo, int64_t hi, bool vec, F4&& four, F1&& one) {
+__device__ __forceinline__ void for_span(int64_t lo, int64_t hi, F4&& four, F1&& one) {
 #pragma unroll 2
   for (int64_t s0 = lo; s0 < hi; s0 += kBlock * 4) {
-    if (vec && s0 + kBlock * 4 <= hi) {
+    if (s0 + kBlock * 4 <= hi) {
       four(s0 + (int64_t)threadIdx.x * 4);
     } else {
 #pragma unroll
@@ -557,8 +555,6 @@ __global__ __launch_bounds__(kBlock) void whiten_partial_multi_kernel(WhitenSegs
   const void* mask = segs.mask[s];
   const int64_t lo = (int64_t)(blockIdx.x - segs.first_wg[s]) * kWhitenSpan;
   const int64_t hi = lo + kWhitenSpan < segs.n[s] ? lo + kWhitenSpan : segs.n[s];
-  const bool vec = (((uintptr_t)x & 15) == 0) &&
-                   (MASK_DT == ORLHF_MASK_NONE || ((uintptr_t)mask & (MASK_DT == ORLHF_MASK_U8 ? 3 : 15)) == 0);
   double sx = 0.0, sxx = 0.0, sm = 0.0;
   auto add = [&](float xv, float mv) {
     const double m = (double)mv, v = (double)xv;
@@ -567,9 +563,9 @@ __global__ __launch_bounds__(kBlock) void whiten_partial_multi_kernel(WhitenSegs
     sm += m;
   };
   for_span(
-      lo, hi, vec,
+      lo, hi,
       [&](int64_t i0) {
-        const f32x4 v = *(const f32x4*)(x + i0);
+        const f32x4 v = *(const f32x4e*)(x + i0);
         float m[4];
         load_mask4<MASK_DT>(mask, i0, m);
 #pragma unroll
@@ -593,16 +589,15 @@ __global__ __launch_bounds__(kBlock) void whiten_apply_multi_kernel(WhitenSegs s
   float* out = segs.out[s];
   const int64_t lo = (int64_t)(blockIdx.x - segs.first_wg[s]) * kWhitenSpan;
   const int64_t hi = lo + kWhitenSpan < segs.n[s] ? lo + kWhitenSpan : segs.n[s];
-  const bool vec = ((((uintptr_t)x) | ((uintptr_t)out)) & 15) == 0;
   const float mean = mean_rstd[0], rstd = mean_rstd[1];
   for_span(
-      lo, hi, vec,
+      lo, hi,
       [&](int64_t i0) {
-        const f32x4 v = *(const f32x4*)(x + i0);
+        const f32x4 v = *(const f32x4e*)(x + i0);
         f32x4 o;
 #pragma unroll
         for (int k = 0; k < 4; ++k) o[k] = (v[k] - mean) * rstd;
-        *(f32x4*)(out + i0) = o;
+        *(f32x4e*)(out + i0) = o;
       },
       [&](int64_t i) { out[i] = (x[i] - mean) * rstd; });
 }
@@ -632,7 +627,7 @@ extern "C" int orlhf_compute_reward(const float* r, float kl_coef, const float* 
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(r && reward && (kl || n_cols == 0), "compute_reward: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
-  const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {kl, reward}) ? 1 : 0};
+  const Rows rows{n_rows, n_cols, cu_seqlens};
   const float neg_coef = -(kl_coef > 0.0f ? kl_coef : 0.0f);
   const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
 #define ORLHF_LAUNCH(M)                                                                                         \
@@ -650,8 +645,7 @@ extern "C" int orlhf_gae_scan(const float* values, const float* rewards, const v
   if (int rc = check_rows("gae_scan", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(values && rewards && advantages && returns, "gae_scan: NULL pointer");
-  const Rows rows{n_rows, n_cols, cu_seqlens,
-                  vector_loads_ok(mask, mask_dtype, {values, rewards, advantages, returns}) ? 1 : 0};
+  const Rows rows{n_rows, n_cols, cu_seqlens};
   launch_scan<true, false>(mask_dtype, rows, values, rewards, mask, (double)gamma, (double)gamma * (double)lambd,
                            SeqReward{}, advantages, returns, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_gae_scan");
@@ -664,7 +658,7 @@ extern "C" int orlhf_discounted_returns(const float* rewards, const void* mask, 
   if (int rc = check_rows("discounted_returns", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(rewards && returns, "discounted_returns: NULL pointer");
-  const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {rewards, returns}) ? 1 : 0};
+  const Rows rows{n_rows, n_cols, cu_seqlens};
   launch_scan<false, false>(mask_dtype, rows, nullptr, rewards, mask, (double)gamma, (double)gamma, SeqReward{},
                             nullptr, returns, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_discounted_returns");
@@ -681,8 +675,7 @@ extern "C" int orlhf_reward_scan(const float* r, float kl_coef, const float* kl,
   ORLHF_CHECK_ARG(r != nullptr && returns != nullptr && (kl != nullptr || n_cols == 0), "reward_scan: NULL pointer");
   ORLHF_CHECK_ARG((values == nullptr) == (advantages == nullptr),
                   "reward_scan: values and advantages go together (GAE) or are both NULL (discounted returns)");
-  const Rows rows{n_rows, n_cols, cu_seqlens,
-                  vector_loads_ok(mask, mask_dtype, {kl, values, advantages, returns}) ? 1 : 0};
+  const Rows rows{n_rows, n_cols, cu_seqlens};
   const SeqReward sr{r, -(kl_coef > 0.0f ? kl_coef : 0.0f), has_clip, clip_low, clip_high, reward_sum};
   if (values != nullptr)
     launch_scan<true, true>(mask_dtype, rows, values, kl, mask, (double)gamma, (double)gamma * (double)lambd, sr,
@@ -798,15 +791,13 @@ extern "C" int orlhf_masked_whiten(const float* x, const void* mask, int mask_dt
   float* mean_rstd = (float*)(partial + (int64_t)kWhitenBlocks * 3);
   const int nb = flat_grid(n, kWhitenBlocks);
   const dim3 grid(nb), block(kBlock);
-  const int vec = vector_loads_ok(mask, mask_dtype, {x}) ? 1 : 0;
-#define ORLHF_LAUNCH(M) hipLaunchKernelGGL(whiten_partial_kernel<M>, grid, block, 0, s, x, mask, n, vec, partial)
+#define ORLHF_LAUNCH(M) hipLaunchKernelGGL(whiten_partial_kernel<M>, grid, block, 0, s, x, mask, n, partial)
   ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
 #undef ORLHF_LAUNCH
   ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(partial)");
   hipLaunchKernelGGL(whiten_final_kernel, dim3(1), block, 0, s, partial, nb, std_norm, mean_rstd, stats);
   ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(final)");
-  hipLaunchKernelGGL(whiten_apply_kernel, dim3(flat_grid((n + 3) / 4, 65536)), block, 0, s, x, n,
-                     (aligned_to(x, 16) && aligned_to(out, 16)) ? 1 : 0, mean_rstd, out);
+  hipLaunchKernelGGL(whiten_apply_kernel, dim3(flat_grid((n + 3) / 4, 65536)), block, 0, s, x, n, mean_rstd, out);
   ORLHF_CHECK_LAUNCH("orlhf_masked_whiten(apply)");
   return ORLHF_OK;
 }

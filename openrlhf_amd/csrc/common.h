@@ -1,8 +1,6 @@
 // Shared device/host helpers for the gfx950 (CDNA4, wave64) token-numerics kernels.
 #pragma once
 #include <hip/hip_runtime.h>
-
-#include <initializer_list>
 #include <math.h>
 #include <stdint.h>
 #include <stdio.h>
@@ -119,7 +117,6 @@ inline bool valid_mask_dtype(int m) { return m >= ORLHF_MASK_NONE && m <= ORLHF_
 struct Rows {
   int64_t n_rows, n_cols;
   const int64_t* cu;  // packed layout when non-null
-  int vec;            // chunked kernels: every array is aligned for four-token vector loads
   int chunk;          // chunked kernels: tokens of one row per work item
 };
 
@@ -135,16 +132,14 @@ __device__ __forceinline__ void row_span(const Rows& r, int64_t b, int64_t& star
 
 // ---------------------------------------------------------------- four tokens per lane
 // Kernels whose lanes work on four consecutive tokens load them with one 16-byte instruction per
-// fp32 array (and one load of the four mask elements) when Rows::vec says every array allows it.
-inline bool aligned_to(const void* p, uintptr_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
-
-// True when `mask` and every non-null fp32 array in `arrays` are aligned for those loads;
-// otherwise every token takes the element-wise path.
-inline bool vector_loads_ok(const void* mask, int mask_dt, std::initializer_list<const void*> arrays) {
-  bool ok = mask_dt == ORLHF_MASK_NONE || aligned_to(mask, mask_dt == ORLHF_MASK_U8 ? 4 : 16);
-  for (const void* a : arrays) ok = ok && aligned_to(a, 16);
-  return ok;
-}
+// fp32 array and one load of the four mask elements. The vector types below promise only the
+// element's own alignment: gfx950 global memory takes such accesses as one instruction wherever
+// they start, so arrays at any address take the same path; the row walks still start on 16-byte
+// boundaries of the index space, which keeps the accesses aligned when the arrays are.
+typedef float f32x4e __attribute__((ext_vector_type(4), aligned(4)));
+typedef uint32_t u32x2h __attribute__((ext_vector_type(2), aligned(2)));  // four 2-byte elements
+typedef int64_t i64x2e __attribute__((ext_vector_type(2), aligned(8)));
+typedef uint32_t u32_b __attribute__((aligned(1)));  // four 1-byte elements
 
 template <int MASK_DT>
 __device__ __forceinline__ void load_mask4(const void* mask, int64_t i0, float* m) {
@@ -152,16 +147,15 @@ __device__ __forceinline__ void load_mask4(const void* mask, int64_t i0, float* 
 #pragma unroll
     for (int k = 0; k < 4; ++k) m[k] = 1.0f;
   } else if (MASK_DT == ORLHF_MASK_U8) {
-    const uint32_t w = *(const uint32_t*)((const uint8_t*)mask + i0);
+    const uint32_t w = *(const u32_b*)((const uint8_t*)mask + i0);
 #pragma unroll
     for (int k = 0; k < 4; ++k) m[k] = (float)((w >> (8 * k)) & 0xffu);
   } else if (MASK_DT == ORLHF_MASK_F32) {
-    const f32x4 x = *(const f32x4*)((const float*)mask + i0);
+    const f32x4 x = *(const f32x4e*)((const float*)mask + i0);
 #pragma unroll
     for (int k = 0; k < 4; ++k) m[k] = x[k];
   } else {
-    typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
-    const i64x2 lo = *(const i64x2*)((const int64_t*)mask + i0), hi = *(const i64x2*)((const int64_t*)mask + i0 + 2);
+    const i64x2e lo = *(const i64x2e*)((const int64_t*)mask + i0), hi = *(const i64x2e*)((const int64_t*)mask + i0 + 2);
     m[0] = (float)lo[0];
     m[1] = (float)lo[1];
     m[2] = (float)hi[0];
@@ -169,8 +163,8 @@ __device__ __forceinline__ void load_mask4(const void* mask, int64_t i0, float* 
   }
 }
 
-// A row as the chunked kernels walk it: when vector loads are on, the walk starts at the last
-// 16-byte boundary at or before the row's first token (`lead` tokens early, 0..3), so that every
+// A row as the chunked kernels walk it: the walk starts at the last 16-byte boundary (of the
+// index space) at or before the row's first token (`lead` tokens early, 0..3), so that every
 // whole step of the walk is aligned; tokens before `lead` are not the row's and are skipped.
 struct RowWalk {
   int64_t base, len;  // flat index of the walk's first position; positions in the walk
@@ -180,7 +174,7 @@ __device__ __forceinline__ RowWalk row_walk(const Rows& rows, int64_t b) {
   int64_t start, len;
   row_span(rows, b, start, len);
   RowWalk w;
-  w.lead = (rows.vec && len > 0) ? (int)(start & 3) : 0;
+  w.lead = len > 0 ? (int)(start & 3) : 0;
   w.base = start - w.lead;
   w.len = len > 0 ? len + w.lead : 0;
   return w;
@@ -194,15 +188,15 @@ __device__ __forceinline__ float load_lp(const void* p, int64_t i) {
   return (float)((const _Float16*)p)[i];
 }
 
-// four consecutive elements from index i0 (a multiple of four from a 16-byte aligned base)
+// four consecutive elements from index i0
 template <int DT>
 __device__ __forceinline__ void load_lp4(const void* p, int64_t i0, float* v) {
   if (DT == ORLHF_F32) {
-    const f32x4 x = *(const f32x4*)((const float*)p + i0);
+    const f32x4 x = *(const f32x4e*)((const float*)p + i0);
 #pragma unroll
     for (int k = 0; k < 4; ++k) v[k] = x[k];
   } else {
-    const u32x2 w = *(const u32x2*)((const uint16_t*)p + i0);
+    const u32x2 w = *(const u32x2h*)((const uint16_t*)p + i0);
     if (DT == ORLHF_BF16) {
       v[0] = bf16_lo(w[0]), v[1] = bf16_hi(w[0]), v[2] = bf16_lo(w[1]), v[3] = bf16_hi(w[1]);
     } else {
@@ -212,12 +206,11 @@ __device__ __forceinline__ void load_lp4(const void* p, int64_t i0, float* v) {
   }
 }
 
-// Walks one row with the whole workgroup: four(i0) for each lane's four consecutive tokens
-// (flat index i0, aligned for a 16-byte load) on every step that lies inside the row when vector
-// loads are on, one(i) per token (stride kBlock) on the steps at the row's ends or on all steps
-// otherwise. Every token of the row is visited exactly once.
+// Walks one row with the whole workgroup: four(i0) for each lane's four consecutive tokens (flat
+// index i0) on every step that lies inside the row, one(i) per token (stride kBlock) on the steps
+// at the row's ends. Every token of the row is visited exactly once.
 template <typename F4, typename F1>
-__device__ __forceinline__ void for_row_tokens(const Rows& rows, const RowWalk& rw, F4&& four, F1&& one) {
+__device__ __forceinline__ void for_row_tokens(const RowWalk& rw, F4&& four, F1&& one) {
   constexpr int kStep = kBlock * 4;
   int64_t s0 = 0;
   auto edge = [&](int64_t s) {
@@ -227,14 +220,12 @@ __device__ __forceinline__ void for_row_tokens(const Rows& rows, const RowWalk& 
       if (t >= rw.lead && t < rw.len) one(rw.base + t);
     }
   };
-  if (rows.vec) {
-    if (rw.lead > 0 && s0 < rw.len) {
-      edge(s0);
-      s0 += kStep;
-    }
-#pragma unroll 2
-    for (; s0 + kStep <= rw.len; s0 += kStep) four(rw.base + s0 + (int64_t)threadIdx.x * 4);
+  if (rw.lead > 0 && s0 < rw.len) {
+    edge(s0);
+    s0 += kStep;
   }
+#pragma unroll 2
+  for (; s0 + kStep <= rw.len; s0 += kStep) four(rw.base + s0 + (int64_t)threadIdx.x * 4);
   for (; s0 < rw.len; s0 += kStep) edge(s0);
 }
 

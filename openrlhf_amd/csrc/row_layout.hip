@@ -109,6 +109,20 @@ __global__ __launch_bounds__(kCuBlock) void cu_seqlens_kernel(const int64_t* __r
 // chunk-fastest the chunks that hold tokens of short rows would pile up on a few XCDs.
 constexpr int kCopyChunk = 4096;
 
+// 16 bytes of consecutive elements as one load or store. The type only promises the element's own
+// alignment (source and destination rows start anywhere), which gfx950 global memory accepts.
+typedef uint32_t u32x4_a1 __attribute__((ext_vector_type(4), aligned(1)));
+typedef uint32_t u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+template <int SIZE> struct Vec16Of { typedef u32x4_a4 type; };
+template <> struct Vec16Of<1> { typedef u32x4_a1 type; };
+template <> struct Vec16Of<2> { typedef u32x4_a2 type; };
+template <typename E>
+struct Vec16 {
+  typedef typename Vec16Of<sizeof(E)>::type type;
+  static constexpr int kElems = 16 / sizeof(E);
+};
+
 template <typename E>
 __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__ src, int64_t n_rows, int64_t n_cols,
                                                            const int64_t* __restrict__ first,
@@ -126,8 +140,12 @@ __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__
     stop = stop < n_cols - f ? stop : n_cols - f;
     const E* in = src + b * n_cols + f;
     E* out = dst + start;
-#pragma unroll 4
-    for (int64_t j = j0 + threadIdx.x; j < stop; j += kBlock) out[j] = in[j];
+    constexpr int kE = Vec16<E>::kElems;
+    typedef typename Vec16<E>::type V;
+    const int64_t groups = (stop - j0) / kE;
+#pragma unroll 2
+    for (int64_t g = threadIdx.x; g < groups; g += kBlock) *(V*)(out + j0 + g * kE) = *(const V*)(in + j0 + g * kE);
+    for (int64_t j = j0 + groups * kE + threadIdx.x; j < stop; j += kBlock) out[j] = in[j];
   }
 }
 
@@ -144,8 +162,27 @@ __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ 
     const int64_t shift = left ? n_cols - len : 0;  // column of the row's first token
     const int64_t stop = t0 + kCopyChunk < n_cols ? t0 + kCopyChunk : n_cols;
     E* out = dst + b * n_cols;
-#pragma unroll 4
-    for (int64_t t = t0 + threadIdx.x; t < stop; t += kBlock)
+    constexpr int kE = Vec16<E>::kElems;
+    typedef typename Vec16<E>::type V;
+    E fill_e[kE];
+#pragma unroll
+    for (int k = 0; k < kE; ++k) fill_e[k] = fill;
+    const V fill_v = __builtin_bit_cast(V, fill_e);
+    const int64_t groups = (stop - t0) / kE;
+#pragma unroll 2
+    for (int64_t g = threadIdx.x; g < groups; g += kBlock) {
+      const int64_t t = t0 + g * kE;
+      if (t >= shift && t + kE <= shift + len) {  // all of the group's columns hold tokens
+        *(V*)(out + t) = *(const V*)(src + start + (t - shift));
+      } else if (t + kE <= shift || t >= shift + len) {  // all padding
+        *(V*)(out + t) = fill_v;
+      } else {
+#pragma unroll
+        for (int k = 0; k < kE; ++k)
+          out[t + k] = (t + k >= shift && t + k < shift + len) ? src[start + (t + k - shift)] : fill;
+      }
+    }
+    for (int64_t t = t0 + groups * kE + threadIdx.x; t < stop; t += kBlock)
       out[t] = (t >= shift && t < shift + len) ? src[start + (t - shift)] : fill;
   }
 }

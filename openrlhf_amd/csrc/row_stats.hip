@@ -49,7 +49,7 @@ __global__ __launch_bounds__(kBlock) void kl_rows_kernel(const void* __restrict_
       sm += (double)m;
     };
     for_row_tokens(
-        rows, rw,
+        rw,
         [&](int64_t i0) {
           float x[4] = {0.0f, 0.0f, 0.0f, 0.0f}, y[4] = {0.0f, 0.0f, 0.0f, 0.0f}, m[4];
           if (enabled) {
@@ -64,7 +64,7 @@ __global__ __launch_bounds__(kBlock) void kl_rows_kernel(const void* __restrict_
             token(x[k], y[k], m[k], vk);
             v[k] = vk;
           }
-          if (kl != nullptr) *(f32x4*)(kl + i0) = v;
+          if (kl != nullptr) *(f32x4e*)(kl + i0) = v;
         },
         [&](int64_t i) {
           float v;
@@ -94,9 +94,9 @@ __global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const flo
     const RowWalk rw = row_walk(rows, b);
     double s = 0.0, c = 0.0, z = 0.0;
     for_row_tokens(
-        rows, rw,
+        rw,
         [&](int64_t i0) {
-          const f32x4 v = *(const f32x4*)(x + i0);
+          const f32x4 v = *(const f32x4e*)(x + i0);
           float m[4];
           load_mask4<MASK_DT>(mask, i0, m);
 #pragma unroll
@@ -115,9 +115,9 @@ __global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const flo
     const float mean = (float)(s / cnt);
     double v = 0.0, z1 = 0.0, z2 = 0.0;
     for_row_tokens(
-        rows, rw,
+        rw,
         [&](int64_t i0) {
-          const f32x4 xv = *(const f32x4*)(x + i0);
+          const f32x4 xv = *(const f32x4e*)(x + i0);
           float m[4];
           load_mask4<MASK_DT>(mask, i0, m);
 #pragma unroll
@@ -134,15 +134,15 @@ __global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const flo
     const float var = (float)(v / cnt);
     const float r = 1.0f / sqrtf(var != var ? var : fmaxf(var, eps));
     for_row_tokens(
-        rows, rw,
+        rw,
         [&](int64_t i0) {
-          const f32x4 xv = *(const f32x4*)(x + i0);
+          const f32x4 xv = *(const f32x4e*)(x + i0);
           float m[4];
           load_mask4<MASK_DT>(mask, i0, m);
           f32x4 o;
 #pragma unroll
           for (int k = 0; k < 4; ++k) o[k] = (xv[k] - mean) * m[k] * r;
-          *(f32x4*)(out + i0) = o;
+          *(f32x4e*)(out + i0) = o;
         },
         [&](int64_t i) { out[i] = (x[i] - mean) * load_mask<MASK_DT>(mask, i) * r; });
   }
@@ -162,7 +162,7 @@ extern "C" int orlhf_kl_rows(const void* log_probs, const void* log_probs_base, 
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(!enabled || n_cols == 0 || (log_probs != nullptr && log_probs_base != nullptr),
                   "kl_rows: log_probs / log_probs_base is NULL");
-  const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {log_probs, log_probs_base, kl}) ? 1 : 0};
+  const Rows rows{n_rows, n_cols, cu_seqlens};
   const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_KL(M)                                                                                                  \
@@ -189,7 +189,7 @@ extern "C" int orlhf_masked_normalize_rows(const float* x, const void* mask, int
   if (int rc = check_rows("masked_normalize_rows", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(x != nullptr && out != nullptr, "masked_normalize_rows: NULL argument");
-  const Rows rows{n_rows, n_cols, cu_seqlens, vector_loads_ok(mask, mask_dtype, {x, out}) ? 1 : 0};
+  const Rows rows{n_rows, n_cols, cu_seqlens};
   const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
 #define ORLHF_NORM(M) \

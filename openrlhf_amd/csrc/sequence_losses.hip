@@ -20,7 +20,7 @@ template <int MASK_DT>
 __global__ __launch_bounds__(kBlock) void sequence_logps_fwd_kernel(const float* __restrict__ lp,
                                                                     const void* __restrict__ att,
                                                                     const int64_t* __restrict__ prompt_lens,
-                                                                    int64_t n_rows, int64_t n_cols, int vec,
+                                                                    int64_t n_rows, int64_t n_cols,
                                                                     float* __restrict__ sums,
                                                                     float* __restrict__ means,
                                                                     float* __restrict__ counts) {
@@ -30,20 +30,28 @@ __global__ __launch_bounds__(kBlock) void sequence_logps_fwd_kernel(const float*
     const int64_t b = row_of_slot(slot, slot, slot_b);
     if (b >= n_rows) continue;
     double s = 0.0, c = 0.0;
-    // the mask sits one column to the right in rows one element longer: element-wise loads for it
-    const Rows rows{n_rows, n_cols, nullptr, vec};
+    // the mask sits one column to the right in rows one element longer: loads without alignment
+    const Rows rows{n_rows, n_cols, nullptr};
     const RowWalk rw = row_walk(rows, b);
     auto token = [&](float x, int64_t t) {
       const float m = dpo_mask<MASK_DT>(att, prompt_lens, b, t, n_cols + 1);
       s += (double)(x * m);  // the reference multiplies by the mask (NaN * 0 stays NaN)
       c += (double)m;
     };
+    const int64_t plen = prompt_lens != nullptr ? prompt_lens[b] : 0;
     for_row_tokens(
-        rows, rw,
+        rw,
         [&](int64_t i0) {
-          const f32x4 x = *(const f32x4*)(lp + i0);
+          const f32x4 x = *(const f32x4e*)(lp + i0);
+          const int64_t t0 = i0 - b * n_cols;
+          float a[4];
+          load_mask4<MASK_DT>(att, b * (n_cols + 1) + t0 + 1, a);
 #pragma unroll
-          for (int k = 0; k < 4; ++k) token(x[k], i0 + k - b * n_cols);
+          for (int k = 0; k < 4; ++k) {
+            const float m = (t0 + k + 1 >= plen && a[k] != 0.0f) ? 1.0f : 0.0f;
+            s += (double)(x[k] * m);
+            c += (double)m;
+          }
         },
         [&](int64_t i) { token(lp[i], i - b * n_cols); });
     s = block_sum(s, lds);
@@ -188,10 +196,9 @@ extern "C" int orlhf_sequence_logps_fwd(const float* per_token_logps, const void
   ORLHF_CHECK_ARG(per_token_logps != nullptr || n_cols == 0, "sequence_logps_fwd: per_token_logps is NULL");
   const dim3 grid(slot_grid(row_slots(n_rows), 65536)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
-  const int vec = aligned_to(per_token_logps, 16) ? 1 : 0;
 #define ORLHF_LAUNCH(M)                                                                                        \
   hipLaunchKernelGGL(sequence_logps_fwd_kernel<M>, grid, block, 0, s, per_token_logps, attention_mask, prompt_id_lens, \
-                     n_rows, n_cols, vec, sums, means, counts)
+                     n_rows, n_cols, sums, means, counts)
   ORLHF_FOR_MASK_DTYPE(mask_dtype, ORLHF_LAUNCH)
 #undef ORLHF_LAUNCH
   ORLHF_CHECK_LAUNCH("orlhf_sequence_logps_fwd");

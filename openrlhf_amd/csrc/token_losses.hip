@@ -4,11 +4,11 @@
 // Layout: a [n_rows, n_cols] problem is cut into chunks of 1024 to 8192 tokens of one row (8192
 // on large batches); a workgroup walks one chunk in steps of 1024 tokens, four consecutive tokens
 // per lane, and reduces the quantities it needs to one fp64 partial per (row, chunk), all
-// quantities through the cross-lane steps together. When every array is 16-byte aligned a step
-// is one 16-byte load per lane and array (and one load of four mask elements): a row that does
-// not start on a 16-byte boundary is walked from the boundary before it, so that only its first
-// and last step take the element-wise path (against 4-byte loads: PolicyLoss forward 206 -> 174 us,
-// backward 286 -> 214 us on 67 M padded tokens). A fold kernel sums the chunks of each row, a
+// quantities through the cross-lane steps together. A step is one 16-byte load per lane and array
+// (and one load of four mask elements): a row that does not start on a multiple of four elements
+// is walked from the multiple before it, so that the loads are 16-byte aligned whenever the
+// arrays are, and only its first and last step go token by token (against 4-byte loads:
+// PolicyLoss forward 206 -> 174 us, backward 286 -> 214 us on 67 M padded tokens). A fold kernel sums the chunks of each row, a
 // single-workgroup kernel folds the rows in a fixed order and writes the scalars plus a per-row
 // aggregation weight that the backward kernels multiply with. Chunks past the end of a short
 // packed row return at once. No atomics anywhere: the result is bit-reproducible. All of these
@@ -32,18 +32,17 @@ constexpr int64_t kMaxItemsGrid = 1 << 22;
 // Chunks a row of up to n_cols tokens can span: a vector walk starts up to 3 tokens before the row
 // unless every row starts on a 16-byte boundary (padded rows whose length is a multiple of four).
 static inline int64_t chunks_of(const Rows& r) {
-  const int64_t lead = (r.vec && (r.cu != nullptr || (r.n_cols & 3) != 0)) ? 3 : 0;
+  const int64_t lead = (r.cu != nullptr || (r.n_cols & 3) != 0) ? 3 : 0;
   return r.n_cols > 0 ? (r.n_cols + lead + r.chunk - 1) / r.chunk : 1;
 }
 
-static Rows make_rows(int64_t n_rows, int64_t n_cols, const int64_t* cu, const void* mask, int mask_dt,
-                      std::initializer_list<const void*> arrays) {
-  const bool vec = vector_loads_ok(mask, mask_dt, arrays);
+// Rows of a chunked launch with the chunk length chosen for the problem size.
+static Rows make_rows(int64_t n_rows, int64_t n_cols, const int64_t* cu) {
   // 8 steps per work item measured fastest on large batches (16 the same, 4: +8%, 2: +35%);
   // smaller problems get shorter chunks so that a thousand workgroups still exist.
   int steps = 8;
   while (steps > 1 && n_rows * ((n_cols + (int64_t)kSubChunk * steps - 1) / ((int64_t)kSubChunk * steps)) < 1024) steps /= 2;
-  return Rows{n_rows, n_cols, cu, vec ? 1 : 0, kSubChunk * steps};
+  return Rows{n_rows, n_cols, cu, kSubChunk * steps};
 }
 
 struct NormArg {
@@ -147,8 +146,8 @@ struct GspoGradTok {  // backward row sum: m * d(token loss)/d(ratio_t) * d(rati
 };
 
 // ---------------------------------------------------------------- token loads
-// A lane works on four consecutive tokens. Where the row layout allows it (Rows::vec) they come
-// in with one 16-byte load per input array and one load of the four mask elements.
+// A lane works on four consecutive tokens: one 16-byte load per input array and one load of the
+// four mask elements.
 template <typename Tok>
 struct TokIn {
   static constexpr int kN = Tok::kIn > 0 ? Tok::kIn : 1;
@@ -163,14 +162,14 @@ __device__ __forceinline__ void load_inputs(const Tok& tok, int64_t i, float* v)
   }
 }
 
-// i0: index of the first of four tokens, a multiple of four elements from 16-byte aligned bases
+// i0: index of the first of four tokens
 template <typename Tok>
 __device__ __forceinline__ void load_inputs4(const Tok& tok, int64_t i0, float (*v)[TokIn<Tok>::kN]) {
 #pragma unroll
   for (int j = 0; j < Tok::kIn; ++j) {
     const float* p = tok.in(j);
     f32x4 x = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (p != nullptr) x = *(const f32x4*)(p + i0);
+    if (p != nullptr) x = *(const f32x4e*)(p + i0);
 #pragma unroll
     for (int k = 0; k < 4; ++k) v[k][j] = x[k];
   }
@@ -200,7 +199,7 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
     for (int i = 0; i < NQ; ++i) acc[i] = 0.0;
 #pragma unroll 1
     for (int64_t s0 = c0; s0 < c0 + rows.chunk && s0 < rw.len; s0 += kSubChunk) {
-      if (rows.vec && s0 >= rw.lead && s0 + kSubChunk <= rw.len) {  // whole step inside the row
+      if (s0 >= rw.lead && s0 + kSubChunk <= rw.len) {  // whole step inside the row
         const int64_t i0 = rw.base + s0 + threadIdx.x * kTokPerLane;
         float v[kTokPerLane][TokIn<Tok>::kN], m[kTokPerLane], q[kTokPerLane][NQ];
         load_inputs4(tok, i0, v);
@@ -441,7 +440,7 @@ __global__ __launch_bounds__(kBlock) void rows_grad_kernel(Rows rows, const void
     const float w = (g_per_row ? g_out[b] : g_out[0]) * row_coef[b];
 #pragma unroll 1
     for (int64_t s0 = c0; s0 < c0 + rows.chunk && s0 < rw.len; s0 += kSubChunk) {
-      if (rows.vec && s0 >= rw.lead && s0 + kSubChunk <= rw.len) {
+      if (s0 >= rw.lead && s0 + kSubChunk <= rw.len) {
         const int64_t i0 = rw.base + s0 + threadIdx.x * kTokPerLane;
         float v[kTokPerLane][TokIn<Tok>::kN], m[kTokPerLane];
         load_inputs4(tok, i0, v);
@@ -449,7 +448,7 @@ __global__ __launch_bounds__(kBlock) void rows_grad_kernel(Rows rows, const void
         f32x4 out;
 #pragma unroll
         for (int k = 0; k < kTokPerLane; ++k) out[k] = w * m[k] * tok.grad(b, v[k], m[k]);
-        *(f32x4*)(g + i0) = out;
+        *(f32x4e*)(g + i0) = out;
       } else {
 #pragma unroll
         for (int k = 0; k < kTokPerLane; ++k) {
@@ -498,13 +497,12 @@ __global__ __launch_bounds__(kBlock) void gspo_grad_kernel(Rows rows, const void
 }
 
 // ---------------------------------------------------------------- approximate KL (flat)
-// vec: every array allows 16-byte (fp32) / 8-byte (half) loads of four consecutive elements
 template <int DT>
 __global__ __launch_bounds__(kBlock) void approx_kl_fwd_kernel(const void* __restrict__ lp,
                                                                const void* __restrict__ base, int64_t n, int est,
-                                                               int vec, float* __restrict__ out) {
+                                                               float* __restrict__ out) {
   const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
-  const int64_t groups = vec ? n / 4 : 0;
+  const int64_t groups = n / 4;
 #pragma unroll 2
   for (int64_t g = first; g < groups; g += stride) {
     float x[4], y[4];
@@ -517,7 +515,7 @@ __global__ __launch_bounds__(kBlock) void approx_kl_fwd_kernel(const void* __res
       kl_value(est, x[k] - y[k], v, dv);
       o[k] = v;
     }
-    *(f32x4*)(out + g * 4) = o;
+    *(f32x4e*)(out + g * 4) = o;
   }
   for (int64_t i = groups * 4 + first; i < n; i += stride) {
     float v, dv;
@@ -529,16 +527,16 @@ __global__ __launch_bounds__(kBlock) void approx_kl_fwd_kernel(const void* __res
 template <int DT>
 __global__ __launch_bounds__(kBlock) void approx_kl_bwd_kernel(const void* __restrict__ lp,
                                                                const void* __restrict__ base, int64_t n, int est,
-                                                               int vec, const float* __restrict__ g_out,
+                                                               const float* __restrict__ g_out,
                                                                float* __restrict__ g_lp, float* __restrict__ g_base) {
   const int64_t first = (int64_t)blockIdx.x * kBlock + threadIdx.x, stride = (int64_t)gridDim.x * kBlock;
-  const int64_t groups = vec ? n / 4 : 0;
+  const int64_t groups = n / 4;
 #pragma unroll 2
   for (int64_t g = first; g < groups; g += stride) {
     float x[4], y[4];
     load_lp4<DT>(lp, g * 4, x);
     load_lp4<DT>(base, g * 4, y);
-    const f32x4 up = *(const f32x4*)(g_out + g * 4);
+    const f32x4 up = *(const f32x4e*)(g_out + g * 4);
     f32x4 o, neg;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
@@ -547,8 +545,8 @@ __global__ __launch_bounds__(kBlock) void approx_kl_bwd_kernel(const void* __res
       o[k] = up[k] * dv;
       neg[k] = -o[k];
     }
-    if (g_lp != nullptr) *(f32x4*)(g_lp + g * 4) = o;
-    if (g_base != nullptr) *(f32x4*)(g_base + g * 4) = neg;
+    if (g_lp != nullptr) *(f32x4e*)(g_lp + g * 4) = o;
+    if (g_base != nullptr) *(f32x4e*)(g_base + g * 4) = neg;
   }
   for (int64_t i = groups * 4 + first; i < n; i += stride) {
     float v, dv;
@@ -651,11 +649,10 @@ extern "C" int orlhf_approx_kl_fwd(const void* log_probs, const void* log_probs_
   ORLHF_CHECK_ARG(log_probs && log_probs_base && out, "approx_kl_fwd: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(flat_grid((n + 3) / 4)), block(kBlock);
-  const int vec = vector_loads_ok(nullptr, ORLHF_MASK_NONE, {log_probs, log_probs_base, out}) ? 1 : 0;
   switch (dtype) {
-    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, out); break;
-    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, out); break;
-    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, out); break;
+    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
+    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
+    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_fwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, out); break;
     default: return fail(ORLHF_ERR_INVALID_ARG, "approx_kl_fwd: unknown dtype %d", dtype);
   }
   ORLHF_CHECK_LAUNCH("orlhf_approx_kl_fwd");
@@ -671,11 +668,10 @@ extern "C" int orlhf_approx_kl_bwd(const void* log_probs, const void* log_probs_
   ORLHF_CHECK_ARG(log_probs && log_probs_base && g_out && (g_lp || g_base), "approx_kl_bwd: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid(flat_grid((n + 3) / 4)), block(kBlock);
-  const int vec = vector_loads_ok(nullptr, ORLHF_MASK_NONE, {log_probs, log_probs_base, g_out, g_lp, g_base}) ? 1 : 0;
   switch (dtype) {
-    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, g_out, g_lp, g_base); break;
-    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, g_out, g_lp, g_base); break;
-    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, vec, g_out, g_lp, g_base); break;
+    case ORLHF_F32: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F32>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
+    case ORLHF_BF16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_BF16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
+    case ORLHF_F16: hipLaunchKernelGGL(approx_kl_bwd_kernel<ORLHF_F16>, grid, block, 0, s, log_probs, log_probs_base, n, estimator, g_out, g_lp, g_base); break;
     default: return fail(ORLHF_ERR_INVALID_ARG, "approx_kl_bwd: unknown dtype %d", dtype);
   }
   ORLHF_CHECK_LAUNCH("orlhf_approx_kl_bwd");
@@ -691,7 +687,7 @@ extern "C" int orlhf_masked_aggregate_fwd(const float* x, const void* mask, int 
   ORLHF_CHECK_ARG(out != nullptr && workspace != nullptr, "masked_aggregate_fwd: NULL out / workspace");
   ORLHF_CHECK_ARG(x != nullptr || n_rows * n_cols == 0, "masked_aggregate_fwd: x is NULL");
   hipStream_t s = (hipStream_t)stream;
-  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens, mask, mask_dtype, {x});
+  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
   const int n_chunks = (int)chunks_of(rows);
   double* partial = (double*)workspace;
   if (n_rows > 0) {
@@ -709,7 +705,7 @@ extern "C" int orlhf_mask_counts(const void* mask, int mask_dtype, int64_t n_row
   if (int rc = check_rows("mask_counts", n_rows, n_cols, mask, mask_dtype)) return rc;
   ORLHF_CHECK_ARG(out2 != nullptr && workspace != nullptr, "mask_counts: NULL out2 / workspace");
   hipStream_t s = (hipStream_t)stream;
-  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens, mask, mask_dtype, {});
+  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
   const int n_chunks = (int)chunks_of(rows);
   double* partial = (double*)workspace;
   if (n_rows > 0) {
@@ -729,7 +725,7 @@ extern "C" int orlhf_masked_aggregate_bwd(const float* g_out, const void* mask, 
   ORLHF_CHECK_ARG(mode >= ORLHF_AGG_TOKEN_MEAN && mode <= ORLHF_AGG_SEQ_MEAN_TOKEN_SUM, "masked_aggregate_bwd: unknown mode %d", mode);
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(g_out && row_coef && g_x, "masked_aggregate_bwd: NULL pointer");
-  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens, mask, mask_dtype, {g_x});
+  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
   launch_grad(mask_dtype, rows, mask, UnitGrad{}, g_out, mode == ORLHF_AGG_ROW_MEAN, row_coef, g_x, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_masked_aggregate_bwd");
   return ORLHF_OK;
@@ -745,7 +741,7 @@ extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_lo
   ORLHF_CHECK_ARG(out4 && workspace && row_aux, "policy_loss_fwd: NULL out4 / workspace / row_aux");
   ORLHF_CHECK_ARG((log_probs && old_log_probs && advantages) || n_rows * n_cols == 0, "policy_loss_fwd: NULL input");
   hipStream_t s = (hipStream_t)stream;
-  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens, mask, mask_dtype, {log_probs, old_log_probs, advantages, rollout_log_probs});
+  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
   const int n_chunks = (int)chunks_of(rows);
   double* partial = (double*)workspace;
   const bool gspo = params->policy_type == ORLHF_POLICY_GSPO;
@@ -789,7 +785,7 @@ extern "C" int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs,
   ORLHF_CHECK_ARG(g_out && log_probs && old_log_probs && advantages && row_coef && row_aux && g_log_probs,
                   "policy_loss_bwd: NULL pointer");
   hipStream_t s = (hipStream_t)stream;
-  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens, mask, mask_dtype, {log_probs, old_log_probs, advantages, rollout_log_probs, g_log_probs});
+  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
   PolicyTok tok = policy_tok(log_probs, old_log_probs, advantages, rollout_log_probs, row_aux, params);
   if (!tok.gspo) {
     launch_grad(mask_dtype, rows, mask, tok, g_out, 0, row_coef, g_log_probs, s);
@@ -821,7 +817,7 @@ extern "C" int orlhf_value_loss_fwd(const float* values, const float* old_values
   ORLHF_CHECK_ARG(out && workspace, "value_loss_fwd: NULL out / workspace");
   ORLHF_CHECK_ARG((values && returns && (old_values || !has_clip)) || n_rows * n_cols == 0, "value_loss_fwd: NULL input");
   hipStream_t s = (hipStream_t)stream;
-  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens, mask, mask_dtype, {values, old_values, returns});
+  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
   const int n_chunks = (int)chunks_of(rows);
   double* partial = (double*)workspace;
   if (n_rows > 0) {
@@ -843,7 +839,7 @@ extern "C" int orlhf_value_loss_bwd(const float* g_out, const float* values, con
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(g_out && values && returns && (old_values || !has_clip) && row_coef && g_values,
                   "value_loss_bwd: NULL pointer");
-  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens, mask, mask_dtype, {values, old_values, returns, g_values});
+  const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
   ValueTok tok{values, old_values, returns, has_clip, clip_eps};
   launch_grad(mask_dtype, rows, mask, tok, g_out, 0, row_coef, g_values, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_value_loss_bwd");

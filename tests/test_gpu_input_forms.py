@@ -99,8 +99,8 @@ def _at_offset(t, off):
 
 @pytest.mark.parametrize("off", [1, 2, 3])
 def test_per_token_arrays_off_the_16_byte_boundary(cuda, off):
-    """Arrays on 16-byte boundaries take four-token vector loads, others the element-wise walk:
-    same losses and gradients (the sums differ in their order only)."""
+    """The four-token vector loads promise the element's alignment only: arrays that start off a
+    16-byte boundary give the same losses and gradients."""
     from openrlhf_amd.models.loss import PolicyLoss, ValueLoss, aggregate_loss
     from openrlhf_amd.trainer.ppo_utils.experience import PackedSteps
 
@@ -143,7 +143,7 @@ def test_per_token_arrays_off_the_16_byte_boundary(cuda, off):
 def test_flat_kernels_off_the_16_byte_boundary(cuda, off, dtype):
     """The flat kernels (approximate KL forward / backward, global whitening) on storage that
     does not start on a 16-byte boundary and with a length that is not a multiple of four: the
-    element-wise path gives the same bits as the vector path on aligned storage."""
+    same bits as on aligned storage."""
     from openrlhf_amd.models.utils import compute_approx_kl
     from openrlhf_amd.trainer.ppo_utils.experience_maker import whiten_advantages
 
