@@ -82,8 +82,19 @@ __global__ __launch_bounds__(kBlock) void sequence_logps_bwd_kernel(const float*
     float up = g_sums != nullptr ? g_sums[b] : 0.0f;
     if (g_means != nullptr) up += g_means[b] / counts[b];
     const int64_t stop = t0 + kSeqChunk < n_cols ? t0 + kSeqChunk : n_cols;
-#pragma unroll 4
-    for (int64_t t = t0 + threadIdx.x; t < stop; t += kBlock)
+    const int64_t plen = prompt_lens != nullptr ? prompt_lens[b] : 0;
+    const int64_t groups = (stop - t0) / 4;  // four columns per lane: one mask load, one 16-byte store
+#pragma unroll 2
+    for (int64_t q = threadIdx.x; q < groups; q += kBlock) {
+      const int64_t t = t0 + q * 4;
+      float a[4];
+      load_mask4<MASK_DT>(att, b * (n_cols + 1) + t + 1, a);
+      f32x4 o;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) o[k] = up * ((t + k + 1 >= plen && a[k] != 0.0f) ? 1.0f : 0.0f);
+      *(f32x4e*)(g + b * n_cols + t) = o;
+    }
+    for (int64_t t = t0 + groups * 4 + threadIdx.x; t < stop; t += kBlock)
       g[b * n_cols + t] = up * dpo_mask<MASK_DT>(att, prompt_lens, b, t, n_cols + 1);
   }
 }
