@@ -52,7 +52,7 @@ __device__ __forceinline__ int64_t last_max_of_mask(const Rows& rows, const RowW
     // byte masks: 16 tokens per lane and load between the row's first and last 16-byte boundary
     // (a quarter of the steps of the four-token walk; this pass is latency-bound)
     const uint8_t* bytes = (const uint8_t*)mask + start;
-    const int64_t len = rw.len - rw.lead;
+    const int64_t len = rw.len;
     int64_t head = (int64_t)((16 - ((uintptr_t)bytes & 15)) & 15);
     head = head < len ? head : len;
     const int64_t groups = (len - head) / 16;
@@ -178,11 +178,11 @@ struct ScanTile {
 // compute_reward_kernel writes it; `sum` collects the row's token rewards.
 struct RowReward {
   float seq, neg_coef;
-  int64_t eos;  // position in the walk (RowWalk::lead + index in the row)
+  int64_t eos;  // index in the row
   double sum;
 };
 
-// `whole`: the tile lies inside the row. Must be called by
+// `whole`: the tile lies inside the row (no lane needs to look at the row's end). Must be called by
 // all lanes of the workgroup (it exchanges the following value across lanes).
 template <int MASK_DT, bool GAE, bool REWARD>
 __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t tile0, bool whole,
@@ -198,7 +198,7 @@ __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t ti
     rr.sum += (double)tok;
     return tok;
   };
-  if (whole) {
+  if (whole || p0 + kScanItems <= rw.len) {  // this lane's four tokens lie in the row
     float m[kScanItems];
     load_mask4<MASK_DT>(mask, rw.base + p0, m);
     const f32x4 r4 = *(const f32x4e*)(rewards + rw.base + p0);
@@ -209,13 +209,13 @@ __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t ti
       t.r[j] = m[j] * reward_of(r4[j], p0 + j);
       t.v[j] = m[j] * v4[j];
     }
-  } else {
+  } else {  // the lane that meets the row's end, and the lanes past it
 #pragma unroll
     for (int j = 0; j < kScanItems; ++j) {
       const int64_t p = p0 + j;
       t.r[j] = 0.0f;
       t.v[j] = 0.0f;
-      if (p >= rw.lead && p < rw.len) {
+      if (p < rw.len) {
         const float m = load_mask<MASK_DT>(mask, rw.base + p);
         t.r[j] = m * reward_of(rewards[rw.base + p], p);
         if (GAE) t.v[j] = m * values[rw.base + p];
@@ -281,12 +281,12 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
       rr.neg_coef = sr.neg_coef;
       rr.eos = MASK_DT == ORLHF_MASK_NONE  // without a mask the last column is the last maximum
                    ? rw.len - 1
-                   : rw.lead + last_max_of_mask<MASK_DT>(rows, rw, rw.base + rw.lead, mask, lds_val, lds_idx);
+                   : last_max_of_mask<MASK_DT>(rows, rw, rw.base, mask, lds_val, lds_idx);
     }
     const int64_t n_tiles = (rw.len + kScanTile - 1) / kScanTile;
     double tile_carry = 0.0;  // A at the first token of the previous (later) tile
     auto whole = [&](int64_t tile) {
-      return tile * kScanTile >= rw.lead && (tile + 1) * kScanTile <= rw.len;
+      return (tile + 1) * kScanTile <= rw.len;
     };
     ScanTile cur =
         load_scan_tile<MASK_DT, GAE, REWARD>(rw, (n_tiles - 1) * kScanTile, whole(n_tiles - 1), values, rewards, mask, rr);
@@ -341,7 +341,7 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
         out_a[j] = (float)a_t;
         out_r[j] = (float)(a_t + (double)cur.v[j]);
       }
-      if (whole(tile)) {
+      if (whole(tile) || p0 + kScanItems <= rw.len) {
         if (GAE) {
           *(f32x4e*)(adv + rw.base + p0) = out_a;
           *(f32x4e*)(ret + rw.base + p0) = out_r;
@@ -352,7 +352,7 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
 #pragma unroll
         for (int j = 0; j < kScanItems; ++j) {
           const int64_t p = p0 + j;
-          if (p >= rw.lead && p < rw.len) {
+          if (p < rw.len) {
             if (GAE) {
               adv[rw.base + p] = out_a[j];
               ret[rw.base + p] = out_r[j];

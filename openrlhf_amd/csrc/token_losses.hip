@@ -5,10 +5,9 @@
 // on large batches); a workgroup walks one chunk in steps of 1024 tokens, four consecutive tokens
 // per lane, and reduces the quantities it needs to one fp64 partial per (row, chunk), all
 // quantities through the cross-lane steps together. A step is one 16-byte load per lane and array
-// (and one load of four mask elements): a row that does not start on a multiple of four elements
-// is walked from the multiple before it, so that the loads are 16-byte aligned whenever the
-// arrays are, and only its first and last step go token by token (against 4-byte loads:
-// PolicyLoss forward 206 -> 174 us, backward 286 -> 214 us on 67 M padded tokens). A fold kernel sums the chunks of each row, a
+// (and one load of four mask elements), wherever the row starts; only the lane that meets the
+// row's end goes token by token (against 4-byte loads: PolicyLoss forward 206 -> 174 us,
+// backward 286 -> 214 us on 67 M padded tokens). A fold kernel sums the chunks of each row, a
 // single-workgroup kernel folds the rows in a fixed order and writes the scalars plus a per-row
 // aggregation weight that the backward kernels multiply with. Chunks past the end of a short
 // packed row return at once. No atomics anywhere: the result is bit-reproducible. All of these
@@ -29,12 +28,8 @@ constexpr int kMaxQ = 6;                      // quantities reduced per token
 constexpr int64_t kMaxItemsGrid = 1 << 22;
 
 
-// Chunks a row of up to n_cols tokens can span: a vector walk starts up to 3 tokens before the row
-// unless every row starts on a 16-byte boundary (padded rows whose length is a multiple of four).
-static inline int64_t chunks_of(const Rows& r) {
-  const int64_t lead = (r.cu != nullptr || (r.n_cols & 3) != 0) ? 3 : 0;
-  return r.n_cols > 0 ? (r.n_cols + lead + r.chunk - 1) / r.chunk : 1;
-}
+// Chunks a row of up to n_cols tokens can span.
+static inline int64_t chunks_of(const Rows& r) { return r.n_cols > 0 ? (r.n_cols + r.chunk - 1) / r.chunk : 1; }
 
 // Rows of a chunked launch with the chunk length chosen for the problem size.
 static Rows make_rows(int64_t n_rows, int64_t n_cols, const int64_t* cu) {
@@ -199,8 +194,9 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
     for (int i = 0; i < NQ; ++i) acc[i] = 0.0;
 #pragma unroll 1
     for (int64_t s0 = c0; s0 < c0 + rows.chunk && s0 < rw.len; s0 += kSubChunk) {
-      if (s0 >= rw.lead && s0 + kSubChunk <= rw.len) {  // whole step inside the row
-        const int64_t i0 = rw.base + s0 + threadIdx.x * kTokPerLane;
+      const int64_t t0 = s0 + (int64_t)threadIdx.x * kTokPerLane;
+      if (t0 + kTokPerLane <= rw.len) {  // this lane's four tokens lie in the row
+        const int64_t i0 = rw.base + t0;
         float v[kTokPerLane][TokIn<Tok>::kN], m[kTokPerLane], q[kTokPerLane][NQ];
         load_inputs4(tok, i0, v);
         load_mask4<MASK_DT>(mask, i0, m);
@@ -211,14 +207,13 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
 #pragma unroll
           for (int i = 0; i < NQ; ++i) acc[i] += (double)q[k][i];
         }
-      } else {
+      } else {  // the lane that meets the row's end, and the lanes past it
 #pragma unroll
         for (int k = 0; k < kTokPerLane; ++k) {
-          const int64_t t = s0 + threadIdx.x + k * kBlock;
-          if (t >= rw.lead && t < rw.len) {
-            const float m = load_mask<MASK_DT>(mask, rw.base + t);
+          if (t0 + k < rw.len) {
+            const float m = load_mask<MASK_DT>(mask, rw.base + t0 + k);
             float v[TokIn<Tok>::kN], q[NQ];
-            load_inputs(tok, rw.base + t, v);
+            load_inputs(tok, rw.base + t0 + k, v);
             tok.eval(b, v, m, q);
 #pragma unroll
             for (int i = 0; i < NQ; ++i) acc[i] += (double)q[i];
@@ -440,8 +435,9 @@ __global__ __launch_bounds__(kBlock) void rows_grad_kernel(Rows rows, const void
     const float w = (g_per_row ? g_out[b] : g_out[0]) * row_coef[b];
 #pragma unroll 1
     for (int64_t s0 = c0; s0 < c0 + rows.chunk && s0 < rw.len; s0 += kSubChunk) {
-      if (s0 >= rw.lead && s0 + kSubChunk <= rw.len) {
-        const int64_t i0 = rw.base + s0 + threadIdx.x * kTokPerLane;
+      const int64_t t0 = s0 + (int64_t)threadIdx.x * kTokPerLane;
+      if (t0 + kTokPerLane <= rw.len) {
+        const int64_t i0 = rw.base + t0;
         float v[kTokPerLane][TokIn<Tok>::kN], m[kTokPerLane];
         load_inputs4(tok, i0, v);
         load_mask4<MASK_DT>(mask, i0, m);
@@ -452,12 +448,11 @@ __global__ __launch_bounds__(kBlock) void rows_grad_kernel(Rows rows, const void
       } else {
 #pragma unroll
         for (int k = 0; k < kTokPerLane; ++k) {
-          const int64_t t = s0 + threadIdx.x + k * kBlock;
-          if (t >= rw.lead && t < rw.len) {
-            const float m = load_mask<MASK_DT>(mask, rw.base + t);
+          if (t0 + k < rw.len) {
+            const float m = load_mask<MASK_DT>(mask, rw.base + t0 + k);
             float v[TokIn<Tok>::kN];
-            load_inputs(tok, rw.base + t, v);
-            g[rw.base + t] = w * m * tok.grad(b, v, m);
+            load_inputs(tok, rw.base + t0 + k, v);
+            g[rw.base + t0 + k] = w * m * tok.grad(b, v, m);
           }
         }
       }
@@ -637,7 +632,7 @@ using namespace orlhf;
 extern "C" int64_t orlhf_token_workspace_bytes(int64_t n_rows, int64_t n_cols) {
   if (n_rows < 0 || n_cols < 0) return 0;
   // chunk partials, then one folded entry per row
-  const int64_t chunks = n_cols > 0 ? (n_cols + 3 + kMinChunk - 1) / kMinChunk : 1;  // the most chunks_of() returns
+  const int64_t chunks = n_cols > 0 ? (n_cols + kMinChunk - 1) / kMinChunk : 1;  // the most chunks_of() returns
   return (n_rows > 0 ? n_rows : 1) * (chunks + 1) * kMaxQ * (int64_t)sizeof(double) + 256;
 }
 
