@@ -16,7 +16,7 @@
 
 namespace orlhf {
 
-constexpr int kTokPerLane = 4;                // loads in flight per lane and array
+constexpr int kTokPerLane = 4;                // consecutive tokens per lane and step: one 16-byte load per array
 constexpr int kSubChunk = kBlock * kTokPerLane;
 constexpr int kMinChunk = kSubChunk;          // fewest tokens of one row per work item
 constexpr int kMaxQ = 6;                      // quantities reduced per token
@@ -128,6 +128,31 @@ struct RatioTok {  // row prepass: sum(lr*m), sum(m) with lr = a - b
   __device__ __forceinline__ void eval(int64_t, const float* v, float m, float* q) const {
     q[0] = (v[0] - v[1]) * m;
     q[1] = m;
+  }
+};
+
+// PPO without importance correction and not GSPO: the common training configuration, with its
+// branches settled at compile time (the general functor decides them per token at run time).
+struct PlainPolicyTok {
+  static constexpr int kQ = PolicyTok::kQ, kIn = 3;
+  PolicyTok p;
+  __device__ __forceinline__ const float* in(int j) const { return j == 0 ? p.lp : (j == 1 ? p.old : p.adv); }
+  __device__ __forceinline__ void eval(int64_t, const float* v, float m, float* q) const {
+    const float raw = v[0] - v[1];
+    float ratio, dr, loss, dratio, clipped;
+    p.ppo_ratio(raw, ratio, dr);
+    p.surrogate(ratio, v[2], loss, dratio, clipped);
+    q[0] = loss * m;
+    q[1] = m;
+    q[2] = clipped * m;
+    q[3] = -raw * m;
+    q[4] = 0.0f;
+  }
+  __device__ __forceinline__ float grad(int64_t, const float* v, float) const {
+    float ratio, dr, loss, dratio, clipped;
+    p.ppo_ratio(v[0] - v[1], ratio, dr);
+    p.surrogate(ratio, v[2], loss, dratio, clipped);
+    return dratio * dr;
   }
 };
 
@@ -758,7 +783,10 @@ extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_lo
   }
   if (n_rows > 0) {
     PolicyTok tok = policy_tok(log_probs, old_log_probs, advantages, rollout_log_probs, row_aux, params);
-    launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
+    if (!gspo && !use_is)
+      launch_partial(mask_dtype, rows, mask, PlainPolicyTok{tok}, partial, n_chunks, s);
+    else
+      launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
     ORLHF_CHECK_LAUNCH("orlhf_policy_loss_fwd(partial)");
   }
   const int mode = (params->token_level && !gspo) ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN;
@@ -783,7 +811,10 @@ extern "C" int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs,
   const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
   PolicyTok tok = policy_tok(log_probs, old_log_probs, advantages, rollout_log_probs, row_aux, params);
   if (!tok.gspo) {
-    launch_grad(mask_dtype, rows, mask, tok, g_out, 0, row_coef, g_log_probs, s);
+    if (tok.is_mode == ORLHF_IS_NONE)
+      launch_grad(mask_dtype, rows, mask, PlainPolicyTok{tok}, g_out, 0, row_coef, g_log_probs, s);
+    else
+      launch_grad(mask_dtype, rows, mask, tok, g_out, 0, row_coef, g_log_probs, s);
     ORLHF_CHECK_LAUNCH("orlhf_policy_loss_bwd");
     return ORLHF_OK;
   }
