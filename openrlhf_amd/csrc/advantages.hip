@@ -38,7 +38,7 @@ __device__ __forceinline__ void mask_as_int4(const void* mask, int64_t i0, int64
 // Index (from the row's first token) of the last position where (int64)mask is maximal: the
 // arg-max over the flipped row that the reference takes. Called by the whole workgroup.
 template <int MASK_DT>
-__device__ __forceinline__ int64_t last_max_of_mask(const Rows& rows, const RowWalk& rw, int64_t start,
+__device__ __forceinline__ int64_t last_max_of_mask(const RowWalk& rw, int64_t start,
                                                     const void* __restrict__ mask, int64_t* lds_val,
                                                     int64_t* lds_idx) {
   int64_t best_v = INT64_MIN, best_i = -1;
@@ -135,7 +135,7 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
       continue;
     }
     const RowWalk rw = row_walk(rows, b);
-    const int64_t best_i = last_max_of_mask<MASK_DT>(rows, rw, start, mask, lds_val, lds_idx);
+    const int64_t best_i = last_max_of_mask<MASK_DT>(rw, start, mask, lds_val, lds_idx);
     const float rb = clipped_reward(r[b], has_clip, clip_lo, clip_hi);
     for_row_tokens(
         rw,
@@ -281,7 +281,7 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
       rr.neg_coef = sr.neg_coef;
       rr.eos = MASK_DT == ORLHF_MASK_NONE  // without a mask the last column is the last maximum
                    ? rw.len - 1
-                   : last_max_of_mask<MASK_DT>(rows, rw, rw.base, mask, lds_val, lds_idx);
+                   : last_max_of_mask<MASK_DT>(rw, rw.base, mask, lds_val, lds_idx);
     }
     const int64_t n_tiles = (rw.len + kScanTile - 1) / kScanTile;
     double tile_carry = 0.0;  // A at the first token of the previous (later) tile

@@ -117,7 +117,7 @@ inline bool valid_mask_dtype(int m) { return m >= ORLHF_MASK_NONE && m <= ORLHF_
 struct Rows {
   int64_t n_rows, n_cols;
   const int64_t* cu;  // packed layout when non-null
-  int chunk;          // chunked kernels: tokens of one row per work item
+  int chunk = 0;      // chunked kernels: tokens of one row per work item
 };
 
 __device__ __forceinline__ void row_span(const Rows& r, int64_t b, int64_t& start, int64_t& len) {
