@@ -124,7 +124,7 @@ class _PolicyLossFn(torch.autograd.Function):
         out4 = torch.empty(4, dtype=torch.float32, device=dev)
         row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
         row_aux = torch.empty(max(n_rows, 1) * 2, dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_policy_loss_fwd", ptr(lp), ptr(old), ptr(adv), mptr, mcode, ptr(rollout), n_rows, n_cols,
                  ptr(cu), params, ptr(ws), ptr(out4), ptr(row_coef), ptr(row_aux), stream_of(dev))
         ctx.params, ctx.keep, ctx.dims, ctx.mcode = params, keep, (n_rows, n_cols), mcode
@@ -142,7 +142,7 @@ class _PolicyLossFn(torch.autograd.Function):
         g = _f32(g_loss).reshape(-1)
         g_lp = torch.empty(lp.shape, dtype=torch.float32, device=dev)
         ws = _workspace(n_rows, n_cols, dev) if ctx.params.policy_type == _lib.POLICY_GSPO else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_policy_loss_bwd", ptr(g), ptr(lp), ptr(old), ptr(adv), ptr(mkeep), ctx.mcode, ptr(rollout),
                  n_rows, n_cols, ptr(cu), ctx.params, ptr(row_coef), ptr(row_aux), ptr(ws), ptr(g_lp),
                  stream_of(dev))
@@ -246,7 +246,7 @@ class _ValueLossFn(torch.autograd.Function):
         out = torch.empty(1, dtype=torch.float32, device=dev)
         row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
         has_clip = clip_eps is not None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_value_loss_fwd", ptr(v), ptr(old), ptr(ret), mptr, mcode, n_rows, n_cols, ptr(cu),
                  1 if has_clip else 0, float(clip_eps) if has_clip else 0.0, 1 if token_level else 0, norm,
                  ptr(ws), ptr(out), ptr(row_coef), stream_of(dev))
@@ -262,7 +262,7 @@ class _ValueLossFn(torch.autograd.Function):
         n_rows, n_cols = ctx.dims
         g = _f32(g_out).reshape(-1)
         g_v = torch.empty(v.shape, dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_value_loss_bwd", ptr(g), ptr(v), ptr(old), ptr(ret), ptr(mkeep), ctx.mcode, n_rows, n_cols,
                  ptr(cu), 1 if ctx.clip[0] else 0, ctx.clip[1], ptr(row_coef), ptr(g_v), stream_of(dev))
         return g_v.view(ctx.v_shape).to(ctx.v_dtype), None, None, None, None, None, None, None, None
@@ -311,7 +311,7 @@ class _PairLossFn(torch.autograd.Function):
         loss = torch.empty(1, dtype=torch.float32, device=dev)
         cr = torch.empty(n, dtype=torch.float32, device=dev) if want_rewards else None
         rr = torch.empty(n, dtype=torch.float32, device=dev) if want_rewards else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_pair_loss_fwd", ptr(a), ptr(b), ptr(c), ptr(d), n, kind, float(beta), float(label_smoothing),
                  ptr(loss), ptr(cr), ptr(rr), stream_of(dev))
         ctx.save_for_backward(a, b, c, d)
@@ -329,7 +329,7 @@ class _PairLossFn(torch.autograd.Function):
         g = g_loss.reshape(1).to(torch.float32).contiguous()
         ga = torch.empty_like(a) if ctx.needs_input_grad[0] else None
         gb = torch.empty_like(b) if ctx.needs_input_grad[1] else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_pair_loss_bwd", ptr(g), ptr(a), ptr(b), ptr(c), ptr(d), a.numel(), kind, beta, smooth,
                  ptr(ga), ptr(gb), stream_of(dev))
         ga = None if ga is None else ga.view(shape).to(dt_a)

@@ -74,7 +74,7 @@ class _LogprobEntropy(torch.autograd.Function):
         logprob = torch.empty(n_rows, **opts) if want_logprob else None
         entropy = torch.empty(n_rows, **opts) if want_entropy else None
         stats = torch.empty(n_rows, 4, **opts) if needs_grad else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call(
                 "orlhf_logprob_entropy_fwd", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
                 float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), 0, stream_of(dev),
@@ -106,7 +106,7 @@ class _LogprobEntropy(torch.autograd.Function):
         else:
             grad_rows = torch.empty((n_rows, vocab), device=dev, dtype=rows.dtype)
             grad_stride = vocab
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call(
                 "orlhf_logprob_entropy_bwd", ptr(rows), ptr(grad_rows), code, n_rows, vocab,
                 ctx.row_stride, grad_stride, ptr(lab), ctx.temperature, ptr(glp), ptr(gent),
@@ -167,7 +167,7 @@ def log_probs_from_logits(
         rows, row_stride, aliases = _as_rows(logits.detach())
         if not aliases:
             raise ValueError("mutate_logits=True needs logits whose rows can be addressed in place")
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_divide_rows_inplace", ptr(rows), _lib.dtype_code(rows), rows.shape[0], rows.shape[1],
                  row_stride, float(temperature), stream_of(dev))
         torch.autograd.graph.increment_version(rows)
@@ -240,7 +240,7 @@ class _ApproxKL(torch.autograd.Function):
         lp, base = torch.broadcast_tensors(lp, base)
         lp, base = lp.contiguous(), base.contiguous()
         out = torch.empty(lp.shape, dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_approx_kl_fwd", ptr(lp), ptr(base), _lib.dtype_code(lp), lp.numel(), estimator,
                  ptr(out), stream_of(dev))
         ctx.estimator = estimator
@@ -258,7 +258,7 @@ class _ApproxKL(torch.autograd.Function):
         g_lp = torch.empty(lp.shape, dtype=torch.float32, device=dev) if need_lp else None
         g_base = torch.empty(lp.shape, dtype=torch.float32, device=dev) if need_base else None
         if need_lp or need_base:
-            with torch.cuda.device(dev):
+            with _lib.on_device(dev):
                 call("orlhf_approx_kl_bwd", ptr(lp), ptr(base), _lib.dtype_code(lp), lp.numel(),
                      ctx.estimator, ptr(g_out), ptr(g_lp), ptr(g_base), stream_of(dev))
 
@@ -301,7 +301,7 @@ class _Aggregate(torch.autograd.Function):
         ws = _workspace(n_rows, n_cols, dev)
         out = torch.empty(n_rows if mode == _lib.AGG_ROW_MEAN else 1, dtype=torch.float32, device=dev)
         row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_masked_aggregate_fwd", ptr(xf), mptr, mcode, n_rows, n_cols, ptr(cu), mode, norm,
                  ptr(ws), ptr(out), ptr(row_coef), stream_of(dev))
         ctx.mode, ctx.dims, ctx.mcode = mode, (n_rows, n_cols), mcode
@@ -318,7 +318,7 @@ class _Aggregate(torch.autograd.Function):
         n_rows, n_cols = ctx.dims
         g = _f32(g_out).reshape(-1)
         g_x = torch.empty(ctx.x_shape, dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_masked_aggregate_bwd", ptr(g), ptr(mkeep), ctx.mcode, n_rows, n_cols, ptr(cu), ctx.mode,
                  ptr(row_coef), ptr(g_x), stream_of(dev))
         return g_x.to(ctx.x_dtype), None, None, None, None, None
@@ -360,7 +360,7 @@ def compute_reward(
     cu = _cu_arg(cu_seqlens, dev)
     out = torch.empty_like(klf)
     lo, hi = (reward_clip_range[0], reward_clip_range[1]) if reward_clip_range else (0.0, 0.0)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_compute_reward", ptr(rf), float(kl_coef), ptr(klf), mptr, mcode, n_rows, n_cols, ptr(cu),
              1 if reward_clip_range else 0, float(lo), float(hi), ptr(out), None, stream_of(dev))
     return out
@@ -381,7 +381,7 @@ def masked_normalize(tensor: torch.Tensor, mask: torch.Tensor, dim: int = 1, eps
     n_cols = x.shape[-1]
     n_rows = x.numel() // n_cols if n_cols else 0
     out = torch.empty_like(x)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_masked_normalize_rows", ptr(x), mptr, mcode, n_rows, n_cols, None, float(eps), ptr(out),
              stream_of(dev))
     out = out.movedim(-1, d) if d != nd - 1 else out
@@ -435,7 +435,7 @@ def fused_logprob_entropy_fwd_bwd(
     same_phase = ((rows.data_ptr() ^ grad_rows.data_ptr()) & 15) == 0 and (
         ((row_stride - grad_stride) * rows.element_size()) & 15
     ) == 0
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         if fits and same_phase:
             call("orlhf_logprob_entropy_fwd_bwd", ptr(rows), ptr(grad_rows), code, n_rows, vocab, row_stride,
                  grad_stride, ptr(lab), float(temperature), ptr(wlp), ptr(went), ptr(logprob), ptr(entropy),

@@ -37,7 +37,7 @@ class _SequenceLogps(torch.autograd.Function):
         mkeep, mptr, mcode = _lib.mask_arg(attention_mask)
         sums = torch.empty(n_rows, dtype=torch.float32, device=dev)
         means, counts = torch.empty_like(sums), torch.empty_like(sums)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_sequence_logps_fwd", ptr(lp), mptr, mcode, ptr(prompt_lens), n_rows, n_cols, ptr(sums),
                  ptr(means), ptr(counts), stream_of(dev))
         ctx.save_for_backward(mkeep, prompt_lens, counts)
@@ -51,7 +51,7 @@ class _SequenceLogps(torch.autograd.Function):
         dev = counts.device
         gs, gm = _f32(g_sums), _f32(g_means)
         g = torch.empty(n_rows, n_cols, dtype=torch.float32, device=dev)
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_sequence_logps_bwd", ptr(gs), ptr(gm), ptr(mkeep), mcode, ptr(prompt_lens), ptr(counts),
                  n_rows, n_cols, ptr(g), stream_of(dev))
         return g.to(dtype), None, None

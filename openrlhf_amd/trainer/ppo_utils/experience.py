@@ -38,7 +38,7 @@ def row_extents(mask: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor, torch.T
     mkeep, mptr, mcode = _lib.mask_arg(mask)
     first = torch.empty(n_rows, dtype=torch.int64, device=dev)
     end, length = torch.empty_like(first), torch.empty_like(first)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_row_extents", mptr, mcode, n_rows, n_cols, ptr(first), ptr(end), ptr(length), stream_of(dev))
     return first, end, length
 
@@ -48,7 +48,7 @@ def cu_seqlens_of(lengths: torch.Tensor) -> torch.Tensor:
     dev = require_gpu(lengths)
     lens = lengths.reshape(-1).to(torch.int64).contiguous()
     cu = torch.empty(lens.numel() + 1, dtype=torch.int64, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_cu_seqlens", ptr(lens), lens.numel(), ptr(cu), stream_of(dev))
     return cu
 
@@ -71,7 +71,7 @@ def pack_padded(x: torch.Tensor, cu_seqlens: torch.Tensor, first: Optional[torch
         return out
     cu = cu_seqlens.to(torch.int64).contiguous()
     f = None if first is None else first.to(torch.int64).contiguous()
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_pack_rows", ptr(src), src.element_size(), x.shape[0], x.shape[1], ptr(f), ptr(cu), ptr(out),
              stream_of(dev))
     return out
@@ -90,7 +90,7 @@ def pad_packed(flat: torch.Tensor, cu_seqlens: torch.Tensor, n_cols: int, side: 
     n_rows = cu_seqlens.numel() - 1
     cu = cu_seqlens.to(torch.int64).contiguous()
     out = torch.empty(n_rows, int(n_cols), dtype=flat.dtype, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_pad_rows", ptr(src), src.element_size(), ptr(cu), n_rows, int(n_cols), 1 if side == "left" else 0,
              _fill_bits(value, flat.dtype), ptr(out), stream_of(dev))
     return out

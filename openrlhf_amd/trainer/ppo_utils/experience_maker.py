@@ -95,7 +95,7 @@ def experience_kl(
     kl_mean = torch.empty(n_rows, dtype=torch.float32, device=dev)
     diff_mean = torch.empty(n_rows, dtype=torch.float32, device=dev)
     code = _lib.dtype_code(lp) if enabled else _lib.F32
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_kl_rows", ptr(lp) if enabled else None, ptr(base), code, mptr, mcode, n_rows, n_cols, ptr(cu),
              _KL_CODES[kl_estimator], 1 if enabled else 0, ptr(kl), ptr(kl_mean), ptr(diff_mean), stream_of(dev))
     if not enabled:  # the reference keeps the log-prob dtype for its zeros
@@ -123,7 +123,7 @@ def get_advantages_and_returns(
     n_rows, n_cols = _rows_of(v, _packed(cu_seqlens, max_seqlen if max_seqlen is not None else v.numel()))
     cu = _cu_arg(cu_seqlens, dev)
     adv, ret = torch.empty_like(v), torch.empty_like(v)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_gae_scan", ptr(v), ptr(r), mptr, mcode, n_rows, n_cols, ptr(cu), float(gamma), float(lambd),
              ptr(adv), ptr(ret), stream_of(dev))
     return adv.to(home), ret.to(home)
@@ -144,7 +144,7 @@ def get_cumulative_returns(
     n_rows, n_cols = _rows_of(r, _packed(cu_seqlens, max_seqlen if max_seqlen is not None else r.numel()))
     cu = _cu_arg(cu_seqlens, dev)
     ret = torch.empty_like(r)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_discounted_returns", ptr(r), mptr, mcode, n_rows, n_cols, ptr(cu), float(gamma), ptr(ret),
              stream_of(dev))
     return ret.to(home)
@@ -183,7 +183,7 @@ def reward_advantages_and_returns(
     ret = torch.empty_like(klf)
     total = torch.empty(n_rows, dtype=torch.float32, device=dev)
     lo, hi = (reward_clip_range[0], reward_clip_range[1]) if reward_clip_range else (0.0, 0.0)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_reward_scan", ptr(rf), float(kl_coef), ptr(klf), ptr(v), mptr, mcode, n_rows, n_cols, ptr(cu),
              1 if reward_clip_range else 0, float(lo), float(hi), float(gamma), float(lambd), ptr(adv), ptr(ret),
              ptr(total), stream_of(dev))
@@ -216,7 +216,7 @@ def group_normalize_rewards(
     out = torch.empty_like(r)
     std = torch.empty_like(r) if n > 1 else None
     ws = torch.empty(max(n_total, 1), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_group_normalize", ptr(r), ptr(idx), n_total // n, n, _GROUP_CODES[estimator], ptr(out), ptr(std),
              ptr(ws), stream_of(dev))
     return out.to(home), (None if std is None else std.to(home))
@@ -253,7 +253,7 @@ def whiten_advantages(
     x_ptrs = (ctypes.c_void_p * k)(*[x.data_ptr() for x in xs])
     m_ptrs = (ctypes.c_void_p * k)(*[mp for _, mp, _ in masks])
     o_ptrs = (ctypes.c_void_p * k)(*[o.data_ptr() for o in outs])
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_masked_whiten_multi", x_ptrs, m_ptrs, mcode, ns, k, 0 if no_std_norm else 1, ptr(ws), o_ptrs,
              None, stream_of(dev))
     return [o.view(a.shape).to(home) for o, a in zip(outs, advantages)]

@@ -69,7 +69,7 @@ def _aggregation_coef(action_mask, token_level, dp_size, norm_value):
     dummy = torch.zeros(b, a, dtype=torch.float32, device=dev)
     out = torch.empty(1, dtype=torch.float32, device=dev)
     row_coef = torch.empty(max(b, 1), dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_masked_aggregate_fwd", ptr(dummy), mptr, mcode, b, a, None,
              _lib.AGG_TOKEN_MEAN if token_level else _lib.AGG_SEQ_MEAN, norm, ptr(ws), ptr(out), ptr(row_coef),
              stream_of(dev))
@@ -92,7 +92,7 @@ class _HandOverGradient(torch.autograd.Function):
         (grad,) = ctx.saved_tensors
         dev = grad.device
         gf = g.reshape(-1)[:1].to(torch.float32).contiguous()
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_rescale_inplace_if", ptr(grad), _lib.dtype_code(grad), grad.numel(), ptr(gf),
                  ctx.produced_scale, stream_of(dev))
         return grad, None, None, None
@@ -184,7 +184,7 @@ def fused_actor_loss_step(
 
         lp_r = torch.empty(n_rows, dtype=torch.float32, device=dev)
         ent_r = torch.empty(n_rows, dtype=torch.float32, device=dev) if want_entropy else None
-        with torch.cuda.device(dev):
+        with _lib.on_device(dev):
             call("orlhf_policy_step_fwd_bwd", ptr(rows), ptr(rows), code, n_rows, vocab, row_stride, row_stride,
                  ptr(labels), float(temperature), terms, ptr(lp_r), ptr(ent_r), ptr(need_r), stream_of(dev))
         torch.autograd.graph.increment_version(rows)

@@ -34,7 +34,7 @@ def mask_counts(loss_mask: torch.Tensor):
     mkeep, mptr, mcode = _lib.mask_arg(rows)
     ws = _workspace(b, a, dev)
     out = torch.empty(2, dtype=torch.float32, device=dev)
-    with torch.cuda.device(dev):
+    with _lib.on_device(dev):
         call("orlhf_mask_counts", mptr, mcode, b, a, None, ptr(ws), ptr(out), stream_of(dev))
     return out[0], out[1]
 
