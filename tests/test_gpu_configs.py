@@ -154,6 +154,11 @@ def test_config3_critic_gae_path(cuda):
     for got, want in ((rew, rew64), (adv, adv64), (ret, ret64), (white, white64)):
         scale = want.abs().max().item()
         assert (got.cpu().double() - want).abs().max().item() <= 1e-5 * scale
+    # reward shaping and GAE in one pass: the same bits, and the row sums of the reward
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import reward_advantages_and_returns
+    adv1, ret1, total = reward_advantages_and_returns(r.to(d), 0.01, kl, values.to(d), mask.to(d), 1.0, 0.95)
+    assert torch.equal(adv1, adv) and torch.equal(ret1, ret)
+    assert (total.cpu().double() - rew64.sum(1)).abs().max().item() <= 1e-5 * rew64.sum(1).abs().max().item()
     v = new_values.to(d).requires_grad_(True)
     loss = ValueLoss(0.2)(v, values.to(d), ret, action_mask=mask.to(d))
     assert abs(loss.item() - loss64.item()) <= 1e-5
