@@ -140,7 +140,7 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
     for_row_tokens(
         rw,
         [&](int64_t i0) {
-          const f32x4 k4 = *(const f32x4e*)(kl + i0);
+          const f32x4 k4 = stream_load4(kl + i0);
           f32x4 o;
 #pragma unroll
           for (int k = 0; k < 4; ++k) o[k] = ((i0 + k - start == best_i) ? rb : 0.0f) + neg_coef * k4[k];
@@ -201,9 +201,9 @@ __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t ti
   if (whole || p0 + kScanItems <= rw.len) {  // this lane's four tokens lie in the row
     float m[kScanItems];
     load_mask4<MASK_DT>(mask, rw.base + p0, m);
-    const f32x4 r4 = *(const f32x4e*)(rewards + rw.base + p0);
+    const f32x4 r4 = stream_load4(rewards + rw.base + p0);
     f32x4 v4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (GAE) v4 = *(const f32x4e*)(values + rw.base + p0);
+    if (GAE) v4 = *(const f32x4e*)(values + rw.base + p0);  // plain: the last lane re-reads across the wave's end
 #pragma unroll
     for (int j = 0; j < kScanItems; ++j) {
       t.r[j] = m[j] * reward_of(r4[j], p0 + j);
@@ -500,7 +500,7 @@ __global__ __launch_bounds__(kBlock) void whiten_apply_kernel(const float* x, in
   const int64_t groups = n / 4;
 #pragma unroll 2
   for (int64_t g = first; g < groups; g += stride) {
-    const f32x4 v = *(const f32x4e*)(x + g * 4);
+    const f32x4 v = stream_load4(x + g * 4);
     f32x4 o;
 #pragma unroll
     for (int k = 0; k < 4; ++k) o[k] = (v[k] - mean) * rstd;
@@ -593,7 +593,7 @@ __global__ __launch_bounds__(kBlock) void whiten_apply_multi_kernel(WhitenSegs s
   for_span(
       lo, hi,
       [&](int64_t i0) {
-        const f32x4 v = *(const f32x4e*)(x + i0);
+        const f32x4 v = stream_load4(x + i0);
         f32x4 o;
 #pragma unroll
         for (int k = 0; k < 4; ++k) o[k] = (v[k] - mean) * rstd;

@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__
     typedef typename Vec16<E>::type V;
     const int64_t groups = (stop - j0) / kE;
 #pragma unroll 2
-    for (int64_t g = threadIdx.x; g < groups; g += kBlock) *(V*)(out + j0 + g * kE) = *(const V*)(in + j0 + g * kE);
+    for (int64_t g = threadIdx.x; g < groups; g += kBlock) *(V*)(out + j0 + g * kE) = __builtin_nontemporal_load((const V*)(in + j0 + g * kE));
     for (int64_t j = j0 + groups * kE + threadIdx.x; j < stop; j += kBlock) out[j] = in[j];
   }
 }
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ 
     for (int64_t g = threadIdx.x; g < groups; g += kBlock) {
       const int64_t t = t0 + g * kE;
       if (t >= shift && t + kE <= shift + len) {  // all of the group's columns hold tokens
-        *(V*)(out + t) = *(const V*)(src + start + (t - shift));
+        *(V*)(out + t) = __builtin_nontemporal_load((const V*)(src + start + (t - shift)));
       } else if (t + kE <= shift || t >= shift + len) {  // all padding
         *(V*)(out + t) = fill_v;
       } else {

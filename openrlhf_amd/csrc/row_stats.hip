@@ -136,7 +136,7 @@ __global__ __launch_bounds__(kBlock) void masked_normalize_rows_kernel(const flo
     for_row_tokens(
         rw,
         [&](int64_t i0) {
-          const f32x4 xv = *(const f32x4e*)(x + i0);
+          const f32x4 xv = stream_load4(x + i0);
           float m[4];
           load_mask4<MASK_DT>(mask, i0, m);
           f32x4 o;

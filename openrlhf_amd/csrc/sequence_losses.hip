@@ -42,7 +42,7 @@ __global__ __launch_bounds__(kBlock) void sequence_logps_fwd_kernel(const float*
     for_row_tokens(
         rw,
         [&](int64_t i0) {
-          const f32x4 x = *(const f32x4e*)(lp + i0);
+          const f32x4 x = stream_load4(lp + i0);
           const int64_t t0 = i0 - b * n_cols;
           float a[4];
           load_mask4<MASK_DT>(att, b * (n_cols + 1) + t0 + 1, a);

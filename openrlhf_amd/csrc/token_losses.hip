@@ -189,7 +189,7 @@ __device__ __forceinline__ void load_inputs4(const Tok& tok, int64_t i0, float (
   for (int j = 0; j < Tok::kIn; ++j) {
     const float* p = tok.in(j);
     f32x4 x = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (p != nullptr) x = *(const f32x4e*)(p + i0);
+    if (p != nullptr) x = stream_load4(p + i0);
 #pragma unroll
     for (int k = 0; k < 4; ++k) v[k][j] = x[k];
   }
@@ -556,7 +556,7 @@ __global__ __launch_bounds__(kBlock) void approx_kl_bwd_kernel(const void* __res
     float x[4], y[4];
     load_lp4<DT>(lp, g * 4, x);
     load_lp4<DT>(base, g * 4, y);
-    const f32x4 up = *(const f32x4e*)(g_out + g * 4);
+    const f32x4 up = stream_load4(g_out + g * 4);
     f32x4 o, neg;
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
