@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
           f32x4 o;
 #pragma unroll
           for (int k = 0; k < 4; ++k) o[k] = ((i0 + k - start == best_i) ? rb : 0.0f) + neg_coef * k4[k];
-          *(f32x4e*)(reward + i0) = o;
+          __builtin_nontemporal_store(o, (f32x4e*)(reward + i0));
         },
         [&](int64_t i) { reward[i] = ((i - start == best_i) ? rb : 0.0f) + neg_coef * kl[i]; });
     if (threadIdx.x == 0 && eos_index != nullptr) eos_index[b] = best_i;
@@ -342,9 +342,9 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
         out_r[j] = (float)(a_t + (double)cur.v[j]);
       }
       if (whole(tile) || p0 + kScanItems <= rw.len) {
-        if (GAE) {
-          *(f32x4e*)(adv + rw.base + p0) = out_a;
-          *(f32x4e*)(ret + rw.base + p0) = out_r;
+        if (GAE) {  // non-temporal: 10 % faster here (not for the single output of the returns)
+          __builtin_nontemporal_store(out_a, (f32x4e*)(adv + rw.base + p0));
+          __builtin_nontemporal_store(out_r, (f32x4e*)(ret + rw.base + p0));
         } else {
           *(f32x4e*)(ret + rw.base + p0) = out_a;
         }
