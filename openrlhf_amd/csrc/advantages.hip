@@ -2,10 +2,10 @@
 // parallel reverse-time scan, group baselines and global masked whitening. Forward only.
 //
 // The scan: A_t = delta_t + c * A_{t+1} is a linear recurrence with a constant coefficient, so a
-// lane that owns kScanItems consecutive tokens reduces them to an affine map C -> b + a*C of the
+// lane that owns ITEMS consecutive tokens reduces them to an affine map C -> b + a*C of the
 // carry C entering from later tokens. Maps compose associatively; a wave composes its 64 maps with
 // log2(64) cross-lane steps, the 4 waves of the workgroup chain through LDS, and a row longer than
-// one tile (kBlock * kScanItems tokens) walks its tiles from the end carrying one number. Carries
+// one tile (kBlock * ITEMS tokens) walks its tiles from the end carrying one number. Carries
 // and the in-lane recurrence are fp64, inputs and outputs fp32. A tile goes through LDS both ways
 // so that global loads and stores are coalesced while each lane works on consecutive tokens.
 #include "common.h"
@@ -152,8 +152,9 @@ __global__ __launch_bounds__(kBlock) void compute_reward_kernel(Rows rows, const
 }
 
 // ---------------------------------------------------------------- reverse scan (GAE, returns)
-constexpr int kScanItems = 4;  // tokens per lane and tile; 8 and 16 measured 25 % and 60 % slower
-constexpr int kScanTile = kBlock * kScanItems;
+// Tokens per lane and tile (ITEMS below): 4 for GAE (8 is 75 % slower there: registers), 8 for the
+// discounted returns with their single input and output (8 % faster than 4).
+constexpr int kGaeItems = 4, kReturnItems = 8;
 
 struct Affine {  // C -> b + a * C
   double a, b;
@@ -166,11 +167,12 @@ __device__ __forceinline__ Affine compose(const Affine& outer, const Affine& inn
   return r;
 }
 
-// One tile of a row in registers: this lane's kScanItems consecutive tokens, masked, plus the
+// One tile of a row in registers: this lane's ITEMS consecutive tokens, masked, plus the
 // value that follows them (the next lane's first; the next tile's first for the last lane).
+template <int ITEMS>
 struct ScanTile {
-  float r[kScanItems];
-  float v[kScanItems + 1];
+  float r[ITEMS];
+  float v[ITEMS + 1];
 };
 
 // Per-token rewards made on the fly from the KL estimate (REWARD mode of the scan): the token
@@ -184,34 +186,37 @@ struct RowReward {
 
 // `whole`: the tile lies inside the row (no lane needs to look at the row's end). Must be called by
 // all lanes of the workgroup (it exchanges the following value across lanes).
-template <int MASK_DT, bool GAE, bool REWARD>
-__device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t tile0, bool whole,
+template <int MASK_DT, bool GAE, bool REWARD, int ITEMS>
+__device__ __forceinline__ ScanTile<ITEMS> load_scan_tile(const RowWalk& rw, int64_t tile0, bool whole,
                                                    const float* __restrict__ values,
                                                    const float* __restrict__ rewards,
                                                    const void* __restrict__ mask, RowReward& rr) {
-  static_assert(kScanItems == 4, "a lane's tokens are one 16-byte load");
-  ScanTile t;
-  const int64_t p0 = tile0 + (int64_t)threadIdx.x * kScanItems;
+  static_assert(ITEMS == 4 || ITEMS == 8, "a lane's tokens are one or two 16-byte loads");
+  ScanTile<ITEMS> t;
+  const int64_t p0 = tile0 + (int64_t)threadIdx.x * ITEMS;
   auto reward_of = [&](float raw, int64_t p) {
     if (!REWARD) return raw;
     const float tok = ((p == rr.eos) ? rr.seq : 0.0f) + rr.neg_coef * raw;
     rr.sum += (double)tok;
     return tok;
   };
-  if (whole || p0 + kScanItems <= rw.len) {  // this lane's four tokens lie in the row
-    float m[kScanItems];
-    load_mask4<MASK_DT>(mask, rw.base + p0, m);
-    const f32x4 r4 = stream_load4(rewards + rw.base + p0);
-    f32x4 v4 = {0.0f, 0.0f, 0.0f, 0.0f};
-    if (GAE) v4 = *(const f32x4e*)(values + rw.base + p0);  // plain: the last lane re-reads across the wave's end
+  if (whole || p0 + ITEMS <= rw.len) {  // this lane's four tokens lie in the row
 #pragma unroll
-    for (int j = 0; j < kScanItems; ++j) {
-      t.r[j] = m[j] * reward_of(r4[j], p0 + j);
-      t.v[j] = m[j] * v4[j];
+    for (int q = 0; q < ITEMS / 4; ++q) {
+      float m[4];
+      load_mask4<MASK_DT>(mask, rw.base + p0 + q * 4, m);
+      const f32x4 r4 = stream_load4(rewards + rw.base + p0 + q * 4);
+      f32x4 v4 = {0.0f, 0.0f, 0.0f, 0.0f};
+      if (GAE) v4 = *(const f32x4e*)(values + rw.base + p0 + q * 4);  // plain: the last lane re-reads across the wave's end
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        t.r[q * 4 + j] = m[j] * reward_of(r4[j], p0 + q * 4 + j);
+        t.v[q * 4 + j] = m[j] * v4[j];
+      }
     }
   } else {  // the lane that meets the row's end, and the lanes past it
 #pragma unroll
-    for (int j = 0; j < kScanItems; ++j) {
+    for (int j = 0; j < ITEMS; ++j) {
       const int64_t p = p0 + j;
       t.r[j] = 0.0f;
       t.v[j] = 0.0f;
@@ -222,16 +227,31 @@ __device__ __forceinline__ ScanTile load_scan_tile(const RowWalk& rw, int64_t ti
       }
     }
   }
-  t.v[kScanItems] = 0.0f;
+  t.v[ITEMS] = 0.0f;
   if (GAE) {
     const float from_next_lane = __shfl_down(t.v[0], 1, kWave);
-    const int64_t p = p0 + kScanItems;  // first token of the next wave (or tile) for the last lane
+    const int64_t p = p0 + ITEMS;  // first token of the next wave (or tile) for the last lane
     float after = 0.0f;
     if ((threadIdx.x & (kWave - 1)) == kWave - 1 && p < rw.len)
       after = load_mask<MASK_DT>(mask, rw.base + p) * values[rw.base + p];
-    t.v[kScanItems] = (threadIdx.x & (kWave - 1)) == kWave - 1 ? after : from_next_lane;
+    t.v[ITEMS] = (threadIdx.x & (kWave - 1)) == kWave - 1 ? after : from_next_lane;
   }
   return t;
+}
+
+// Four consecutive outputs of a lane. GAE's two outputs leave with non-temporal stores (10 %
+// faster there; the single output of the returns is faster with plain stores).
+template <bool GAE>
+__device__ __forceinline__ void store_scan4(float* __restrict__ adv, float* __restrict__ ret, int64_t i0,
+                                            const float* a, const float* r) {
+  const f32x4 a4 = {a[0], a[1], a[2], a[3]};
+  if (GAE) {
+    const f32x4 r4 = {r[0], r[1], r[2], r[3]};
+    __builtin_nontemporal_store(a4, (f32x4e*)(adv + i0));
+    __builtin_nontemporal_store(r4, (f32x4e*)(ret + i0));
+  } else {
+    *(f32x4e*)(ret + i0) = a4;
+  }
 }
 
 // One workgroup per row, walking it backwards in tiles of kScanTile tokens; the tile before the
@@ -253,6 +273,7 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
                                                               const void* __restrict__ mask, double gamma,
                                                               double coef, SeqReward sr, float* __restrict__ adv,
                                                               float* __restrict__ ret) {
+  constexpr int ITEMS = GAE ? kGaeItems : kReturnItems, kScanTile = kBlock * ITEMS;
   __shared__ Affine lds_wave[2][kWavesPerBlock];  // alternating: one barrier per tile is enough
   __shared__ int64_t lds_val[kWavesPerBlock];
   __shared__ int64_t lds_idx[kWavesPerBlock];
@@ -260,10 +281,10 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
 
-  double pw[kScanItems + 1];  // coef^k
+  double pw[ITEMS + 1];  // coef^k
   pw[0] = 1.0;
 #pragma unroll
-  for (int k = 1; k <= kScanItems; ++k) pw[k] = pw[k - 1] * coef;
+  for (int k = 1; k <= ITEMS; ++k) pw[k] = pw[k - 1] * coef;
 
   const int slot_b = slot_bits(rows.n_rows);
   int buf = 0;
@@ -288,18 +309,18 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
     auto whole = [&](int64_t tile) {
       return (tile + 1) * kScanTile <= rw.len;
     };
-    ScanTile cur =
-        load_scan_tile<MASK_DT, GAE, REWARD>(rw, (n_tiles - 1) * kScanTile, whole(n_tiles - 1), values, rewards, mask, rr);
+    ScanTile<ITEMS> cur =
+        load_scan_tile<MASK_DT, GAE, REWARD, ITEMS>(rw, (n_tiles - 1) * kScanTile, whole(n_tiles - 1), values, rewards, mask, rr);
     for (int64_t tile = n_tiles - 1; tile >= 0; --tile) {
       const int64_t tile0 = tile * kScanTile;
-      ScanTile nxt = cur;
+      ScanTile<ITEMS> nxt = cur;
       if (tile > 0)
-        nxt = load_scan_tile<MASK_DT, GAE, REWARD>(rw, tile0 - kScanTile, whole(tile - 1), values, rewards, mask, rr);
+        nxt = load_scan_tile<MASK_DT, GAE, REWARD, ITEMS>(rw, tile0 - kScanTile, whole(tile - 1), values, rewards, mask, rr);
       // in-lane recurrence with zero carry-in
-      double local[kScanItems];
+      double local[ITEMS];
       double run = 0.0;
 #pragma unroll
-      for (int j = kScanItems - 1; j >= 0; --j) {
+      for (int j = ITEMS - 1; j >= 0; --j) {
         const double delta =
             GAE ? ((double)cur.r[j] + gamma * (double)cur.v[j + 1]) - (double)cur.v[j] : (double)cur.r[j];
         run = delta + coef * run;
@@ -307,7 +328,7 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
       }
       // inclusive suffix composition over the wave: lane i ends with the map of lanes i..63
       Affine f;
-      f.a = pw[kScanItems];
+      f.a = pw[ITEMS];
       f.b = local[0];
 #pragma unroll
       for (int d = 1; d < kWave; d <<= 1) {
@@ -333,24 +354,20 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
       after.a = __shfl_down(f.a, 1, kWave);
       after.b = __shfl_down(f.b, 1, kWave);
       const double carry = (lane == kWave - 1) ? wave_carry : after.b + after.a * wave_carry;
-      const int64_t p0 = tile0 + (int64_t)threadIdx.x * kScanItems;
-      f32x4 out_a, out_r;
+      const int64_t p0 = tile0 + (int64_t)threadIdx.x * ITEMS;
+      float out_a[ITEMS], out_r[ITEMS];
 #pragma unroll
-      for (int j = 0; j < kScanItems; ++j) {
-        const double a_t = local[j] + pw[kScanItems - j] * carry;
+      for (int j = 0; j < ITEMS; ++j) {
+        const double a_t = local[j] + pw[ITEMS - j] * carry;
         out_a[j] = (float)a_t;
         out_r[j] = (float)(a_t + (double)cur.v[j]);
       }
-      if (whole(tile) || p0 + kScanItems <= rw.len) {
-        if (GAE) {  // non-temporal: 10 % faster here (not for the single output of the returns)
-          __builtin_nontemporal_store(out_a, (f32x4e*)(adv + rw.base + p0));
-          __builtin_nontemporal_store(out_r, (f32x4e*)(ret + rw.base + p0));
-        } else {
-          *(f32x4e*)(ret + rw.base + p0) = out_a;
-        }
+      if (whole(tile) || p0 + ITEMS <= rw.len) {
+        store_scan4<GAE>(adv, ret, rw.base + p0, out_a, out_r);
+        if (ITEMS == 8) store_scan4<GAE>(adv, ret, rw.base + p0 + 4, out_a + 4, out_r + 4);
       } else {
 #pragma unroll
-        for (int j = 0; j < kScanItems; ++j) {
+        for (int j = 0; j < ITEMS; ++j) {
           const int64_t p = p0 + j;
           if (p < rw.len) {
             if (GAE) {
