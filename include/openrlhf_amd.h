@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 11
+#define ORLHF_ABI_VERSION 12
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -287,11 +287,13 @@ int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs, const floa
 /*
  * ValueLoss.forward (openrlhf/models/loss.py:244-269): 0.5 * aggregate(max((vc-R)^2, (v-R)^2)),
  * vc = old + clamp(v - old, -eps, eps); has_clip == 0 gives 0.5 * aggregate((v-R)^2).
+ *   out2 float [2]: loss, masked mean of the values (the "values" status of
+ *   openrlhf/trainer/ray/ppo_critic.py:174, from the same pass)
  */
 int orlhf_value_loss_fwd(const float* values, const float* old_values, const float* returns,
                          const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
                          const int64_t* cu_seqlens, int has_clip, float clip_eps, int token_level,
-                         const orlhf_norm* norm, void* workspace, float* out, float* row_coef,
+                         const orlhf_norm* norm, void* workspace, float* out2, float* row_coef,
                          orlhf_stream_t stream);
 int orlhf_value_loss_bwd(const float* g_out, const float* values, const float* old_values,
                          const float* returns, const void* mask, int mask_dtype, int64_t n_rows,

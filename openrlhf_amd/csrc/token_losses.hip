@@ -78,8 +78,8 @@ struct AggTok {  // aggregate_loss / masked_mean: x*m and m
   }
 };
 
-struct ValueTok {
-  static constexpr int kQ = 2, kIn = 3;
+struct ValueTok {  // quantities: masked loss, mask, masked value (for the mean value the trainer logs)
+  static constexpr int kQ = 3, kIn = 3;
   const float *v, *old, *ret;
   int has_clip;
   float eps;
@@ -113,6 +113,7 @@ struct ValueTok {
     both(in, loss, dv);
     q[0] = loss * m;
     q[1] = m;
+    q[2] = in[0] * m;
   }
   __device__ __forceinline__ float grad(int64_t, const float* in, float) const {
     float loss, dv;
@@ -837,10 +838,10 @@ extern "C" int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs,
 extern "C" int orlhf_value_loss_fwd(const float* values, const float* old_values, const float* returns,
                                     const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
                                     const int64_t* cu_seqlens, int has_clip, float clip_eps, int token_level,
-                                    const orlhf_norm* norm, void* workspace, float* out, float* row_coef,
+                                    const orlhf_norm* norm, void* workspace, float* out2, float* row_coef,
                                     orlhf_stream_t stream) {
   if (int rc = check_rows("value_loss_fwd", n_rows, n_cols, mask, mask_dtype)) return rc;
-  ORLHF_CHECK_ARG(out && workspace, "value_loss_fwd: NULL out / workspace");
+  ORLHF_CHECK_ARG(out2 && workspace, "value_loss_fwd: NULL out / workspace");
   ORLHF_CHECK_ARG((values && returns && (old_values || !has_clip)) || n_rows * n_cols == 0, "value_loss_fwd: NULL input");
   hipStream_t s = (hipStream_t)stream;
   const Rows rows = make_rows(n_rows, n_cols, cu_seqlens);
@@ -851,8 +852,8 @@ extern "C" int orlhf_value_loss_fwd(const float* values, const float* old_values
     launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
     ORLHF_CHECK_LAUNCH("orlhf_value_loss_fwd(partial)");
   }
-  launch_final<2>(n_rows, n_chunks, partial, token_level ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN, norm_arg(norm),
-                  0.5f, 1, out, row_coef, s);
+  launch_final<3>(n_rows, n_chunks, partial, token_level ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN, norm_arg(norm),
+                  0.5f, 2, out2, row_coef, s);
   ORLHF_CHECK_LAUNCH("orlhf_value_loss_fwd(final)");
   return ORLHF_OK;
 }

@@ -243,7 +243,7 @@ class _ValueLossFn(torch.autograd.Function):
         keep = []
         norm = _lib.make_norm(dp_size, norm_value, keep)
         ws = _workspace(n_rows, n_cols, dev)
-        out = torch.empty(1, dtype=torch.float32, device=dev)
+        out = torch.empty(2, dtype=torch.float32, device=dev)  # loss, masked mean of the values
         row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
         has_clip = clip_eps is not None
         with _lib.on_device(dev):
@@ -253,10 +253,12 @@ class _ValueLossFn(torch.autograd.Function):
         ctx.clip, ctx.dims, ctx.mcode = (has_clip, float(clip_eps) if has_clip else 0.0), (n_rows, n_cols), mcode
         ctx.v_shape, ctx.v_dtype = values.shape, values.dtype
         ctx.save_for_backward(v, old, ret, mkeep, cu, row_coef)
-        return out.view(())
+        loss, values_mean = out[0], out[1]
+        ctx.mark_non_differentiable(values_mean)
+        return loss, values_mean
 
     @staticmethod
-    def backward(ctx, g_out):
+    def backward(ctx, g_out, _g_mean):
         v, old, ret, mkeep, cu, row_coef = ctx.saved_tensors
         dev = v.device
         n_rows, n_cols = ctx.dims
@@ -289,6 +291,14 @@ class ValueLoss(nn.Module):
         cu_seqlens: Optional[torch.Tensor] = None,
         max_seqlen: Optional[int] = None,
     ) -> torch.Tensor:
+        return self.loss_and_values_mean(values, old_values, returns, action_mask, dp_size, batch_num_tokens,
+                                         global_batch_size, cu_seqlens, max_seqlen)[0]
+
+    def loss_and_values_mean(self, values, old_values, returns, action_mask=None, dp_size=1, batch_num_tokens=None,
+                             global_batch_size=None, cu_seqlens=None, max_seqlen=None):
+        """(loss, masked_mean(values, action_mask)) from one pass: the second is the "values"
+        status the critic trainer logs next to the loss (openrlhf/trainer/ray/ppo_critic.py:174),
+        detached."""
         norm_value = batch_num_tokens if self.token_level_loss else global_batch_size
         return _ValueLossFn.apply(
             values, old_values if self.clip_eps is not None else None, returns, action_mask, self.clip_eps,

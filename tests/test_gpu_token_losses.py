@@ -329,6 +329,60 @@ def test_value_loss_matches_oracle(cuda, clip_eps, token_level):
         assert abs(big.item() - plain.item()) <= 1e-6 * max(1.0, plain.item())
 
 
+@pytest.mark.parametrize("token_level", [True, False])
+@pytest.mark.parametrize("packed", [False, True])
+def test_critic_loss_step_matches_oracle(cuda, token_level, packed):
+    """critic_loss_step (openrlhf/trainer/ray/ppo_critic.py:151-176): value loss, masked mean of the
+    values from the same pass, loss = critic_loss + aux * coef; the gradient reaches the values."""
+    from openrlhf_amd.models.loss import ValueLoss
+    from openrlhf_amd.trainer.ray.ppo_critic import critic_loss_step
+
+    g = torch.Generator().manual_seed(77)
+    b, a = 19, 2300
+    _, _, _, _, mask = _tok(b, a, seed=77)
+    values = torch.randn(b, a, generator=g) + 0.7
+    old = values + torch.randn(b, a, generator=g) * 0.3
+    ret = torch.randn(b, a, generator=g)
+    info = dict(dp_size=2, batch_num_tokens=float(mask.sum()) * 2 + 5, global_batch_size=float(b * 2))
+    ref_v = values.double().requires_grad_(True)
+    ref = ol.value_loss(ref_v, old.double(), ret.double(), mask.double(), clip_eps=0.2,
+                        token_level_loss=token_level, **info)
+    (ref + 0.25 * 0.01).backward()
+    ref_mean = otn.masked_mean(values.double(), mask.double())
+    if packed:  # real tokens only: rows cut at their last unmasked column, holes kept with mask 0
+        lens = [int(mask[i].nonzero().max()) + 1 for i in range(b)]
+        flat = lambda t: torch.cat([t[i, :lens[i]] for i in range(b)]).to(cuda)
+        cu = torch.tensor([0] + lens).cumsum(0).to(cuda)
+        args = (flat(values).requires_grad_(True), flat(old), flat(ret), flat(mask))
+        extra = dict(cu_seqlens=cu, max_seqlen=max(lens))
+    else:
+        args = (values.to(cuda).requires_grad_(True), old.to(cuda), ret.to(cuda), mask.to(cuda))
+        extra = {}
+    out = critic_loss_step(*args, ValueLoss(0.2, token_level_loss=token_level), aux_loss=0.25, aux_loss_coef=0.01,
+                           **info, **extra)
+    _close(out["critic_loss"], ref)
+    _close(out["loss"], ref + 0.25 * 0.01)
+    _close(out["values_mean"], ref_mean)
+    assert not out["values_mean"].requires_grad
+    out["loss"].backward()
+    got = args[0].grad
+    want = ref_v.grad if not packed else torch.cat([ref_v.grad[i, :lens[i]] for i in range(b)])
+    _close(got, want, 1e-9 + 2e-5 * want.abs().max().item())
+    # the plain module still returns the scalar alone, equal to the step's critic_loss bit for bit
+    alone = ValueLoss(0.2, token_level_loss=token_level)(args[0].detach(), *args[1:3], action_mask=args[3], **info, **extra)
+    assert alone.dim() == 0 and torch.equal(alone, out["critic_loss"].detach())
+
+
+def test_critic_loss_step_empty_mask_is_nan(cuda):
+    """No unmasked token: the reference's masked_mean divides 0 by 0 (openrlhf/models/utils.py:166-169)."""
+    from openrlhf_amd.models.loss import ValueLoss
+    from openrlhf_amd.trainer.ray.ppo_critic import critic_loss_step
+
+    z = torch.zeros(3, 40, device=cuda)
+    out = critic_loss_step(torch.randn(3, 40, device=cuda), z, z, z, ValueLoss(0.2))
+    assert math.isnan(out["values_mean"].item()) and math.isnan(out["critic_loss"].item())
+
+
 # ------------------------------------------------------------------ config 1 end to end
 def test_config1_plumbing(cuda):
     """The CPU-runnable configuration: fp32 logits [4, 256, 32000] ~ N(0, 2), labels uniform, action mask with
