@@ -25,6 +25,11 @@ def _case(rng):
     return dtype, vocab, rows, pad, shift, temperature, std
 
 
+def _maxabs(t):
+    """max |t|, 0 for an empty selection (every row masked out)."""
+    return t.abs().max().item() if t.numel() else 0.0
+
+
 @pytest.mark.parametrize("seed", range(48))
 def test_random_case(cuda, seed):
     from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
@@ -58,8 +63,8 @@ def test_random_case(cuda, seed):
     rm = None if keep is None else keep.to(cuda)
     lp, ent = logprobs_and_entropy_from_logits(xd, labels.to(cuda), temperature, row_mask=rm)
     sel = torch.ones(rows, dtype=torch.bool) if keep is None else keep
-    assert (lp.cpu().double() - lp_ref.detach())[sel].abs().max().item() <= atol * max(1.0, std), info
-    assert (ent.cpu().double() - ent_ref.detach())[sel].abs().max().item() <= atol * max(1.0, std), info
+    assert _maxabs((lp.cpu().double() - lp_ref.detach())[sel]) <= atol * max(1.0, std), info
+    assert _maxabs((ent.cpu().double() - ent_ref.detach())[sel]) <= atol * max(1.0, std), info
     if keep is not None:
         assert (lp.cpu()[~keep] == 0).all() and (ent.cpu()[~keep] == 0).all(), info
     (gd,) = torch.autograd.grad((lp * g_lp.to(cuda)).sum() + (ent * g_ent.to(cuda)).sum(), xd)
@@ -68,6 +73,6 @@ def test_random_case(cuda, seed):
     xf = device_rows()
     lp1, ent1, grad1 = fused_logprob_entropy_fwd_bwd(xf, labels.to(cuda), g_lp.to(cuda), g_ent.to(cuda),
                                                      temperature=temperature, inplace=bool(seed % 2), row_mask=rm)
-    assert (lp1.cpu().double() - lp_ref.detach())[sel].abs().max().item() <= atol * max(1.0, std), info
-    assert (ent1.cpu().double() - ent_ref.detach())[sel].abs().max().item() <= atol * max(1.0, std), info
+    assert _maxabs((lp1.cpu().double() - lp_ref.detach())[sel]) <= atol * max(1.0, std), info
+    assert _maxabs((ent1.cpu().double() - ent_ref.detach())[sel]) <= atol * max(1.0, std), info
     assert (grad1.cpu().double() - g_ref).abs().max().item() <= gtol * gscale + 1e-12, info
