@@ -357,6 +357,124 @@ def bench_per_token(args, dev, emit=True):
     return res
 
 
+def bench_torch_eager(args, dev):
+    """`--workload torch_eager`: what stock OpenRLHF executes on this GPU for the same inputs - its op
+    sequence in eager torch (fp32 up-cast of the logits, compute_entropy, gather - logsumexp in
+    1024-row blocks, autograd backward: openrlhf/models/actor.py:267-285, models/utils.py:129-186;
+    PolicyLoss and the k3 KL as elementwise chains: models/loss.py:157-230, models/utils.py:64-95;
+    GAE as a Python loop over columns: experience_maker.py:358-376) - timed next to the HIP path.
+    Plain torch written out here, nothing of the product runs in the eager legs; the logits leg
+    uses --rows rows of config 2's shape (the eager chain holds several fp32 copies of them)."""
+    from openrlhf_amd.models.loss import PolicyLoss
+    from openrlhf_amd.models.utils import compute_approx_kl, fused_logprob_entropy_fwd_bwd, \
+        logprobs_and_entropy_from_logits
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import get_advantages_and_returns
+
+    def wall_ms(fn, n, warm=1):
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / n * 1e3
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    n, vocab = args.rows, args.vocab
+    logits = (torch.randn(n, vocab, device=dev, generator=g) * 3).to(torch.bfloat16)
+    labels = torch.randint(0, vocab, (n,), device=dev, generator=g)
+    g_lp, g_ent = torch.randn(n, device=dev, generator=g), torch.randn(n, device=dev, generator=g)
+
+    def eager_logits_step():
+        x = logits.detach().clone().requires_grad_(True)  # stands for the lm head's output
+        f = x.to(torch.float32)
+        pd = torch.softmax(f, dim=-1)
+        ent = torch.logsumexp(f, dim=-1) - torch.sum(pd * f, dim=-1)
+        picked = torch.gather(f, -1, labels.unsqueeze(-1)).squeeze(-1)
+        lse = torch.empty(n, device=dev, dtype=f.dtype)
+        for lo in range(0, n, 1024):
+            lse[lo:lo + 1024] = torch.logsumexp(f[lo:lo + 1024], dim=-1)
+        torch.autograd.backward([picked - lse, ent], [g_lp, g_ent])
+        return x.grad
+
+    eager_ms = wall_ms(eager_logits_step, 3) - wall_ms(lambda: logits.detach().clone(), 3)
+    bufs = [logits.clone() for _ in range(4)]
+    turn = [0]
+
+    def hip_one_pass():
+        turn[0] = (turn[0] + 1) % len(bufs)
+        return fused_logprob_entropy_fwd_bwd(bufs[turn[0]], labels, g_lp, g_ent, 1.0, inplace=True)
+
+    def hip_two_kernels():
+        turn[0] = (turn[0] + 1) % len(bufs)
+        x = bufs[turn[0]].detach().requires_grad_(True)
+        lp, ent = logprobs_and_entropy_from_logits(x, labels, 1.0, inplace_backward=True)
+        return torch.autograd.grad([lp, ent], [x], [g_lp, g_ent])
+
+    res = {"logprob_entropy_fwd_bwd": {"rows": n, "vocab": vocab, "torch_eager_ms": eager_ms,
+                                       "hip_one_pass_ms": wall_ms(hip_one_pass, 8, 2),
+                                       "hip_two_kernels_ms": wall_ms(hip_two_kernels, 8, 2)}}
+    del bufs, logits
+    torch.cuda.empty_cache()
+
+    b, a = 4096, 16384  # config 4
+    lens = torch.randint(64, a + 1, (b,), device=dev, generator=g)
+    mask = (torch.arange(a, device=dev)[None, :] < lens[:, None]).float()
+    lp = -torch.rand(b, a, device=dev, generator=g) * 3
+    old = lp + torch.randn(b, a, device=dev, generator=g) * 0.02
+    ref_lp = lp + torch.randn(b, a, device=dev, generator=g) * 0.1
+    adv = torch.randn(b, a, device=dev, generator=g)
+
+    def eager_policy():
+        x = lp.detach().requires_grad_(True)
+        raw = x - old
+        ratio = raw.clamp(min=-20.0, max=20.0).exp()
+        s1, s2 = ratio * adv, ratio.clamp(0.8, 1.2) * adv
+        c1 = torch.min(s1, s2)
+        loss = -torch.where(adv < 0, torch.max(c1, 3.0 * adv), c1)
+        cnt = mask.sum(dim=-1)
+        seq, seq_mask = (loss * mask).sum(dim=-1) / (cnt + 1e-8), (cnt > 0).float()
+        total = (seq * seq_mask).sum() / seq_mask.sum()
+        _ = ((s2 < s1).float() * mask).sum() / mask.sum(), ((-raw.detach()) * mask).sum() / mask.sum()
+        total.backward()
+        return x.grad
+
+    loss_fn = PolicyLoss(0.2, 0.2, dual_clip=3.0, token_level_loss=False)
+
+    def hip_policy():
+        x = lp.detach().requires_grad_(True)
+        loss_fn(x, old, adv, action_mask=mask)[0].backward()
+        return x.grad
+
+    def eager_kl():
+        d = lp.float() - ref_lp.float()
+        return ((-d).exp() - 1 + d).clamp(min=-10, max=10)
+
+    res["config4_policy_loss_fwd_bwd"] = {"torch_eager_ms": wall_ms(eager_policy, 5), "hip_ms": wall_ms(hip_policy, 20, 3)}
+    res["config4_k3_kl"] = {"torch_eager_ms": wall_ms(eager_kl, 5),
+                            "hip_ms": wall_ms(lambda: compute_approx_kl(lp, ref_lp, "k3"), 20, 3)}
+    values, rewards = torch.randn(b, a, device=dev, generator=g), torch.randn(b, a, device=dev, generator=g)
+
+    def eager_gae():
+        v, r, last, cols = mask * values, mask * rewards, 0, []
+        for t in reversed(range(a)):
+            nxt = v[:, t + 1] if t < a - 1 else 0.0
+            last = r[:, t] + 1.0 * nxt - v[:, t] + 0.95 * last
+            cols.append(last)
+        adv_ = torch.stack(cols[::-1], dim=1)
+        return adv_, adv_ + v
+
+    res["config4_gae"] = {"torch_eager_ms": wall_ms(eager_gae, 1),
+                          "hip_ms": wall_ms(lambda: get_advantages_and_returns(values, rewards, mask, 1.0, 0.95), 20, 3)}
+    for entry in res.values():
+        hip = entry.get("hip_ms", entry.get("hip_one_pass_ms"))
+        entry["speedup"] = entry["torch_eager_ms"] / hip
+    print(json.dumps({"workload": "the reference's eager torch op sequence on the same GPU beside the HIP path "
+                                  "(wall ms per call through the Python API)", "n_gpus": 1, "entries": res}), flush=True)
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -364,8 +482,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--ring", type=int, default=6, help="distinct logits buffers per timed segment")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU-baseline sample")
-    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token", "kernels"],
-                    help="logprob: the headline step (default); per_token: the small kernels of configs 3/4")
+    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token", "kernels", "torch_eager"],
+                    help="logprob: the headline step (default); per_token: the small kernels of configs 3/4; "
+                         "torch_eager: the reference's eager torch op sequence on this GPU beside the HIP path")
     ap.add_argument("--rows", type=int, default=8192, help="rows of logits for --workload kernels")
     ap.add_argument("--vocab", type=int, default=VOCAB, help="vocabulary for --workload kernels")
     ap.add_argument("--temperature", type=float, default=1.0, help="temperature for --workload kernels")
@@ -390,6 +509,9 @@ def main():
         return
     if args.workload == "per_token":
         bench_per_token(args, dev)
+        return
+    if args.workload == "torch_eager":
+        bench_torch_eager(args, dev)
         return
     pristine, labels, g_lp, g_ent, cu = make_workload(dev)
     n_tok = pristine.shape[0]
