@@ -324,6 +324,19 @@ def bench_per_token(args, dev, emit=True):
         torch.autograd.grad(out[0], x)
 
     record("config4.policy_loss_fwd_bwd", timed(policy_step), padded, 13 + 17)
+    # token mean: without a given count the gradient needs its own pass; with the trainers'
+    # batch_num_tokens the forward writes it (13 bytes in, 4 out)
+    pl_tok = PolicyLoss(0.2, 0.2, dual_clip=3.0)
+    n_tok_given = float(mask.sum()) * 2
+
+    def policy_step_token_mean():
+        torch.autograd.grad(pl_tok(x, old, adv, action_mask=mask)[0], x)
+
+    def policy_step_given_count():
+        torch.autograd.grad(pl_tok(x, old, adv, action_mask=mask, dp_size=2, batch_num_tokens=n_tok_given)[0], x)
+
+    record("config4.policy_loss_token_mean_fwd_bwd", timed(policy_step_token_mean), padded, 13 + 17)
+    record("config4.policy_loss_token_mean_given_count_fwd_bwd", timed(policy_step_given_count), padded, 13 + 4)
 
     # the same batch packed once (flat tokens + cu_seqlens): padding is neither stored nor read
     from openrlhf_amd.trainer.dpo_trainer import get_batch_logps

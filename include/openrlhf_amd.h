@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 12
+#define ORLHF_ABI_VERSION 13
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -275,6 +275,20 @@ int orlhf_policy_loss_fwd(const float* log_probs, const float* old_log_probs,
                           const int64_t* cu_seqlens, const orlhf_policy_params* params,
                           void* workspace, float* out4, float* row_coef, float* row_aux,
                           orlhf_stream_t stream);
+/*
+ * The same forward that also writes g_log_probs = d out4[0] / d log_probs (upstream gradient 1) in
+ * the same pass: 4 more bytes per token instead of the 21 of orlhf_policy_loss_bwd, bit-identical
+ * to what that writes for g_out = 1. Only where a token's weight is known before the pass: PPO,
+ * token_level = 1 and a given count in params->norm (what the trainer passes as batch_num_tokens,
+ * openrlhf/trainer/ray/ppo_actor.py:306-318); anything else is ORLHF_ERR_INVALID_ARG.
+ * No reference counterpart (the reference leaves the backward to autograd).
+ */
+int orlhf_policy_loss_fwd_grad(const float* log_probs, const float* old_log_probs,
+                               const float* advantages, const void* mask, int mask_dtype,
+                               const float* rollout_log_probs, int64_t n_rows, int64_t n_cols,
+                               const int64_t* cu_seqlens, const orlhf_policy_params* params,
+                               void* workspace, float* out4, float* row_coef, float* row_aux,
+                               float* g_log_probs, orlhf_stream_t stream);
 /* grad wrt log_probs only (everything else is detached in the callers). g_out: device scalar.
  * workspace (orlhf_token_workspace_bytes) is used by GSPO only and may be NULL otherwise. */
 int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs, const float* old_log_probs,
@@ -295,6 +309,13 @@ int orlhf_value_loss_fwd(const float* values, const float* old_values, const flo
                          const int64_t* cu_seqlens, int has_clip, float clip_eps, int token_level,
                          const orlhf_norm* norm, void* workspace, float* out2, float* row_coef,
                          orlhf_stream_t stream);
+/* Forward plus g_values = d out2[0] / d values in one pass; token mean over a given count only
+ * (see orlhf_policy_loss_fwd_grad). No reference counterpart. */
+int orlhf_value_loss_fwd_grad(const float* values, const float* old_values, const float* returns,
+                              const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                              const int64_t* cu_seqlens, int has_clip, float clip_eps,
+                              const orlhf_norm* norm, void* workspace, float* out2, float* row_coef,
+                              float* g_values, orlhf_stream_t stream);
 int orlhf_value_loss_bwd(const float* g_out, const float* values, const float* old_values,
                          const float* returns, const void* mask, int mask_dtype, int64_t n_rows,
                          int64_t n_cols, const int64_t* cu_seqlens, int has_clip, float clip_eps,

@@ -197,12 +197,20 @@ __device__ __forceinline__ void load_inputs4(const Tok& tok, int64_t i0, float (
 }
 
 // ---------------------------------------------------------------- stage 1: chunk partials
-template <int MASK_DT, typename Tok>
+// STORE_GRAD: the aggregation weight of a token is known before the pass (token mean over a given
+// count), so d(loss)/d(input 0) for a unit upstream gradient is written in the same pass:
+// g_store[i] = w * m * tok.grad(...) with w = post_scale * dp_size / count, the float the finaliser
+// puts into row_coef - the values rows_grad_kernel writes for g_out = 1, bit for bit.
+template <int MASK_DT, typename Tok, bool STORE_GRAD>
 __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const void* __restrict__ mask,
                                                               Tok tok, double* __restrict__ partial,
-                                                              int n_chunks) {
+                                                              int n_chunks, float* __restrict__ g_store,
+                                                              NormArg norm, float post_scale) {
   constexpr int NQ = Tok::kQ;
   __shared__ double lds[NQ][kWavesPerBlock];
+  float w = 0.0f;
+  if (STORE_GRAD)
+    w = (float)((double)post_scale * (norm.dp_size / (norm.dev != nullptr ? (double)norm.dev[0] : norm.value)));
   const int64_t slots = row_slots(rows.n_rows), items = slots * n_chunks;
   const int slot_b = slot_bits(rows.n_rows);
   for (int64_t item = blockIdx.x; item < items; item += gridDim.x) {
@@ -233,6 +241,12 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
 #pragma unroll
           for (int i = 0; i < NQ; ++i) acc[i] += (double)q[k][i];
         }
+        if constexpr (STORE_GRAD) {
+          f32x4 go;
+#pragma unroll
+          for (int k = 0; k < kTokPerLane; ++k) go[k] = w * m[k] * tok.grad(b, v[k], m[k]);
+          *(f32x4e*)(g_store + i0) = go;
+        }
       } else {  // the lane that meets the row's end, and the lanes past it
 #pragma unroll
         for (int k = 0; k < kTokPerLane; ++k) {
@@ -243,6 +257,7 @@ __global__ __launch_bounds__(kBlock) void rows_partial_kernel(Rows rows, const v
             tok.eval(b, v, m, q);
 #pragma unroll
             for (int i = 0; i < NQ; ++i) acc[i] += (double)q[i];
+            if constexpr (STORE_GRAD) g_store[rw.base + t0 + k] = w * m * tok.grad(b, v, m);
           }
         }
       }
@@ -587,8 +602,26 @@ template <typename Tok>
 static void launch_partial(int mask_dt, Rows rows, const void* mask, const Tok& tok, double* partial,
                            int n_chunks, hipStream_t s) {
   const dim3 grid = row_grid(rows), block(kBlock);
-#define ORLHF_LAUNCH(M) \
-  hipLaunchKernelGGL((rows_partial_kernel<M, Tok>), grid, block, 0, s, rows, mask, tok, partial, n_chunks)
+#define ORLHF_LAUNCH(M)                                                                                      \
+  hipLaunchKernelGGL((rows_partial_kernel<M, Tok, false>), grid, block, 0, s, rows, mask, tok, partial, n_chunks, \
+                     (float*)nullptr, NormArg{1.0, 1.0, nullptr}, 1.0f)
+  ORLHF_FOR_MASK_DTYPE(mask_dt, ORLHF_LAUNCH)
+#undef ORLHF_LAUNCH
+}
+
+// Chunk partials plus the gradient for a unit upstream gradient in the same pass (token mean over a
+// given count only: see rows_partial_kernel). g_store == nullptr is the plain launch.
+template <typename Tok>
+static void launch_partial_grad(int mask_dt, Rows rows, const void* mask, const Tok& tok, double* partial,
+                                int n_chunks, float* g_store, const NormArg& norm, float post_scale, hipStream_t s) {
+  if (g_store == nullptr) {
+    launch_partial(mask_dt, rows, mask, tok, partial, n_chunks, s);
+    return;
+  }
+  const dim3 grid = row_grid(rows), block(kBlock);
+#define ORLHF_LAUNCH(M)                                                                                     \
+  hipLaunchKernelGGL((rows_partial_kernel<M, Tok, true>), grid, block, 0, s, rows, mask, tok, partial, n_chunks, \
+                     g_store, norm, post_scale)
   ORLHF_FOR_MASK_DTYPE(mask_dt, ORLHF_LAUNCH)
 #undef ORLHF_LAUNCH
 }
@@ -752,11 +785,14 @@ extern "C" int orlhf_masked_aggregate_bwd(const float* g_out, const void* mask, 
   return ORLHF_OK;
 }
 
-extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_log_probs, const float* advantages,
-                                     const void* mask, int mask_dtype, const float* rollout_log_probs,
-                                     int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
-                                     const orlhf_policy_params* params, void* workspace, float* out4,
-                                     float* row_coef, float* row_aux, orlhf_stream_t stream) {
+// The weight of a token in the loss is known before the pass: token mean over a count the caller gives.
+static bool norm_given(const orlhf_norm* n) { return n != nullptr && (n->norm_dev != nullptr || n->norm_value == n->norm_value); }
+
+static int policy_loss_fwd_impl(const float* log_probs, const float* old_log_probs, const float* advantages,
+                                const void* mask, int mask_dtype, const float* rollout_log_probs,
+                                int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
+                                const orlhf_policy_params* params, void* workspace, float* out4,
+                                float* row_coef, float* row_aux, float* g_store, orlhf_stream_t stream) {
   if (int rc = check_rows("policy_loss_fwd", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (int rc = check_policy("policy_loss_fwd", params, rollout_log_probs)) return rc;
   ORLHF_CHECK_ARG(out4 && workspace && row_aux, "policy_loss_fwd: NULL out4 / workspace / row_aux");
@@ -784,10 +820,11 @@ extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_lo
   }
   if (n_rows > 0) {
     PolicyTok tok = policy_tok(log_probs, old_log_probs, advantages, rollout_log_probs, row_aux, params);
+    const NormArg na = norm_arg(&params->norm);
     if (!gspo && !use_is)
-      launch_partial(mask_dtype, rows, mask, PlainPolicyTok{tok}, partial, n_chunks, s);
+      launch_partial_grad(mask_dtype, rows, mask, PlainPolicyTok{tok}, partial, n_chunks, g_store, na, 1.0f, s);
     else
-      launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
+      launch_partial_grad(mask_dtype, rows, mask, tok, partial, n_chunks, g_store, na, 1.0f, s);
     ORLHF_CHECK_LAUNCH("orlhf_policy_loss_fwd(partial)");
   }
   const int mode = (params->token_level && !gspo) ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN;
@@ -795,6 +832,29 @@ extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_lo
   launch_final<5>(n_rows, n_chunks, partial, mode, norm_arg(&params->norm), 1.0f, n_out, out4, row_coef, s);
   ORLHF_CHECK_LAUNCH("orlhf_policy_loss_fwd(final)");
   return ORLHF_OK;
+}
+
+extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_log_probs, const float* advantages,
+                                     const void* mask, int mask_dtype, const float* rollout_log_probs,
+                                     int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
+                                     const orlhf_policy_params* params, void* workspace, float* out4,
+                                     float* row_coef, float* row_aux, orlhf_stream_t stream) {
+  return policy_loss_fwd_impl(log_probs, old_log_probs, advantages, mask, mask_dtype, rollout_log_probs, n_rows,
+                              n_cols, cu_seqlens, params, workspace, out4, row_coef, row_aux, nullptr, stream);
+}
+
+extern "C" int orlhf_policy_loss_fwd_grad(const float* log_probs, const float* old_log_probs,
+                                          const float* advantages, const void* mask, int mask_dtype,
+                                          const float* rollout_log_probs, int64_t n_rows, int64_t n_cols,
+                                          const int64_t* cu_seqlens, const orlhf_policy_params* params,
+                                          void* workspace, float* out4, float* row_coef, float* row_aux,
+                                          float* g_log_probs, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(params != nullptr && g_log_probs != nullptr, "policy_loss_fwd_grad: NULL params / g_log_probs");
+  ORLHF_CHECK_ARG(params->token_level && params->policy_type == ORLHF_POLICY_PPO && norm_given(&params->norm),
+                  "policy_loss_fwd_grad: needs the token mean over a given count (token_level, PPO, norm value or "
+                  "device scalar); other modes learn a token's weight only after the pass");
+  return policy_loss_fwd_impl(log_probs, old_log_probs, advantages, mask, mask_dtype, rollout_log_probs, n_rows,
+                              n_cols, cu_seqlens, params, workspace, out4, row_coef, row_aux, g_log_probs, stream);
 }
 
 extern "C" int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs, const float* old_log_probs,
@@ -835,11 +895,11 @@ extern "C" int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs,
   return ORLHF_OK;
 }
 
-extern "C" int orlhf_value_loss_fwd(const float* values, const float* old_values, const float* returns,
-                                    const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
-                                    const int64_t* cu_seqlens, int has_clip, float clip_eps, int token_level,
-                                    const orlhf_norm* norm, void* workspace, float* out2, float* row_coef,
-                                    orlhf_stream_t stream) {
+static int value_loss_fwd_impl(const float* values, const float* old_values, const float* returns,
+                               const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                               const int64_t* cu_seqlens, int has_clip, float clip_eps, int token_level,
+                               const orlhf_norm* norm, void* workspace, float* out2, float* row_coef,
+                               float* g_store, orlhf_stream_t stream) {
   if (int rc = check_rows("value_loss_fwd", n_rows, n_cols, mask, mask_dtype)) return rc;
   ORLHF_CHECK_ARG(out2 && workspace, "value_loss_fwd: NULL out / workspace");
   ORLHF_CHECK_ARG((values && returns && (old_values || !has_clip)) || n_rows * n_cols == 0, "value_loss_fwd: NULL input");
@@ -849,13 +909,34 @@ extern "C" int orlhf_value_loss_fwd(const float* values, const float* old_values
   double* partial = (double*)workspace;
   if (n_rows > 0) {
     ValueTok tok{values, old_values, returns, has_clip, clip_eps};
-    launch_partial(mask_dtype, rows, mask, tok, partial, n_chunks, s);
+    launch_partial_grad(mask_dtype, rows, mask, tok, partial, n_chunks, g_store, norm_arg(norm), 0.5f, s);
     ORLHF_CHECK_LAUNCH("orlhf_value_loss_fwd(partial)");
   }
   launch_final<3>(n_rows, n_chunks, partial, token_level ? ORLHF_AGG_TOKEN_MEAN : ORLHF_AGG_SEQ_MEAN, norm_arg(norm),
                   0.5f, 2, out2, row_coef, s);
   ORLHF_CHECK_LAUNCH("orlhf_value_loss_fwd(final)");
   return ORLHF_OK;
+}
+
+extern "C" int orlhf_value_loss_fwd(const float* values, const float* old_values, const float* returns,
+                                    const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                                    const int64_t* cu_seqlens, int has_clip, float clip_eps, int token_level,
+                                    const orlhf_norm* norm, void* workspace, float* out2, float* row_coef,
+                                    orlhf_stream_t stream) {
+  return value_loss_fwd_impl(values, old_values, returns, mask, mask_dtype, n_rows, n_cols, cu_seqlens, has_clip,
+                             clip_eps, token_level, norm, workspace, out2, row_coef, nullptr, stream);
+}
+
+extern "C" int orlhf_value_loss_fwd_grad(const float* values, const float* old_values, const float* returns,
+                                         const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                                         const int64_t* cu_seqlens, int has_clip, float clip_eps,
+                                         const orlhf_norm* norm, void* workspace, float* out2, float* row_coef,
+                                         float* g_values, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(g_values != nullptr, "value_loss_fwd_grad: NULL g_values");
+  ORLHF_CHECK_ARG(norm_given(norm), "value_loss_fwd_grad: needs the token mean over a given count (norm value or "
+                                    "device scalar); other modes learn a token's weight only after the pass");
+  return value_loss_fwd_impl(values, old_values, returns, mask, mask_dtype, n_rows, n_cols, cu_seqlens, has_clip,
+                             clip_eps, 1, norm, workspace, out2, row_coef, g_values, stream);
 }
 
 extern "C" int orlhf_value_loss_bwd(const float* g_out, const float* values, const float* old_values,

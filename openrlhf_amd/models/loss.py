@@ -97,10 +97,26 @@ class SFTLoss(nn.Module):
 _IS_CODES = {"tis": _lib.IS_TIS, "icepop": _lib.IS_ICEPOP, "seq-mask-tis": _lib.IS_SEQ_MASK_TIS}
 
 
+def _weights_known(token_level, norm_value):
+    """A token's weight in the loss is known before any token is read: token mean over a given count."""
+    return bool(token_level) and norm_value is not None
+
+
+def _hand_over(ctx, g, dev):
+    """The gradient the forward already wrote for a unit upstream gradient, multiplied in place by
+    the upstream gradient on the device (the kernel returns at once when that is 1). The stored
+    tensor is given away: a second backward through the same node (retain_graph) recomputes."""
+    grad, ctx.ready_grad = ctx.ready_grad, None
+    with _lib.on_device(dev):
+        call("orlhf_rescale_inplace_if", ptr(grad), _lib.F32, grad.numel(), ptr(g), 1.0, stream_of(dev))
+    return grad
+
+
 class _PolicyLossFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, log_probs, old_log_probs, advantages, action_mask, rollout_log_probs, cfg, dp_size,
                 norm_value, cu_seqlens):
+        ctx.set_materialize_grads(False)  # no zero-filled gradients for the three statistics
         dev = require_gpu(log_probs, old_log_probs, advantages, action_mask, rollout_log_probs)
         lp, old, adv = _f32(log_probs), _f32(old_log_probs.detach()), _f32(advantages.detach())
         if old.shape != lp.shape or adv.shape != lp.shape:
@@ -124,9 +140,20 @@ class _PolicyLossFn(torch.autograd.Function):
         out4 = torch.empty(4, dtype=torch.float32, device=dev)
         row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
         row_aux = torch.empty(max(n_rows, 1) * 2, dtype=torch.float32, device=dev)
+        # token mean over a given count (the trainers' loss_batch_info): every token's weight is known
+        # before the pass, so the gradient for a unit upstream gradient is written by the forward
+        ctx.ready_grad = None
+        if ctx.needs_input_grad[0] and _weights_known(cfg["token_level"], norm_value) \
+                and cfg["policy_type"] == _lib.POLICY_PPO:
+            ctx.ready_grad = torch.empty(lp.shape, dtype=torch.float32, device=dev)
         with _lib.on_device(dev):
-            call("orlhf_policy_loss_fwd", ptr(lp), ptr(old), ptr(adv), mptr, mcode, ptr(rollout), n_rows, n_cols,
-                 ptr(cu), params, ptr(ws), ptr(out4), ptr(row_coef), ptr(row_aux), stream_of(dev))
+            if ctx.ready_grad is not None:
+                call("orlhf_policy_loss_fwd_grad", ptr(lp), ptr(old), ptr(adv), mptr, mcode, ptr(rollout), n_rows,
+                     n_cols, ptr(cu), params, ptr(ws), ptr(out4), ptr(row_coef), ptr(row_aux), ptr(ctx.ready_grad),
+                     stream_of(dev))
+            else:
+                call("orlhf_policy_loss_fwd", ptr(lp), ptr(old), ptr(adv), mptr, mcode, ptr(rollout), n_rows, n_cols,
+                     ptr(cu), params, ptr(ws), ptr(out4), ptr(row_coef), ptr(row_aux), stream_of(dev))
         ctx.params, ctx.keep, ctx.dims, ctx.mcode = params, keep, (n_rows, n_cols), mcode
         ctx.lp_shape, ctx.lp_dtype = log_probs.shape, log_probs.dtype
         ctx.save_for_backward(lp, old, adv, mkeep, rollout, cu, row_coef, row_aux)
@@ -136,10 +163,14 @@ class _PolicyLossFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, _g1, _g2, _g3):
+        if g_loss is None:
+            return (None,) * 9
         lp, old, adv, mkeep, rollout, cu, row_coef, row_aux = ctx.saved_tensors
         dev = lp.device
         n_rows, n_cols = ctx.dims
         g = _f32(g_loss).reshape(-1)
+        if ctx.ready_grad is not None:
+            return (_hand_over(ctx, g, dev).view(ctx.lp_shape).to(ctx.lp_dtype),) + (None,) * 8
         g_lp = torch.empty(lp.shape, dtype=torch.float32, device=dev)
         ws = _workspace(n_rows, n_cols, dev) if ctx.params.policy_type == _lib.POLICY_GSPO else None
         with _lib.on_device(dev):
@@ -232,6 +263,7 @@ class _ValueLossFn(torch.autograd.Function):
     @staticmethod
     def forward(ctx, values, old_values, returns, action_mask, clip_eps, token_level, dp_size, norm_value,
                 cu_seqlens):
+        ctx.set_materialize_grads(False)  # no zero-filled gradient for the mean of the values
         dev = require_gpu(values, old_values, returns, action_mask)
         v, ret = _f32(values), _f32(returns.detach())
         old = None if old_values is None else _f32(old_values.detach())
@@ -246,10 +278,18 @@ class _ValueLossFn(torch.autograd.Function):
         out = torch.empty(2, dtype=torch.float32, device=dev)  # loss, masked mean of the values
         row_coef = torch.empty(max(n_rows, 1), dtype=torch.float32, device=dev)
         has_clip = clip_eps is not None
+        ctx.ready_grad = None
+        if ctx.needs_input_grad[0] and _weights_known(token_level, norm_value):
+            ctx.ready_grad = torch.empty(v.shape, dtype=torch.float32, device=dev)
         with _lib.on_device(dev):
-            call("orlhf_value_loss_fwd", ptr(v), ptr(old), ptr(ret), mptr, mcode, n_rows, n_cols, ptr(cu),
-                 1 if has_clip else 0, float(clip_eps) if has_clip else 0.0, 1 if token_level else 0, norm,
-                 ptr(ws), ptr(out), ptr(row_coef), stream_of(dev))
+            if ctx.ready_grad is not None:
+                call("orlhf_value_loss_fwd_grad", ptr(v), ptr(old), ptr(ret), mptr, mcode, n_rows, n_cols, ptr(cu),
+                     1 if has_clip else 0, float(clip_eps) if has_clip else 0.0, norm, ptr(ws), ptr(out),
+                     ptr(row_coef), ptr(ctx.ready_grad), stream_of(dev))
+            else:
+                call("orlhf_value_loss_fwd", ptr(v), ptr(old), ptr(ret), mptr, mcode, n_rows, n_cols, ptr(cu),
+                     1 if has_clip else 0, float(clip_eps) if has_clip else 0.0, 1 if token_level else 0, norm,
+                     ptr(ws), ptr(out), ptr(row_coef), stream_of(dev))
         ctx.clip, ctx.dims, ctx.mcode = (has_clip, float(clip_eps) if has_clip else 0.0), (n_rows, n_cols), mcode
         ctx.v_shape, ctx.v_dtype = values.shape, values.dtype
         ctx.save_for_backward(v, old, ret, mkeep, cu, row_coef)
@@ -259,10 +299,14 @@ class _ValueLossFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_out, _g_mean):
+        if g_out is None:
+            return (None,) * 9
         v, old, ret, mkeep, cu, row_coef = ctx.saved_tensors
         dev = v.device
         n_rows, n_cols = ctx.dims
         g = _f32(g_out).reshape(-1)
+        if ctx.ready_grad is not None:
+            return (_hand_over(ctx, g, dev).view(ctx.v_shape).to(ctx.v_dtype),) + (None,) * 8
         g_v = torch.empty(v.shape, dtype=torch.float32, device=dev)
         with _lib.on_device(dev):
             call("orlhf_value_loss_bwd", ptr(g), ptr(v), ptr(old), ptr(ret), ptr(mkeep), ctx.mcode, n_rows, n_cols,
@@ -311,6 +355,7 @@ class _PairLossFn(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, chosen, rejected, ref_chosen, ref_rejected, kind, beta, label_smoothing, want_rewards):
+        ctx.set_materialize_grads(False)  # no zero-filled gradients for the two reward estimates
         dev = require_gpu(chosen, rejected, ref_chosen, ref_rejected)
         if chosen.shape != rejected.shape:
             raise ValueError(f"chosen {tuple(chosen.shape)} and rejected {tuple(rejected.shape)} differ in shape")
@@ -333,6 +378,8 @@ class _PairLossFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_loss, _g_cr, _g_rr):
+        if g_loss is None:
+            return (None,) * 8
         a, b, c, d = ctx.saved_tensors
         kind, beta, smooth, shape, dt_a, dt_b = ctx.cfg
         dev = a.device

@@ -66,6 +66,20 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     p.dual_clip, p.is_correction = 0.0, 1
     assert lib.orlhf_policy_loss_fwd(None, None, None, None, 0, None, 0, 0, None, p, None, None, None, None, None) == -1
     assert "rollout" in err()
+    # forward + gradient in one pass: only for the token mean over a given count
+    q = _lib.PolicyParams()
+    q.token_level = 1  # PPO, but no count given
+    q.norm = _lib.make_norm(1, None, [])
+    assert lib.orlhf_policy_loss_fwd_grad(None, None, None, None, 0, None, 0, 0, None, q, None, None, None, None, 8, None) == -1
+    assert "given count" in err()
+    q.norm = _lib.make_norm(1, 100.0, [])
+    q.token_level = 0
+    assert lib.orlhf_policy_loss_fwd_grad(None, None, None, None, 0, None, 0, 0, None, q, None, None, None, None, 8, None) == -1
+    q.token_level = 1
+    assert lib.orlhf_policy_loss_fwd_grad(None, None, None, None, 0, None, 0, 0, None, q, None, None, None, None, None, None) == -1
+    assert "g_log_probs" in err()
+    assert lib.orlhf_value_loss_fwd_grad(None, None, None, None, 0, 0, 0, None, 0, 0.0, _lib.make_norm(1, None, []), None, None, None, 8, None) == -1
+    assert "given count" in err()
     assert lib.orlhf_group_normalize(None, None, 3, 0, 0, None, None, None, None) == -1
     assert lib.orlhf_group_normalize(None, None, 3, 2, 9, None, None, None, None) == -1
     assert lib.orlhf_gae_scan(None, None, None, 0, -1, 4, None, 1.0, 1.0, None, None, None) == -1

@@ -383,6 +383,90 @@ def test_critic_loss_step_empty_mask_is_nan(cuda):
     assert math.isnan(out["values_mean"].item()) and math.isnan(out["critic_loss"].item())
 
 
+# ------------------------------------------------------------------ forward that also writes the gradient
+@pytest.mark.parametrize("is_type", [None, "tis", "icepop", "seq-mask-tis"])
+@pytest.mark.parametrize("count_on_device", [False, True])
+@pytest.mark.parametrize("packed", [False, True])
+def test_policy_loss_gradient_from_the_forward_pass(cuda, is_type, count_on_device, packed):
+    """Token mean over a given count (the trainers' loss_batch_info): the forward writes the gradient
+    and backward hands it over. Checked against autograd through the oracle for an upstream gradient
+    of 0.37, and bit for bit against the separate backward kernel (which a second backward through a
+    retained graph runs) for an upstream gradient of 1."""
+    from openrlhf_amd.models.loss import PolicyLoss
+
+    b, a = 23, 1900
+    lp, old, rollout, adv, mask = _tok(b, a, seed=5)
+    count = float(mask.sum()) * 2 + 3
+    kw = dict(clip_eps_low=0.2, clip_eps_high=0.3, dual_clip=3.0)
+    if is_type is not None:
+        kw.update(enable_vllm_is_correction=True, vllm_is_truncated_threshold=[0.8, 1.25], vllm_is_correction_type=is_type)
+    ref_x = lp.double().requires_grad_(True)
+    ref = ol.policy_loss(ref_x, old.double(), adv.double(), mask.double(), rollout.double() if is_type else None,
+                         dp_size=2, batch_num_tokens=count, **kw)[0]
+    (ref * 0.37).backward()
+    if packed:
+        lens = [int(mask[i].nonzero().max()) + 1 for i in range(b)]
+        flat = lambda t: torch.cat([t[i, :lens[i]] for i in range(b)]).to(cuda)
+        extra = dict(cu_seqlens=torch.tensor([0] + lens).cumsum(0).to(cuda), max_seqlen=max(lens))
+        want = torch.cat([ref_x.grad[i, :lens[i]] for i in range(b)])
+    else:
+        flat, extra, want = (lambda t: t.to(cuda)), {}, ref_x.grad
+    n = torch.tensor(count, device=cuda) if count_on_device else count
+    fn = PolicyLoss(**kw)
+
+    def run(upstream, retain=False):
+        x = flat(lp).requires_grad_(True)
+        out = fn(x, flat(old), flat(adv), action_mask=flat(mask), rollout_log_probs=flat(rollout) if is_type else None,
+                 dp_size=2, batch_num_tokens=n, **extra)
+        (out[0] * upstream).backward(retain_graph=retain)
+        return x, out
+
+    x, out = run(0.37)
+    _close(out[0], ref)
+    _close(x.grad, want, 1e-9 + 2e-5 * want.abs().max().item())
+    x, out = run(1.0, retain=True)
+    first = x.grad.clone()
+    x.grad = None
+    out[0].backward()  # the stored gradient is gone: the separate backward kernel runs
+    assert torch.equal(first, x.grad)
+
+
+@pytest.mark.parametrize("clip_eps", [None, 0.2])
+def test_value_loss_gradient_from_the_forward_pass(cuda, clip_eps):
+    from openrlhf_amd.models.loss import ValueLoss
+
+    g = torch.Generator().manual_seed(12)
+    b, a = 17, 2500
+    _, _, _, _, mask = _tok(b, a, seed=12)
+    values = torch.randn(b, a, generator=g)
+    old = values + torch.randn(b, a, generator=g) * 0.3
+    ret = torch.randn(b, a, generator=g)
+    count = float(mask.sum()) + 11
+    ref_v = values.double().requires_grad_(True)
+    ref = ol.value_loss(ref_v, old.double(), ret.double(), mask.double(), clip_eps=clip_eps, dp_size=4, batch_num_tokens=count)
+    (ref * 2.5).backward()
+    fn = ValueLoss(clip_eps)
+
+    def run(upstream, retain=False):
+        x = values.to(cuda).requires_grad_(True)
+        out = fn(x, old.to(cuda), ret.to(cuda), action_mask=mask.to(cuda), dp_size=4,
+                 batch_num_tokens=torch.tensor(count, device=cuda))
+        (out * upstream).backward(retain_graph=retain)
+        return x, out
+
+    x, out = run(2.5)
+    _close(out, ref)
+    _close(x.grad, ref_v.grad, 1e-9 + 2e-5 * ref_v.grad.abs().max().item())
+    x, out = run(1.0, retain=True)
+    first = x.grad.clone()
+    x.grad = None
+    out.backward()
+    assert torch.equal(first, x.grad)
+    with torch.no_grad():  # nothing to differentiate: the plain forward, same value
+        plain = fn(values.to(cuda), old.to(cuda), ret.to(cuda), action_mask=mask.to(cuda), dp_size=4, batch_num_tokens=count)
+    assert torch.equal(plain, out.detach())
+
+
 # ------------------------------------------------------------------ config 1 end to end
 def test_config1_plumbing(cuda):
     """The CPU-runnable configuration: fp32 logits [4, 256, 32000] ~ N(0, 2), labels uniform, action mask with
