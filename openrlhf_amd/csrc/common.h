@@ -149,22 +149,29 @@ __device__ __forceinline__ f32x4 stream_load4(const float* p) {
   return __builtin_nontemporal_load((const f32x4e*)p);
 }
 
-template <int MASK_DT>
+// STREAM = false: cached loads, for a lane that comes back to the same cache lines with its next
+// load (two groups of four tokens per lane): non-temporal there fetches the lines twice.
+template <bool STREAM, typename T>
+__device__ __forceinline__ T load_once(const T* p) {
+  return STREAM ? __builtin_nontemporal_load(p) : *p;
+}
+
+template <int MASK_DT, bool STREAM = true>
 __device__ __forceinline__ void load_mask4(const void* mask, int64_t i0, float* m) {
   if (MASK_DT == ORLHF_MASK_NONE) {
 #pragma unroll
     for (int k = 0; k < 4; ++k) m[k] = 1.0f;
   } else if (MASK_DT == ORLHF_MASK_U8) {
-    const uint32_t w = __builtin_nontemporal_load((const u32_b*)((const uint8_t*)mask + i0));
+    const uint32_t w = load_once<STREAM>((const u32_b*)((const uint8_t*)mask + i0));
 #pragma unroll
     for (int k = 0; k < 4; ++k) m[k] = (float)((w >> (8 * k)) & 0xffu);
   } else if (MASK_DT == ORLHF_MASK_F32) {
-    const f32x4 x = stream_load4((const float*)mask + i0);
+    const f32x4 x = load_once<STREAM>((const f32x4e*)((const float*)mask + i0));
 #pragma unroll
     for (int k = 0; k < 4; ++k) m[k] = x[k];
   } else {
-    const i64x2e lo = __builtin_nontemporal_load((const i64x2e*)((const int64_t*)mask + i0)),
-                 hi = __builtin_nontemporal_load((const i64x2e*)((const int64_t*)mask + i0 + 2));
+    const i64x2e lo = load_once<STREAM>((const i64x2e*)((const int64_t*)mask + i0)),
+                 hi = load_once<STREAM>((const i64x2e*)((const int64_t*)mask + i0 + 2));
     m[0] = (float)lo[0];
     m[1] = (float)lo[1];
     m[2] = (float)hi[0];
