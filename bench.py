@@ -533,6 +533,7 @@ def main():
     bufs = [torch.empty_like(pristine) for _ in range(ring)]
 
     fwd_ms, bwd_ms, fused_ms = [], [], []
+    last_fused = []
 
     def step_two_kernels(buf, timed):
         x = buf.requires_grad_(True)
@@ -557,10 +558,29 @@ def main():
             e0.record()
         lp, ent, grad = fused_logprob_entropy_fwd_bwd(buf, labels, g_lp, g_ent, 1.0, inplace=True)
         assert grad.data_ptr() == buf.data_ptr()
+        last_fused[:] = [buf, lp, ent]
         if timed:
             e1.record()
             return e0, e1
         return None
+
+    def check_last_fused(sample=64):
+        """Outside the timed region: a row sample of the last timed buffer (now holding the one-pass
+        kernel's gradient) and its log-probs / entropies against the separate forward and backward
+        kernels run on the same rows of the pristine logits."""
+        buf, lp, ent = last_fused
+        pick = torch.randperm(n_tok, generator=torch.Generator().manual_seed(5))[:sample].to(dev)
+        x = pristine[pick].clone().requires_grad_(True)
+        lp2, ent2 = logprobs_and_entropy_from_logits(x, labels[pick], 1.0)
+        (g2,) = torch.autograd.grad([lp2, ent2], [x], [g_lp[pick], g_ent[pick]])
+        got, want = buf[pick].float(), g2.float()
+        e_lp = (lp[pick] - lp2).abs().max().item()
+        e_ent = (ent[pick] - ent2).abs().max().item()
+        e_grad = ((got - want).abs() - 2.0 ** -7 * want.abs()).max().item()
+        ok = e_lp <= 2e-5 and e_ent <= 2e-5 and e_grad <= 4e-6 and bool(torch.isfinite(got).all())
+        return ok, {"rows": sample, "logprob_abs_err": e_lp, "entropy_abs_err": e_ent,
+                    "grad_excess_over_bf16_rounding": e_grad,
+                    "against": "logprobs_and_entropy_from_logits + autograd on the same rows of the pristine logits"}
 
     def run_segment(step, count, timed):
         for b in bufs[:count]:
@@ -594,6 +614,7 @@ def main():
 
     total_two = run(step_two_kernels)
     total = run(step_fused)
+    checked, check_detail = check_last_fused()
     ppo = None if args.no_ppo_step else bench_ppo_step(args, pristine, bufs, cu, ring, dev)
 
     ms_per_step = total / args.steps * 1e3
@@ -624,6 +645,8 @@ def main():
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
+        "checked": checked,
+        "check": check_detail,
         "config": {
             "workload": "BASELINE config 2: 16 sequences, lengths uniform in [512,3072], packed to one row; bf16 "
                         "logits [T_total,151936] ~N(0,3), 1% of rows with one +15 spike, temperature 1.0; "

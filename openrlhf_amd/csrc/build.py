@@ -7,6 +7,8 @@ import argparse
 import os
 import shutil
 import subprocess
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 CSRC = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(CSRC)
@@ -23,7 +25,6 @@ HIPCC_FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
@@ -38,11 +39,7 @@ def find_hipcc():
     raise RuntimeError("hipcc not found (set HIPCC or install ROCm under /opt/rocm)")
 
 
-def build(extra_flags=(), out=LIB_PATH, verbose=True, sources=None):
-    srcs = [os.path.join(CSRC, s) for s in (sources or SOURCES) if os.path.exists(os.path.join(CSRC, s))]
-    os.makedirs(os.path.dirname(out), exist_ok=True)
-    tmp = out + ".tmp"
-    cmd = [find_hipcc(), *HIPCC_FLAGS, *extra_flags, "-I", os.path.join(PKG, "..", "include"), *srcs, "-o", tmp]
+def _run(cmd, verbose):
     if verbose:
         print("+", " ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)
@@ -50,6 +47,24 @@ def build(extra_flags=(), out=LIB_PATH, verbose=True, sources=None):
     log = "\n".join(l for l in (res.stdout + res.stderr).splitlines() if not any(n in l for n in noise))
     if res.returncode != 0:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{log}")
+    return log
+
+
+def build(extra_flags=(), out=LIB_PATH, verbose=True, sources=None, jobs=None):
+    """Compiles every source to an object (in parallel, one hipcc per file) and links them."""
+    srcs = [os.path.join(CSRC, s) for s in (sources or SOURCES) if os.path.exists(os.path.join(CSRC, s))]
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    hipcc = find_hipcc()
+    include = os.path.join(PKG, "..", "include")
+    jobs = jobs or min(len(srcs), max(1, min(8, os.cpu_count() or 1)))
+    with tempfile.TemporaryDirectory(prefix="orlhf_build_") as tmpdir:
+        objs = [os.path.join(tmpdir, os.path.basename(s) + ".o") for s in srcs]
+        cmds = [[hipcc, *HIPCC_FLAGS, *extra_flags, "-I", include, "-c", s, "-o", o] for s, o in zip(srcs, objs)]
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            logs = list(pool.map(lambda c: _run(c, verbose), cmds))
+        tmp = out + ".tmp"
+        logs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", tmp], verbose))
+    log = "\n".join(l for l in logs if l.strip())
     if verbose and log.strip():
         print(log)
     os.replace(tmp, out)

@@ -213,3 +213,133 @@ def test_config4_grpo_group_step(cuda):
     out[0].backward()
     ref[0].backward()
     assert (x.grad.cpu().double() - x64.grad).abs().max().item() <= 1e-5 * x64.grad.abs().max().item() + 1e-12
+
+
+def _rounding_excess(got, want, eps, slab=2048):
+    """max over all elements of |got - want| - eps * |want|, slab by slab on the device."""
+    worst = -1.0
+    for lo in range(0, got.shape[0], slab):
+        a, b = got[lo:lo + slab].float(), want[lo:lo + slab].float()
+        worst = max(worst, ((a - b).abs() - eps * b.abs()).max().item())
+    return worst
+
+
+def _one_pass_config(cuda, n, vocab, std, temperature, seed, spike_frac, sample):
+    """The one-pass forward+backward kernel on a full-size batch: every row against the separate
+    forward and in-place backward kernels (run on a copy), a row sample against the fp64 oracle."""
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
+
+    g = torch.Generator().manual_seed(seed)
+    x = _fill_normal(n, vocab, std, cuda, seed)
+    if spike_frac:
+        k = max(1, int(n * spike_frac))
+        x[torch.randperm(n, generator=g)[:k].to(cuda), torch.randint(0, vocab, (k,), generator=g).to(cuda)] += 15.0
+    labels = torch.randint(0, vocab, (n,), generator=g).to(cuda)
+    g_lp, g_ent = torch.randn(n, generator=g).to(cuda), torch.randn(n, generator=g).to(cuda)
+    dead = torch.randperm(n, generator=g)[: n // 50].to(cuda)
+    g_lp[dead] = 0
+    g_ent[dead] = 0
+    pick = torch.randperm(n, generator=g)[:sample].to(cuda)
+    x_pick = x[pick].cpu()
+
+    xa = x.clone().requires_grad_(True)
+    lp2, ent2 = logprobs_and_entropy_from_logits(xa, labels, temperature, inplace_backward=True)
+    (g2,) = torch.autograd.grad([lp2, ent2], [xa], [g_lp, g_ent])
+    lp, ent, grad = fused_logprob_entropy_fwd_bwd(x, labels, g_lp, g_ent, temperature, inplace=True)
+    assert grad.data_ptr() == x.data_ptr() and g2.data_ptr() == xa.data_ptr()
+    assert (lp - lp2).abs().max().item() <= 2e-5 and (ent - ent2).abs().max().item() <= 2e-5
+    assert _rounding_excess(grad, g2, 2.0 ** -7) <= 4e-6
+    assert grad[dead].abs().max().item() == 0.0
+    lp64 = otn.log_probs_from_logits(x_pick.double(), labels[pick].cpu(), temperature)
+    ent64 = otn.compute_entropy(x_pick.double())
+    assert (lp[pick].cpu().double() - lp64).abs().max().item() <= 2e-3
+    assert (ent[pick].cpu().double() - ent64).abs().max().item() <= 2e-3
+    ref = _analytic_grad64(x_pick, labels[pick].cpu(), temperature, g_lp[pick].cpu(), g_ent[pick].cpu())
+    err = (grad[pick].cpu().double() - ref).abs()
+    assert (err <= 2.0 ** -8 * ref.abs() + 1e-6).all(), err.max().item()
+
+
+def test_config2_one_pass_kernel_full_size(cuda):
+    """Config 2 through the one-pass kernel the benchmark times: ~30 K rows on one workgroup per
+    CU, i.e. ~120 rows per workgroup through the row-to-row register pipeline."""
+    g = torch.Generator().manual_seed(2)
+    n = int(torch.randint(512, 3073, (16,), generator=g).sum())
+    _one_pass_config(cuda, n, 151936, 3.0, 1.0, seed=23, spike_frac=0.01, sample=48)
+    torch.cuda.empty_cache()
+
+
+def test_config5_one_pass_kernel_full_size(cuda):
+    """Config 5 through the one-pass kernel: 65536 rows of 262144 bf16 logits at T = 0.6, half of
+    every row resident in registers and half streamed twice, two statistic sets."""
+    _one_pass_config(cuda, 65536, 262144, 4.0, 0.6, seed=56, spike_frac=0.0, sample=16)
+    torch.cuda.empty_cache()
+
+
+def test_config2_fused_actor_step_full_size(cuda):
+    """The whole PPO actor loss step at config 2's size from one pass over the packed logits,
+    against the composed step on the separate kernels (values and all gradient rows), and a row
+    sample against the oracle: d(loss)/d(logprob) and d(loss)/d(entropy) from torch autograd
+    through the oracle's losses in fp64, pushed through the analytic row gradient."""
+    from openrlhf_amd.models.actor import unpad_indices
+    from openrlhf_amd.models.loss import PolicyLoss
+    from openrlhf_amd.trainer.ray.ppo_actor import actor_loss_step, fused_actor_loss_step
+
+    vocab = 151936
+    g = torch.Generator().manual_seed(2)
+    lens = torch.randint(512, 3073, (16,), generator=g)
+    b, t = 16, int(lens.max())
+    n = int(lens.sum())
+    attn = (torch.arange(t)[None, :] < lens[:, None]).long()
+    seqs = torch.randint(1, vocab, (b, t), generator=g) * attn
+    a = t - 1
+    amask = attn[:, 1:].bool().clone()
+    amask[:, :200] = False                      # prompt
+    amask[3, 700:760] = False                   # a hole (environment tokens)
+    old = -torch.rand(b, a, generator=g) * 14
+    base = -torch.rand(b, a, generator=g) * 14
+    adv = torch.randn(b, a, generator=g)
+    x = _fill_normal(n, vocab, 3.0, cuda, 24)
+    d = cuda
+    idx = unpad_indices(attn.to(d))
+    labels_rows = torch.roll(seqs, -1, 1).reshape(-1)[idx.cpu()]
+    pick = torch.randperm(n, generator=g)[:32]
+    x_pick = x[pick.to(d)].cpu()
+    fn = PolicyLoss(0.2, 0.28, dual_clip=3.0)
+    kw = dict(base_action_log_probs=base.to(d), kl_estimator="k3", kl_coef=0.01, entropy_coef=0.001,
+              packed_indices=idx)
+    tensors = (seqs.to(d), attn.to(d), amask.to(d), old.to(d), adv.to(d), fn)
+
+    xa = x.clone().requires_grad_(True)
+    ref = actor_loss_step(xa, *tensors, inplace_backward=True, **kw)
+    ref["loss"].backward()
+    out = fused_actor_loss_step(x, *tensors, **kw)
+    grad = out["grad_logits"]
+    assert grad.data_ptr() == x.data_ptr()
+    for key in ("loss", "actor_loss", "kl_loss", "entropy_loss", "clip_ratio", "ppo_kl"):
+        assert abs(out[key].item() - ref[key].item()) <= 2e-5 * max(1.0, abs(ref[key].item())), key
+    assert (out["action_log_probs"] - ref["action_log_probs"]).abs().max().item() <= 2e-5
+    gscale = xa.grad.float().abs().max().item()
+    assert _rounding_excess(grad, xa.grad, 2.0 ** -7) <= 1e-6 * gscale + 1e-12
+
+    # oracle: the losses in fp64 on the action log-probs / entropy the device produced
+    alp = out["action_log_probs"].cpu().double().requires_grad_(True)
+    ent = out["entropy"].cpu().double().requires_grad_(True)
+    m = amask.double()
+    pl = ol.policy_loss(alp, old.double(), adv.double(), m, dual_clip=3.0, clip_eps_low=0.2, clip_eps_high=0.28)
+    kl_loss = ol.aggregate_loss(otn.compute_approx_kl(alp, base.double(), "k3"), m)
+    ent_loss = ol.aggregate_loss(ent, m)
+    loss = pl[0] + kl_loss * 0.01 - ent_loss * 0.001
+    assert abs(out["loss"].item() - loss.item()) <= 1e-5
+    loss.backward()
+
+    def rows_of(t_ba):  # [B, A] -> one value per packed logits row
+        full = torch.zeros(b, t, dtype=torch.float64)
+        full[:, : t - 1] = t_ba
+        return full.reshape(-1)[idx.cpu()]
+
+    w_lp, w_ent = rows_of(alp.grad * m), rows_of(ent.grad)
+    want = _analytic_grad64(x_pick, labels_rows[pick], 1.0, w_lp[pick], w_ent[pick])
+    got = grad[pick.to(d)].cpu().double()
+    err = (got - want).abs()
+    assert (err <= 2.0 ** -7 * want.abs() + 1e-4 * want.abs().max().item() + 1e-12).all(), err.max().item()
+    torch.cuda.empty_cache()

@@ -171,3 +171,90 @@ def test_fused_extreme_rows(cuda):
     assert lp[3] == float("-inf") and math.isnan(ent[3])
     assert math.isnan(lp[4]) and math.isnan(ent[4])
     assert torch.equal(lp2.cpu().isnan(), lp.isnan()) and torch.equal(ent2.cpu().isnan(), ent.isnan())
+
+
+def _device_case(cuda, rows, vocab, dtype, std, seed):
+    g = torch.Generator(device=cuda).manual_seed(seed)
+    x = torch.empty(rows, vocab, dtype=dtype, device=cuda)
+    for lo in range(0, rows, 512):
+        hi = min(lo + 512, rows)
+        x[lo:hi] = (torch.randn(hi - lo, vocab, generator=g, device=cuda) * std).to(dtype)
+    spiked = torch.randperm(rows, generator=g, device=cuda)[: max(1, rows // 50)]
+    x[spiked, torch.randint(0, vocab, (len(spiked),), generator=g, device=cuda)] += 15.0
+    labels = torch.randint(0, vocab, (rows,), generator=g, device=cuda)
+    w_lp = torch.randn(rows, generator=g, device=cuda)
+    w_ent = torch.randn(rows, generator=g, device=cuda)
+    return x, labels, w_lp, w_ent
+
+
+def _close_to_rounding(got, want, dtype, slab=1024):
+    """got / want: [N, V] gradients of two kernels that round the same fp32 value independently."""
+    eps = {torch.bfloat16: 2.0 ** -7, torch.float16: 2.0 ** -10, torch.float32: 2e-5}[dtype]
+    worst = 0.0
+    for lo in range(0, got.shape[0], slab):
+        a, b = got[lo:lo + slab].float(), want[lo:lo + slab].float()
+        excess = ((a - b).abs() - eps * b.abs()).max().item()
+        worst = max(worst, excess)
+    return worst
+
+
+@pytest.mark.parametrize(
+    "rows,vocab,dtype,std,temperature",
+    [
+        (1200, 151936, torch.bfloat16, 3.0, 1.0),   # 4-5 rows per workgroup, all 38 register chunks refilled
+        (700, 151936, torch.bfloat16, 3.0, 0.8),    # the same with two statistic sets
+        (600, 200003, torch.bfloat16, 3.0, 1.0),    # register part + streamed tail, odd vocabulary (scalar tail)
+        (530, 262144, torch.bfloat16, 4.0, 0.6),    # config-5 row shape, streamed half, two statistic sets
+        (2000, 32000, torch.float32, 2.0, 1.0),     # fp32, 16 of 38 chunks live
+        (1500, 50257, torch.bfloat16, 3.0, 1.0),    # scalar tail, 13 of 38 chunks live
+        (300, 77825, torch.float32, 2.0, 1.3),      # fp32 row one element longer than the registers hold
+        (257, 155648, torch.float16, 2.0, 1.0),     # exactly the register capacity; one workgroup gets a second row
+    ],
+)
+@pytest.mark.parametrize("masked", [False, True])
+def test_fused_many_rows_per_workgroup(cuda, rows, vocab, dtype, std, temperature, masked):
+    """More rows than workgroups (one per CU): the row-to-row pipeline, where every register chunk
+    is refilled from the workgroup's next row while the current row's gradient is stored. All rows
+    against the separate forward and backward kernels, a row sample against the fp64 oracle. With
+    `masked`, half of the rows are switched off at random, so unwanted rows fall before, between
+    and after the wanted rows of one workgroup."""
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, logprobs_and_entropy_from_logits
+
+    x, labels, w_lp, w_ent = _device_case(cuda, rows, vocab, dtype, std, seed=rows * 7 + vocab)
+    g = torch.Generator().manual_seed(rows + 1)
+    row_mask = None
+    if masked:
+        row_mask = (torch.rand(rows, generator=g) < 0.5)
+        row_mask[:3] = torch.tensor([False, True, False])
+        row_mask[256:259] = False  # second rows of workgroups 0-2 off
+        row_mask[-2:] = False
+        row_mask = row_mask.to(cuda)
+    keep = torch.ones(rows, dtype=torch.bool, device=cuda) if row_mask is None else row_mask
+    pick = torch.nonzero(keep).squeeze(-1)
+    pick = pick[torch.randperm(len(pick), generator=g)[:12].to(cuda)]
+    x_pick = x[pick].cpu()
+
+    xa = x.clone().requires_grad_(True)
+    lp2, ent2 = logprobs_and_entropy_from_logits(xa, labels, temperature, inplace_backward=True, row_mask=row_mask)
+    (g2,) = torch.autograd.grad([lp2, ent2], [xa], [w_lp, w_ent])
+    lp, ent, grad = fused_logprob_entropy_fwd_bwd(x, labels, w_lp, w_ent, temperature, inplace=True, row_mask=row_mask)
+    assert grad.data_ptr() == x.data_ptr()
+
+    atol = 1e-5 if dtype == torch.float32 else 2e-3
+    assert (lp - lp2).abs().max().item() <= 2e-5 and (ent - ent2).abs().max().item() <= 2e-5
+    assert _close_to_rounding(grad, g2, dtype) <= 4e-6
+    if masked:
+        off = ~keep
+        assert lp[off].abs().max().item() == 0.0 and ent[off].abs().max().item() == 0.0
+        assert grad[off].abs().max().item() == 0.0
+    ref_lp = otn.log_probs_from_logits(x_pick.double(), labels[pick].cpu(), temperature)
+    ref_ent = otn.compute_entropy(x_pick.double())
+    assert (lp[pick].cpu().double() - ref_lp).abs().max().item() <= atol
+    assert (ent[pick].cpu().double() - ref_ent).abs().max().item() <= atol
+    ref = _analytic_grad64(x_pick, labels[pick].cpu(), temperature, w_lp[pick].cpu(), w_ent[pick].cpu())
+    err = (grad[pick].cpu().double() - ref).abs()
+    if dtype == torch.float32:
+        assert err.max().item() <= 1e-5 * max(1.0, ref.abs().max().item())
+    else:
+        eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -11
+        assert (err <= eps * ref.abs() + 1e-6).all(), err.max().item()
