@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 13
+#define ORLHF_ABI_VERSION 14
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -289,6 +289,23 @@ int orlhf_policy_loss_fwd_grad(const float* log_probs, const float* old_log_prob
                                const int64_t* cu_seqlens, const orlhf_policy_params* params,
                                void* workspace, float* out4, float* row_coef, float* row_aux,
                                float* g_log_probs, orlhf_stream_t stream);
+/*
+ * orlhf_policy_loss_fwd for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): the same kernels and the same
+ * results, bit for bit, with the partial sums in a scratch array built into the library
+ * (ORLHF_NOALLOC_SCRATCH_BYTES per GPU, held from the first call on that GPU until the process
+ * ends) instead of a caller's workspace. It calls no hipMalloc / hipFree and no allocating
+ * routine. No counterpart in the reference. Problems whose orlhf_token_workspace_bytes(n_rows,
+ * n_cols) exceeds the scratch return ORLHF_ERR_UNSUPPORTED. All calls on one GPU share that GPU's
+ * scratch: calls that overlap on one GPU (different streams or host threads) race; serialise them.
+ */
+#define ORLHF_NOALLOC_SCRATCH_BYTES (8 << 20)
+int orlhf_policy_loss_fwd_noalloc(const float* log_probs, const float* old_log_probs,
+                                  const float* advantages, const void* mask, int mask_dtype,
+                                  const float* rollout_log_probs, int64_t n_rows, int64_t n_cols,
+                                  const int64_t* cu_seqlens, const orlhf_policy_params* params,
+                                  float* out4, float* row_coef, float* row_aux,
+                                  orlhf_stream_t stream);
 /* grad wrt log_probs only (everything else is detached in the callers). g_out: device scalar.
  * workspace (orlhf_token_workspace_bytes) is used by GSPO only and may be NULL otherwise. */
 int orlhf_policy_loss_bwd(const float* g_out, const float* log_probs, const float* old_log_probs,

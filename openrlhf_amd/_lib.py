@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 
 class Norm(Structure):
@@ -85,6 +85,7 @@ SIGNATURES = {
     "orlhf_masked_aggregate_bwd": (c_int, [P, P, c_int, I64, I64, P, c_int, P, P, P]),
     "orlhf_policy_loss_fwd": (c_int, [P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P]),
     "orlhf_policy_loss_fwd_grad": (c_int, [P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P, P]),
+    "orlhf_policy_loss_fwd_noalloc": (c_int, [P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P]),
     "orlhf_policy_loss_bwd": (c_int, [P, P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P]),
     "orlhf_value_loss_fwd": (c_int, [P, P, P, P, c_int, I64, I64, P, c_int, c_float, c_int, POINTER(Norm), P, P, P, P]),
     "orlhf_value_loss_fwd_grad": (c_int, [P, P, P, P, c_int, I64, I64, P, c_int, c_float, POINTER(Norm), P, P, P, P, P]),

@@ -12,6 +12,8 @@
 // aggregation weight that the backward kernels multiply with. Chunks past the end of a short
 // packed row return at once. No atomics anywhere: the result is bit-reproducible. All of these
 // are HBM-bound streams of 4-17 bytes per token.
+#include <atomic>
+
 #include "token_terms.h"
 
 namespace orlhf {
@@ -841,6 +843,57 @@ extern "C" int orlhf_policy_loss_fwd(const float* log_probs, const float* old_lo
                                      float* row_coef, float* row_aux, orlhf_stream_t stream) {
   return policy_loss_fwd_impl(log_probs, old_log_probs, advantages, mask, mask_dtype, rollout_log_probs, n_rows,
                               n_cols, cu_seqlens, params, workspace, out4, row_coef, row_aux, nullptr, stream);
+}
+
+// ---------------------------------------------------------------- the entry point that allocates nothing
+// Partial sums of orlhf_policy_loss_fwd_noalloc live in this file-scope device array instead of a
+// caller-provided workspace. Every GPU the library runs on holds its own copy at its own address,
+// taken once per device with hipGetSymbolAddress; host code only ever uses that address.
+static __device__ __align__(256) unsigned char scratch[ORLHF_NOALLOC_SCRATCH_BYTES];
+
+namespace orlhf {
+constexpr int kMaxDevices = 64;
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+
+// Address of `scratch` on the current device (looked up on the first call per device).
+static int scratch_on_current_device(void** out) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "policy_loss_fwd_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  if (device < 0 || device >= kMaxDevices)
+    return fail(ORLHF_ERR_UNSUPPORTED, "policy_loss_fwd_noalloc: device index %d outside [0, %d)", device, kMaxDevices);
+  void* p = g_scratch_ptr[device].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return fail(ORLHF_ERR_LAUNCH, "policy_loss_fwd_noalloc: hipGetSymbolAddress(scratch) on device %d: %s", device,
+                  hipGetErrorString(e));
+    g_scratch_ptr[device].store(p, std::memory_order_release);
+  }
+  *out = p;
+  return ORLHF_OK;
+}
+}  // namespace orlhf
+
+extern "C" int orlhf_policy_loss_fwd_noalloc(const float* log_probs, const float* old_log_probs,
+                                             const float* advantages, const void* mask, int mask_dtype,
+                                             const float* rollout_log_probs, int64_t n_rows, int64_t n_cols,
+                                             const int64_t* cu_seqlens, const orlhf_policy_params* params,
+                                             float* out4, float* row_coef, float* row_aux,
+                                             orlhf_stream_t stream) {
+  if (int rc = check_rows("policy_loss_fwd_noalloc", n_rows, n_cols, mask, mask_dtype)) return rc;
+  const int64_t need = orlhf_token_workspace_bytes(n_rows, n_cols);
+  if (need > (int64_t)ORLHF_NOALLOC_SCRATCH_BYTES)
+    return fail(ORLHF_ERR_UNSUPPORTED,
+                "policy_loss_fwd_noalloc: %lld rows x %lld columns need %lld bytes of partial sums, the built-in "
+                "scratch holds %lld; use orlhf_policy_loss_fwd with a workspace",
+                (long long)n_rows, (long long)n_cols, (long long)need, (long long)ORLHF_NOALLOC_SCRATCH_BYTES);
+  void* ws = nullptr;
+  if (int rc = scratch_on_current_device(&ws)) return rc;
+  // every (row, chunk) partial the later stages read is written by the first stage of this call:
+  // nothing in the scratch has to start at zero
+  return policy_loss_fwd_impl(log_probs, old_log_probs, advantages, mask, mask_dtype, rollout_log_probs, n_rows,
+                              n_cols, cu_seqlens, params, ws, out4, row_coef, row_aux, nullptr, stream);
 }
 
 extern "C" int orlhf_policy_loss_fwd_grad(const float* log_probs, const float* old_log_probs,
