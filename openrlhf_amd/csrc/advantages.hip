@@ -6,8 +6,10 @@
 // carry C entering from later tokens. Maps compose associatively; a wave composes its 64 maps with
 // log2(64) cross-lane steps, the 4 waves of the workgroup chain through LDS, and a row longer than
 // one tile (kBlock * ITEMS tokens) walks its tiles from the end carrying one number. Carries
-// and the in-lane recurrence are fp64, inputs and outputs fp32. A tile goes through LDS both ways
-// so that global loads and stores are coalesced while each lane works on consecutive tokens.
+// and the in-lane recurrence are fp64, inputs and outputs fp32. A lane loads its consecutive
+// tokens straight into registers with one 16-byte load per array (the value after them comes from
+// the next lane by a shuffle) and stores its outputs the same way; only the per-wave affine
+// carries go through LDS.
 #include "common.h"
 
 namespace orlhf {

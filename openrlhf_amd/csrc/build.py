@@ -27,6 +27,7 @@ HIPCC_FLAGS = [
     "-fPIC",
     "-ffp-contract=off",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Werror=align-mismatch",
     "-Wno-unused-command-line-argument",
     "-Wno-option-ignored",
 ]

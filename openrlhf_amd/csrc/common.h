@@ -139,6 +139,7 @@ __device__ __forceinline__ void row_span(const Rows& r, int64_t b, int64_t& star
 // (one more step per row; the scans 10-15 % on ragged packed batches).
 typedef float f32x4e __attribute__((ext_vector_type(4), aligned(4)));
 typedef uint32_t u32x2h __attribute__((ext_vector_type(2), aligned(2)));  // four 2-byte elements
+typedef int64_t i64x2 __attribute__((ext_vector_type(2)));
 typedef int64_t i64x2e __attribute__((ext_vector_type(2), aligned(8)));
 typedef uint32_t u32_b __attribute__((aligned(1)));  // four 1-byte elements
 
@@ -151,8 +152,18 @@ __device__ __forceinline__ f32x4 stream_load4(const float* p) {
 
 // STREAM = false: cached loads, for a lane that comes back to the same cache lines with its next
 // load (two groups of four tokens per lane): non-temporal there fetches the lines twice.
-template <bool STREAM, typename T>
-__device__ __forceinline__ T load_once(const T* p) {
+// One overload per element-aligned type: the parameter keeps the typedef, so the load inside is
+// compiled with the element's alignment, not the natural alignment of the vector.
+template <bool STREAM>
+__device__ __forceinline__ f32x4 load_once(const f32x4e* p) {
+  return STREAM ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool STREAM>
+__device__ __forceinline__ i64x2 load_once(const i64x2e* p) {
+  return STREAM ? __builtin_nontemporal_load(p) : *p;
+}
+template <bool STREAM>
+__device__ __forceinline__ uint32_t load_once(const u32_b* p) {
   return STREAM ? __builtin_nontemporal_load(p) : *p;
 }
 
@@ -170,8 +181,8 @@ __device__ __forceinline__ void load_mask4(const void* mask, int64_t i0, float* 
 #pragma unroll
     for (int k = 0; k < 4; ++k) m[k] = x[k];
   } else {
-    const i64x2e lo = load_once<STREAM>((const i64x2e*)((const int64_t*)mask + i0)),
-                 hi = load_once<STREAM>((const i64x2e*)((const int64_t*)mask + i0 + 2));
+    const i64x2 lo = load_once<STREAM>((const i64x2e*)((const int64_t*)mask + i0)),
+                hi = load_once<STREAM>((const i64x2e*)((const int64_t*)mask + i0 + 2));
     m[0] = (float)lo[0];
     m[1] = (float)lo[1];
     m[2] = (float)hi[0];
