@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 14
+#define ORLHF_ABI_VERSION 15
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -148,6 +148,49 @@ int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logits, int dty
                                   const int64_t* labels, double temperature, const float* w_logprob,
                                   const float* w_entropy, float* logprob, float* entropy,
                                   const uint8_t* row_mask, orlhf_stream_t stream);
+
+/*
+ * lm-head + log-prob + entropy with the logits never in memory: what Actor.forward does between
+ * the last hidden states and the action log-probs (openrlhf/models/actor.py:263-285: the model's
+ * lm_head projection, output["logits"].to(float32), compute_entropy, log_probs_from_logits) as
+ * matrix-core tiles whose logits are folded into per-token statistics in registers.
+ *   logits[i, v] = sum_h hidden[i, h] * weight[v, h]        (fp32 accumulation, never stored)
+ *   logprob / entropy / row_stats as orlhf_logprob_entropy_fwd on those logits
+ *   hidden  [n_rows, hidden_dim] and weight [vocab, hidden_dim] (the nn.Linear layout), bf16 or
+ *           fp16 (`dtype`), element stride 1, row strides in elements; both 4-byte aligned with
+ *           even strides and an even hidden_dim (else ORLHF_ERR_UNSUPPORTED)
+ *   labels  int64 [n_rows] (-100: logprob 0; any other label outside [0, vocab): NaN)
+ *   workspace: orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, 0) bytes, 256-byte aligned
+ * The reference rounds the logits to the 16-bit dtype before the fp32 up-cast; here they stay fp32,
+ * which is the value-preserving side (the same decision as for 16-bit logits above).
+ */
+int64_t orlhf_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab, int backward);
+int orlhf_lmhead_logprob_entropy_fwd(const void* hidden, const void* weight, int dtype, int64_t n_rows,
+                                     int64_t hidden_dim, int64_t vocab, int64_t hidden_stride,
+                                     int64_t weight_stride, const int64_t* labels, double temperature,
+                                     float* logprob, float* entropy, float* row_stats, void* workspace,
+                                     int64_t workspace_bytes, orlhf_stream_t stream);
+/*
+ * Backward of the above down to the hidden states and the lm_head weight (torch autograd through
+ * openrlhf/models/actor.py:263-285 and the projection): with P = d(loss)/d(logits) as in
+ * orlhf_logprob_entropy_bwd, rounded to `dtype` (the dtype the reference's logits gradient has),
+ *   grad_hidden[i, h] = sum_v P[i, v] * weight[v, h]         grad_weight[v, h] = sum_i P[i, v] * hidden[i, h]
+ * both accumulated in fp32 and rounded once to `dtype`. The vocabulary is processed in chunks: per
+ * chunk the logits tiles are recomputed, P is written to the workspace and multiplied twice on the
+ * matrix cores. grad_hidden [n_rows, hidden_dim] / grad_weight [vocab, hidden_dim]: either may be
+ * NULL; row strides in elements. row_stats: from the forward. Rows whose upstream gradients are
+ * both 0 contribute exact zeros.
+ *   workspace: orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, 1) bytes or more (a larger
+ *   workspace means wider chunks), 256-byte aligned.
+ */
+int orlhf_lmhead_logprob_entropy_bwd(const void* hidden, const void* weight, int dtype, int64_t n_rows,
+                                     int64_t hidden_dim, int64_t vocab, int64_t hidden_stride,
+                                     int64_t weight_stride, const int64_t* labels, double temperature,
+                                     const float* g_logprob, const float* g_entropy,
+                                     const float* row_stats, void* grad_hidden,
+                                     int64_t grad_hidden_stride, void* grad_weight,
+                                     int64_t grad_weight_stride, void* workspace,
+                                     int64_t workspace_bytes, orlhf_stream_t stream);
 
 /*
  * The loss assembly of the PPO actor step (openrlhf/trainer/ray/ppo_actor.py:305-352) folded into

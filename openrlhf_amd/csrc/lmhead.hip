@@ -1,0 +1,599 @@
+// Fused lm-head + log-prob / entropy for gfx950: the logits x = hidden @ W^T are produced tile by
+// tile on the matrix cores and consumed on the spot, so the [N, V] logits never exist in memory.
+//
+// Forward: a workgroup owns 256 tokens and a range of vocabulary tiles; for each 256 x 256 tile
+// (vocabulary x tokens, so that one lane holds 64 vocabulary entries of ONE token per MFMA column)
+// it multiplies W[tile] * hidden[block]^T over the hidden dimension and folds the tile into
+// per-token online statistics (max, sum e^(x-m), sum e^(x-m) x, the same at temperature T, and
+// the label's logit), all in registers. Vocabulary ranges are combined by a small second kernel.
+//
+// Backward: the vocabulary is cut into chunks of Vc columns. Per chunk, (1) the logits tiles are
+// recomputed and turned into P = d(loss)/d(logits) in the 16-bit dtype (the rounding the
+// reference's 16-bit logits gradient has), written to a [N, Vc] workspace; (2) dHidden += P @
+// W[chunk] and (3) dW[chunk] = P^T @ hidden run on the same matrix-core tile, which reads operands
+// in either orientation, so no matrix is ever transposed in memory. Only the chunk of P exists at
+// any time (it is written once and read twice, mostly from the Infinity Cache).
+#include "mfma_gemm.h"
+#include "vocab_rows.h"
+
+namespace orlhf {
+namespace lm {
+
+using mm::f32x16;
+using mm::Operand;
+
+// "no value yet" / "not a vocabulary entry". Small enough that e^(kLow - m) is 0 for any real m,
+// large enough that kLow * log2(e) / T stays finite: a lane whose part of a tile lies wholly past
+// the vocabulary keeps (m = kLow, finite sums) and is weighted out exactly when it is merged.
+constexpr float kLow = -1.0e30f;
+constexpr int kMaxSplits = 64;     // vocabulary ranges per token block in the forward
+constexpr int kRec = 8;            // floats per (range, token) record: m, s1, t1, sT, x_label
+constexpr int kParkBytes = 5 * 4 * mm::kThreads * 4;  // running statistics parked in LDS during a product
+constexpr int kFwdLdsBytes = mm::kLdsBytes + kParkBytes;
+
+// Vocabulary offset of accumulator register r of MFMA row-tile mt inside a wave's 128 rows, minus
+// the lane-dependent 4 * (lane >> 5): a compile-time constant per register.
+__device__ __forceinline__ constexpr int reg_off(int mt, int r) { return mt * 32 + 8 * (r >> 2) + (r & 3); }
+
+struct Running {
+  float m, s1, t1, sT, xl;
+};
+
+// Folds one 256 x 256 logits tile into the running statistics of this lane's four tokens.
+// vrem = number of valid vocabulary entries from this lane's first row of the tile on (<= 0: none).
+template <bool BOTH_T, bool EDGE>
+__device__ __forceinline__ void fold_tile(const f32x16 (&acc)[4][4], Running (&run)[4], const int (&lab_rel)[4], int vrem,
+                                          float c1, float cT) {
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    float mx = kLow;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float x = (!EDGE || reg_off(mt, r) < vrem) ? acc[mt][nt][r] : kLow;
+        mx = fmaxf(mx, x);
+      }
+    }
+    const float m_new = fmaxf(run[nt].m, mx);
+    const float n1 = -m_new * c1, nT = -m_new * cT;
+    float s1[2] = {0.0f, 0.0f}, t1[2] = {0.0f, 0.0f}, sT[2] = {0.0f, 0.0f};
+    float xl = run[nt].xl;
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        // entries past the vocabulary (EDGE tiles only) contribute exact zeros, also when the lane
+        // has seen no real entry yet and m_new is still kLow
+        const bool real = !EDGE || reg_off(mt, r) < vrem;
+        const float x = real ? acc[mt][nt][r] : 0.0f;
+        const float e = real ? fast_exp2(fmaf(x, c1, n1)) : 0.0f;
+        s1[r & 1] += e;
+        t1[r & 1] = fmaf(e, x, t1[r & 1]);
+        if (BOTH_T) sT[r & 1] += real ? fast_exp2(fmaf(x, cT, nT)) : 0.0f;
+        xl = (lab_rel[nt] == reg_off(mt, r)) ? x : xl;
+      }
+    }
+    const float d = run[nt].m - m_new;  // <= 0
+    const float q1 = fast_exp2(d * c1);
+    run[nt].s1 = fmaf(run[nt].s1, q1, s1[0] + s1[1]);
+    run[nt].t1 = fmaf(run[nt].t1, q1, t1[0] + t1[1]);
+    if (BOTH_T) run[nt].sT = fmaf(run[nt].sT, fast_exp2(d * cT), sT[0] + sT[1]);
+    run[nt].m = m_new;
+    run[nt].xl = xl;
+  }
+}
+
+__device__ __forceinline__ void merge(Running& a, const Running& b, float c1, float cT, bool both_t) {
+  const float m = fmaxf(a.m, b.m);
+  const float qa = fast_exp2((a.m - m) * c1), qb = fast_exp2((b.m - m) * c1);
+  a.s1 = a.s1 * qa + b.s1 * qb;
+  a.t1 = a.t1 * qa + b.t1 * qb;
+  if (both_t) a.sT = a.sT * fast_exp2((a.m - m) * cT) + b.sT * fast_exp2((b.m - m) * cT);
+  a.xl = fmaxf(a.xl, b.xl);
+  a.m = m;
+}
+
+// ---------------------------------------------------------------- forward: logits tiles -> statistics
+template <int DT, bool BOTH_T>
+__global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, Operand h, const int64_t* __restrict__ labels,
+                                                                     float c1, float cT, float* __restrict__ records,
+                                                                     int64_t n_token_blocks, int n_splits,
+                                                                     int64_t tiles_per_split, int64_t n_vocab_tiles) {
+  extern __shared__ __align__(16) char lds[];
+  const int64_t n_items = n_token_blocks * n_splits;
+  const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
+  if (item >= n_items) return;
+  const int64_t sp = item / n_token_blocks, tb = item - sp * n_token_blocks;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wm = wave & 1u, wn = wave >> 1;
+  const int64_t n_tokens = h.rows, vocab = w.rows;
+
+  // The running statistics of this lane's four tokens wait in LDS while a tile is multiplied:
+  // the product needs every register (256 accumulators, staging, fragments).
+  float* parked = (float*)(lds + mm::kLdsBytes);  // [5 fields][4 tokens][256 threads]
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    parked[(0 * 4 + nt) * 256 + tid] = kLow;
+    parked[(1 * 4 + nt) * 256 + tid] = 0.0f;
+    parked[(2 * 4 + nt) * 256 + tid] = 0.0f;
+    parked[(3 * 4 + nt) * 256 + tid] = 0.0f;
+    parked[(4 * 4 + nt) * 256 + tid] = kLow;
+  }
+  Running run[4];
+  const int64_t vt_end = (sp + 1) * tiles_per_split < n_vocab_tiles ? (sp + 1) * tiles_per_split : n_vocab_tiles;
+  for (int64_t vt = sp * tiles_per_split; vt < vt_end; ++vt) {
+    f32x16 acc[4][4];
+    mm::tile_product<DT, false, false>(acc, w, h, vt * 256, tb * 256, lds);
+    const int64_t vbase = vt * 256 + wm * 128 + 4 * (lane >> 5);  // vocabulary index of this lane's register offset 0
+    int lab_rel[4];
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int64_t tok = tb * 256 + mm::acc_col(wn, nt, lane);
+      const int64_t d = ((labels != nullptr && tok < n_tokens) ? labels[tok] : -1) - vbase;
+      lab_rel[nt] = (d >= 0 && d < 128) ? (int)d : -1;
+      run[nt] = Running{parked[(0 * 4 + nt) * 256 + tid], parked[(1 * 4 + nt) * 256 + tid], parked[(2 * 4 + nt) * 256 + tid],
+                        parked[(3 * 4 + nt) * 256 + tid], parked[(4 * 4 + nt) * 256 + tid]};
+    }
+    if (vt * 256 + 256 <= vocab) {
+      fold_tile<BOTH_T, false>(acc, run, lab_rel, 128, c1, cT);
+    } else {
+      const int64_t left = vocab - vbase;
+      fold_tile<BOTH_T, true>(acc, run, lab_rel, left > 128 ? 128 : (left < 0 ? 0 : (int)left), c1, cT);
+    }
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      parked[(0 * 4 + nt) * 256 + tid] = run[nt].m;
+      parked[(1 * 4 + nt) * 256 + tid] = run[nt].s1;
+      parked[(2 * 4 + nt) * 256 + tid] = run[nt].t1;
+      parked[(3 * 4 + nt) * 256 + tid] = run[nt].sT;
+      parked[(4 * 4 + nt) * 256 + tid] = run[nt].xl;
+    }
+  }
+  // the two lane halves and the two waves along the vocabulary hold parts of the same tokens
+  float* ex = (float*)lds;  // the slab buffers are free after the last product's closing barrier
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    Running o;
+    o.m = __shfl_xor(run[nt].m, 32, kWave);
+    o.s1 = __shfl_xor(run[nt].s1, 32, kWave);
+    o.t1 = __shfl_xor(run[nt].t1, 32, kWave);
+    o.sT = __shfl_xor(run[nt].sT, 32, kWave);
+    o.xl = __shfl_xor(run[nt].xl, 32, kWave);
+    merge(run[nt], o, c1, cT, BOTH_T);
+    if (wm == 1 && lane < 32) {
+      float* p = ex + ((wn * 4 + nt) * 32 + lane) * 5;
+      p[0] = run[nt].m, p[1] = run[nt].s1, p[2] = run[nt].t1, p[3] = run[nt].sT, p[4] = run[nt].xl;
+    }
+  }
+  __syncthreads();
+  if (wm == 0 && lane < 32) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const float* p = ex + ((wn * 4 + nt) * 32 + lane) * 5;
+      const Running o{p[0], p[1], p[2], p[3], p[4]};
+      merge(run[nt], o, c1, cT, BOTH_T);
+      const int64_t tok = tb * 256 + mm::acc_col(wn, nt, lane);
+      if (tok < n_tokens) {
+        float* rec = records + (sp * n_tokens + tok) * kRec;
+        *(f32x4*)rec = f32x4{run[nt].m, run[nt].s1, run[nt].t1, run[nt].sT};
+        rec[4] = run[nt].xl;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- forward: vocabulary ranges -> outputs
+__global__ __launch_bounds__(kBlock) void lmhead_combine_kernel(const float* __restrict__ records, int64_t n_tokens,
+                                                                int n_splits, const int64_t* __restrict__ labels,
+                                                                int64_t vocab, double temperature, int both_t,
+                                                                float* __restrict__ logprob, float* __restrict__ entropy,
+                                                                float* __restrict__ row_stats) {
+  const int64_t tok = (int64_t)blockIdx.x * kBlock + threadIdx.x;
+  if (tok >= n_tokens) return;
+  const double inv_t = 1.0 / temperature;
+  float m = kLow;
+  for (int sp = 0; sp < n_splits; ++sp) m = fmaxf(m, records[(sp * n_tokens + tok) * kRec]);
+  double s1 = 0.0, t1 = 0.0, sT = 0.0;
+  float xl = kLow;
+  for (int sp = 0; sp < n_splits; ++sp) {
+    const float* rec = records + (sp * n_tokens + tok) * kRec;
+    const double d = (double)rec[0] - (double)m;
+    const double q1 = exp(d);
+    s1 += (double)rec[1] * q1;
+    t1 += (double)rec[2] * q1;
+    if (both_t) sT += (double)rec[3] * exp(d * inv_t);
+    xl = fmaxf(xl, rec[4]);
+  }
+  const double lse1 = (double)m + log(s1);
+  const double lseT = both_t ? (double)m * inv_t + log(sT) : lse1;
+  const double ex = t1 / s1;
+  if (logprob != nullptr) {
+    const int64_t label = labels[tok];
+    float lp;
+    if (label >= 0 && label < vocab)
+      lp = (float)((double)xl * inv_t - lseT);
+    else
+      lp = (label == -100) ? 0.0f : NAN;
+    logprob[tok] = lp;
+  }
+  if (entropy != nullptr) entropy[tok] = (float)(lse1 - ex);
+  if (row_stats != nullptr) *(f32x4*)(row_stats + tok * 4) = f32x4{(float)lseT, (float)lse1, (float)ex, 0.0f};
+}
+
+// ---------------------------------------------------------------- backward (1): logits tiles -> P chunk
+// P[tok][v - v0] = g_lp * (1[v == label] - softmax(x/T)) / T + g_ent * softmax(x) * (E[x] - x), rounded to DT.
+template <int DT, bool BOTH_T>
+__global__ __launch_bounds__(mm::kThreads, 1) void lmhead_bwd_p_kernel(Operand w, Operand h, const int64_t* __restrict__ labels,
+                                                                       double temperature,
+                                                                       const float* __restrict__ g_logprob,
+                                                                       const float* __restrict__ g_entropy,
+                                                                       const float* __restrict__ row_stats,
+                                                                       uint16_t* __restrict__ p_chunk, int64_t ldp,
+                                                                       int64_t v0, int64_t n_token_blocks,
+                                                                       int64_t n_chunk_tiles) {
+  extern __shared__ __align__(16) char lds[];
+  using E = Elt<DT>;
+  constexpr int MODE = BOTH_T ? kBwdBothT : kBwdBothT1;
+  const int64_t n_items = n_token_blocks * n_chunk_tiles;
+  const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
+  if (item >= n_items) return;
+  const int64_t ct = item / n_token_blocks, tb = item - ct * n_token_blocks;
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wm = wave & 1u, wn = wave >> 1;
+  const int64_t n_tokens = h.rows, vocab = w.rows;
+
+  f32x16 acc[4][4];
+  mm::tile_product<DT, false, false>(acc, w, h, v0 + ct * 256, tb * 256, lds);
+
+  const double inv_t = 1.0 / temperature;
+  const int64_t vbase = v0 + ct * 256 + wm * 128 + 4 * (lane >> 5);
+  const int64_t left = vocab - vbase;
+  const int vrem = left > 128 ? 128 : (int)left;
+#pragma unroll
+  for (int nt = 0; nt < 4; ++nt) {
+    const int64_t tok = tb * 256 + mm::acc_col(wn, nt, lane);
+    if (tok >= n_tokens) continue;
+    const float glp = g_logprob != nullptr ? g_logprob[tok] : 0.0f;
+    const float gh = g_entropy != nullptr ? g_entropy[tok] : 0.0f;
+    const f32x4 st = *(const f32x4*)(row_stats + tok * 4);
+    GradFn<MODE> fn;
+    fn.cT = (float)(1.4426950408889634 * inv_t);
+    fn.c1 = kLog2e;
+    fn.negLT = -(float)((double)st[0] * 1.4426950408889634);
+    fn.negL1 = -(float)((double)st[1] * 1.4426950408889634);
+    fn.a_lp = -(float)((double)glp * inv_t);
+    fn.onehot = (float)((double)glp * inv_t);
+    fn.gh = gh;
+    fn.k1 = gh * st[2] - (MODE == kBwdBothT1 ? glp : 0.0f);
+    const int64_t d = (labels != nullptr ? labels[tok] : -1) - vbase;
+    const int lab_rel = (d >= 0 && d < 128) ? (int)d : -1;
+    const bool dead = glp == 0.0f && gh == 0.0f;  // masked token: exact zeros, whatever its statistics hold
+    uint16_t* out = p_chunk + tok * ldp + (ct * 256 + wm * 128 + 4 * (lane >> 5));
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float v[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int off = reg_off(mt, g * 4 + k);
+          float y = fn.elem(acc[mt][nt][g * 4 + k]);
+          if (lab_rel == off) y += fn.onehot;
+          v[k] = (dead || off >= vrem) ? 0.0f : y;
+        }
+        u32x2 pk;
+        if (DT == ORLHF_BF16) {
+          pk[0] = pack_bf16(v[0], v[1]);
+          pk[1] = pack_bf16(v[2], v[3]);
+        } else {
+          pk[0] = pack_f16(v[0], v[1]);
+          pk[1] = pack_f16(v[2], v[3]);
+        }
+        *(u32x2*)(out + mt * 32 + g * 8) = pk;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- backward (2), (3): the two products
+// C[i][j] (fp32, ldc) = or += sum_k A[i][k] * B[j][k] for the tile at (tm, tn).
+template <int DT, bool A_MN, bool B_MN, bool ACCUMULATE>
+__global__ __launch_bounds__(mm::kThreads, 1) void lmhead_gemm_f32_kernel(Operand a, Operand b, float* __restrict__ c,
+                                                                          int64_t ldc, int64_t tiles_m, int64_t tiles_n) {
+  extern __shared__ __align__(16) char lds[];
+  const int64_t n_items = tiles_m * tiles_n;
+  const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
+  if (item >= n_items) return;
+  const int64_t tn = item / tiles_m, tm = item - tn * tiles_m;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wm = wave & 1u, wn = wave >> 1;
+  f32x16 acc[4][4];
+  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds);
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int64_t j = tn * 256 + mm::acc_col(wn, nt, lane);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t i = tm * 256 + mm::acc_row(wm, mt, r, lane);
+        if (i < a.rows && j < b.rows) {
+          float* p = c + i * ldc + j;
+          *p = ACCUMULATE ? *p + acc[mt][nt][r] : acc[mt][nt][r];
+        }
+      }
+    }
+  }
+}
+
+// C[i][j] (DT, ldc) = sum_k A[i][k] * B[j][k], rounded once.
+template <int DT, bool A_MN, bool B_MN>
+__global__ __launch_bounds__(mm::kThreads, 1) void lmhead_gemm_lowp_kernel(Operand a, Operand b, uint16_t* __restrict__ c,
+                                                                           int64_t ldc, int64_t tiles_m, int64_t tiles_n) {
+  extern __shared__ __align__(16) char lds[];
+  using E = Elt<DT>;
+  const int64_t n_items = tiles_m * tiles_n;
+  const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
+  if (item >= n_items) return;
+  const int64_t tn = item / tiles_m, tm = item - tn * tiles_m;
+  const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wm = wave & 1u, wn = wave >> 1;
+  f32x16 acc[4][4];
+  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds);
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const int64_t j = tn * 256 + mm::acc_col(wn, nt, lane);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int64_t i = tm * 256 + mm::acc_row(wm, mt, r, lane);
+        if (i < a.rows && j < b.rows) E::store1((char*)(c + i * ldc + j), acc[mt][nt][r]);
+      }
+    }
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void lmhead_round_kernel(const float* __restrict__ src, int64_t n_rows, int64_t n_cols,
+                                                              uint16_t* __restrict__ dst, int64_t ld_dst) {
+  using E = Elt<DT>;
+  const int64_t n = n_rows * n_cols;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t r = i / n_cols, c = i - r * n_cols;
+    E::store1((char*)(dst + r * ld_dst + c), src[i]);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(kBlock) void lmhead_zero_kernel(uint16_t* __restrict__ dst, int64_t n_rows, int64_t n_cols, int64_t ld) {
+  const int64_t n = n_rows * n_cols;
+  for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    const int64_t r = i / n_cols, c = i - r * n_cols;
+    dst[r * ld + c] = 0;
+  }
+}
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+inline unsigned grid_for_items(int64_t items) { return (unsigned)(((items + 7) / 8) * 8); }
+
+template <typename K>
+static hipError_t allow_lds(K kernel, int bytes = mm::kLdsBytes) {
+  return hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+}
+
+static int check_operands(const char* what, const void* hidden, const void* weight, int dtype, int64_t n_rows,
+                          int64_t hidden_dim, int64_t vocab, int64_t hidden_stride, int64_t weight_stride) {
+  if (dtype != ORLHF_BF16 && dtype != ORLHF_F16)
+    return fail(ORLHF_ERR_UNSUPPORTED, "%s: the matrix-core path takes bf16 or fp16 operands, got dtype %d", what, dtype);
+  if (n_rows < 0 || hidden_dim <= 0 || vocab <= 0)
+    return fail(ORLHF_ERR_INVALID_ARG, "%s: n_rows=%lld hidden=%lld vocab=%lld", what, (long long)n_rows,
+                (long long)hidden_dim, (long long)vocab);
+  if (hidden_stride < hidden_dim || weight_stride < hidden_dim)
+    return fail(ORLHF_ERR_INVALID_ARG, "%s: row strides %lld/%lld < hidden %lld", what, (long long)hidden_stride,
+                (long long)weight_stride, (long long)hidden_dim);
+  if (n_rows > 0 && (hidden == nullptr || weight == nullptr)) return fail(ORLHF_ERR_INVALID_ARG, "%s: NULL hidden / weight", what);
+  // buffer loads fetch whole dwords: bases on 4 bytes, even strides and an even hidden size
+  if ((((uintptr_t)hidden | (uintptr_t)weight) & 3u) != 0 || ((hidden_stride | weight_stride | hidden_dim) & 1) != 0)
+    return fail(ORLHF_ERR_UNSUPPORTED, "%s: hidden / weight must be 4-byte aligned with even row strides and an even hidden size",
+                what);
+  if (hidden_stride >= (1ll << 30) || weight_stride >= (1ll << 30))
+    return fail(ORLHF_ERR_UNSUPPORTED, "%s: row strides beyond 2^30 elements", what);
+  return ORLHF_OK;
+}
+
+// Vocabulary ranges per token block: enough workgroups for two rounds over the chip, whole tiles each.
+static int pick_splits(int64_t n_token_blocks, int64_t n_vocab_tiles, int n_cu) {
+  int64_t want = (2 * (int64_t)n_cu + n_token_blocks - 1) / n_token_blocks;
+  if (want < 1) want = 1;
+  if (want > kMaxSplits) want = kMaxSplits;
+  if (want > n_vocab_tiles) want = n_vocab_tiles;
+  return (int)want;
+}
+
+static int device_cus() {
+  int device = 0, n_cu = 256;
+  if (hipGetDevice(&device) == hipSuccess) {
+    int v = 0;
+    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) n_cu = v;
+  }
+  return n_cu;
+}
+
+// Bytes of the statistics records of the forward.
+static int64_t records_bytes(int64_t n_rows) { return (int64_t)kMaxSplits * (n_rows > 0 ? n_rows : 1) * kRec * 4; }
+// fp32 accumulator of dHidden.
+static int64_t dhidden_bytes(int64_t n_rows, int64_t hidden_dim) { return round_up(n_rows * hidden_dim * 4, 256); }
+
+template <int DT>
+static int launch_fwd(const void* hidden, const void* weight, int64_t n_rows, int64_t hidden_dim, int64_t vocab,
+                      int64_t hidden_stride, int64_t weight_stride, const int64_t* labels, double temperature,
+                      float* logprob, float* entropy, float* row_stats, float* records, hipStream_t s) {
+  const Operand w{(const uint16_t*)weight, weight_stride, vocab, hidden_dim};
+  const Operand h{(const uint16_t*)hidden, hidden_stride, n_rows, hidden_dim};
+  const int64_t n_tb = (n_rows + 255) / 256, n_vt = (vocab + 255) / 256;
+  const int n_splits = pick_splits(n_tb, n_vt, device_cus());
+  const int64_t per = (n_vt + n_splits - 1) / n_splits;
+  const int used_splits = (int)((n_vt + per - 1) / per);  // ranges that hold at least one tile
+  const bool both_t = temperature != 1.0;
+  const float c1 = kLog2e, cT = (float)(1.4426950408889634 / temperature);
+  const dim3 grid(grid_for_items(n_tb * used_splits)), block(mm::kThreads);
+  if (both_t) {
+    if (allow_lds(lmhead_fwd_kernel<DT, true>, kFwdLdsBytes) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", kFwdLdsBytes);
+    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, true>), grid, block, kFwdLdsBytes, s, w, h, labels, c1, cT, records, n_tb,
+                       used_splits, per, n_vt);
+  } else {
+    if (allow_lds(lmhead_fwd_kernel<DT, false>, kFwdLdsBytes) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", kFwdLdsBytes);
+    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, false>), grid, block, kFwdLdsBytes, s, w, h, labels, c1, cT, records, n_tb,
+                       used_splits, per, n_vt);
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_fwd(tiles)");
+  hipLaunchKernelGGL(lmhead_combine_kernel, dim3((unsigned)((n_rows + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, records,
+                     n_rows, used_splits, labels, vocab, temperature, both_t ? 1 : 0, logprob, entropy, row_stats);
+  ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_fwd(combine)");
+  return ORLHF_OK;
+}
+
+template <int DT>
+static int launch_bwd(const void* hidden, const void* weight, int64_t n_rows, int64_t hidden_dim, int64_t vocab,
+                      int64_t hidden_stride, int64_t weight_stride, const int64_t* labels, double temperature,
+                      const float* g_logprob, const float* g_entropy, const float* row_stats, void* grad_hidden,
+                      int64_t grad_hidden_stride, void* grad_weight, int64_t grad_weight_stride, char* workspace,
+                      int64_t chunk_cols, hipStream_t s) {
+  const Operand w{(const uint16_t*)weight, weight_stride, vocab, hidden_dim};
+  const Operand h{(const uint16_t*)hidden, hidden_stride, n_rows, hidden_dim};
+  float* dh_acc = (float*)workspace;
+  uint16_t* p_chunk = (uint16_t*)(workspace + dhidden_bytes(n_rows, hidden_dim));
+  const int64_t n_tb = (n_rows + 255) / 256, tiles_h = (hidden_dim + 255) / 256;
+  const bool both_t = temperature != 1.0;
+  const dim3 block(mm::kThreads);
+  if (allow_lds(lmhead_bwd_p_kernel<DT, true>) != hipSuccess || allow_lds(lmhead_bwd_p_kernel<DT, false>) != hipSuccess ||
+      allow_lds(lmhead_gemm_f32_kernel<DT, false, true, false>) != hipSuccess ||
+      allow_lds(lmhead_gemm_f32_kernel<DT, false, true, true>) != hipSuccess ||
+      allow_lds(lmhead_gemm_lowp_kernel<DT, true, true>) != hipSuccess)
+    return fail(ORLHF_ERR_LAUNCH, "lmhead_bwd: cannot get %d bytes of LDS", mm::kLdsBytes);
+  for (int64_t v0 = 0; v0 < vocab; v0 += chunk_cols) {
+    const int64_t cols = vocab - v0 < chunk_cols ? vocab - v0 : chunk_cols;  // valid vocabulary entries of this chunk
+    const int64_t ctiles = (cols + 255) / 256;
+    const int64_t ldp = chunk_cols;
+    // (1) P chunk
+    {
+      const dim3 grid(grid_for_items(n_tb * ctiles));
+      if (both_t)
+        hipLaunchKernelGGL((lmhead_bwd_p_kernel<DT, true>), grid, block, mm::kLdsBytes, s, w, h, labels, temperature,
+                           g_logprob, g_entropy, row_stats, p_chunk, ldp, v0, n_tb, ctiles);
+      else
+        hipLaunchKernelGGL((lmhead_bwd_p_kernel<DT, false>), grid, block, mm::kLdsBytes, s, w, h, labels, temperature,
+                           g_logprob, g_entropy, row_stats, p_chunk, ldp, v0, n_tb, ctiles);
+      ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(P)");
+    }
+    // (2) dHidden[n][h] (+)= sum_v P[n][v] * W[v0 + v][h]
+    if (grad_hidden != nullptr) {
+      const Operand a{p_chunk, ldp, n_rows, ctiles * 256};  // whole tiles: the pad columns hold zeros
+      const Operand b{(const uint16_t*)weight + v0 * weight_stride, weight_stride, hidden_dim, cols};
+      const dim3 grid(grid_for_items(n_tb * tiles_h));
+      if (v0 == 0)
+        hipLaunchKernelGGL((lmhead_gemm_f32_kernel<DT, false, true, false>), grid, block, mm::kLdsBytes, s, a, b, dh_acc,
+                           hidden_dim, n_tb, tiles_h);
+      else
+        hipLaunchKernelGGL((lmhead_gemm_f32_kernel<DT, false, true, true>), grid, block, mm::kLdsBytes, s, a, b, dh_acc,
+                           hidden_dim, n_tb, tiles_h);
+      ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(dHidden)");
+    }
+    // (3) dW[v0 + v][h] = sum_n P[n][v] * hidden[n][h]
+    if (grad_weight != nullptr) {
+      const Operand a{p_chunk, ldp, cols, n_rows};
+      const Operand b{(const uint16_t*)hidden, hidden_stride, hidden_dim, n_rows};
+      const dim3 grid(grid_for_items(ctiles * tiles_h));
+      hipLaunchKernelGGL((lmhead_gemm_lowp_kernel<DT, true, true>), grid, block, mm::kLdsBytes, s, a, b,
+                         (uint16_t*)grad_weight + v0 * grad_weight_stride, grad_weight_stride, ctiles, tiles_h);
+      ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(dW)");
+    }
+  }
+  if (grad_hidden != nullptr) {
+    hipLaunchKernelGGL(lmhead_round_kernel<DT>, dim3(flat_grid(n_rows * hidden_dim, 16384)), dim3(kBlock), 0, s, dh_acc,
+                       n_rows, hidden_dim, (uint16_t*)grad_hidden, grad_hidden_stride);
+    ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(round)");
+  }
+  return ORLHF_OK;
+}
+
+}  // namespace lm
+}  // namespace orlhf
+
+using namespace orlhf;
+
+extern "C" int64_t orlhf_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab, int backward) {
+  if (n_rows < 0 || hidden_dim <= 0 || vocab <= 0) return 0;
+  if (!backward) return lm::records_bytes(n_rows);
+  // the fp32 dHidden accumulator plus a chunk of P of about 256 MiB (at least one tile column, at most the vocabulary)
+  const int64_t rows = n_rows > 0 ? n_rows : 1;
+  int64_t cols = ((256ll << 20) / (2 * rows)) / 256 * 256;
+  const int64_t vpad = lm::round_up(vocab, 256);
+  cols = cols < 256 ? 256 : (cols > vpad ? vpad : cols);
+  return lm::dhidden_bytes(n_rows, hidden_dim) + rows * cols * 2;
+}
+
+extern "C" int orlhf_lmhead_logprob_entropy_fwd(const void* hidden, const void* weight, int dtype, int64_t n_rows,
+                                                int64_t hidden_dim, int64_t vocab, int64_t hidden_stride,
+                                                int64_t weight_stride, const int64_t* labels, double temperature,
+                                                float* logprob, float* entropy, float* row_stats, void* workspace,
+                                                int64_t workspace_bytes, orlhf_stream_t stream) {
+  if (int rc = lm::check_operands("lmhead_logprob_entropy_fwd", hidden, weight, dtype, n_rows, hidden_dim, vocab,
+                                  hidden_stride, weight_stride))
+    return rc;
+  ORLHF_CHECK_ARG(temperature > 0.0 && temperature == temperature, "lmhead_logprob_entropy_fwd: temperature must be > 0");
+  if (n_rows == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(logprob != nullptr || entropy != nullptr || row_stats != nullptr, "lmhead_logprob_entropy_fwd: nothing to compute");
+  ORLHF_CHECK_ARG(logprob == nullptr || labels != nullptr, "lmhead_logprob_entropy_fwd: labels is NULL");
+  ORLHF_CHECK_ARG(workspace != nullptr && workspace_bytes >= lm::records_bytes(n_rows),
+                  "lmhead_logprob_entropy_fwd: workspace of %lld bytes needed (orlhf_lmhead_workspace_bytes), got %lld",
+                  (long long)lm::records_bytes(n_rows), (long long)workspace_bytes);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == ORLHF_BF16)
+    return lm::launch_fwd<ORLHF_BF16>(hidden, weight, n_rows, hidden_dim, vocab, hidden_stride, weight_stride, labels,
+                                      temperature, logprob, entropy, row_stats, (float*)workspace, s);
+  return lm::launch_fwd<ORLHF_F16>(hidden, weight, n_rows, hidden_dim, vocab, hidden_stride, weight_stride, labels,
+                                   temperature, logprob, entropy, row_stats, (float*)workspace, s);
+}
+
+extern "C" int orlhf_lmhead_logprob_entropy_bwd(const void* hidden, const void* weight, int dtype, int64_t n_rows,
+                                                int64_t hidden_dim, int64_t vocab, int64_t hidden_stride,
+                                                int64_t weight_stride, const int64_t* labels, double temperature,
+                                                const float* g_logprob, const float* g_entropy, const float* row_stats,
+                                                void* grad_hidden, int64_t grad_hidden_stride, void* grad_weight,
+                                                int64_t grad_weight_stride, void* workspace, int64_t workspace_bytes,
+                                                orlhf_stream_t stream) {
+  if (int rc = lm::check_operands("lmhead_logprob_entropy_bwd", hidden, weight, dtype, n_rows, hidden_dim, vocab,
+                                  hidden_stride, weight_stride))
+    return rc;
+  ORLHF_CHECK_ARG(temperature > 0.0 && temperature == temperature, "lmhead_logprob_entropy_bwd: temperature must be > 0");
+  ORLHF_CHECK_ARG(grad_hidden != nullptr || grad_weight != nullptr, "lmhead_logprob_entropy_bwd: nothing to compute");
+  ORLHF_CHECK_ARG(grad_hidden == nullptr || grad_hidden_stride >= hidden_dim, "lmhead_logprob_entropy_bwd: grad_hidden_stride %lld < hidden %lld",
+                  (long long)grad_hidden_stride, (long long)hidden_dim);
+  ORLHF_CHECK_ARG(grad_weight == nullptr || grad_weight_stride >= hidden_dim, "lmhead_logprob_entropy_bwd: grad_weight_stride %lld < hidden %lld",
+                  (long long)grad_weight_stride, (long long)hidden_dim);
+  hipStream_t s = (hipStream_t)stream;
+  if (n_rows == 0) {  // no token: dW is all zeros, dHidden is empty
+    if (grad_weight != nullptr) {
+      hipLaunchKernelGGL(lm::lmhead_zero_kernel<ORLHF_BF16>, dim3(flat_grid(vocab * hidden_dim, 16384)), dim3(kBlock), 0, s,
+                         (uint16_t*)grad_weight, vocab, hidden_dim, grad_weight_stride);
+      ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(zero)");
+    }
+    return ORLHF_OK;
+  }
+  ORLHF_CHECK_ARG(row_stats != nullptr && (g_logprob != nullptr || g_entropy != nullptr),
+                  "lmhead_logprob_entropy_bwd: row_stats and at least one upstream gradient are needed");
+  ORLHF_CHECK_ARG(g_logprob == nullptr || labels != nullptr, "lmhead_logprob_entropy_bwd: labels is NULL");
+  const int64_t fixed = lm::dhidden_bytes(n_rows, hidden_dim);
+  int64_t cols = workspace != nullptr && workspace_bytes > fixed ? ((workspace_bytes - fixed) / (2 * n_rows)) / 256 * 256 : 0;
+  const int64_t vpad = lm::round_up(vocab, 256);
+  if (cols > vpad) cols = vpad;
+  ORLHF_CHECK_ARG(cols >= 256, "lmhead_logprob_entropy_bwd: workspace of %lld bytes is too small (orlhf_lmhead_workspace_bytes gives %lld)",
+                  (long long)workspace_bytes, (long long)orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, 1));
+  ORLHF_CHECK_ARG(((uintptr_t)workspace & 255u) == 0, "lmhead_logprob_entropy_bwd: workspace must be 256-byte aligned");
+  if (dtype == ORLHF_BF16)
+    return lm::launch_bwd<ORLHF_BF16>(hidden, weight, n_rows, hidden_dim, vocab, hidden_stride, weight_stride, labels,
+                                      temperature, g_logprob, g_entropy, row_stats, grad_hidden, grad_hidden_stride,
+                                      grad_weight, grad_weight_stride, (char*)workspace, cols, s);
+  return lm::launch_bwd<ORLHF_F16>(hidden, weight, n_rows, hidden_dim, vocab, hidden_stride, weight_stride, labels,
+                                   temperature, g_logprob, g_entropy, row_stats, grad_hidden, grad_hidden_stride,
+                                   grad_weight, grad_weight_stride, (char*)workspace, cols, s);
+}

@@ -1,0 +1,238 @@
+// bf16 / fp16 matrix-core tile for gfx950 (CDNA4): C[256 x 256] += A[256 x K] * B[256 x K]^T with
+// fp32 accumulation on v_mfma_f32_32x32x16, shared by the lm-head kernels (logits tile, and the
+// two gradient products of the backward).
+//
+// One 256-thread workgroup (4 wave64, one per SIMD) owns a 256 x 256 output tile; wave (wm, wn)
+// owns its 128 x 128 quadrant as 4 x 4 MFMA tiles of 32 x 32 (256 accumulator registers per lane).
+// The K dimension is walked in slabs of 64: a slab of A and of B (32 KiB each) is fetched from
+// global memory into registers (16-byte loads) while the previous slab is multiplied out of LDS,
+// then written to the other LDS buffer (two buffers of 64 KiB, one barrier per slab).
+//
+// LDS layout of a slab: [256 rows][64 k] 16-bit elements, i.e. 8 chunks of 16 bytes per row; chunk
+// kc of row r sits at position kc ^ swz(r), swz(r) = (r ^ (r >> 3)) & 7, which makes the staging
+// writes and the fragment reads (32 consecutive rows, one chunk each) conflict-free.
+//
+// Global loads are buffer loads: a resource covering the operand from the slab's first element to
+// the end of the matrix makes rows past the edge read as zero in hardware (no branches); only a k
+// tail of a K-major operand (depth not a multiple of 64) is masked in registers, in a separate
+// copy of the loop that runs for the last slab alone. Operand bases must be 4-byte aligned and
+// leading dimensions even.
+//
+// An operand may be K-major in memory (element (r, k) at r * ld + k: copied chunk by chunk) or
+// MN-major (element (r, k) at k * ld + r: each thread fetches an 8 x 8 block, transposes it in
+// registers with byte permutes and writes 8 chunks), so the three products of the lm-head path
+// need no transposed copy of any matrix.
+//
+// MFMA 32x32x16 operand layout: lane l supplies row (l & 31), 8 consecutive k starting at
+// (l >> 5) * 8; result register r of lane l is C[8 * (r / 4) + 4 * (l >> 5) + (r & 3)][l & 31].
+#pragma once
+#include "common.h"
+
+namespace orlhf {
+namespace mm {
+
+constexpr int kTile = 256;            // output tile edge
+constexpr int kSlab = 64;             // k elements per slab
+constexpr int kThreads = 256;
+constexpr int kSlabBytes = kTile * kSlab * 2;      // one operand, one slab
+constexpr int kStageBytes = 2 * kSlabBytes;        // A + B
+constexpr int kLdsBytes = 2 * kStageBytes;         // two stages
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4u __attribute__((ext_vector_type(4), aligned(2)));  // 16 bytes at element alignment
+
+__device__ __forceinline__ uint32_t swz(uint32_t row) { return (row ^ (row >> 3)) & 7u; }
+
+// One operand of the product: `rows` x `depth` elements (rows = the M or N extent, depth = K).
+struct Operand {
+  const uint16_t* base;
+  int64_t ld;      // elements between consecutive rows (K-major) or consecutive k (MN-major)
+  int64_t rows;    // valid rows; rows beyond read as zero
+  int64_t depth;   // valid k; k beyond reads as zero
+};
+
+// Buffer resource over the operand's memory from the element at (row0, k0) to the end of the
+// matrix: loads past the end return zero in hardware, so rows beyond the operand need no branch.
+// Offsets inside one slab are 32-bit; the 64-bit part lives in the resource's base.
+template <bool MN_MAJOR>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t slab_resource(const Operand& op, int64_t row0, int64_t k0) {
+  const int64_t first = MN_MAJOR ? k0 * op.ld + row0 : row0 * op.ld + k0;
+  const int64_t end = MN_MAJOR ? (op.depth - 1) * op.ld + op.rows : (op.rows - 1) * op.ld + op.depth;
+  int64_t bytes = ((end - first) * 2 + 3) & ~(int64_t)3;  // whole dwords: the range check is per dword
+  bytes = bytes < 0 ? 0 : (bytes > 0xffffffffll ? 0xffffffffll : bytes);
+  return __builtin_amdgcn_make_buffer_rsrc((void*)(op.base + first), 0, (int)(uint32_t)bytes, 0x00020000);
+}
+
+// ---- global -> registers: the 8 chunks of one thread for the slab starting at k0, rows row0..
+// Rows beyond the operand read as zero (K-major) or as whatever follows (MN-major, where they
+// only reach output rows nobody stores); k beyond the operand must read as zero for both, which
+// the resource does for MN-major and TAIL masks in registers for K-major (the elements past
+// `depth` in a row belong to the next row).
+template <bool MN_MAJOR, bool TAIL>
+__device__ __forceinline__ void fetch_slab(u32x4 (&r)[8], const Operand& op, int64_t row0, int64_t k0, uint32_t tid) {
+  const __amdgpu_buffer_rsrc_t rs = slab_resource<MN_MAJOR>(op, row0, k0);
+  const uint32_t ld2 = (uint32_t)op.ld * 2u;
+  if (!MN_MAJOR) {
+    const uint32_t kc = tid & 7u, rb = tid >> 3;
+    const uint32_t voff = rb * ld2 + kc * 16u;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)(32 * i) * ld2, 0);
+    if (TAIL) {
+      const int64_t valid = op.depth - (k0 + kc * 8);  // elements of this thread's chunks inside the operand
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const uint32_t m = (2 * w < valid ? 0x0000ffffu : 0u) | (2 * w + 1 < valid ? 0xffff0000u : 0u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i][w] &= m;
+      }
+    }
+  } else {
+    const uint32_t c = tid & 31u, kb = tid >> 5;
+    const uint32_t voff = kb * 8u * ld2 + c * 16u;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)i * ld2, 0);
+  }
+}
+
+// ---- registers -> LDS slab ([256][64] swizzled)
+template <bool MN_MAJOR>
+__device__ __forceinline__ void stage_slab(const u32x4 (&r)[8], char* slab, uint32_t tid) {
+  if (!MN_MAJOR) {
+    const uint32_t kc = tid & 7u, rb = tid >> 3;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t row = rb + 32 * i;
+      *(u32x4*)(slab + row * 128u + ((kc ^ swz(row)) << 4)) = r[i];
+    }
+  } else {
+    // r[i] = 8 consecutive rows at k = 8*kb + i  ->  t[e] = 8 consecutive k of row 8*c + e
+    const uint32_t c = tid & 31u, kb = tid >> 5;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      u32x4 t;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint32_t lo = r[2 * j][e >> 1], hi = r[2 * j + 1][e >> 1];
+        t[j] = (e & 1) ? __builtin_amdgcn_perm(hi, lo, 0x07060302u) : __builtin_amdgcn_perm(hi, lo, 0x05040100u);
+      }
+      const uint32_t row = c * 8 + e;
+      *(u32x4*)(slab + row * 128u + ((kb ^ swz(row)) << 4)) = t;
+    }
+  }
+}
+
+template <int DT>
+struct Mfma;
+template <>
+struct Mfma<ORLHF_BF16> {
+  static __device__ __forceinline__ f32x16 run(const u32x4& a, const u32x4& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<ORLHF_F16> {
+  static __device__ __forceinline__ f32x16 run(const u32x4& a, const u32x4& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  }
+};
+
+// ---- one slab out of LDS into the accumulators of this wave
+template <int DT>
+__device__ __forceinline__ void multiply_slab(f32x16 (&acc)[4][4], const char* slab_a, const char* slab_b,
+                                              uint32_t wm, uint32_t wn, uint32_t lane) {
+  const uint32_t lr = lane & 31u, lk = lane >> 5;
+#pragma unroll
+  for (int ks = 0; ks < kSlab / 16; ++ks) {
+    u32x4 a[4], b[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const uint32_t ra = wm * 128u + t * 32u + lr, rb = wn * 128u + t * 32u + lr;
+      a[t] = *(const u32x4*)(slab_a + ra * 128u + (((ks * 2u + lk) ^ swz(ra)) << 4));
+      b[t] = *(const u32x4*)(slab_b + rb * 128u + (((ks * 2u + lk) ^ swz(rb)) << 4));
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = Mfma<DT>::run(a[mt], b[nt], acc[mt][nt]);
+    }
+  }
+}
+
+// ---- the whole product of one output tile: acc = A[row0_a.., :] * B[row0_b.., :]^T over k in [0, depth)
+// `lds` = kLdsBytes of dynamic shared memory. Ends with all waves past their last LDS read.
+//
+// Pipeline: while slab s is multiplied out of one LDS buffer, slab s + 1 (fetched into registers
+// during the previous iteration) is written to the other buffer and the fetch of slab s + 2 is
+// issued into the registers it leaves, so a global load has a whole slab of MFMAs to land.
+template <int DT, bool A_MN_MAJOR, bool B_MN_MAJOR>
+__device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand& a, const Operand& b, int64_t row0_a,
+                                             int64_t row0_b, char* lds) {
+  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+  const uint32_t wm = wave & 1u, wn = wave >> 1;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[mt][nt][r] = 0.0f;
+    }
+  }
+  const int64_t depth = a.depth;
+  const int64_t n_slabs = (depth + kSlab - 1) / kSlab;
+  const int64_t full = depth / kSlab;  // slabs 0 .. full-1 need no masking of a k tail
+  u32x4 ra[8], rb[8];
+  fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, 0, tid);
+  fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, 0, tid);
+  stage_slab<A_MN_MAJOR>(ra, lds, tid);
+  stage_slab<B_MN_MAJOR>(rb, lds + kSlabBytes, tid);
+  if (n_slabs > 1) {
+    fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, kSlab, tid);
+    fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, kSlab, tid);
+  }
+  __syncthreads();
+  int64_t s = 0;
+  for (; s + 2 < full; ++s) {  // steady state: slab s + 2 is whole
+    char* cur = lds + (s & 1) * kStageBytes;
+    char* nxt = lds + ((s + 1) & 1) * kStageBytes;
+    stage_slab<A_MN_MAJOR>(ra, nxt, tid);
+    stage_slab<B_MN_MAJOR>(rb, nxt + kSlabBytes, tid);
+    fetch_slab<A_MN_MAJOR, false>(ra, a, row0_a, (s + 2) * kSlab, tid);
+    fetch_slab<B_MN_MAJOR, false>(rb, b, row0_b, (s + 2) * kSlab, tid);
+    __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, not where the scheduler would sink them
+    multiply_slab<DT>(acc, cur, cur + kSlabBytes, wm, wn, lane);
+    __syncthreads();
+  }
+  for (; s < n_slabs; ++s) {  // the last slabs: a k tail may need masking, fetches run out
+    char* cur = lds + (s & 1) * kStageBytes;
+    char* nxt = lds + ((s + 1) & 1) * kStageBytes;
+    if (s + 1 < n_slabs) {
+      stage_slab<A_MN_MAJOR>(ra, nxt, tid);
+      stage_slab<B_MN_MAJOR>(rb, nxt + kSlabBytes, tid);
+    }
+    if (s + 2 < n_slabs) {
+      fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, (s + 2) * kSlab, tid);
+      fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, (s + 2) * kSlab, tid);
+    }
+    multiply_slab<DT>(acc, cur, cur + kSlabBytes, wm, wn, lane);
+    __syncthreads();
+  }
+}
+
+// Position of accumulator register r of tile (mt, nt) inside the 256 x 256 output tile.
+__device__ __forceinline__ uint32_t acc_row(uint32_t wm, int mt, int r, uint32_t lane) {
+  return wm * 128u + mt * 32u + 8u * (r >> 2) + 4u * (lane >> 5) + (r & 3);
+}
+__device__ __forceinline__ uint32_t acc_col(uint32_t wn, int nt, uint32_t lane) { return wn * 128u + nt * 32u + (lane & 31u); }
+
+// Workgroup index -> tile index such that the workgroups of one XCD (indices congruent modulo 8)
+// work on a contiguous range of tiles and share operand rows through that XCD's L2.
+__device__ __forceinline__ int64_t xcd_contiguous(int64_t wg, int64_t n) {
+  const int64_t per = (n + 7) / 8;
+  const int64_t t = (wg & 7) * per + (wg >> 3);
+  return t;  // may be >= n for the last XCD's slack: callers skip those
+}
+
+}  // namespace mm
+}  // namespace orlhf

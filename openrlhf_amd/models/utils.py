@@ -8,7 +8,9 @@ Mirrors (paths relative to the OpenRLHF tree):
   masked_normalize         openrlhf/models/utils.py:172-179
   compute_entropy          openrlhf/models/utils.py:182-186
 plus ``logprobs_and_entropy_from_logits``, the one-pass form of what Actor.forward does with
-two calls (openrlhf/models/actor.py:269-285).
+two calls (openrlhf/models/actor.py:269-285), and ``lm_head_logprobs_and_entropy``, the same from
+the last hidden states and the lm_head weight with the logits never stored
+(openrlhf/models/actor.py:263-285).
 
 Every function launches hand-written HIP kernels through the C ABI; tensors must be on the GPU.
 
@@ -180,6 +182,96 @@ def compute_entropy(logits: torch.Tensor, inplace_backward: bool = False) -> tor
     """logsumexp(x) - sum(softmax(x) * x) over the last dim (openrlhf/models/utils.py:182-186),
     fp32 result."""
     return _LogprobEntropy.apply(logits, None, 1.0, False, True, inplace_backward)[1]
+
+
+# ------------------------------------------------------------------ lm-head + log-prob, logits never stored
+class _LmHeadLogprobEntropy(torch.autograd.Function):
+    """(hidden states, lm_head weight) -> (log-prob of label, entropy) on matrix-core tiles."""
+
+    @staticmethod
+    def forward(ctx, hidden, weight, labels, temperature):
+        dev = require_gpu(hidden, weight, labels)
+        if hidden.dtype != weight.dtype or hidden.dtype not in (torch.bfloat16, torch.float16):
+            raise TypeError(f"hidden ({hidden.dtype}) and weight ({weight.dtype}) must both be bfloat16 or float16")
+        if hidden.dim() != 2 or weight.dim() != 2 or hidden.shape[1] != weight.shape[1]:
+            raise ValueError(f"hidden {tuple(hidden.shape)} and weight {tuple(weight.shape)} must be [N, H] and [V, H]")
+        if labels.shape != hidden.shape[:1]:
+            raise ValueError(f"labels shape {tuple(labels.shape)} != ({hidden.shape[0]},)")
+        h = hidden.detach()
+        w = weight.detach()
+        h = h if h.stride(1) == 1 and h.stride(0) % 2 == 0 and h.data_ptr() % 4 == 0 else h.contiguous()
+        w = w if w.stride(1) == 1 and w.stride(0) % 2 == 0 and w.data_ptr() % 4 == 0 else w.contiguous()
+        n, hdim = h.shape
+        vocab = w.shape[0]
+        lab = labels.to(torch.int64).contiguous()
+        code = _lib.dtype_code(h)
+        opts = dict(device=dev, dtype=torch.float32)
+        logprob, entropy, stats = torch.empty(n, **opts), torch.empty(n, **opts), torch.empty(n, 4, **opts)
+        lib = _lib.load()
+        ws = torch.empty(lib.orlhf_lmhead_workspace_bytes(n, hdim, vocab, 0), dtype=torch.uint8, device=dev)
+        with _lib.on_device(dev):
+            call("orlhf_lmhead_logprob_entropy_fwd", ptr(h), ptr(w), code, n, hdim, vocab, h.stride(0), w.stride(0),
+                 ptr(lab), float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(ws), ws.numel(), stream_of(dev))
+        ctx.temperature = float(temperature)
+        ctx.set_materialize_grads(False)
+        ctx.save_for_backward(h, w, lab, stats)
+        return logprob, entropy
+
+    @staticmethod
+    def backward(ctx, g_logprob, g_entropy):
+        h, w, lab, stats = ctx.saved_tensors
+        need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        if (g_logprob is None and g_entropy is None) or not (need_h or need_w):
+            return None, None, None, None
+        dev = h.device
+        n, hdim = h.shape
+        vocab = w.shape[0]
+        glp = None if g_logprob is None else g_logprob.reshape(-1).to(torch.float32).contiguous()
+        gent = None if g_entropy is None else g_entropy.reshape(-1).to(torch.float32).contiguous()
+        grad_h = torch.empty((n, hdim), device=dev, dtype=h.dtype) if need_h else None
+        grad_w = torch.empty((vocab, hdim), device=dev, dtype=w.dtype) if need_w else None
+        lib = _lib.load()
+        ws = torch.empty(lib.orlhf_lmhead_workspace_bytes(n, hdim, vocab, 1), dtype=torch.uint8, device=dev)
+        with _lib.on_device(dev):
+            call("orlhf_lmhead_logprob_entropy_bwd", ptr(h), ptr(w), _lib.dtype_code(h), n, hdim, vocab, h.stride(0),
+                 w.stride(0), ptr(lab), ctx.temperature, ptr(glp), ptr(gent), ptr(stats), ptr(grad_h), hdim,
+                 ptr(grad_w), hdim, ptr(ws), ws.numel(), stream_of(dev))
+        return grad_h, grad_w, None, None
+
+
+def lm_head_logprobs_and_entropy(
+    hidden_states: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    labels: torch.Tensor,
+    temperature: float = 1.0,
+    row_mask: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``logits = hidden_states @ lm_head_weight.T`` followed by ``log_probs_from_logits(logits,
+    labels, temperature)`` and ``compute_entropy(logits)`` (openrlhf/models/actor.py:263-285 with
+    the projection that produces ``output["logits"]``), without the ``[..., V]`` logits ever being
+    stored: matrix-core tiles of the projection are folded into per-token statistics on chip, and
+    the backward recomputes them chunk by chunk to produce the gradients of the hidden states and
+    of the weight. The logits stay in fp32 between the projection and the softmax (the reference
+    rounds them to the 16-bit dtype first). fp32 results.
+
+    hidden_states ``[..., H]`` and lm_head_weight ``[V, H]`` in bfloat16 or float16; labels
+    ``[...]``. ``row_mask`` (same shape as labels): positions with 0 are left out of the projection
+    altogether; their outputs are 0 and they receive zero gradient."""
+    batch_shape = hidden_states.shape[:-1]
+    if labels.shape != batch_shape:
+        raise ValueError(f"labels shape {tuple(labels.shape)} != hidden batch shape {tuple(batch_shape)}")
+    rows = hidden_states.reshape(-1, hidden_states.shape[-1])
+    lab = labels.reshape(-1)
+    if row_mask is None:
+        lp, ent = _LmHeadLogprobEntropy.apply(rows, lm_head_weight, lab, temperature)
+        return lp.view(batch_shape), ent.view(batch_shape)
+    if row_mask.shape != batch_shape:
+        raise ValueError(f"row_mask shape {tuple(row_mask.shape)} != hidden batch shape {tuple(batch_shape)}")
+    keep = torch.nonzero(row_mask.reshape(-1) != 0, as_tuple=False).squeeze(-1)
+    lp_k, ent_k = _LmHeadLogprobEntropy.apply(rows[keep], lm_head_weight, lab[keep], temperature)
+    lp = torch.zeros(rows.shape[0], dtype=torch.float32, device=rows.device).index_copy(0, keep, lp_k)
+    ent = torch.zeros(rows.shape[0], dtype=torch.float32, device=rows.device).index_copy(0, keep, ent_k)
+    return lp.view(batch_shape), ent.view(batch_shape)
 
 
 # ------------------------------------------------------------------ per-token helpers
