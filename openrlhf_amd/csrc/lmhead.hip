@@ -1,11 +1,12 @@
 // Fused lm-head + log-prob / entropy for gfx950: the logits x = hidden @ W^T are produced tile by
 // tile on the matrix cores and consumed on the spot, so the [N, V] logits never exist in memory.
 //
-// Forward: a workgroup owns 256 tokens and a range of vocabulary tiles; for each 256 x 256 tile
-// (vocabulary x tokens, so that one lane holds 64 vocabulary entries of ONE token per MFMA column)
+// Forward: a workgroup owns one 256 x 256 tile of the logits
+// (vocabulary x tokens, so that one lane holds 64 vocabulary entries of ONE token per MFMA column):
 // it multiplies W[tile] * hidden[block]^T over the hidden dimension and folds the tile into
-// per-token online statistics (max, sum e^(x-m), sum e^(x-m) x, the same at temperature T, and
-// the label's logit), all in registers. Vocabulary ranges are combined by a small second kernel.
+// per-token statistics (max, sum e^(x-m), sum e^(x-m) x, the same at temperature T, and the
+// label's logit), all in registers; 16 bytes per (tile, token) leave the chip. The tiles of a
+// token are combined by a small second kernel.
 //
 // Backward: the vocabulary is cut into chunks of Vc columns. Per chunk, (1) the logits tiles are
 // recomputed and turned into P = d(loss)/d(logits) in the 16-bit dtype (the rounding the
@@ -26,10 +27,7 @@ using mm::Operand;
 // large enough that kLow * log2(e) / T stays finite: a lane whose part of a tile lies wholly past
 // the vocabulary keeps (m = kLow, finite sums) and is weighted out exactly when it is merged.
 constexpr float kLow = -1.0e30f;
-constexpr int kMaxSplits = 64;     // vocabulary ranges per token block in the forward
-constexpr int kRec = 8;            // floats per (range, token) record: m, s1, t1, sT, x_label
-constexpr int kParkBytes = 5 * 4 * mm::kThreads * 4;  // running statistics parked in LDS during a product
-constexpr int kFwdLdsBytes = mm::kLdsBytes + kParkBytes;
+constexpr int kRec = 4;            // floats per (vocabulary tile, token) record: m, s1, t1, sT
 
 // Vocabulary offset of accumulator register r of MFMA row-tile mt inside a wave's 128 rows, minus
 // the lane-dependent 4 * (lane >> 5): a compile-time constant per register.
@@ -95,96 +93,77 @@ __device__ __forceinline__ void merge(Running& a, const Running& b, float c1, fl
 }
 
 // ---------------------------------------------------------------- forward: logits tiles -> statistics
+// One workgroup per (vocabulary tile, token block): the tile's statistics of each of its 256 tokens
+// go to records[vt][token] = {m, s1, t1, sT}; the lane that holds a token's label writes its logit.
 template <int DT, bool BOTH_T>
 __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, Operand h, const int64_t* __restrict__ labels,
                                                                      float c1, float cT, float* __restrict__ records,
-                                                                     int64_t n_token_blocks, int n_splits,
-                                                                     int64_t tiles_per_split, int64_t n_vocab_tiles) {
+                                                                     float* __restrict__ x_label, int64_t n_token_blocks,
+                                                                     int64_t n_vocab_tiles) {
   extern __shared__ __align__(16) char lds[];
-  const int64_t n_items = n_token_blocks * n_splits;
+  const int64_t n_items = n_token_blocks * n_vocab_tiles;
   const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
   if (item >= n_items) return;
-  const int64_t sp = item / n_token_blocks, tb = item - sp * n_token_blocks;
+  int64_t tb, vt;
+  mm::grouped_tile(item, n_token_blocks, n_vocab_tiles, tb, vt);
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wm = wave & 1u, wn = wave >> 1;
   const int64_t n_tokens = h.rows, vocab = w.rows;
 
-  // The running statistics of this lane's four tokens wait in LDS while a tile is multiplied:
-  // the product needs every register (256 accumulators, staging, fragments).
-  float* parked = (float*)(lds + mm::kLdsBytes);  // [5 fields][4 tokens][256 threads]
+  f32x16 acc[4][4];
+  mm::Chain chain;
+  mm::tile_product<DT, false, false>(acc, w, h, vt * 256, tb * 256, lds, chain);
+
+  const int64_t vbase = vt * 256 + wm * 128 + 4 * (lane >> 5);  // vocabulary index of this lane's register offset 0
+  Running run[4];
+  int lab_rel[4];
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
-    parked[(0 * 4 + nt) * 256 + tid] = kLow;
-    parked[(1 * 4 + nt) * 256 + tid] = 0.0f;
-    parked[(2 * 4 + nt) * 256 + tid] = 0.0f;
-    parked[(3 * 4 + nt) * 256 + tid] = 0.0f;
-    parked[(4 * 4 + nt) * 256 + tid] = kLow;
+    run[nt] = Running{kLow, 0.0f, 0.0f, 0.0f, kLow};
+    const int64_t tok = tb * 256 + mm::acc_col(wn, nt, lane);
+    const int64_t d = ((labels != nullptr && tok < n_tokens) ? labels[tok] : -1) - vbase;
+    lab_rel[nt] = (d >= 0 && d < 128) ? (int)d : -1;
   }
-  Running run[4];
-  const int64_t vt_end = (sp + 1) * tiles_per_split < n_vocab_tiles ? (sp + 1) * tiles_per_split : n_vocab_tiles;
-  for (int64_t vt = sp * tiles_per_split; vt < vt_end; ++vt) {
-    f32x16 acc[4][4];
-    mm::tile_product<DT, false, false>(acc, w, h, vt * 256, tb * 256, lds);
-    const int64_t vbase = vt * 256 + wm * 128 + 4 * (lane >> 5);  // vocabulary index of this lane's register offset 0
-    int lab_rel[4];
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      const int64_t tok = tb * 256 + mm::acc_col(wn, nt, lane);
-      const int64_t d = ((labels != nullptr && tok < n_tokens) ? labels[tok] : -1) - vbase;
-      lab_rel[nt] = (d >= 0 && d < 128) ? (int)d : -1;
-      run[nt] = Running{parked[(0 * 4 + nt) * 256 + tid], parked[(1 * 4 + nt) * 256 + tid], parked[(2 * 4 + nt) * 256 + tid],
-                        parked[(3 * 4 + nt) * 256 + tid], parked[(4 * 4 + nt) * 256 + tid]};
-    }
-    if (vt * 256 + 256 <= vocab) {
-      fold_tile<BOTH_T, false>(acc, run, lab_rel, 128, c1, cT);
-    } else {
-      const int64_t left = vocab - vbase;
-      fold_tile<BOTH_T, true>(acc, run, lab_rel, left > 128 ? 128 : (left < 0 ? 0 : (int)left), c1, cT);
-    }
-#pragma unroll
-    for (int nt = 0; nt < 4; ++nt) {
-      parked[(0 * 4 + nt) * 256 + tid] = run[nt].m;
-      parked[(1 * 4 + nt) * 256 + tid] = run[nt].s1;
-      parked[(2 * 4 + nt) * 256 + tid] = run[nt].t1;
-      parked[(3 * 4 + nt) * 256 + tid] = run[nt].sT;
-      parked[(4 * 4 + nt) * 256 + tid] = run[nt].xl;
-    }
+  if (vt * 256 + 256 <= vocab) {
+    fold_tile<BOTH_T, false>(acc, run, lab_rel, 128, c1, cT);
+  } else {
+    const int64_t left = vocab - vbase;
+    fold_tile<BOTH_T, true>(acc, run, lab_rel, left > 128 ? 128 : (left < 0 ? 0 : (int)left), c1, cT);
   }
   // the two lane halves and the two waves along the vocabulary hold parts of the same tokens
-  float* ex = (float*)lds;  // the slab buffers are free after the last product's closing barrier
+  __syncthreads();  // every wave is done with the slab buffers: they serve as the exchange area now
+  float* ex = (float*)lds;  // [2 wn][4 tokens][32 lanes][4 fields]
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
+    if (run[nt].xl != kLow) {  // exactly one lane of the grid holds a token's label
+      const int64_t tok = tb * 256 + mm::acc_col(wn, nt, lane);
+      if (tok < n_tokens) x_label[tok] = run[nt].xl;
+    }
     Running o;
     o.m = __shfl_xor(run[nt].m, 32, kWave);
     o.s1 = __shfl_xor(run[nt].s1, 32, kWave);
     o.t1 = __shfl_xor(run[nt].t1, 32, kWave);
     o.sT = __shfl_xor(run[nt].sT, 32, kWave);
-    o.xl = __shfl_xor(run[nt].xl, 32, kWave);
+    o.xl = kLow;
     merge(run[nt], o, c1, cT, BOTH_T);
-    if (wm == 1 && lane < 32) {
-      float* p = ex + ((wn * 4 + nt) * 32 + lane) * 5;
-      p[0] = run[nt].m, p[1] = run[nt].s1, p[2] = run[nt].t1, p[3] = run[nt].sT, p[4] = run[nt].xl;
-    }
+    if (wm == 1 && lane < 32) *(f32x4*)(ex + ((wn * 4 + nt) * 32 + lane) * 4) = f32x4{run[nt].m, run[nt].s1, run[nt].t1, run[nt].sT};
   }
   __syncthreads();
   if (wm == 0 && lane < 32) {
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
-      const float* p = ex + ((wn * 4 + nt) * 32 + lane) * 5;
-      const Running o{p[0], p[1], p[2], p[3], p[4]};
+      const f32x4 p = *(const f32x4*)(ex + ((wn * 4 + nt) * 32 + lane) * 4);
+      const Running o{p[0], p[1], p[2], p[3], kLow};
       merge(run[nt], o, c1, cT, BOTH_T);
       const int64_t tok = tb * 256 + mm::acc_col(wn, nt, lane);
-      if (tok < n_tokens) {
-        float* rec = records + (sp * n_tokens + tok) * kRec;
-        *(f32x4*)rec = f32x4{run[nt].m, run[nt].s1, run[nt].t1, run[nt].sT};
-        rec[4] = run[nt].xl;
-      }
+      if (tok < n_tokens) *(f32x4*)(records + (vt * n_tokens + tok) * kRec) = f32x4{run[nt].m, run[nt].s1, run[nt].t1, run[nt].sT};
     }
   }
 }
 
 // ---------------------------------------------------------------- forward: vocabulary ranges -> outputs
-__global__ __launch_bounds__(kBlock) void lmhead_combine_kernel(const float* __restrict__ records, int64_t n_tokens,
-                                                                int n_splits, const int64_t* __restrict__ labels,
+__global__ __launch_bounds__(kBlock) void lmhead_combine_kernel(const float* __restrict__ records,
+                                                                const float* __restrict__ x_label, int64_t n_tokens,
+                                                                int64_t n_tiles, const int64_t* __restrict__ labels,
                                                                 int64_t vocab, double temperature, int both_t,
                                                                 float* __restrict__ logprob, float* __restrict__ entropy,
                                                                 float* __restrict__ row_stats) {
@@ -192,17 +171,15 @@ __global__ __launch_bounds__(kBlock) void lmhead_combine_kernel(const float* __r
   if (tok >= n_tokens) return;
   const double inv_t = 1.0 / temperature;
   float m = kLow;
-  for (int sp = 0; sp < n_splits; ++sp) m = fmaxf(m, records[(sp * n_tokens + tok) * kRec]);
+  for (int64_t t = 0; t < n_tiles; ++t) m = fmaxf(m, records[(t * n_tokens + tok) * kRec]);
   double s1 = 0.0, t1 = 0.0, sT = 0.0;
-  float xl = kLow;
-  for (int sp = 0; sp < n_splits; ++sp) {
-    const float* rec = records + (sp * n_tokens + tok) * kRec;
+  for (int64_t t = 0; t < n_tiles; ++t) {
+    const f32x4 rec = *(const f32x4*)(records + (t * n_tokens + tok) * kRec);
     const double d = (double)rec[0] - (double)m;
     const double q1 = exp(d);
     s1 += (double)rec[1] * q1;
     t1 += (double)rec[2] * q1;
     if (both_t) sT += (double)rec[3] * exp(d * inv_t);
-    xl = fmaxf(xl, rec[4]);
   }
   const double lse1 = (double)m + log(s1);
   const double lseT = both_t ? (double)m * inv_t + log(sT) : lse1;
@@ -211,7 +188,7 @@ __global__ __launch_bounds__(kBlock) void lmhead_combine_kernel(const float* __r
     const int64_t label = labels[tok];
     float lp;
     if (label >= 0 && label < vocab)
-      lp = (float)((double)xl * inv_t - lseT);
+      lp = (float)((double)x_label[tok] * inv_t - lseT);
     else
       lp = (label == -100) ? 0.0f : NAN;
     logprob[tok] = lp;
@@ -237,12 +214,14 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_bwd_p_kernel(Operand w
   const int64_t n_items = n_token_blocks * n_chunk_tiles;
   const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
   if (item >= n_items) return;
-  const int64_t ct = item / n_token_blocks, tb = item - ct * n_token_blocks;
+  int64_t tb, ct;
+  mm::grouped_tile(item, n_token_blocks, n_chunk_tiles, tb, ct);
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wm = wave & 1u, wn = wave >> 1;
   const int64_t n_tokens = h.rows, vocab = w.rows;
 
   f32x16 acc[4][4];
-  mm::tile_product<DT, false, false>(acc, w, h, v0 + ct * 256, tb * 256, lds);
+  mm::Chain chain;
+  mm::tile_product<DT, false, false>(acc, w, h, v0 + ct * 256, tb * 256, lds, chain);
 
   const double inv_t = 1.0 / temperature;
   const int64_t vbase = v0 + ct * 256 + wm * 128 + 4 * (lane >> 5);
@@ -303,10 +282,12 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_gemm_f32_kernel(Operan
   const int64_t n_items = tiles_m * tiles_n;
   const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
   if (item >= n_items) return;
-  const int64_t tn = item / tiles_m, tm = item - tn * tiles_m;
+  int64_t tm, tn;
+  mm::grouped_tile(item, tiles_m, tiles_n, tm, tn);
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wm = wave & 1u, wn = wave >> 1;
   f32x16 acc[4][4];
-  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds);
+  mm::Chain chain;
+  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds, chain);
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
@@ -333,10 +314,12 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_gemm_lowp_kernel(Opera
   const int64_t n_items = tiles_m * tiles_n;
   const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
   if (item >= n_items) return;
-  const int64_t tn = item / tiles_m, tm = item - tn * tiles_m;
+  int64_t tm, tn;
+  mm::grouped_tile(item, tiles_m, tiles_n, tm, tn);
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wm = wave & 1u, wn = wave >> 1;
   f32x16 acc[4][4];
-  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds);
+  mm::Chain chain;
+  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds, chain);
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
@@ -399,26 +382,11 @@ static int check_operands(const char* what, const void* hidden, const void* weig
   return ORLHF_OK;
 }
 
-// Vocabulary ranges per token block: enough workgroups for two rounds over the chip, whole tiles each.
-static int pick_splits(int64_t n_token_blocks, int64_t n_vocab_tiles, int n_cu) {
-  int64_t want = (2 * (int64_t)n_cu + n_token_blocks - 1) / n_token_blocks;
-  if (want < 1) want = 1;
-  if (want > kMaxSplits) want = kMaxSplits;
-  if (want > n_vocab_tiles) want = n_vocab_tiles;
-  return (int)want;
+// Bytes of the forward's workspace: one record per (vocabulary tile, token), then the label logits.
+static int64_t records_bytes(int64_t n_rows, int64_t vocab) {
+  const int64_t rows = n_rows > 0 ? n_rows : 1;
+  return ((vocab + 255) / 256) * rows * kRec * 4 + round_up(rows * 4, 256);
 }
-
-static int device_cus() {
-  int device = 0, n_cu = 256;
-  if (hipGetDevice(&device) == hipSuccess) {
-    int v = 0;
-    if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess && v > 0) n_cu = v;
-  }
-  return n_cu;
-}
-
-// Bytes of the statistics records of the forward.
-static int64_t records_bytes(int64_t n_rows) { return (int64_t)kMaxSplits * (n_rows > 0 ? n_rows : 1) * kRec * 4; }
 // fp32 accumulator of dHidden.
 static int64_t dhidden_bytes(int64_t n_rows, int64_t hidden_dim) { return round_up(n_rows * hidden_dim * 4, 256); }
 
@@ -429,24 +397,20 @@ static int launch_fwd(const void* hidden, const void* weight, int64_t n_rows, in
   const Operand w{(const uint16_t*)weight, weight_stride, vocab, hidden_dim};
   const Operand h{(const uint16_t*)hidden, hidden_stride, n_rows, hidden_dim};
   const int64_t n_tb = (n_rows + 255) / 256, n_vt = (vocab + 255) / 256;
-  const int n_splits = pick_splits(n_tb, n_vt, device_cus());
-  const int64_t per = (n_vt + n_splits - 1) / n_splits;
-  const int used_splits = (int)((n_vt + per - 1) / per);  // ranges that hold at least one tile
+  float* x_label = records + n_vt * n_rows * kRec;
   const bool both_t = temperature != 1.0;
   const float c1 = kLog2e, cT = (float)(1.4426950408889634 / temperature);
-  const dim3 grid(grid_for_items(n_tb * used_splits)), block(mm::kThreads);
+  const dim3 grid(grid_for_items(n_tb * n_vt)), block(mm::kThreads);
   if (both_t) {
-    if (allow_lds(lmhead_fwd_kernel<DT, true>, kFwdLdsBytes) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", kFwdLdsBytes);
-    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, true>), grid, block, kFwdLdsBytes, s, w, h, labels, c1, cT, records, n_tb,
-                       used_splits, per, n_vt);
+    if (allow_lds(lmhead_fwd_kernel<DT, true>) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", mm::kLdsBytes);
+    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, true>), grid, block, mm::kLdsBytes, s, w, h, labels, c1, cT, records, x_label, n_tb, n_vt);
   } else {
-    if (allow_lds(lmhead_fwd_kernel<DT, false>, kFwdLdsBytes) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", kFwdLdsBytes);
-    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, false>), grid, block, kFwdLdsBytes, s, w, h, labels, c1, cT, records, n_tb,
-                       used_splits, per, n_vt);
+    if (allow_lds(lmhead_fwd_kernel<DT, false>) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", mm::kLdsBytes);
+    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, false>), grid, block, mm::kLdsBytes, s, w, h, labels, c1, cT, records, x_label, n_tb, n_vt);
   }
   ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_fwd(tiles)");
   hipLaunchKernelGGL(lmhead_combine_kernel, dim3((unsigned)((n_rows + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, records,
-                     n_rows, used_splits, labels, vocab, temperature, both_t ? 1 : 0, logprob, entropy, row_stats);
+                     x_label, n_rows, n_vt, labels, vocab, temperature, both_t ? 1 : 0, logprob, entropy, row_stats);
   ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_fwd(combine)");
   return ORLHF_OK;
 }
@@ -522,7 +486,7 @@ using namespace orlhf;
 
 extern "C" int64_t orlhf_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab, int backward) {
   if (n_rows < 0 || hidden_dim <= 0 || vocab <= 0) return 0;
-  if (!backward) return lm::records_bytes(n_rows);
+  if (!backward) return lm::records_bytes(n_rows, vocab);
   // the fp32 dHidden accumulator plus a chunk of P of about 256 MiB (at least one tile column, at most the vocabulary)
   const int64_t rows = n_rows > 0 ? n_rows : 1;
   int64_t cols = ((256ll << 20) / (2 * rows)) / 256 * 256;
@@ -543,9 +507,10 @@ extern "C" int orlhf_lmhead_logprob_entropy_fwd(const void* hidden, const void* 
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(logprob != nullptr || entropy != nullptr || row_stats != nullptr, "lmhead_logprob_entropy_fwd: nothing to compute");
   ORLHF_CHECK_ARG(logprob == nullptr || labels != nullptr, "lmhead_logprob_entropy_fwd: labels is NULL");
-  ORLHF_CHECK_ARG(workspace != nullptr && workspace_bytes >= lm::records_bytes(n_rows),
+  ORLHF_CHECK_ARG(workspace != nullptr && workspace_bytes >= lm::records_bytes(n_rows, vocab),
                   "lmhead_logprob_entropy_fwd: workspace of %lld bytes needed (orlhf_lmhead_workspace_bytes), got %lld",
-                  (long long)lm::records_bytes(n_rows), (long long)workspace_bytes);
+                  (long long)lm::records_bytes(n_rows, vocab), (long long)workspace_bytes);
+  ORLHF_CHECK_ARG(((uintptr_t)workspace & 15u) == 0, "lmhead_logprob_entropy_fwd: workspace must be 16-byte aligned");
   hipStream_t s = (hipStream_t)stream;
   if (dtype == ORLHF_BF16)
     return lm::launch_fwd<ORLHF_BF16>(hidden, weight, n_rows, hidden_dim, vocab, hidden_stride, weight_stride, labels,

@@ -4,9 +4,9 @@
 //
 // One 256-thread workgroup (4 wave64, one per SIMD) owns a 256 x 256 output tile; wave (wm, wn)
 // owns its 128 x 128 quadrant as 4 x 4 MFMA tiles of 32 x 32 (256 accumulator registers per lane).
-// The K dimension is walked in slabs of 64: a slab of A and of B (32 KiB each) is fetched from
-// global memory into registers (16-byte loads) while the previous slab is multiplied out of LDS,
-// then written to the other LDS buffer (two buffers of 64 KiB, one barrier per slab).
+// The K dimension is walked in slabs of 64: a slab of A and of B (32 KiB each) arrives in one LDS
+// buffer while the previous slab is multiplied out of the other (two buffers of 64 KiB, one
+// barrier per slab).
 //
 // LDS layout of a slab: [256 rows][64 k] 16-bit elements, i.e. 8 chunks of 16 bytes per row; chunk
 // kc of row r sits at position kc ^ swz(r), swz(r) = (r ^ (r >> 3)) & 7, which makes the staging
@@ -70,7 +70,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t slab_resource(const Operand& o
 // only reach output rows nobody stores); k beyond the operand must read as zero for both, which
 // the resource does for MN-major and TAIL masks in registers for K-major (the elements past
 // `depth` in a row belong to the next row).
-template <bool MN_MAJOR, bool TAIL>
+template <bool MN_MAJOR, bool TAIL, int I0 = 0, int I1 = 8>
 __device__ __forceinline__ void fetch_slab(u32x4 (&r)[8], const Operand& op, int64_t row0, int64_t k0, uint32_t tid) {
   const __amdgpu_buffer_rsrc_t rs = slab_resource<MN_MAJOR>(op, row0, k0);
   const uint32_t ld2 = (uint32_t)op.ld * 2u;
@@ -78,31 +78,52 @@ __device__ __forceinline__ void fetch_slab(u32x4 (&r)[8], const Operand& op, int
     const uint32_t kc = tid & 7u, rb = tid >> 3;
     const uint32_t voff = rb * ld2 + kc * 16u;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)(32 * i) * ld2, 0);
+    for (int i = I0; i < I1; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)(32 * i) * ld2, 0);
     if (TAIL) {
       const int64_t valid = op.depth - (k0 + kc * 8);  // elements of this thread's chunks inside the operand
 #pragma unroll
       for (int w = 0; w < 4; ++w) {
         const uint32_t m = (2 * w < valid ? 0x0000ffffu : 0u) | (2 * w + 1 < valid ? 0xffff0000u : 0u);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) r[i][w] &= m;
+        for (int i = I0; i < I1; ++i) r[i][w] &= m;
       }
     }
   } else {
     const uint32_t c = tid & 31u, kb = tid >> 5;
     const uint32_t voff = kb * 8u * ld2 + c * 16u;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)i * ld2, 0);
+    for (int i = I0; i < I1; ++i) r[i] = __builtin_amdgcn_raw_buffer_load_b128(rs, voff, (uint32_t)i * ld2, 0);
   }
 }
 
-// ---- registers -> LDS slab ([256][64] swizzled)
-template <bool MN_MAJOR>
+// ---- global -> LDS directly (K-major operands, whole slabs): buffer loads that write LDS without
+// passing through registers. One wave-instruction fills 1 KiB of LDS, lane L at byte 16 * L: 8 rows
+// of the slab, so lane L fetches the chunk that the swizzle puts at position (L & 7) of row
+// (L >> 3) of those 8 rows. Rows past the operand arrive as zeros (resource bounds). The caller
+// waits for these loads (vmcnt) before the barrier that publishes the slab.
+__device__ __forceinline__ void dma_slab(const Operand& op, int64_t row0, int64_t k0, char* slab, uint32_t wave_u,
+                                         uint32_t lane) {
+  const __amdgpu_buffer_rsrc_t rs = slab_resource<false>(op, row0, k0);
+  const uint32_t ld2 = (uint32_t)op.ld * 2u;
+  const uint32_t lrow = lane >> 3, x = (lane & 7u) ^ lrow;
+  const uint32_t vbase = lrow * ld2;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    // rows (wave_u * 8 + i) * 8 .. + 7: swz(row) = (row & 7) ^ ((row >> 3) & 7) = lrow ^ i
+    const uint32_t voff = vbase + ((x ^ (uint32_t)i) << 4);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(slab + (wave_u * 8u + i) * 1024u), 16,
+                                             voff, (wave_u * 64u + (uint32_t)i * 8u) * ld2, 0, 0);
+  }
+}
+
+// ---- registers -> LDS slab ([256][64] swizzled). K-major: chunks I0 .. I1-1 of this thread.
+// MN-major: the 8 x 8 block is transposed as a whole; output rows E0 .. E1-1 are written.
+template <bool MN_MAJOR, int I0 = 0, int I1 = 8>
 __device__ __forceinline__ void stage_slab(const u32x4 (&r)[8], char* slab, uint32_t tid) {
   if (!MN_MAJOR) {
     const uint32_t kc = tid & 7u, rb = tid >> 3;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
+    for (int i = I0; i < I1; ++i) {
       const uint32_t row = rb + 32 * i;
       *(u32x4*)(slab + row * 128u + ((kc ^ swz(row)) << 4)) = r[i];
     }
@@ -110,7 +131,7 @@ __device__ __forceinline__ void stage_slab(const u32x4 (&r)[8], char* slab, uint
     // r[i] = 8 consecutive rows at k = 8*kb + i  ->  t[e] = 8 consecutive k of row 8*c + e
     const uint32_t c = tid & 31u, kb = tid >> 5;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
+    for (int e = I0; e < I1; ++e) {
       u32x4 t;
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -138,38 +159,66 @@ struct Mfma<ORLHF_F16> {
   }
 };
 
-// ---- one slab out of LDS into the accumulators of this wave
-template <int DT>
-__device__ __forceinline__ void multiply_slab(f32x16 (&acc)[4][4], const char* slab_a, const char* slab_b,
-                                              uint32_t wm, uint32_t wn, uint32_t lane) {
+// ---- fragments of one k-step (16 k) of a slab: 4 row-tiles of A and 4 of B for this wave
+struct Frags {
+  u32x4 a[4], b[4];
+};
+
+__device__ __forceinline__ void load_frags(Frags& f, const char* slab_a, const char* slab_b, int ks, uint32_t wm,
+                                           uint32_t wn, uint32_t lane) {
   const uint32_t lr = lane & 31u, lk = lane >> 5;
 #pragma unroll
-  for (int ks = 0; ks < kSlab / 16; ++ks) {
-    u32x4 a[4], b[4];
+  for (int t = 0; t < 4; ++t) {
+    const uint32_t ra = wm * 128u + t * 32u + lr, rb = wn * 128u + t * 32u + lr;
+    f.a[t] = *(const u32x4*)(slab_a + ra * 128u + (((ks * 2u + lk) ^ swz(ra)) << 4));
+    f.b[t] = *(const u32x4*)(slab_b + rb * 128u + (((ks * 2u + lk) ^ swz(rb)) << 4));
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void mfma_step(f32x16 (&acc)[4][4], const Frags& f) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const uint32_t ra = wm * 128u + t * 32u + lr, rb = wn * 128u + t * 32u + lr;
-      a[t] = *(const u32x4*)(slab_a + ra * 128u + (((ks * 2u + lk) ^ swz(ra)) << 4));
-      b[t] = *(const u32x4*)(slab_b + rb * 128u + (((ks * 2u + lk) ^ swz(rb)) << 4));
-    }
+  for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-#pragma unroll
-      for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = Mfma<DT>::run(a[mt], b[nt], acc[mt][nt]);
-    }
+    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = Mfma<DT>::run(f.a[mt], f.b[nt], acc[mt][nt]);
   }
 }
 
 // ---- the whole product of one output tile: acc = A[row0_a.., :] * B[row0_b.., :]^T over k in [0, depth)
-// `lds` = kLdsBytes of dynamic shared memory. Ends with all waves past their last LDS read.
+// `lds` = kLdsBytes of dynamic shared memory.
 //
-// Pipeline: while slab s is multiplied out of one LDS buffer, slab s + 1 (fetched into registers
-// during the previous iteration) is written to the other buffer and the fetch of slab s + 2 is
-// issued into the registers it leaves, so a global load has a whole slab of MFMAs to land.
+// Iteration s multiplies slab s out of one LDS buffer while slab s + 1 arrives in the other:
+//  * a K-major operand's slab is loaded straight into LDS (dma_slab), issued at the top of the
+//    iteration; only a slab that crosses the end of the depth goes through registers (masking);
+//  * an MN-major operand's slab s + 1 sits in registers (fetched during iteration s - 1), is
+//    transposed and written to LDS during the first k-steps, and the fetch of slab s + 2 is issued
+//    into the registers it leaves.
+// The fragments of k-step ks + 1 are read from LDS while k-step ks is multiplied; the single
+// barrier of the iteration sits before the LAST k-step's MFMAs, which then cover the read of the
+// next slab's first fragments: the matrix pipe does not drain at a slab boundary.
+// State carried from one product to the next by a workgroup that multiplies several tiles in a
+// row: which LDS buffer the next slab 0 goes to, and whether the previous product already issued
+// its load (during its own last iteration, so that it lands while that tile's epilogue runs).
+struct Chain {
+  uint32_t phase = 0;
+  bool primed = false;
+};
+
+// has_next / next_row0_*: the tile this workgroup multiplies next (same operands), only used with
+// two K-major operands. The function ends WITHOUT a barrier: no wave reads the slab buffers after
+// the barrier inside the last iteration, but a caller that reuses them as scratch must synchronise.
 template <int DT, bool A_MN_MAJOR, bool B_MN_MAJOR>
 __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand& a, const Operand& b, int64_t row0_a,
-                                             int64_t row0_b, char* lds) {
-  const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+                                             int64_t row0_b, char* lds, Chain& chain, bool has_next = false,
+                                             int64_t next_row0_a = 0, int64_t next_row0_b = 0) {
+  constexpr bool kCanChain = !A_MN_MAJOR && !B_MN_MAJOR;
+  // Everything addressed below derives from the thread index: making it opaque keeps a caller's
+  // loop over tiles from hoisting a hundred address registers out of the product and holding
+  // them (spilled) across its epilogue; they are recomputed per tile instead.
+  uint32_t tid = threadIdx.x;
+  asm volatile("" : "+v"(tid));
+  const uint32_t lane = tid & 63u, wave = tid >> 6;
+  const uint32_t wave_u = __builtin_amdgcn_readfirstlane(wave);
   const uint32_t wm = wave & 1u, wn = wave >> 1;
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
@@ -181,43 +230,89 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
   }
   const int64_t depth = a.depth;
   const int64_t n_slabs = (depth + kSlab - 1) / kSlab;
-  const int64_t full = depth / kSlab;  // slabs 0 .. full-1 need no masking of a k tail
+  const int64_t full = depth / kSlab;  // slabs 0 .. full-1 are whole
+  const uint32_t phase = chain.phase;
+  auto buffer = [&](int64_t slab) -> char* { return lds + ((phase + (uint32_t)slab) & 1u) * kStageBytes; };
   u32x4 ra[8], rb[8];
-  fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, 0, tid);
-  fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, 0, tid);
-  stage_slab<A_MN_MAJOR>(ra, lds, tid);
-  stage_slab<B_MN_MAJOR>(rb, lds + kSlabBytes, tid);
-  if (n_slabs > 1) {
-    fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, kSlab, tid);
-    fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, kSlab, tid);
+  if (!(kCanChain && chain.primed)) {
+    fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, 0, tid);
+    fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, 0, tid);
+    stage_slab<A_MN_MAJOR>(ra, buffer(0), tid);
+    stage_slab<B_MN_MAJOR>(rb, buffer(0) + kSlabBytes, tid);
   }
-  __syncthreads();
+  if (n_slabs > 1) {  // MN-major operands carry slab s + 1 in registers from one iteration to the next
+    if (A_MN_MAJOR) fetch_slab<true, true>(ra, a, row0_a, kSlab, tid);
+    if (B_MN_MAJOR) fetch_slab<true, true>(rb, b, row0_b, kSlab, tid);
+  }
+  __syncthreads();  // slab 0 is complete in LDS (also when the previous product loaded it)
+  Frags f0, f1;
+  load_frags(f0, buffer(0), buffer(0) + kSlabBytes, 0, wm, wn, lane);
   int64_t s = 0;
-  for (; s + 2 < full; ++s) {  // steady state: slab s + 2 is whole
-    char* cur = lds + (s & 1) * kStageBytes;
-    char* nxt = lds + ((s + 1) & 1) * kStageBytes;
-    stage_slab<A_MN_MAJOR>(ra, nxt, tid);
-    stage_slab<B_MN_MAJOR>(rb, nxt + kSlabBytes, tid);
-    fetch_slab<A_MN_MAJOR, false>(ra, a, row0_a, (s + 2) * kSlab, tid);
-    fetch_slab<B_MN_MAJOR, false>(rb, b, row0_b, (s + 2) * kSlab, tid);
-    __builtin_amdgcn_sched_barrier(0);  // the loads are issued here, not where the scheduler would sink them
-    multiply_slab<DT>(acc, cur, cur + kSlabBytes, wm, wn, lane);
-    __syncthreads();
+  for (; s + 2 < full; ++s) {  // steady state: slabs s + 1 and s + 2 exist and are whole
+    const char* cur = buffer(s);
+    char* nxt = buffer(s + 1);
+    const int64_t k1 = (s + 1) * kSlab, k2 = (s + 2) * kSlab;
+    // k-step 0
+    if (!A_MN_MAJOR) dma_slab(a, row0_a, k1, nxt, wave_u, lane);
+    if (!B_MN_MAJOR) dma_slab(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);
+    load_frags(f1, cur, cur + kSlabBytes, 1, wm, wn, lane);
+    if (A_MN_MAJOR) stage_slab<true, 0, 4>(ra, nxt, tid);
+    if (B_MN_MAJOR) stage_slab<true, 0, 4>(rb, nxt + kSlabBytes, tid);
+    mfma_step<DT>(acc, f0);
+    __builtin_amdgcn_sched_barrier(0);
+    // k-step 1
+    load_frags(f0, cur, cur + kSlabBytes, 2, wm, wn, lane);
+    if (A_MN_MAJOR) stage_slab<true, 4, 8>(ra, nxt, tid);
+    if (B_MN_MAJOR) stage_slab<true, 4, 8>(rb, nxt + kSlabBytes, tid);
+    mfma_step<DT>(acc, f1);
+    __builtin_amdgcn_sched_barrier(0);
+    // k-step 2
+    load_frags(f1, cur, cur + kSlabBytes, 3, wm, wn, lane);
+    if (A_MN_MAJOR) fetch_slab<true, false>(ra, a, row0_a, k2, tid);
+    if (B_MN_MAJOR) fetch_slab<true, false>(rb, b, row0_b, k2, tid);
+    mfma_step<DT>(acc, f0);
+    __syncthreads();  // every wave holds its last fragments of `cur`; slab s + 1 is complete in `nxt`
+    // k-step 3, over the read of the next slab's first fragments
+    load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
+    mfma_step<DT>(acc, f1);
+    __builtin_amdgcn_sched_barrier(0);
   }
-  for (; s < n_slabs; ++s) {  // the last slabs: a k tail may need masking, fetches run out
-    char* cur = lds + (s & 1) * kStageBytes;
-    char* nxt = lds + ((s + 1) & 1) * kStageBytes;
-    if (s + 1 < n_slabs) {
-      stage_slab<A_MN_MAJOR>(ra, nxt, tid);
-      stage_slab<B_MN_MAJOR>(rb, nxt + kSlabBytes, tid);
+  const bool prime_next = kCanChain && has_next && depth >= kSlab;  // the next tile's slab 0 is whole
+  for (; s < n_slabs; ++s) {  // the last slabs: a k tail may need masking, slabs run out
+    const char* cur = buffer(s);
+    char* nxt = buffer(s + 1);
+    const bool has1 = s + 1 < n_slabs, has2 = s + 2 < n_slabs;
+    if (has1) {
+      if (!A_MN_MAJOR) fetch_slab<false, true>(ra, a, row0_a, (s + 1) * kSlab, tid);
+      if (!B_MN_MAJOR) fetch_slab<false, true>(rb, b, row0_b, (s + 1) * kSlab, tid);
+      if (A_MN_MAJOR) stage_slab<true>(ra, nxt, tid);
+      if (B_MN_MAJOR) stage_slab<true>(rb, nxt + kSlabBytes, tid);
+    } else if (kCanChain && prime_next) {  // the other buffer is free: the next tile's first slab goes there
+      dma_slab(a, next_row0_a, 0, nxt, wave_u, lane);
+      dma_slab(b, next_row0_b, 0, nxt + kSlabBytes, wave_u, lane);
     }
-    if (s + 2 < n_slabs) {
-      fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, (s + 2) * kSlab, tid);
-      fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, (s + 2) * kSlab, tid);
+    if (has2) {
+      if (A_MN_MAJOR) fetch_slab<true, true>(ra, a, row0_a, (s + 2) * kSlab, tid);
+      if (B_MN_MAJOR) fetch_slab<true, true>(rb, b, row0_b, (s + 2) * kSlab, tid);
     }
-    multiply_slab<DT>(acc, cur, cur + kSlabBytes, wm, wn, lane);
-    __syncthreads();
+    load_frags(f1, cur, cur + kSlabBytes, 1, wm, wn, lane);
+    mfma_step<DT>(acc, f0);
+    load_frags(f0, cur, cur + kSlabBytes, 2, wm, wn, lane);
+    mfma_step<DT>(acc, f1);
+    load_frags(f1, cur, cur + kSlabBytes, 3, wm, wn, lane);
+    mfma_step<DT>(acc, f0);
+    if (has1) {
+      if (!A_MN_MAJOR) stage_slab<false>(ra, nxt, tid);
+      if (!B_MN_MAJOR) stage_slab<false>(rb, nxt + kSlabBytes, tid);
+      __syncthreads();
+      load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
+    }
+    // (last iteration: nothing to publish, and the next tile's load is not waited for here; `cur`
+    // is refilled only after the barrier that opens the next product)
+    mfma_step<DT>(acc, f1);
   }
+  chain.phase = phase + (uint32_t)n_slabs;
+  chain.primed = prime_next;
 }
 
 // Position of accumulator register r of tile (mt, nt) inside the 256 x 256 output tile.
@@ -232,6 +327,18 @@ __device__ __forceinline__ int64_t xcd_contiguous(int64_t wg, int64_t n) {
   const int64_t per = (n + 7) / 8;
   const int64_t t = (wg & 7) * per + (wg >> 3);
   return t;  // may be >= n for the last XCD's slack: callers skip those
+}
+
+// Work item t of a tiles_m x tiles_n grid -> (tm, tn) such that 32 consecutive items (what one
+// XCD runs at a time) form an 8 x 4 block: 12 distinct operand row-blocks for 32 tiles, so most
+// slab loads hit that XCD's L2.
+__device__ __forceinline__ void grouped_tile(int64_t t, int64_t tiles_m, int64_t tiles_n, int64_t& tm, int64_t& tn) {
+  const int64_t per_group = 8 * tiles_n;
+  const int64_t group = t / per_group, in_group = t - group * per_group;
+  const int64_t first = group * 8;
+  const int64_t height = tiles_m - first < 8 ? tiles_m - first : 8;
+  tn = in_group / height;
+  tm = first + (in_group - tn * height);
 }
 
 }  // namespace mm
