@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 15
+#define ORLHF_ABI_VERSION 16
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -230,6 +230,55 @@ int orlhf_policy_step_fwd_bwd(const void* logits, void* grad_logits, int dtype, 
                               orlhf_stream_t stream);
 
 /*
+ * Index work around orlhf_policy_step_fwd_bwd, one launch instead of a dozen framework launches.
+ * The per-token terms of the actor step live in [B, A] tensors (the last A of the first T-1
+ * columns of a padded [B, T] batch, openrlhf/models/actor.py:287-296); the vocabulary-row kernel
+ * wants one value per logits row: row r is flat position packed_indices[r] (or r when
+ * packed_indices is NULL and n_rows = B*T) of the [B, T] grid, i.e. (b, t) with action column
+ * t - (T - 1 - A). For every row this writes
+ *   labels_rows      sequences[b, (t + 1) mod T]  (torch.roll(sequences, -1, 1): actor.py:273-276)
+ *   weight_rows      action_mask[b, col] as a float, 0 outside the action columns; need_rows = (weight != 0)
+ *   old / adv / rollout / base rows: the [B, A] value at (b, col), 0 outside the action columns
+ *   policy_coef_rows = row_coef_policy[b] * weight * loss_scale, token_coef_rows likewise with
+ *                      row_coef_token (row_coef of orlhf_masked_aggregate_fwd: the weight of a
+ *                      token in aggregate_loss, openrlhf/models/loss.py:11-39)
+ * rollout / base inputs and outputs are nullable together. Replaces the slicing / masking /
+ * re-padding index arithmetic of openrlhf/models/actor.py:273-296 and
+ * openrlhf/models/ring_attn_utils.py:129-140,181 for the fused step.
+ */
+int orlhf_actor_step_gather(const int64_t* sequences, const void* action_mask, int mask_dtype,
+                            const int64_t* packed_indices, int64_t batch, int64_t seqlen, int64_t width,
+                            int64_t n_rows, const float* old_log_probs, const float* advantages,
+                            const float* rollout_log_probs, const float* base_log_probs,
+                            const float* row_coef_policy, const float* row_coef_token, float loss_scale,
+                            int64_t* labels_rows, uint8_t* need_rows, float* weight_rows, float* old_rows,
+                            float* adv_rows, float* rollout_rows, float* base_rows,
+                            float* policy_coef_rows, float* token_coef_rows, orlhf_stream_t stream);
+/*
+ * Every value the actor training step reports (openrlhf/trainer/ray/ppo_actor.py:305-352), from the
+ * per-row log-probs / entropies orlhf_policy_step_fwd_bwd returned and the per-row arrays above,
+ * in two launches (deterministic two-stage fp64 sums), plus the scatter of the per-row results
+ * back to [B, A]:
+ *   out8 = { loss, actor_loss, clip_ratio, ppo_kl, vllm_kl, kl_loss, entropy_loss, logprobs_diff }
+ *   loss = actor_loss + kl_coef * kl_loss - entropy_coef * entropy_loss (the last only if
+ *   entropy_in_loss); vllm_kl / kl_loss / logprobs_diff / entropy_loss are NaN when their inputs
+ *   (rollout_rows / base_rows / entropy_rows) are NULL.
+ *   action_log_probs [B, A] <- logprob * weight and action_entropy [B, A] <- entropy at the rows'
+ *   action columns; positions no row maps to are left untouched (the caller zero-fills).
+ * Since policy_coef / token_coef are exactly d(aggregate_loss)/d(token loss) (times loss_scale),
+ * the aggregated losses are their dot products with the token losses.
+ * workspace: orlhf_actor_step_values_workspace_bytes(n_rows) bytes.
+ */
+int64_t orlhf_actor_step_values_workspace_bytes(int64_t n_rows);
+int orlhf_actor_step_values(const float* logprob_rows, const float* entropy_rows, const float* weight_rows,
+                            const float* old_rows, const float* adv_rows, const float* rollout_rows,
+                            const float* base_rows, const float* policy_coef_rows,
+                            const float* token_coef_rows, const int64_t* packed_indices, int64_t seqlen,
+                            int64_t width, int64_t n_rows, const orlhf_step_terms* terms, float loss_scale,
+                            int entropy_in_loss, void* workspace, float* action_log_probs,
+                            float* action_entropy, float* out8, orlhf_stream_t stream);
+
+/*
  * data[i] *= g[0] / expected, skipped entirely (every workgroup returns at once) when the ratio
  * is 1: lets an autograd backward hand out a gradient that was produced ahead of time with the
  * scale `expected` and still be correct if the upstream gradient turns out different, without a
@@ -287,6 +336,15 @@ int orlhf_masked_aggregate_fwd(const float* x, const void* mask, int mask_dtype,
  */
 int orlhf_mask_counts(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
                       const int64_t* cu_seqlens, void* workspace, float* out2, orlhf_stream_t stream);
+
+/*
+ * row_coef alone, from the mask: the weight of row b's masked token sum in aggregate_loss
+ * (openrlhf/models/loss.py:11-39) for TOKEN_MEAN / SEQ_MEAN (/ SEQ_MEAN_TOKEN_SUM), known before
+ * any loss value is, which is what lets the fused actor step differentiate in its single pass.
+ * Padded layout. workspace: orlhf_token_workspace_bytes(n_rows, n_cols).
+ */
+int orlhf_mask_row_coef(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols, int mode,
+                        const orlhf_norm* norm, void* workspace, float* row_coef, orlhf_stream_t stream);
 
 /* g_x[b,t] = g(b) * row_coef[b] * mask[b,t]; g(b) = g_out[0] (scalar modes) or g_out[b]. */
 int orlhf_masked_aggregate_bwd(const float* g_out, const void* mask, int mask_dtype,

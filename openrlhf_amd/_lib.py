@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 
 class Norm(Structure):
@@ -80,12 +80,18 @@ SIGNATURES = {
     "orlhf_lmhead_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, P, c_double, P, P, P, P, I64, P,
                                                  I64, P, I64, P]),
     "orlhf_policy_step_fwd_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, POINTER(StepTerms), P, P, P, P]),
+    "orlhf_actor_step_gather": (c_int, [P, P, c_int, P, I64, I64, I64, I64, P, P, P, P, P, P, c_float, P, P, P, P, P, P, P, P,
+                                        P, P]),
+    "orlhf_actor_step_values_workspace_bytes": (I64, [I64]),
+    "orlhf_actor_step_values": (c_int, [P, P, P, P, P, P, P, P, P, P, I64, I64, I64, POINTER(StepTerms), c_float, c_int, P, P,
+                                        P, P, P]),
     "orlhf_rescale_inplace_if": (c_int, [P, c_int, I64, P, c_float, P]),
     "orlhf_approx_kl_fwd": (c_int, [P, P, c_int, I64, c_int, P, P]),
     "orlhf_approx_kl_bwd": (c_int, [P, P, c_int, I64, c_int, P, P, P, P]),
     "orlhf_token_workspace_bytes": (I64, [I64, I64]),
     "orlhf_masked_aggregate_fwd": (c_int, [P, P, c_int, I64, I64, P, c_int, POINTER(Norm), P, P, P, P]),
     "orlhf_mask_counts": (c_int, [P, c_int, I64, I64, P, P, P, P]),
+    "orlhf_mask_row_coef": (c_int, [P, c_int, I64, I64, c_int, POINTER(Norm), P, P, P]),
     "orlhf_masked_aggregate_bwd": (c_int, [P, P, c_int, I64, I64, P, c_int, P, P, P]),
     "orlhf_policy_loss_fwd": (c_int, [P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P]),
     "orlhf_policy_loss_fwd_grad": (c_int, [P, P, P, P, c_int, P, I64, I64, P, POINTER(PolicyParams), P, P, P, P, P, P]),

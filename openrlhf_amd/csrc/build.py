@@ -16,7 +16,7 @@ LIB_DIR = os.path.join(PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libopenrlhf_amd.so")
 
 SOURCES = ["abi.hip", "logprob_entropy.hip", "logprob_entropy_fused.hip", "token_losses.hip", "advantages.hip",
-           "sequence_losses.hip", "row_layout.hip", "row_stats.hip", "lmhead.hip"]
+           "sequence_losses.hip", "row_layout.hip", "row_stats.hip", "lmhead.hip", "actor_rows.hip"]
 
 # -packed-fp32-ops off: v_pk_*_f32 forms generated from plain float code are not trusted on the
 # target machines; the flag only concerns device code (the host pass warns that it is unknown).

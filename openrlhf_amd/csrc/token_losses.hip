@@ -774,6 +774,27 @@ extern "C" int orlhf_mask_counts(const void* mask, int mask_dtype, int64_t n_row
   return ORLHF_OK;
 }
 
+extern "C" int orlhf_mask_row_coef(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols, int mode,
+                                   const orlhf_norm* norm, void* workspace, float* row_coef, orlhf_stream_t stream) {
+  if (int rc = check_rows("mask_row_coef", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(mode == ORLHF_AGG_TOKEN_MEAN || mode == ORLHF_AGG_SEQ_MEAN || mode == ORLHF_AGG_SEQ_MEAN_TOKEN_SUM,
+                  "mask_row_coef: mode %d has no scalar aggregate", mode);
+  ORLHF_CHECK_ARG(row_coef != nullptr && workspace != nullptr, "mask_row_coef: NULL row_coef / workspace");
+  hipStream_t s = (hipStream_t)stream;
+  const Rows rows = make_rows(n_rows, n_cols, nullptr);
+  const int n_chunks = (int)chunks_of(rows);
+  double* partial = (double*)workspace;
+  if (n_rows > 0) {
+    launch_partial(mask_dtype, rows, mask, CountTok{}, partial, n_chunks, s);
+    ORLHF_CHECK_LAUNCH("orlhf_mask_row_coef(partial)");
+  }
+  // the aggregate of the mask itself is of no interest: it goes to the spare tail of the workspace
+  float* unused = (float*)((char*)workspace + orlhf_token_workspace_bytes(n_rows, n_cols) - 256);
+  launch_final<2>(n_rows, n_chunks, partial, mode, norm_arg(norm), 1.0f, 1, unused, row_coef, s);
+  ORLHF_CHECK_LAUNCH("orlhf_mask_row_coef(final)");
+  return ORLHF_OK;
+}
+
 extern "C" int orlhf_masked_aggregate_bwd(const float* g_out, const void* mask, int mask_dtype, int64_t n_rows,
                                           int64_t n_cols, const int64_t* cu_seqlens, int mode,
                                           const float* row_coef, float* g_x, orlhf_stream_t stream) {

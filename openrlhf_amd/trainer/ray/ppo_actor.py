@@ -24,7 +24,7 @@ from ... import _lib
 from ..._lib import call, ptr, require_gpu, stream_of
 from ...models.actor import actor_forward_tail
 from ...models.loss import PolicyLoss, aggregate_loss
-from ...models.utils import _KL_CODES, _as_rows, _workspace, compute_approx_kl
+from ...models.utils import _KL_CODES, _as_rows, _workspace, compute_approx_kl, masked_mean
 
 
 def actor_loss_step(
@@ -44,11 +44,15 @@ def actor_loss_step(
         action_log_probs, old_action_log_probs, advantages, action_mask=action_mask,
         rollout_log_probs=rollout_log_probs, **info)
     result = dict(actor_loss=actor_loss, clip_ratio=clip_ratio, ppo_kl=ppo_kl, vllm_kl=vllm_kl,
-                  action_log_probs=action_log_probs, entropy=entropy, kl_loss=None, entropy_loss=None)
+                  action_log_probs=action_log_probs, entropy=entropy, kl_loss=None, entropy_loss=None,
+                  logprobs_diff=None)
     loss = actor_loss
     if base_action_log_probs is not None:
         kl = compute_approx_kl(action_log_probs, base_action_log_probs, kl_estimator=kl_estimator)
         result["kl_loss"] = aggregate_loss(kl, action_mask, **info)
+        # the "logprobs_diff" status of the step (ppo_actor.py:327-333): masked mean of lp - base
+        with torch.no_grad():
+            result["logprobs_diff"] = masked_mean(action_log_probs.float() - base_action_log_probs.float(), action_mask)
         loss = loss + result["kl_loss"] * kl_coef
     if want_entropy:
         result["entropy_loss"] = aggregate_loss(entropy[:, -action_mask.shape[1]:], action_mask, **info)
@@ -58,22 +62,24 @@ def actor_loss_step(
     return result
 
 
-def _aggregation_coef(action_mask, token_level, dp_size, norm_value):
-    """d(aggregate_loss)/d(token loss) for every [B, A] position: row weight times the mask."""
+def _row_coef(action_mask, token_level, dp_size, norm_value):
+    """d(aggregate_loss)/d(masked token sum of row b) for every row: the weight of a token of row b
+    in the aggregated loss is row_coef[b] * mask[b, t]."""
     dev = action_mask.device
     b, a = action_mask.shape
     mkeep, mptr, mcode = _lib.mask_arg(action_mask)
     keep = []
     norm = _lib.make_norm(dp_size, norm_value, keep)
     ws = _workspace(b, a, dev)
-    dummy = torch.zeros(b, a, dtype=torch.float32, device=dev)
-    out = torch.empty(1, dtype=torch.float32, device=dev)
     row_coef = torch.empty(max(b, 1), dtype=torch.float32, device=dev)
     with _lib.on_device(dev):
-        call("orlhf_masked_aggregate_fwd", ptr(dummy), mptr, mcode, b, a, None,
-             _lib.AGG_TOKEN_MEAN if token_level else _lib.AGG_SEQ_MEAN, norm, ptr(ws), ptr(out), ptr(row_coef),
-             stream_of(dev))
-    return row_coef[:b, None] * action_mask.to(torch.float32)
+        call("orlhf_mask_row_coef", mptr, mcode, b, a, _lib.AGG_TOKEN_MEAN if token_level else _lib.AGG_SEQ_MEAN, norm,
+             ptr(ws), ptr(row_coef), stream_of(dev))
+    return row_coef
+
+
+def _f32c(t):
+    return t.to(torch.float32).contiguous()
 
 
 class _HandOverGradient(torch.autograd.Function):
@@ -90,6 +96,10 @@ class _HandOverGradient(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         (grad,) = ctx.saved_tensors
+        if getattr(ctx, "handed_over", False):
+            # the stored gradient may have been rescaled in place by the first backward
+            raise RuntimeError("the gradient of a fused actor step can be handed over once; run the step again")
+        ctx.handed_over = True
         dev = grad.device
         gf = g.reshape(-1)[:1].to(torch.float32).contiguous()
         with _lib.on_device(dev):
@@ -131,41 +141,38 @@ def fused_actor_loss_step(
     info = dict(dp_size=dp_size, batch_num_tokens=batch_num_tokens, global_batch_size=global_batch_size)
 
     with torch.no_grad():
-        pol_norm = batch_num_tokens if policy_loss_fn.token_level_loss else global_batch_size
-        policy_coef = _aggregation_coef(action_mask, policy_loss_fn.token_level_loss, dp_size, pol_norm) * loss_scale
-        token_coef = _aggregation_coef(action_mask, True, dp_size, batch_num_tokens) * loss_scale
-
-        def to_rows(t):  # [B, A] -> one value per logits row
-            if t is None:
-                return None
-            full = torch.zeros(batch, seqlen, dtype=torch.float32, device=dev)
-            full[:, lo_col:hi_col] = t.to(torch.float32)
-            flat = full.reshape(-1)
-            return (flat if packed_indices is None else flat[packed_indices]).contiguous()
-
-        old_r, adv_r = to_rows(old_action_log_probs), to_rows(advantages)
-        roll_r = to_rows(rollout_log_probs) if use_is else None
-        base_r = to_rows(base_action_log_probs)
-        pc_r, tc_r = to_rows(policy_coef), to_rows(token_coef)
-        need = torch.zeros(batch, seqlen, dtype=torch.uint8, device=dev)
-        need[:, lo_col:hi_col] = (action_mask != 0).to(torch.uint8)
-        labels = torch.roll(sequences, shifts=-1, dims=1).reshape(-1)
-        if packed_indices is not None:
-            need_r, labels = need.reshape(-1)[packed_indices].contiguous(), labels[packed_indices]
-        else:
-            need_r = need.reshape(-1)
-        labels = labels.to(torch.int64).contiguous()
-
         rows, row_stride, aliases = _as_rows(logits.detach().reshape(-1, logits.shape[-1]) if logits.dim() == 3
                                             else logits.detach())
         if not aliases or rows.data_ptr() != logits.data_ptr():
             raise ValueError("fused_actor_loss_step needs logits it can overwrite: contiguous [B, T, V] or [Ttot, V]")
         n_rows, vocab = rows.shape
-        if n_rows != labels.numel():
-            raise ValueError(f"{n_rows} logits rows for {labels.numel()} token positions")
+        expect_rows = batch * seqlen if packed_indices is None else packed_indices.numel()
+        if n_rows != expect_rows:
+            raise ValueError(f"{n_rows} logits rows for {expect_rows} token positions")
         code = _lib.dtype_code(rows)
         if vocab > _lib.load().orlhf_logprob_entropy_fwd_bwd_max_vocab(code):
             raise ValueError(f"a row of {vocab} {rows.dtype} logits is too long for the one-pass kernel; use actor_loss_step")
+
+        # aggregation weights per batch row (they only depend on the mask and the normalisers)
+        token_rc = _row_coef(action_mask, True, dp_size, batch_num_tokens)
+        policy_rc = token_rc if policy_loss_fn.token_level_loss else _row_coef(action_mask, False, dp_size, global_batch_size)
+
+        # one gather launch: everything the vocabulary-row kernel needs per logits row
+        want_entropy = entropy_coef is not None
+        has_base = base_action_log_probs is not None
+        f32 = dict(dtype=torch.float32, device=dev)
+        per_row = torch.empty(7, n_rows, **f32)
+        weight_r, old_r, adv_r, pc_r, tc_r = per_row[0], per_row[1], per_row[2], per_row[3], per_row[4]
+        roll_r = per_row[5] if use_is else None
+        base_r = per_row[6] if has_base else None
+        labels = torch.empty(n_rows, dtype=torch.int64, device=dev)
+        need_r = torch.empty(n_rows, dtype=torch.uint8, device=dev)
+        mkeep, mptr, mcode = _lib.mask_arg(action_mask)
+        seqs = sequences.to(torch.int64).contiguous()
+        idx = None if packed_indices is None else packed_indices.to(torch.int64).contiguous()
+        old_in, adv_in = _f32c(old_action_log_probs), _f32c(advantages)
+        roll_in = _f32c(rollout_log_probs) if use_is else None
+        base_in = _f32c(base_action_log_probs) if has_base else None
 
         terms = _lib.StepTerms()
         terms.old_log_probs, terms.advantages = ptr(old_r), ptr(adv_r)
@@ -178,43 +185,38 @@ def fused_actor_loss_step(
         if use_is:
             terms.is_low, terms.is_high = (float(v) for v in policy_loss_fn.vllm_is_truncated_threshold)
         terms.kl_estimator = _KL_CODES.get(kl_estimator, 0)
-        terms.kl_coef = float(kl_coef) if base_r is not None else 0.0
-        want_entropy = entropy_coef is not None
+        terms.kl_coef = float(kl_coef) if has_base else 0.0
         terms.entropy_coef = float(entropy_coef) if want_entropy else 0.0
 
-        lp_r = torch.empty(n_rows, dtype=torch.float32, device=dev)
-        ent_r = torch.empty(n_rows, dtype=torch.float32, device=dev) if want_entropy else None
+        lp_r = torch.empty(n_rows, **f32)
+        ent_r = torch.empty(n_rows, **f32) if want_entropy else None
+        action_log_probs = torch.zeros(batch, width, **f32)
+        entropy = torch.zeros(batch, width, **f32) if want_entropy else None
+        out8 = torch.empty(8, **f32)
+        lib = _lib.load()
+        ws = torch.empty(lib.orlhf_actor_step_values_workspace_bytes(n_rows), dtype=torch.uint8, device=dev)
         with _lib.on_device(dev):
+            stream = stream_of(dev)
+            call("orlhf_actor_step_gather", ptr(seqs), mptr, mcode, ptr(idx), batch, seqlen, width, n_rows, ptr(old_in),
+                 ptr(adv_in), ptr(roll_in), ptr(base_in), ptr(policy_rc), ptr(token_rc), float(loss_scale), ptr(labels),
+                 ptr(need_r), ptr(weight_r), ptr(old_r), ptr(adv_r), ptr(roll_r), ptr(base_r), ptr(pc_r), ptr(tc_r), stream)
             call("orlhf_policy_step_fwd_bwd", ptr(rows), ptr(rows), code, n_rows, vocab, row_stride, row_stride,
-                 ptr(labels), float(temperature), terms, ptr(lp_r), ptr(ent_r), ptr(need_r), stream_of(dev))
+                 ptr(labels), float(temperature), terms, ptr(lp_r), ptr(ent_r), ptr(need_r), stream)
+            # every value of the step from the per-row results, and their scatter back to [B, A]
+            call("orlhf_actor_step_values", ptr(lp_r), ptr(ent_r), ptr(weight_r), ptr(old_r), ptr(adv_r), ptr(roll_r),
+                 ptr(base_r), ptr(pc_r), ptr(tc_r), ptr(idx), seqlen, width, n_rows, terms, float(loss_scale),
+                 1 if (want_entropy and entropy_coef != 0) else 0, ptr(ws), ptr(action_log_probs), ptr(entropy),
+                 ptr(out8), stream)
         torch.autograd.graph.increment_version(rows)
-
-        def from_rows(t):  # one value per logits row -> [B, A]
-            if packed_indices is not None:
-                t = torch.zeros(batch * seqlen, dtype=torch.float32, device=dev).index_copy(0, packed_indices, t)
-            return t.view(batch, seqlen)[:, lo_col:hi_col]
-
-        action_log_probs = from_rows(lp_r) * action_mask.float()
-        entropy = from_rows(ent_r) if want_entropy else None
-
-        # the values, from the per-token outputs (17 B/token kernels)
-        actor_loss, clip_ratio, ppo_kl, vllm_kl = policy_loss_fn(
-            action_log_probs, old_action_log_probs, advantages, action_mask=action_mask,
-            rollout_log_probs=rollout_log_probs, **info)
-        loss = actor_loss
-        kl_loss = entropy_loss = None
-        if base_action_log_probs is not None:
-            kl_loss = aggregate_loss(compute_approx_kl(action_log_probs, base_action_log_probs, kl_estimator),
-                                     action_mask, **info)
-            loss = loss + kl_loss * kl_coef
-        if want_entropy:
-            entropy_loss = aggregate_loss(entropy, action_mask, **info)
-            if entropy_coef != 0:
-                loss = loss - entropy_loss * entropy_coef
+        loss, actor_loss, clip_ratio, ppo_kl = out8[0], out8[1], out8[2], out8[3]
+        vllm_kl = out8[4] if use_is else None
+        kl_loss = out8[5] if has_base else None
+        entropy_loss = out8[6] if want_entropy else None
+        logprobs_diff = out8[7] if has_base else None
 
     grad_logits = rows if rows.shape == logits.shape else rows.view(logits.shape)
     if logits.requires_grad:
         loss = _HandOverGradient.apply(logits, loss, grad_logits, loss_scale)
     return dict(loss=loss, actor_loss=actor_loss, clip_ratio=clip_ratio, ppo_kl=ppo_kl, vllm_kl=vllm_kl,
-                kl_loss=kl_loss, entropy_loss=entropy_loss, action_log_probs=action_log_probs, entropy=entropy,
-                grad_logits=grad_logits)
+                kl_loss=kl_loss, entropy_loss=entropy_loss, logprobs_diff=logprobs_diff,
+                action_log_probs=action_log_probs, entropy=entropy, grad_logits=grad_logits)

@@ -48,9 +48,12 @@ def _oracle_step(logits64, seqs, attn, amask, old, adv, base, roll, temperature,
     pl = ol.policy_loss(alp, old.double(), adv.double(), m, roll.double() if pol_cfg.get("enable_vllm_is_correction") else None,
                         **pol_cfg, **info)
     loss = pl[0]
-    out = dict(actor_loss=pl[0], clip_ratio=pl[1], ppo_kl=pl[2], vllm_kl=pl[3], kl_loss=None, entropy_loss=None)
+    out = dict(actor_loss=pl[0], clip_ratio=pl[1], ppo_kl=pl[2], vllm_kl=pl[3], kl_loss=None, entropy_loss=None,
+               logprobs_diff=None)
     if base is not None:
         out["kl_loss"] = ol.aggregate_loss(otn.compute_approx_kl(alp, base.double(), kl_est), m, **info)
+        # the step's "logprobs_diff" status (openrlhf/trainer/ray/ppo_actor.py:327-333)
+        out["logprobs_diff"] = otn.masked_mean(alp.detach() - base.double(), m)
         loss = loss + out["kl_loss"] * kl_coef
     if ent_coef is not None:
         out["entropy_loss"] = ol.aggregate_loss(ent, m, **info)
@@ -115,7 +118,7 @@ def test_actor_step_matches_oracle(cuda, case, dtype, packed, fused):
         out = actor_loss_step(*args, **kw)
         (out["loss"] * scale).backward()
     atol = 1e-5 if dtype == torch.float32 else 2e-3
-    for key in ("loss", "actor_loss", "clip_ratio", "ppo_kl", "vllm_kl", "kl_loss", "entropy_loss"):
+    for key in ("loss", "actor_loss", "clip_ratio", "ppo_kl", "vllm_kl", "kl_loss", "entropy_loss", "logprobs_diff"):
         if ref[key] is None:
             assert out[key] is None, key
         else:
@@ -146,6 +149,12 @@ def test_fused_step_rescales_when_upstream_differs(cuda):
         (out["loss"] * upstream).backward()
         grads.append(xd.grad.clone())
     assert torch.allclose(grads[1], grads[0] * 0.5, rtol=1e-6, atol=0)
+    # the stored gradient is handed over once: a second backward through the node must not rescale it again
+    xd = logits.to(d).requires_grad_(True)
+    out = fused_actor_loss_step(xd, seqs.to(d), attn.to(d), amask.to(d), old.to(d), adv.to(d), PolicyLoss())
+    (out["loss"] * 0.5).backward(retain_graph=True)
+    with pytest.raises(RuntimeError, match="once"):
+        (out["loss"] * 0.5).backward()
     with pytest.raises(ValueError):
         fused_actor_loss_step(logits.to(d), seqs.to(d), attn.to(d), amask.to(d), old.to(d), adv.to(d),
                               PolicyLoss(policy_loss_type="gspo"))
