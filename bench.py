@@ -478,6 +478,14 @@ def bench_per_token(args, dev, emit=True):
            timed(rot(lambda k: get_cumulative_returns(ps[k]["adv"], ps[k]["mask"], 1.0, cu_seqlens=ps[k].cu_seqlens, max_seqlen=a))), real, 9)
     record("config4.gae_scan_packed",
            timed(rot(lambda k: get_advantages_and_returns(ps[k]["old"], ps[k]["adv"], ps[k]["mask"], 1.0, 0.95, cu_seqlens=ps[k].cu_seqlens))), real, 17)
+    # the same with the rows handed out longest first (the order is computed once per packed batch)
+    order = [p_.longest_first for p_ in ps]
+    record("config4.discounted_returns_packed_longest_first",
+           timed(rot(lambda k: get_cumulative_returns(ps[k]["adv"], ps[k]["mask"], 1.0, cu_seqlens=ps[k].cu_seqlens, max_seqlen=a,
+                                                      row_order=order[k]))), real, 9)
+    record("config4.gae_scan_packed_longest_first",
+           timed(rot(lambda k: get_advantages_and_returns(ps[k]["old"], ps[k]["adv"], ps[k]["mask"], 1.0, 0.95,
+                                                          cu_seqlens=ps[k].cu_seqlens, row_order=order[k]))), real, 17)
     xk = [p_["lp"].clone().requires_grad_(True) for p_ in ps]
 
     def policy_step_packed(k):

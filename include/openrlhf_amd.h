@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 16
+#define ORLHF_ABI_VERSION 17
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -458,15 +458,21 @@ int orlhf_compute_reward(const float* r, float kl_coef, const float* kl, const v
  * v = m*values, r = m*rewards, delta_t = r_t + gamma*v_{t+1} - v_t, A_t = delta_t +
  * gamma*lambd*A_{t+1}, returns = A + v; every column takes part and nothing is re-masked.
  * Parallel reverse scan per row, fp64 carries.
+ * row_order (int64 [n_rows], nullable; also in the two scans below): a permutation of the rows;
+ * workgroup slot s walks row row_order[s]. Results do not depend on it; a caller that knows the
+ * row lengths of a ragged packed batch passes the rows longest first, so that no long row's
+ * sequential walk is left running alone at the end of the launch.
  */
 int orlhf_gae_scan(const float* values, const float* rewards, const void* mask, int mask_dtype,
-                   int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens, float gamma,
-                   float lambd, float* advantages, float* returns, orlhf_stream_t stream);
+                   int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
+                   const int64_t* row_order, float gamma, float lambd, float* advantages,
+                   float* returns, orlhf_stream_t stream);
 
 /* get_cumulative_returns (experience_maker.py:379-411): G_t = m_t*r_t + gamma*G_{t+1}. */
 int orlhf_discounted_returns(const float* rewards, const void* mask, int mask_dtype,
                              int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
-                             float gamma, float* returns, orlhf_stream_t stream);
+                             const int64_t* row_order, float gamma, float* returns,
+                             orlhf_stream_t stream);
 
 /*
  * The per-experience body of compute_advantages_and_returns (experience_maker.py:276-312) in one
@@ -480,9 +486,9 @@ int orlhf_discounted_returns(const float* rewards, const void* mask, int mask_dt
  */
 int orlhf_reward_scan(const float* r, float kl_coef, const float* kl, const float* values,
                       const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
-                      const int64_t* cu_seqlens, int has_clip, float clip_low, float clip_high,
-                      float gamma, float lambd, float* advantages, float* returns,
-                      float* reward_sum, orlhf_stream_t stream);
+                      const int64_t* cu_seqlens, const int64_t* row_order, int has_clip,
+                      float clip_low, float clip_high, float gamma, float lambd, float* advantages,
+                      float* returns, float* reward_sum, orlhf_stream_t stream);
 
 /*
  * Group baseline / normalisation of scalar rewards (experience_maker.py:246-272).

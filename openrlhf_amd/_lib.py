@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 
 class Norm(Structure):
@@ -101,9 +101,9 @@ SIGNATURES = {
     "orlhf_value_loss_fwd_grad": (c_int, [P, P, P, P, c_int, I64, I64, P, c_int, c_float, POINTER(Norm), P, P, P, P, P]),
     "orlhf_value_loss_bwd": (c_int, [P, P, P, P, P, c_int, I64, I64, P, c_int, c_float, P, P, P]),
     "orlhf_compute_reward": (c_int, [P, c_float, P, P, c_int, I64, I64, P, c_int, c_float, c_float, P, P, P]),
-    "orlhf_gae_scan": (c_int, [P, P, P, c_int, I64, I64, P, c_float, c_float, P, P, P]),
-    "orlhf_discounted_returns": (c_int, [P, P, c_int, I64, I64, P, c_float, P, P]),
-    "orlhf_reward_scan": (c_int, [P, c_float, P, P, P, c_int, I64, I64, P, c_int, c_float, c_float, c_float, c_float,
+    "orlhf_gae_scan": (c_int, [P, P, P, c_int, I64, I64, P, P, c_float, c_float, P, P, P]),
+    "orlhf_discounted_returns": (c_int, [P, P, c_int, I64, I64, P, P, c_float, P, P]),
+    "orlhf_reward_scan": (c_int, [P, c_float, P, P, P, c_int, I64, I64, P, P, c_int, c_float, c_float, c_float, c_float,
                                   P, P, P, P]),
     "orlhf_group_normalize": (c_int, [P, P, I64, I64, c_int, P, P, P, P]),
     "orlhf_whiten_workspace_bytes": (I64, [I64]),

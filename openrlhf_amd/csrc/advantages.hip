@@ -292,9 +292,13 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
 
   const int slot_b = slot_bits(rows.n_rows);
   int buf = 0;
-  for (int64_t slot = blockIdx.x; slot < row_slots(rows.n_rows); slot += gridDim.x) {
-    const int64_t b = row_of_slot(slot, slot, slot_b);
-    if (b >= rows.n_rows) continue;
+  // A caller that knows the row lengths hands the rows out longest first (rows.order): the last
+  // workgroups to start then hold the shortest rows, instead of a long row's sequential walk
+  // ending alone. Otherwise rows are spread by row_of_slot().
+  const int64_t n_slots = rows.order != nullptr ? rows.n_rows : row_slots(rows.n_rows);
+  for (int64_t slot = blockIdx.x; slot < n_slots; slot += gridDim.x) {
+    const int64_t b = rows.order != nullptr ? rows.order[slot] : row_of_slot(slot, slot, slot_b);
+    if (b < 0 || b >= rows.n_rows) continue;
     const RowWalk rw = row_walk(rows, b);
     if (rw.len <= 0) {
       if (REWARD && threadIdx.x == 0 && sr.reward_sum != nullptr) sr.reward_sum[b] = 0.0f;
@@ -661,12 +665,12 @@ extern "C" int orlhf_compute_reward(const float* r, float kl_coef, const float* 
 }
 
 extern "C" int orlhf_gae_scan(const float* values, const float* rewards, const void* mask, int mask_dtype,
-                              int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens, float gamma, float lambd,
-                              float* advantages, float* returns, orlhf_stream_t stream) {
+                              int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens, const int64_t* row_order,
+                              float gamma, float lambd, float* advantages, float* returns, orlhf_stream_t stream) {
   if (int rc = check_rows("gae_scan", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(values && rewards && advantages && returns, "gae_scan: NULL pointer");
-  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const Rows rows{n_rows, n_cols, cu_seqlens, 0, row_order};
   launch_scan<true, false>(mask_dtype, rows, values, rewards, mask, (double)gamma, (double)gamma * (double)lambd,
                            SeqReward{}, advantages, returns, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_gae_scan");
@@ -674,12 +678,12 @@ extern "C" int orlhf_gae_scan(const float* values, const float* rewards, const v
 }
 
 extern "C" int orlhf_discounted_returns(const float* rewards, const void* mask, int mask_dtype, int64_t n_rows,
-                                        int64_t n_cols, const int64_t* cu_seqlens, float gamma, float* returns,
-                                        orlhf_stream_t stream) {
+                                        int64_t n_cols, const int64_t* cu_seqlens, const int64_t* row_order,
+                                        float gamma, float* returns, orlhf_stream_t stream) {
   if (int rc = check_rows("discounted_returns", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(rewards && returns, "discounted_returns: NULL pointer");
-  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const Rows rows{n_rows, n_cols, cu_seqlens, 0, row_order};
   launch_scan<false, false>(mask_dtype, rows, nullptr, rewards, mask, (double)gamma, (double)gamma, SeqReward{},
                             nullptr, returns, (hipStream_t)stream);
   ORLHF_CHECK_LAUNCH("orlhf_discounted_returns");
@@ -688,15 +692,15 @@ extern "C" int orlhf_discounted_returns(const float* rewards, const void* mask, 
 
 extern "C" int orlhf_reward_scan(const float* r, float kl_coef, const float* kl, const float* values,
                                  const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
-                                 const int64_t* cu_seqlens, int has_clip, float clip_low, float clip_high,
-                                 float gamma, float lambd, float* advantages, float* returns, float* reward_sum,
-                                 orlhf_stream_t stream) {
+                                 const int64_t* cu_seqlens, const int64_t* row_order, int has_clip, float clip_low,
+                                 float clip_high, float gamma, float lambd, float* advantages, float* returns,
+                                 float* reward_sum, orlhf_stream_t stream) {
   if (int rc = check_rows("reward_scan", n_rows, n_cols, mask, mask_dtype)) return rc;
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(r != nullptr && returns != nullptr && (kl != nullptr || n_cols == 0), "reward_scan: NULL pointer");
   ORLHF_CHECK_ARG((values == nullptr) == (advantages == nullptr),
                   "reward_scan: values and advantages go together (GAE) or are both NULL (discounted returns)");
-  const Rows rows{n_rows, n_cols, cu_seqlens};
+  const Rows rows{n_rows, n_cols, cu_seqlens, 0, row_order};
   const SeqReward sr{r, -(kl_coef > 0.0f ? kl_coef : 0.0f), has_clip, clip_low, clip_high, reward_sum};
   if (values != nullptr)
     launch_scan<true, true>(mask_dtype, rows, values, kl, mask, (double)gamma, (double)gamma * (double)lambd, sr,

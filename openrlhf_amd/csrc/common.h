@@ -118,6 +118,7 @@ struct Rows {
   int64_t n_rows, n_cols;
   const int64_t* cu;  // packed layout when non-null
   int chunk = 0;      // chunked kernels: tokens of one row per work item
+  const int64_t* order = nullptr;  // one-workgroup-per-row kernels: slot s works on row order[s] (a permutation)
 };
 
 __device__ __forceinline__ void row_span(const Rows& r, int64_t b, int64_t& start, int64_t& len) {

@@ -125,6 +125,18 @@ class PackedSteps:
         """A bound on the longest row, known without reading anything back: the padded width."""
         return self.n_cols
 
+    @property
+    def longest_first(self) -> torch.Tensor:
+        """The rows ordered by decreasing length (int64 [B], computed once per batch): what the
+        one-workgroup-per-row scans take as ``row_order`` so that a ragged batch does not end on a
+        single long row's walk."""
+        order = getattr(self, "_longest_first", None)
+        if order is None:
+            lengths = self.cu_seqlens[1:] - self.cu_seqlens[:-1]
+            order = torch.argsort(lengths, descending=True, stable=True)
+            object.__setattr__(self, "_longest_first", order)
+        return order
+
     def to_padded(self, name: str, side: str = "right", value=0) -> torch.Tensor:
         """The named field back as a right- (or left-) padded ``[B, n_cols]`` tensor."""
         return pad_packed(self.fields[name], self.cu_seqlens, self.n_cols, side, value)

@@ -103,6 +103,15 @@ def experience_kl(
     return kl.to(home), kl_mean.to(home), diff_mean.to(home)
 
 
+def _order_arg(row_order, n_rows, dev):
+    """A row permutation as the kernels take it (int64 on the device), or None."""
+    if row_order is None:
+        return None
+    if row_order.numel() != n_rows:
+        raise ValueError(f"row_order has {row_order.numel()} entries for {n_rows} rows")
+    return row_order.to(device=dev, dtype=torch.int64).contiguous()
+
+
 @torch.no_grad()
 def get_advantages_and_returns(
     values: torch.Tensor,
@@ -112,10 +121,13 @@ def get_advantages_and_returns(
     lambd: float,
     cu_seqlens: Optional[torch.Tensor] = None,
     max_seqlen: Optional[int] = None,
+    row_order: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """GAE (experience_maker.py:332-377): with v = mask*values, r = mask*rewards,
     delta_t = r_t + gamma*v_{t+1} - v_t, A_t = delta_t + gamma*lambd*A_{t+1}; returns = A + v.
-    Every column of the [B, A] block takes part and the outputs are not re-masked."""
+    Every column of the [B, A] block takes part and the outputs are not re-masked.
+    ``row_order`` (int64 permutation of the rows, e.g. ``PackedSteps.longest_first``): the order
+    rows are handed to workgroups in; it changes the schedule of a ragged batch, never a result."""
     dev, home = _device_for(values, rewards, action_mask)
     v, r = _f32(_on_gpu(values, dev)), _f32(_on_gpu(rewards, dev))
     mkeep, mptr, mcode = _lib.mask_arg(_on_gpu(action_mask, dev))
@@ -124,8 +136,8 @@ def get_advantages_and_returns(
     cu = _cu_arg(cu_seqlens, dev)
     adv, ret = torch.empty_like(v), torch.empty_like(v)
     with _lib.on_device(dev):
-        call("orlhf_gae_scan", ptr(v), ptr(r), mptr, mcode, n_rows, n_cols, ptr(cu), float(gamma), float(lambd),
-             ptr(adv), ptr(ret), stream_of(dev))
+        call("orlhf_gae_scan", ptr(v), ptr(r), mptr, mcode, n_rows, n_cols, ptr(cu), ptr(_order_arg(row_order, n_rows, dev)),
+             float(gamma), float(lambd), ptr(adv), ptr(ret), stream_of(dev))
     return adv.to(home), ret.to(home)
 
 
@@ -136,6 +148,7 @@ def get_cumulative_returns(
     gamma: float,
     cu_seqlens: Optional[torch.Tensor] = None,
     max_seqlen: Optional[int] = None,
+    row_order: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Discounted reward-to-go G_t = mask_t*r_t + gamma*G_{t+1} (experience_maker.py:379-411)."""
     dev, home = _device_for(rewards, action_mask)
@@ -145,8 +158,8 @@ def get_cumulative_returns(
     cu = _cu_arg(cu_seqlens, dev)
     ret = torch.empty_like(r)
     with _lib.on_device(dev):
-        call("orlhf_discounted_returns", ptr(r), mptr, mcode, n_rows, n_cols, ptr(cu), float(gamma), ptr(ret),
-             stream_of(dev))
+        call("orlhf_discounted_returns", ptr(r), mptr, mcode, n_rows, n_cols, ptr(cu), ptr(_order_arg(row_order, n_rows, dev)),
+             float(gamma), ptr(ret), stream_of(dev))
     return ret.to(home)
 
 
@@ -161,6 +174,7 @@ def reward_advantages_and_returns(
     lambd: float = 1.0,
     reward_clip_range: Optional[Tuple[float, float]] = None,
     cu_seqlens: Optional[torch.Tensor] = None,
+    row_order: Optional[torch.Tensor] = None,
 ) -> Tuple[Optional[torch.Tensor], torch.Tensor, torch.Tensor]:
     """``compute_reward`` followed by GAE (``values`` given) or by the discounted returns
     (``values=None``) in one pass that never stores the per-token reward: the per-experience body
@@ -185,7 +199,7 @@ def reward_advantages_and_returns(
     lo, hi = (reward_clip_range[0], reward_clip_range[1]) if reward_clip_range else (0.0, 0.0)
     with _lib.on_device(dev):
         call("orlhf_reward_scan", ptr(rf), float(kl_coef), ptr(klf), ptr(v), mptr, mcode, n_rows, n_cols, ptr(cu),
-             1 if reward_clip_range else 0, float(lo), float(hi), float(gamma), float(lambd), ptr(adv), ptr(ret),
+             ptr(_order_arg(row_order, n_rows, dev)), 1 if reward_clip_range else 0, float(lo), float(hi), float(gamma), float(lambd), ptr(adv), ptr(ret),
              ptr(total), stream_of(dev))
     return (None if adv is None else adv.to(home)), ret.to(home), total.to(home)
 

@@ -82,7 +82,7 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert "given count" in err()
     assert lib.orlhf_group_normalize(None, None, 3, 0, 0, None, None, None, None) == -1
     assert lib.orlhf_group_normalize(None, None, 3, 2, 9, None, None, None, None) == -1
-    assert lib.orlhf_gae_scan(None, None, None, 0, -1, 4, None, 1.0, 1.0, None, None, None) == -1
+    assert lib.orlhf_gae_scan(None, None, None, 0, -1, 4, None, None, 1.0, 1.0, None, None, None) == -1
     assert lib.orlhf_token_workspace_bytes(4096, 16383) >= 4096 * 4 * 6 * 8  # 4096-token chunks, 6 quantities, fp64
     assert lib.orlhf_whiten_workspace_bytes(10) > 0
 

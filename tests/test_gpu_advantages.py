@@ -151,6 +151,26 @@ def test_packed_scan_equals_padded(cuda):
     g1 = get_cumulative_returns(rewards.to(cuda), inner.to(cuda), 0.99)
     g2 = get_cumulative_returns(rewards[valid].to(cuda), inner[valid].to(cuda), 0.99, cu_seqlens=cu)
     assert torch.equal(g2, g1[valid.to(cuda)])
+    # rows handed out longest first (any permutation): the schedule changes, no bit of the results does
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import reward_advantages_and_returns
+    for order in (torch.argsort(lens, descending=True), torch.randperm(21, generator=g)):
+        adv_o, ret_o = get_advantages_and_returns(values[valid].to(cuda), rewards[valid].to(cuda), inner[valid].to(cuda),
+                                                  1.0, 0.95, cu_seqlens=cu, row_order=order.to(cuda))
+        assert torch.equal(adv_o, adv_p) and torch.equal(ret_o, ret_p)
+        g3 = get_cumulative_returns(rewards[valid].to(cuda), inner[valid].to(cuda), 0.99, cu_seqlens=cu,
+                                    row_order=order.to(cuda))
+        assert torch.equal(g3, g2)
+        adv_o2, ret_o2 = get_advantages_and_returns(values.to(cuda), rewards.to(cuda), inner.to(cuda), 1.0, 0.95,
+                                                    row_order=order.to(cuda))
+        assert torch.equal(adv_o2, adv) and torch.equal(ret_o2, ret)
+        r_seq = torch.randn(21, generator=torch.Generator().manual_seed(1)).to(cuda)
+        one = reward_advantages_and_returns(r_seq, 0.01, rewards[valid].to(cuda), values[valid].to(cuda),
+                                            inner[valid].to(cuda), 1.0, 0.95, cu_seqlens=cu)
+        two = reward_advantages_and_returns(r_seq, 0.01, rewards[valid].to(cuda), values[valid].to(cuda),
+                                            inner[valid].to(cuda), 1.0, 0.95, cu_seqlens=cu, row_order=order.to(cuda))
+        assert all(torch.equal(x, y) for x, y in zip(one, two))
+    with pytest.raises(ValueError):
+        get_cumulative_returns(rewards.to(cuda), inner.to(cuda), 0.99, row_order=torch.arange(5, device=cuda))
 
 
 # ------------------------------------------------------------------ group baselines
