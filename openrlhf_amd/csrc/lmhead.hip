@@ -161,20 +161,38 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, 
 }
 
 // ---------------------------------------------------------------- forward: vocabulary ranges -> outputs
-__global__ __launch_bounds__(kBlock) void lmhead_combine_kernel(const float* __restrict__ records,
-                                                                const float* __restrict__ x_label, int64_t n_tokens,
-                                                                int64_t n_tiles, const int64_t* __restrict__ labels,
-                                                                int64_t vocab, double temperature, int both_t,
-                                                                float* __restrict__ logprob, float* __restrict__ entropy,
-                                                                float* __restrict__ row_stats) {
-  const int64_t tok = (int64_t)blockIdx.x * kBlock + threadIdx.x;
-  if (tok >= n_tokens) return;
-  const double inv_t = 1.0 / temperature;
+constexpr int kCombineBlock = 1024;  // 16 waves: lane = token, the waves split the vocabulary tiles
+
+__global__ __launch_bounds__(kCombineBlock) void lmhead_combine_kernel(const float* __restrict__ records,
+                                                                       const float* __restrict__ x_label, int64_t n_tokens,
+                                                                       int64_t n_tiles, const int64_t* __restrict__ labels,
+                                                                       int64_t vocab, double temperature, int both_t,
+                                                                       float* __restrict__ logprob, float* __restrict__ entropy,
+                                                                       float* __restrict__ row_stats) {
+  constexpr int kWaves = kCombineBlock / kWave;
+  __shared__ f32x4 lds[kWaves][kWave];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t tok = (int64_t)blockIdx.x * kWave + lane;
+  const float c1 = kLog2e, cT = (float)(1.4426950408889634 / temperature);
+  Running run{kLow, 0.0f, 0.0f, 0.0f, kLow};
+  if (tok < n_tokens) {
+    for (int64_t t = wave; t < n_tiles; t += kWaves) {  // 64 consecutive tokens of one tile: one 1 KiB read per wave
+      const f32x4 rec = *(const f32x4*)(records + (t * n_tokens + tok) * kRec);
+      merge(run, Running{rec[0], rec[1], rec[2], rec[3], kLow}, c1, cT, both_t != 0);
+    }
+  }
+  lds[wave][lane] = f32x4{run.m, run.s1, run.t1, run.sT};
+  __syncthreads();
+  if (wave != 0 || tok >= n_tokens) return;
+  // the 16 partial results of this token, folded in fp64
   float m = kLow;
-  for (int64_t t = 0; t < n_tiles; ++t) m = fmaxf(m, records[(t * n_tokens + tok) * kRec]);
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) m = fmaxf(m, lds[w][lane][0]);
+  const double inv_t = 1.0 / temperature;
   double s1 = 0.0, t1 = 0.0, sT = 0.0;
-  for (int64_t t = 0; t < n_tiles; ++t) {
-    const f32x4 rec = *(const f32x4*)(records + (t * n_tokens + tok) * kRec);
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w) {
+    const f32x4 rec = lds[w][lane];
     const double d = (double)rec[0] - (double)m;
     const double q1 = exp(d);
     s1 += (double)rec[1] * q1;
@@ -409,7 +427,7 @@ static int launch_fwd(const void* hidden, const void* weight, int64_t n_rows, in
     hipLaunchKernelGGL((lmhead_fwd_kernel<DT, false>), grid, block, mm::kLdsBytes, s, w, h, labels, c1, cT, records, x_label, n_tb, n_vt);
   }
   ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_fwd(tiles)");
-  hipLaunchKernelGGL(lmhead_combine_kernel, dim3((unsigned)((n_rows + kBlock - 1) / kBlock)), dim3(kBlock), 0, s, records,
+  hipLaunchKernelGGL(lmhead_combine_kernel, dim3((unsigned)((n_rows + kWave - 1) / kWave)), dim3(kCombineBlock), 0, s, records,
                      x_label, n_rows, n_vt, labels, vocab, temperature, both_t ? 1 : 0, logprob, entropy, row_stats);
   ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_fwd(combine)");
   return ORLHF_OK;
