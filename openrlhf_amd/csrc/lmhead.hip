@@ -110,8 +110,7 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, 
   const int64_t n_tokens = h.rows, vocab = w.rows;
 
   f32x16 acc[4][4];
-  mm::Chain chain;
-  mm::tile_product<DT, false, false>(acc, w, h, vt * 256, tb * 256, lds, chain);
+  mm::tile_product<DT, false, false>(acc, w, h, vt * 256, tb * 256, lds);
 
   const int64_t vbase = vt * 256 + wm * 128 + 4 * (lane >> 5);  // vocabulary index of this lane's register offset 0
   Running run[4];
@@ -238,8 +237,7 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_bwd_p_kernel(Operand w
   const int64_t n_tokens = h.rows, vocab = w.rows;
 
   f32x16 acc[4][4];
-  mm::Chain chain;
-  mm::tile_product<DT, false, false>(acc, w, h, v0 + ct * 256, tb * 256, lds, chain);
+  mm::tile_product<DT, false, false>(acc, w, h, v0 + ct * 256, tb * 256, lds);
 
   const double inv_t = 1.0 / temperature;
   const int64_t vbase = v0 + ct * 256 + wm * 128 + 4 * (lane >> 5);
@@ -304,8 +302,7 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_gemm_f32_kernel(Operan
   mm::grouped_tile(item, tiles_m, tiles_n, tm, tn);
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wm = wave & 1u, wn = wave >> 1;
   f32x16 acc[4][4];
-  mm::Chain chain;
-  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds, chain);
+  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds);
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
@@ -336,8 +333,7 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_gemm_lowp_kernel(Opera
   mm::grouped_tile(item, tiles_m, tiles_n, tm, tn);
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wm = wave & 1u, wn = wave >> 1;
   f32x16 acc[4][4];
-  mm::Chain chain;
-  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds, chain);
+  mm::tile_product<DT, A_MN, B_MN>(acc, a, b, tm * 256, tn * 256, lds);
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll

@@ -26,6 +26,8 @@
 // MFMA 32x32x16 operand layout: lane l supplies row (l & 31), 8 consecutive k starting at
 // (l >> 5) * 8; result register r of lane l is C[8 * (r / 4) + 4 * (l >> 5) + (r & 3)][l & 31].
 #pragma once
+#include <type_traits>
+
 #include "common.h"
 
 namespace orlhf {
@@ -196,22 +198,11 @@ __device__ __forceinline__ void mfma_step(f32x16 (&acc)[4][4], const Frags& f) {
 // The fragments of k-step ks + 1 are read from LDS while k-step ks is multiplied; the single
 // barrier of the iteration sits before the LAST k-step's MFMAs, which then cover the read of the
 // next slab's first fragments: the matrix pipe does not drain at a slab boundary.
-// State carried from one product to the next by a workgroup that multiplies several tiles in a
-// row: which LDS buffer the next slab 0 goes to, and whether the previous product already issued
-// its load (during its own last iteration, so that it lands while that tile's epilogue runs).
-struct Chain {
-  uint32_t phase = 0;
-  bool primed = false;
-};
-
-// has_next / next_row0_*: the tile this workgroup multiplies next (same operands), only used with
-// two K-major operands. The function ends WITHOUT a barrier: no wave reads the slab buffers after
-// the barrier inside the last iteration, but a caller that reuses them as scratch must synchronise.
+// (Touching slab s + 2 an iteration early to warm the L2 changed nothing: the counters put the
+// average L2 read latency of these loads at ~270 cycles, far below an iteration.)
 template <int DT, bool A_MN_MAJOR, bool B_MN_MAJOR>
 __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand& a, const Operand& b, int64_t row0_a,
-                                             int64_t row0_b, char* lds, Chain& chain, bool has_next = false,
-                                             int64_t next_row0_a = 0, int64_t next_row0_b = 0) {
-  constexpr bool kCanChain = !A_MN_MAJOR && !B_MN_MAJOR;
+                                             int64_t row0_b, char* lds) {
   // Everything addressed below derives from the thread index: making it opaque keeps a caller's
   // loop over tiles from hoisting a hundred address registers out of the product and holding
   // them (spilled) across its epilogue; they are recomputed per tile instead.
@@ -231,27 +222,26 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
   const int64_t depth = a.depth;
   const int64_t n_slabs = (depth + kSlab - 1) / kSlab;
   const int64_t full = depth / kSlab;  // slabs 0 .. full-1 are whole
-  const uint32_t phase = chain.phase;
-  auto buffer = [&](int64_t slab) -> char* { return lds + ((phase + (uint32_t)slab) & 1u) * kStageBytes; };
   u32x4 ra[8], rb[8];
-  if (!(kCanChain && chain.primed)) {
-    fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, 0, tid);
-    fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, 0, tid);
-    stage_slab<A_MN_MAJOR>(ra, buffer(0), tid);
-    stage_slab<B_MN_MAJOR>(rb, buffer(0) + kSlabBytes, tid);
-  }
+  fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, 0, tid);
+  fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, 0, tid);
+  stage_slab<A_MN_MAJOR>(ra, lds, tid);
+  stage_slab<B_MN_MAJOR>(rb, lds + kSlabBytes, tid);
   if (n_slabs > 1) {  // MN-major operands carry slab s + 1 in registers from one iteration to the next
     if (A_MN_MAJOR) fetch_slab<true, true>(ra, a, row0_a, kSlab, tid);
     if (B_MN_MAJOR) fetch_slab<true, true>(rb, b, row0_b, kSlab, tid);
   }
-  __syncthreads();  // slab 0 is complete in LDS (also when the previous product loaded it)
+  __syncthreads();
   Frags f0, f1;
-  load_frags(f0, buffer(0), buffer(0) + kSlabBytes, 0, wm, wn, lane);
+  load_frags(f0, lds, lds + kSlabBytes, 0, wm, wn, lane);
   int64_t s = 0;
-  for (; s + 2 < full; ++s) {  // steady state: slabs s + 1 and s + 2 exist and are whole
-    const char* cur = buffer(s);
-    char* nxt = buffer(s + 1);
-    const int64_t k1 = (s + 1) * kSlab, k2 = (s + 2) * kSlab;
+
+  // One steady-state iteration: slab s in buffer PARITY, slab s + 1 arrives in the other.
+  auto steady = [&](auto parity, int64_t it) {
+    constexpr int P = decltype(parity)::value;
+    const char* cur = lds + P * kStageBytes;
+    char* nxt = lds + (1 - P) * kStageBytes;
+    const int64_t k1 = (it + 1) * kSlab, k2 = (it + 2) * kSlab;
     // k-step 0
     if (!A_MN_MAJOR) dma_slab(a, row0_a, k1, nxt, wave_u, lane);
     if (!B_MN_MAJOR) dma_slab(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);
@@ -271,25 +261,26 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     if (A_MN_MAJOR) fetch_slab<true, false>(ra, a, row0_a, k2, tid);
     if (B_MN_MAJOR) fetch_slab<true, false>(rb, b, row0_b, k2, tid);
     mfma_step<DT>(acc, f0);
-    __syncthreads();  // every wave holds its last fragments of `cur`; slab s + 1 is complete in `nxt`
+    // every wave holds its last fragments of `cur`; slab s + 1 is complete in `nxt`
+    __syncthreads();
     // k-step 3, over the read of the next slab's first fragments
     load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
     mfma_step<DT>(acc, f1);
     __builtin_amdgcn_sched_barrier(0);
+  };
+  for (; s + 3 < full; s += 2) {  // pairs of steady iterations: slabs up to s + 3 exist and are whole
+    steady(std::integral_constant<int, 0>{}, s);
+    steady(std::integral_constant<int, 1>{}, s + 1);
   }
-  const bool prime_next = kCanChain && has_next && depth >= kSlab;  // the next tile's slab 0 is whole
   for (; s < n_slabs; ++s) {  // the last slabs: a k tail may need masking, slabs run out
-    const char* cur = buffer(s);
-    char* nxt = buffer(s + 1);
+    const char* cur = lds + (s & 1) * kStageBytes;
+    char* nxt = lds + ((s + 1) & 1) * kStageBytes;
     const bool has1 = s + 1 < n_slabs, has2 = s + 2 < n_slabs;
     if (has1) {
       if (!A_MN_MAJOR) fetch_slab<false, true>(ra, a, row0_a, (s + 1) * kSlab, tid);
       if (!B_MN_MAJOR) fetch_slab<false, true>(rb, b, row0_b, (s + 1) * kSlab, tid);
       if (A_MN_MAJOR) stage_slab<true>(ra, nxt, tid);
       if (B_MN_MAJOR) stage_slab<true>(rb, nxt + kSlabBytes, tid);
-    } else if (kCanChain && prime_next) {  // the other buffer is free: the next tile's first slab goes there
-      dma_slab(a, next_row0_a, 0, nxt, wave_u, lane);
-      dma_slab(b, next_row0_b, 0, nxt + kSlabBytes, wave_u, lane);
     }
     if (has2) {
       if (A_MN_MAJOR) fetch_slab<true, true>(ra, a, row0_a, (s + 2) * kSlab, tid);
@@ -307,12 +298,10 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
       __syncthreads();
       load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
     }
-    // (last iteration: nothing to publish, and the next tile's load is not waited for here; `cur`
-    // is refilled only after the barrier that opens the next product)
     mfma_step<DT>(acc, f1);
   }
-  chain.phase = phase + (uint32_t)n_slabs;
-  chain.primed = prime_next;
+  // no closing barrier: after the barrier inside the last iteration no wave reads the slab
+  // buffers any more, but a caller that reuses them as scratch must synchronise first
 }
 
 // Position of accumulator register r of tile (mt, nt) inside the 256 x 256 output tile.
