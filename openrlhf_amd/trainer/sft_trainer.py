@@ -16,7 +16,7 @@ import torch
 from ..models.actor import actor_forward_tail
 from ..models.loss import SFTLoss
 from ..models.utils import fused_logprob_entropy_fwd_bwd
-from .ray.ppo_actor import _aggregation_coef, _HandOverGradient
+from .ray.ppo_actor import _HandOverGradient, _row_coef
 
 
 def sft_loss_step(logits, inputs, attention_mask, loss_mask, loss_fn: SFTLoss = None, fused: bool = False,
@@ -38,7 +38,7 @@ def sft_loss_step(logits, inputs, attention_mask, loss_mask, loss_fn: SFTLoss = 
 
     with torch.no_grad():
         norm = batch_num_tokens if loss_fn.token_level_loss else global_batch_size
-        coef = _aggregation_coef(shifted, loss_fn.token_level_loss, dp_size, norm)  # [B, T-1], 0 off the mask
+        coef = _row_coef(shifted, loss_fn.token_level_loss, dp_size, norm)[:batch, None] * shifted.to(torch.float32)  # [B, T-1], 0 off the mask
         w = torch.zeros(batch, seqlen, dtype=torch.float32, device=logits.device)
         w[:, : seqlen - 1] = -coef * loss_scale
         need = torch.zeros(batch, seqlen, dtype=torch.uint8, device=logits.device)

@@ -207,3 +207,40 @@ def test_later_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert "separate forward and backward" in err()
     assert lib.orlhf_logprob_entropy_fwd_bwd(16, 32 + 2, 1, 2, 1024, 1024, 1024, 8, 1.0, 8, None, 8, None, None, None) == -3
     assert "16-byte phases" in err()
+
+
+def test_every_intra_package_import_resolves():
+    """Names imported from one module of the package by another (or by a test) exist: a helper
+    renamed in one file must not break a caller that is only imported lazily inside a function."""
+    import ast
+    import glob
+    import importlib
+    import os
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    files = glob.glob(os.path.join(root, "openrlhf_amd", "**", "*.py"), recursive=True)
+    files += glob.glob(os.path.join(root, "tests", "*.py")) + [os.path.join(root, "bench.py")]
+    missing = []
+    for path in files:
+        rel = os.path.relpath(path, root)
+        tree = ast.parse(open(path).read())
+        for node in ast.walk(tree):
+            if not isinstance(node, ast.ImportFrom):
+                continue
+            if node.level > 0:
+                parts = rel[:-3].split(os.sep)
+                base = ".".join(parts[: len(parts) - node.level])
+                mod = base + ("." + node.module if node.module else "")
+            elif node.module and node.module.split(".")[0] == "openrlhf_amd":
+                mod = node.module
+            else:
+                continue
+            m = importlib.import_module(mod)
+            for alias in node.names:
+                if hasattr(m, alias.name):
+                    continue
+                try:
+                    importlib.import_module(mod + "." + alias.name)
+                except ImportError:
+                    missing.append((rel, mod, alias.name))
+    assert not missing, missing
