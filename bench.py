@@ -282,6 +282,67 @@ def bench_lmhead(dev, n=4096, hdim=4096, vocab=VOCAB, reps=4):
     }
 
 
+def bench_few_rows(dev, n=64, vocab=VOCAB, copies=32):
+    """A launch with fewer rows than the GPU has compute units (n x 151936 bf16, 19 MB at n = 64):
+    forward with the rows cut into segments against the whole-row forward on the same rows, and
+    the backward (which cuts its rows itself), through the C ABI. Each timed launch takes the next
+    of `copies` distinct inputs (0.6 GB in all at the defaults: more than the caches hold)."""
+    from openrlhf_amd import _lib
+    from openrlhf_amd._lib import call, ptr, stream_of
+
+    lib = _lib.load()
+    xs = [(torch.randn(n, vocab, device=dev) * 3).to(torch.bfloat16) for _ in range(copies)]
+    grads = torch.empty(n, vocab, device=dev, dtype=torch.bfloat16)
+    labels = torch.randint(0, vocab, (n,), device=dev)
+    g_lp, g_ent = torch.randn(n, device=dev), torch.randn(n, device=dev)
+    lp, ent = torch.empty(n, device=dev), torch.empty(n, device=dev)
+    stats = torch.empty(n, 4, device=dev)
+    ws_bytes = lib.orlhf_logprob_entropy_split_workspace_bytes(_lib.BF16, n, vocab)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
+    st = stream_of(dev)
+
+    def cut(x):
+        call("orlhf_logprob_entropy_fwd_split", ptr(x), _lib.BF16, n, vocab, vocab, ptr(labels), 1.0, ptr(lp), ptr(ent),
+             ptr(stats), None, ptr(ws), ws_bytes, st)
+
+    def whole(x):
+        call("orlhf_logprob_entropy_fwd", ptr(x), _lib.BF16, n, vocab, vocab, ptr(labels), 1.0, ptr(lp), ptr(ent),
+             ptr(stats), None, 0, st)
+
+    def backward(x):
+        call("orlhf_logprob_entropy_bwd", ptr(x), ptr(grads), _lib.BF16, n, vocab, vocab, vocab, ptr(labels), 1.0,
+             ptr(g_lp), ptr(g_ent), ptr(stats), None, st)
+
+    def timed(fn):
+        for x in xs[:4]:
+            fn(x)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for x in xs:
+            fn(x)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / len(xs)
+
+    whole_ms, cut_ms = timed(whole), timed(cut)
+    cut(xs[0])
+    lp_cut = lp.clone()
+    whole(xs[0])
+    bwd_ms = timed(backward)
+    row_bytes = vocab * 2
+    return {
+        "workload": f"{n} rows x {vocab} bf16 logits per launch ({n * row_bytes / 1e6:.1f} MB), {copies} distinct inputs in rotation",
+        "segments_per_row": ws_bytes // (n * 32) if ws_bytes else 1,
+        "forward_whole_rows_us": whole_ms * 1e3, "forward_whole_rows_gbs": n * row_bytes / whole_ms / 1e6,
+        "forward_cut_rows_us": cut_ms * 1e3, "forward_cut_rows_gbs": n * row_bytes / cut_ms / 1e6,
+        "backward_cut_rows_us": bwd_ms * 1e3, "backward_cut_rows_gbs": 2 * n * row_bytes / bwd_ms / 1e6,
+        "max_abs_diff_cut_vs_whole": (lp_cut - lp).abs().max().item(),
+        "note": "a launch this small is a few microseconds: the times include the launch itself and the ramp of the "
+                "first loads, which is what keeps them under the streaming rates of the full-size batch",
+    }
+
+
 def bench_kernels(args, dev):
     """--workload kernels: the three vocabulary-row kernels launched back to back on ONE resident
     buffer of --rows x 151936 bf16 logits (forward, in-place backward, one-pass forward+backward,
@@ -627,7 +688,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--ring", type=int, default=6, help="distinct logits buffers per timed segment")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU-baseline sample")
-    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token", "kernels", "torch_eager", "ceilings", "lmhead"],
+    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token", "kernels", "torch_eager", "ceilings", "lmhead", "few_rows"],
                     help="logprob: the headline step (default); per_token: the small kernels of configs 3/4; "
                          "torch_eager: the reference's eager torch op sequence on this GPU beside the HIP path; "
                          "ceilings: plain read / read+write / copy / fill streams on the headline buffers; "
@@ -664,6 +725,9 @@ def main():
     if args.workload == "lmhead":
         print(json.dumps({"workload": "lm-head + log-prob + entropy, logits never stored", "n_gpus": 1,
                           **bench_lmhead(dev, n=args.rows if args.rows != 8192 else 4096)}), flush=True)
+        return
+    if args.workload == "few_rows":
+        print(json.dumps({"n_gpus": 1, **bench_few_rows(dev, n=args.rows if args.rows != 8192 else 64)}), flush=True)
         return
     pristine, labels, g_lp, g_ent, cu = make_workload(dev)
     n_tok = pristine.shape[0]
@@ -844,6 +908,7 @@ def main():
         torch.cuda.empty_cache()
         out["lmhead_logprob_entropy"] = bench_lmhead(dev)
     if not args.no_per_token:
+        out["few_rows_n64"] = bench_few_rows(dev)
         entries = bench_per_token(args, dev, emit=False)
         out["per_token_config4"] = {
             "note": "the other kernels of the path at BASELINE config 4's size (4096 rows x 16384 columns fp32, 33.7 M real "

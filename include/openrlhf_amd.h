@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 17
+#define ORLHF_ABI_VERSION 18
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -109,6 +109,25 @@ int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows, int
  */
 int orlhf_divide_rows_inplace(void* logits, int dtype, int64_t n_rows, int64_t vocab,
                               int64_t row_stride, double divisor, orlhf_stream_t stream);
+
+/*
+ * The same forward for launches with fewer rows than the GPU has compute units (short rollouts,
+ * a 64-token micro-batch): every row is cut into segments, one workgroup per (row, segment)
+ * writes a partial record (running maxima and sums) into `workspace`, and a second small kernel
+ * merges a row's records in segment order and finishes the row as the whole-row kernel does. Same
+ * arguments, outputs and conventions as orlhf_logprob_entropy_fwd (same reference lines:
+ * openrlhf/models/utils.py:139-163,182-186); results agree with it to the rounding of the fp32
+ * partial sums. orlhf_logprob_entropy_split_workspace_bytes returns the bytes this shape needs, 0
+ * when the rows would not be cut (256 rows or more, or rows shorter than 64 KiB); then the call is
+ * orlhf_logprob_entropy_fwd itself and `workspace` may be NULL. The cut depends on the shape
+ * only. orlhf_logprob_entropy_bwd needs no workspace and cuts its rows by the same rule itself.
+ */
+int64_t orlhf_logprob_entropy_split_workspace_bytes(int dtype, int64_t n_rows, int64_t vocab);
+int orlhf_logprob_entropy_fwd_split(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                                    int64_t row_stride, const int64_t* labels, double temperature,
+                                    float* logprob, float* entropy, float* row_stats,
+                                    const uint8_t* row_mask, void* workspace, int64_t workspace_bytes,
+                                    orlhf_stream_t stream);
 
 /*
  * Backward of the above in one streaming pass, written in the logits dtype:

@@ -10,7 +10,11 @@
 //     nats above the reference, or inf/NaN logits) is re-read once with a classic per-lane online
 //     maximum, so the result never depends on the shortcut;
 //   * sums are kept in fp32 in 4 independent accumulators per lane, reduced over the wave with
-//     cross-lane shuffles and over the 4 waves through LDS; the per-row epilogue runs in fp64.
+//     cross-lane shuffles and over the 4 waves through LDS; the per-row epilogue runs in fp64;
+//   * a launch with fewer rows than the chip has compute units cuts every row into segments, one
+//     workgroup per (row, segment): the backward needs nothing else (an element's gradient depends
+//     on the row only through its saved statistics), the forward writes one partial record per
+//     segment and a small second kernel merges a row's records in a fixed order.
 #include <stdlib.h>
 
 #include "vocab_rows.h"
@@ -180,6 +184,29 @@ struct RowSums {
   float MT, sT, M1, s1, t1;
 };
 
+// How a launch cuts its rows: n segments of seg_elems elements (the last one shorter), work item
+// w = row * n + segment. n == 1: whole rows. partials (forward only, n > 1): kPartial floats per
+// work item {MT, sT, M1, s1, t1, fast-pass flag, the label's logit if it lies in the segment, 0}.
+constexpr int kPartial = 8;
+struct RowSplit {
+  int n;
+  uint32_t seg_elems;
+  float* partials;
+};
+
+struct WorkItem {
+  int64_t row;
+  uint32_t first;  // first element of the segment
+  int64_t len;     // its length
+};
+__device__ __forceinline__ WorkItem work_item(int64_t w, const RowSplit& split, int64_t vocab) {
+  if (split.n == 1) return {w, 0u, vocab};
+  const int64_t row = w / split.n;
+  const uint32_t first = (uint32_t)(w - row * split.n) * split.seg_elems;
+  const int64_t left = vocab - first;
+  return {row, first, left < (int64_t)split.seg_elems ? left : (int64_t)split.seg_elems};
+}
+
 __device__ __forceinline__ bool sums_usable(float s) { return s > 0.0f && s < INFINITY; }
 
 // ---------------------------------------------------------------- forward kernel
@@ -188,7 +215,7 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
     const char* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
     const int64_t* __restrict__ labels, double temperature, float* __restrict__ logprob,
     float* __restrict__ entropy, float* __restrict__ row_stats, const uint8_t* __restrict__ row_mask,
-    int scalar_only) {
+    int scalar_only, RowSplit split) {
   using E = Elt<DT>;
   using MT = ModeTraits<MODE>;
   __shared__ float lds[kWavesPerBlock][8];
@@ -199,8 +226,12 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
   const float c_plain = kLog2e;
   const float c_scaled = (float)(1.4426950408889634 / temperature);
 
-  for (int64_t row_i = blockIdx.x; row_i < n_rows; row_i += gridDim.x) {
+  const int64_t n_work = n_rows * split.n;
+  for (int64_t work = blockIdx.x; work < n_work; work += gridDim.x) {
+    const WorkItem item = work_item(work, split, vocab);
+    const int64_t row_i = item.row;
     if (row_mask != nullptr && row_mask[row_i] == 0) {  // row not wanted: outputs 0, logits not read
+      if (split.n > 1) continue;                        // (the merging kernel writes the zeros)
       if (tid == 0) {
         if (MODE != kEntOnly && logprob != nullptr) logprob[row_i] = 0.0f;
         if (MT::kPlainSet && entropy != nullptr) entropy[row_i] = 0.0f;
@@ -208,8 +239,9 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
       }
       continue;
     }
-    const char* row = logits + row_i * row_stride_bytes;
-    const RowGeom g = row_geom<DT>(row, vocab, scalar_only != 0);
+    const char* row = logits + row_i * row_stride_bytes + (int64_t)item.first * E::kSize;
+    const int64_t seg_len = item.len;
+    const RowGeom g = row_geom<DT>(row, seg_len, scalar_only != 0);
 
     // ---- reference maximum of this wave: first vector (or first scalar) of each lane
     float m_ref = -INFINITY;
@@ -221,7 +253,7 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
 #pragma unroll
       for (int j = 0; j < E::kPerVec; ++j) m_ref = fmaxf(m_ref, x[j]);
     } else {
-      const uint32_t e = (uint32_t)tid < (uint32_t)vocab ? (uint32_t)tid : (uint32_t)vocab - 1;
+      const uint32_t e = (uint32_t)tid < (uint32_t)seg_len ? (uint32_t)tid : (uint32_t)seg_len - 1;
       m_ref = E::load1(row + e * E::kSize);
     }
     m_ref = wave_max(m_ref);
@@ -314,6 +346,20 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
       __syncthreads();
     }
 
+    if (split.n > 1) {  // a segment: its sums go to the merging kernel as they are
+      if (tid == 0) {
+        float x_label = 0.0f;
+        if (MODE != kEntOnly && logprob != nullptr) {
+          const int64_t at = labels[row_i] - (int64_t)item.first;
+          if (at >= 0 && at < seg_len) x_label = E::load1(row + at * E::kSize);
+        }
+        float* rec = split.partials + work * kPartial;
+        *(f32x4*)rec = f32x4{sums.MT, sums.sT, sums.M1, sums.s1};
+        *(f32x4*)(rec + 4) = f32x4{sums.t1, ok ? 1.0f : 0.0f, x_label, 0.0f};
+      }
+      continue;
+    }
+
     // ---- per-row epilogue in fp64
     if (tid == 0) {
       double lse_t = 0.0, lse_1 = 0.0, ex = 0.0;
@@ -347,6 +393,83 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
   }
 }
 
+// Merges the segment records of every row and finishes the row exactly as the whole-row epilogue
+// does: one wave per row, lane k holds segment k (at most 64), maxima and sums go through the
+// fixed butterfly of the wave reductions in fp64, so the result does not depend on scheduling.
+template <int DT>
+__global__ __launch_bounds__(kBlock) void logprob_entropy_merge_kernel(
+    const char* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
+    const int64_t* __restrict__ labels, double temperature, float* __restrict__ logprob,
+    float* __restrict__ entropy, float* __restrict__ row_stats, const uint8_t* __restrict__ row_mask,
+    int mode, RowSplit split) {
+  using E = Elt<DT>;
+  const bool scaled_set = (mode == kLpOnly || mode == kBothT), plain_set = (mode != kLpOnly);
+  const double c_plain = 1.4426950408889634, c_scaled = 1.4426950408889634 / temperature;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t row_i = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
+  if (row_i >= n_rows) return;
+  const bool want_lp = mode != kEntOnly && logprob != nullptr;
+  if (row_mask != nullptr && row_mask[row_i] == 0) {
+    if (lane == 0) {
+      if (want_lp) logprob[row_i] = 0.0f;
+      if (plain_set && entropy != nullptr) entropy[row_i] = 0.0f;
+      if (row_stats != nullptr) *(f32x4*)(row_stats + row_i * 4) = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+    return;
+  }
+  const int64_t label = want_lp ? labels[row_i] : -1;
+  // maxima in log2 units: a fast-pass record holds them so, a safe-pass record holds the segment
+  // maximum in logit units in both fields. Lanes past the last segment hold the neutral record.
+  double mt = -INFINITY, m1 = -INFINITY, sT = 0.0, s1 = 0.0, t1 = 0.0;
+  float x_label = 0.0f;  // the segment that holds the label has read its logit
+  if (lane < split.n) {
+    const float* rec = split.partials + (row_i * split.n + lane) * kPartial;
+    const f32x4 a = *(const f32x4*)rec, b = *(const f32x4*)(rec + 4);
+    const bool fast = b[1] != 0.0f;
+    mt = (double)a[0] * (fast ? 1.0 : c_scaled);
+    m1 = (double)a[2] * (fast ? 1.0 : c_plain);
+    sT = (double)a[1];
+    s1 = (double)a[3];
+    t1 = (double)b[0];
+    if (label >= 0 && label < vocab && (uint32_t)lane == (uint32_t)label / split.seg_elems) x_label = b[2];
+  }
+  x_label = wave_sum(x_label);  // one lane holds it, the others 0
+  double MT = mt, M1 = m1;
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    const double ot = __shfl_xor(MT, o, kWave), o1 = __shfl_xor(M1, o, kWave);
+    MT = ot > MT ? ot : MT;
+    M1 = o1 > M1 ? o1 : M1;
+  }
+  // a segment at the row maximum (or one that saw nothing finite) keeps its sums as they are:
+  // 0, or the NaN markers of the safe pass
+  const double rT = (mt != -INFINITY && mt != MT) ? exp2(mt - MT) : 1.0;
+  const double r1 = (m1 != -INFINITY && m1 != M1) ? exp2(m1 - M1) : 1.0;
+  sT = wave_sum(sT * rT);
+  s1 = wave_sum(s1 * r1);
+  t1 = wave_sum(t1 * r1);
+  if (lane != 0) return;
+  double lse_t = 0.0, lse_1 = 0.0, ex = 0.0;
+  if (scaled_set) lse_t = MT * kLn2d + log(sT);
+  if (plain_set) {
+    lse_1 = M1 * kLn2d + log(s1);
+    ex = t1 / s1;
+    if (!scaled_set) lse_t = lse_1;
+  }
+  if (want_lp) {
+    float lp;
+    if (label >= 0 && label < vocab) {
+      lp = (float)((double)x_label / temperature - lse_t);
+    } else {
+      lp = (label == -100) ? 0.0f : NAN;
+    }
+    logprob[row_i] = lp;
+  }
+  if (plain_set && entropy != nullptr) entropy[row_i] = (float)(lse_1 - ex);
+  if (row_stats != nullptr)
+    *(f32x4*)(row_stats + row_i * 4) = f32x4{(float)lse_t, (float)(plain_set ? lse_1 : lse_t), (float)ex, 0.0f};
+}
+
 // ---------------------------------------------------------------- backward kernel
 // Zero-fills a row without reading it.
 template <int DT>
@@ -368,14 +491,18 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_bwd_kernel(
     const char* logits, char* grad, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
     int64_t grad_stride_bytes, const int64_t* __restrict__ labels, double temperature,
     const float* __restrict__ g_logprob, const float* __restrict__ g_entropy,
-    const float* __restrict__ row_stats, const uint8_t* __restrict__ row_mask, int scalar_only) {
+    const float* __restrict__ row_stats, const uint8_t* __restrict__ row_mask, int scalar_only,
+    RowSplit split) {
   const double inv_t = 1.0 / temperature;
-  for (int64_t row_i = blockIdx.x; row_i < n_rows; row_i += gridDim.x) {
-    const char* row = logits + row_i * row_stride_bytes;
-    char* out_row = grad + row_i * grad_stride_bytes;
+  const int64_t n_work = n_rows * split.n;
+  for (int64_t work = blockIdx.x; work < n_work; work += gridDim.x) {
+    const WorkItem item = work_item(work, split, vocab);
+    const int64_t row_i = item.row;
+    const char* row = logits + row_i * row_stride_bytes + (int64_t)item.first * Elt<DT>::kSize;
+    char* out_row = grad + row_i * grad_stride_bytes + (int64_t)item.first * Elt<DT>::kSize;
     // the geometry follows the OUTPUT row when only zeros are written, the input row otherwise
     // (the host guarantees both have the same 16-byte phase unless scalar_only is set)
-    const RowGeom g = row_geom<DT>(row, vocab, scalar_only != 0);
+    const RowGeom g = row_geom<DT>(row, item.len, scalar_only != 0);
 
     const float glp = (MODE != kBwdEnt) ? g_logprob[row_i] : 0.0f;
     const float gh = (MODE != kBwdLp) ? g_entropy[row_i] : 0.0f;
@@ -394,7 +521,9 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_bwd_kernel(
     fn.onehot = (float)((double)glp * inv_t);
     fn.gh = gh;
     fn.k1 = gh * st[2] - (MODE == kBwdBothT1 ? glp : 0.0f);
-    fn.set_label((MODE != kBwdEnt) ? labels[row_i] : -1, vocab, g, Elt<DT>::kPerVec);
+    // the label relative to this segment; outside it (or outside the vocabulary) no element gets the one-hot term
+    const int64_t label = (MODE != kBwdEnt) ? labels[row_i] : -1;
+    fn.set_label((label >= 0 && label < vocab) ? label - (int64_t)item.first : -1, item.len, g, Elt<DT>::kPerVec);
     traverse_row<DT, true>(row, out_row, g, fn);
   }
 }
@@ -409,10 +538,29 @@ static int grid_for_rows(int64_t n_rows) {
   return (int)(n_rows < cap ? n_rows : cap);
 }
 
+// Rows are cut when there are fewer of them than compute units: enough segments for about two
+// workgroups per CU of a 256-CU part, none shorter than 32 KiB (one full batch of loads per lane),
+// at most 64. Segment lengths are multiples of 16 elements so every segment keeps its row's
+// 16-byte phase. The rule depends on the shape only, so results do not depend on the device.
+static RowSplit row_split(int64_t n_rows, int64_t vocab, int esize) {
+  RowSplit split{1, (uint32_t)vocab, nullptr};
+  constexpr int64_t kWholeRowsFrom = 256, kItems = 512, kMinSegBytes = 32768, kMaxSplit = 64;
+  if (n_rows >= kWholeRowsFrom) return split;
+  int64_t n = (kItems + n_rows - 1) / n_rows;
+  if (n > kMaxSplit) n = kMaxSplit;
+  if (n > vocab * esize / kMinSegBytes) n = vocab * esize / kMinSegBytes;
+  if (n <= 1) return split;
+  const int64_t seg = (((vocab + n - 1) / n) + 15) & ~(int64_t)15;
+  split.n = (int)((vocab + seg - 1) / seg);
+  split.seg_elems = (uint32_t)seg;
+  return split;
+}
+
 template <int DT>
 static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
                       const int64_t* labels, double temperature, float* logprob, float* entropy,
-                      float* row_stats, const uint8_t* row_mask, hipStream_t stream) {
+                      float* row_stats, const uint8_t* row_mask, void* workspace, int64_t workspace_bytes,
+                      hipStream_t stream) {
   using E = Elt<DT>;
   const bool want_lp = logprob != nullptr;
   const bool want_ent = entropy != nullptr;
@@ -421,11 +569,22 @@ static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
   const char* p = (const char*)logits;
   const int64_t stride_bytes = row_stride * E::kSize;
   const int scalar_only = 0;
-  const dim3 grid(grid_for_rows(n_rows)), block(kBlock);
+  RowSplit split{1, (uint32_t)vocab, nullptr};
+  if (workspace != nullptr) {  // the caller offers room for segment records
+    split = row_split(n_rows, vocab, E::kSize);
+    if (split.n > 1) {
+      ORLHF_CHECK_ARG(workspace_bytes >= n_rows * split.n * kPartial * (int64_t)sizeof(float) &&
+                          ((uintptr_t)workspace & 15u) == 0,
+                      "logprob_entropy_fwd_split: workspace of %lld bytes too small or not 16-byte aligned",
+                      (long long)workspace_bytes);
+      split.partials = (float*)workspace;
+    }
+  }
+  const dim3 grid(grid_for_rows(n_rows * split.n)), block(kBlock);
 #define ORLHF_FWD(M)                                                                          \
   hipLaunchKernelGGL((logprob_entropy_fwd_kernel<DT, M>), grid, block, 0, stream, p, n_rows,  \
                      vocab, stride_bytes, labels, temperature, logprob, entropy, row_stats,   \
-                     row_mask, scalar_only)
+                     row_mask, scalar_only, split)
   switch (mode) {
     case kLpOnly: ORLHF_FWD(kLpOnly); break;
     case kEntOnly: ORLHF_FWD(kEntOnly); break;
@@ -434,6 +593,12 @@ static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
   }
 #undef ORLHF_FWD
   ORLHF_CHECK_LAUNCH("orlhf_logprob_entropy_fwd");
+  if (split.n > 1) {
+    hipLaunchKernelGGL((logprob_entropy_merge_kernel<DT>), dim3((unsigned)((n_rows + kWavesPerBlock - 1) / kWavesPerBlock)), block, 0,
+                       stream, p, n_rows, vocab, stride_bytes, labels, temperature, logprob, entropy, row_stats,
+                       row_mask, mode, split);
+    ORLHF_CHECK_LAUNCH("orlhf_logprob_entropy_fwd_split(merge)");
+  }
   return ORLHF_OK;
 }
 
@@ -455,11 +620,12 @@ static int launch_bwd(const void* logits, void* grad, int64_t n_rows, int64_t vo
   const bool same_phase = (((uintptr_t)p ^ (uintptr_t)gp) & 15u) == 0 &&
                           ((stride_bytes - gstride_bytes) & 15) == 0;
   const int scalar_only = same_phase ? 0 : 1;
-  const dim3 grid(grid_for_rows(n_rows)), block(kBlock);
+  const RowSplit split = row_split(n_rows, vocab, E::kSize);
+  const dim3 grid(grid_for_rows(n_rows * split.n)), block(kBlock);
 #define ORLHF_BWD(M)                                                                          \
   hipLaunchKernelGGL((logprob_entropy_bwd_kernel<DT, M>), grid, block, 0, stream, p, gp,      \
                      n_rows, vocab, stride_bytes, gstride_bytes, labels, temperature,         \
-                     g_logprob, g_entropy, row_stats, row_mask, scalar_only)
+                     g_logprob, g_entropy, row_stats, row_mask, scalar_only, split)
   switch (mode) {
     case kBwdLp: ORLHF_BWD(kBwdLp); break;
     case kBwdEnt: ORLHF_BWD(kBwdEnt); break;
@@ -519,11 +685,10 @@ extern "C" int orlhf_divide_rows_inplace(void* logits, int dtype, int64_t n_rows
   return ORLHF_OK;
 }
 
-extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows,
-                                         int64_t vocab, int64_t row_stride, const int64_t* labels,
-                                         double temperature, float* logprob, float* entropy,
-                                         float* row_stats, const uint8_t* row_mask, int flags,
-                                         orlhf_stream_t stream) {
+static int forward_entry(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
+                         const int64_t* labels, double temperature, float* logprob, float* entropy,
+                         float* row_stats, const uint8_t* row_mask, int flags, void* workspace,
+                         int64_t workspace_bytes, orlhf_stream_t stream) {
   ORLHF_CHECK_ARG(n_rows >= 0 && vocab > 0, "logprob_entropy_fwd: n_rows=%lld vocab=%lld",
                   (long long)n_rows, (long long)vocab);
   ORLHF_CHECK_ARG(row_stride >= vocab, "logprob_entropy_fwd: row_stride %lld < vocab %lld",
@@ -543,18 +708,44 @@ extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t 
     case ORLHF_F32:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 3u) == 0, "logprob_entropy_fwd: logits not 4-byte aligned");
       return launch_fwd<ORLHF_F32>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                   entropy, row_stats, row_mask, s);
+                                   entropy, row_stats, row_mask, workspace, workspace_bytes, s);
     case ORLHF_BF16:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 1u) == 0, "logprob_entropy_fwd: logits not 2-byte aligned");
       return launch_fwd<ORLHF_BF16>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                    entropy, row_stats, row_mask, s);
+                                    entropy, row_stats, row_mask, workspace, workspace_bytes, s);
     case ORLHF_F16:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 1u) == 0, "logprob_entropy_fwd: logits not 2-byte aligned");
       return launch_fwd<ORLHF_F16>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                   entropy, row_stats, row_mask, s);
+                                   entropy, row_stats, row_mask, workspace, workspace_bytes, s);
     default:
       return fail(ORLHF_ERR_INVALID_ARG, "logprob_entropy_fwd: unknown dtype %d", dtype);
   }
+}
+
+extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t n_rows,
+                                         int64_t vocab, int64_t row_stride, const int64_t* labels,
+                                         double temperature, float* logprob, float* entropy,
+                                         float* row_stats, const uint8_t* row_mask, int flags,
+                                         orlhf_stream_t stream) {
+  return forward_entry(logits, dtype, n_rows, vocab, row_stride, labels, temperature, logprob, entropy, row_stats,
+                       row_mask, flags, nullptr, 0, stream);
+}
+
+extern "C" int64_t orlhf_logprob_entropy_split_workspace_bytes(int dtype, int64_t n_rows, int64_t vocab) {
+  if (n_rows <= 0 || vocab <= 0 || vocab >= (1ll << 29)) return 0;
+  const RowSplit split = row_split(n_rows, vocab, dtype == ORLHF_F32 ? 4 : 2);
+  return split.n > 1 ? n_rows * split.n * kPartial * (int64_t)sizeof(float) : 0;
+}
+
+extern "C" int orlhf_logprob_entropy_fwd_split(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
+                                               int64_t row_stride, const int64_t* labels, double temperature,
+                                               float* logprob, float* entropy, float* row_stats,
+                                               const uint8_t* row_mask, void* workspace, int64_t workspace_bytes,
+                                               orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(workspace != nullptr || orlhf_logprob_entropy_split_workspace_bytes(dtype, n_rows, vocab) == 0,
+                  "logprob_entropy_fwd_split: this shape needs a workspace (orlhf_logprob_entropy_split_workspace_bytes)");
+  return forward_entry(logits, dtype, n_rows, vocab, row_stride, labels, temperature, logprob, entropy, row_stats,
+                       row_mask, 0, workspace, workspace_bytes, stream);
 }
 
 extern "C" int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, int dtype,

@@ -44,6 +44,20 @@ def _as_rows(logits: torch.Tensor):
     return logits.contiguous().view(-1, vocab), vocab, False
 
 
+
+def _forward_rows(rows, code, n_rows, vocab, row_stride, lab, temperature, logprob, entropy, stats, rmask, dev):
+    """One forward launch over vocabulary rows. With fewer rows than the GPU has compute units the
+    rows are cut into segments (one workgroup each) whose partial sums a second kernel merges."""
+    ws_bytes = _lib.load().orlhf_logprob_entropy_split_workspace_bytes(code, n_rows, vocab)
+    if ws_bytes > 0:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        call("orlhf_logprob_entropy_fwd_split", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
+             float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), ptr(ws), ws_bytes, stream_of(dev))
+    else:
+        call("orlhf_logprob_entropy_fwd", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
+             float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), 0, stream_of(dev))
+
+
 class _LogprobEntropy(torch.autograd.Function):
     """logits -> (log-prob of label, entropy), one vocabulary pass forward, one backward."""
 
@@ -77,10 +91,7 @@ class _LogprobEntropy(torch.autograd.Function):
         entropy = torch.empty(n_rows, **opts) if want_entropy else None
         stats = torch.empty(n_rows, 4, **opts) if needs_grad else None
         with _lib.on_device(dev):
-            call(
-                "orlhf_logprob_entropy_fwd", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
-                float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), 0, stream_of(dev),
-            )
+            _forward_rows(rows, code, n_rows, vocab, row_stride, lab, temperature, logprob, entropy, stats, rmask, dev)
         ctx.temperature = float(temperature)
         ctx.inplace = bool(inplace_backward)
         ctx.row_stride = row_stride
@@ -528,15 +539,15 @@ def fused_logprob_entropy_fwd_bwd(
         ((row_stride - grad_stride) * rows.element_size()) & 15
     ) == 0
     with _lib.on_device(dev):
-        if fits and same_phase:
+        few_rows = lib.orlhf_logprob_entropy_split_workspace_bytes(code, n_rows, vocab) > 0
+        if fits and same_phase and not few_rows:
             call("orlhf_logprob_entropy_fwd_bwd", ptr(rows), ptr(grad_rows), code, n_rows, vocab, row_stride,
                  grad_stride, ptr(lab), float(temperature), ptr(wlp), ptr(went), ptr(logprob), ptr(entropy),
                  ptr(rmask), stream_of(dev))
         else:
             stats = torch.empty(n_rows, 4, **opts)
             zeros = torch.zeros(n_rows, **opts)
-            call("orlhf_logprob_entropy_fwd", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
-                 float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), 0, stream_of(dev))
+            _forward_rows(rows, code, n_rows, vocab, row_stride, lab, temperature, logprob, entropy, stats, rmask, dev)
             call("orlhf_logprob_entropy_bwd", ptr(rows), ptr(grad_rows), code, n_rows, vocab, row_stride,
                  grad_stride, ptr(lab), float(temperature), ptr(wlp if wlp is not None else zeros),
                  ptr(went if went is not None else zeros), ptr(stats), ptr(rmask), stream_of(dev))
