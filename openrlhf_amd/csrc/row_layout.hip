@@ -28,19 +28,36 @@ __global__ __launch_bounds__(kBlock) void row_extents_kernel(const void* __restr
       }
     };
     if (MASK_DT == ORLHF_MASK_U8) {
-      // byte masks: 16 columns per lane and load between the row's 16-byte boundaries
+      // byte masks: 16 columns per load between the row's 16-byte boundaries. A lane visits its
+      // groups in rising order, so it only has to keep the first and the last group that held a
+      // non-zero byte; the bytes themselves are looked at once, after the loop.
       const uint8_t* bytes = (const uint8_t*)mask + b * n_cols;
       int64_t head = (int64_t)((16 - ((uintptr_t)bytes & 15)) & 15);
       head = head < n_cols ? head : n_cols;
       const int64_t groups = (n_cols - head) / 16;
       for (int64_t t = threadIdx.x; t < head; t += kBlock) see(bytes[t] != 0, t);
-#pragma unroll 2
+      int64_t g_first = -1, g_last = -1;
+      u32x4 w_first = {0u, 0u, 0u, 0u}, w_last = {0u, 0u, 0u, 0u};
+#pragma unroll 4
       for (int64_t g = threadIdx.x; g < groups; g += kBlock) {
         const u32x4 w = *(const u32x4*)(bytes + head + g * 16);
         if ((w[0] | w[1] | w[2] | w[3]) != 0u) {
-#pragma unroll
-          for (int k = 0; k < 16; ++k) see(((w[k / 4] >> (8 * (k % 4))) & 0xffu) != 0u, head + g * 16 + k);
+          if (g_first < 0) g_first = g, w_first = w;
+          g_last = g, w_last = w;
         }
+      }
+      // bit 7 of every byte of nz(w) is set iff that byte of w is non-zero
+      auto nz = [](uint32_t w) { return (((w & 0x7f7f7f7fu) + 0x7f7f7f7fu) | w) & 0x80808080u; };
+      if (g_first >= 0) {
+        int at = 0;
+#pragma unroll
+        for (int k = 3; k >= 0; --k)
+          if (w_first[k] != 0u) at = 4 * k + (__builtin_ctz(nz(w_first[k])) >> 3);
+        see(true, head + g_first * 16 + at);
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (w_last[k] != 0u) at = 4 * k + ((31 - __builtin_clz(nz(w_last[k]))) >> 3);
+        see(true, head + g_last * 16 + at);
       }
       for (int64_t t = head + groups * 16 + threadIdx.x; t < n_cols; t += kBlock) see(bytes[t] != 0, t);
     } else {
@@ -104,10 +121,12 @@ __global__ __launch_bounds__(kCuBlock) void cu_seqlens_kernel(const int64_t* __r
   }
 }
 
-// A workgroup moves kCopyChunk consecutive columns of one row. (row, chunk) items are numbered
+// A workgroup moves copy_chunk<E>() consecutive columns of one row (16 KiB whatever the element). (row, chunk) items are numbered
 // with the row varying fastest: workgroups go to the XCDs round-robin by index, and numbered
 // chunk-fastest the chunks that hold tokens of short rows would pile up on a few XCDs.
-constexpr int kCopyChunk = 4096;
+constexpr int kCopyChunkBytes = 16384;
+template <typename E>
+constexpr int copy_chunk() { return kCopyChunkBytes / (int)sizeof(E); }
 
 // 16 bytes of consecutive elements as one load or store. The type only promises the element's own
 // alignment (source and destination rows start anywhere), which gfx950 global memory accepts.
@@ -127,6 +146,7 @@ template <typename E>
 __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__ src, int64_t n_rows, int64_t n_cols,
                                                            const int64_t* __restrict__ first,
                                                            const int64_t* __restrict__ cu, E* __restrict__ dst) {
+  constexpr int kCopyChunk = copy_chunk<E>();
   const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
   const int64_t slots = row_slots(n_rows);
   const int slot_b = slot_bits(n_rows);
@@ -143,7 +163,7 @@ __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__
     constexpr int kE = Vec16<E>::kElems;
     typedef typename Vec16<E>::type V;
     const int64_t groups = (stop - j0) / kE;
-#pragma unroll 2
+#pragma unroll 4
     for (int64_t g = threadIdx.x; g < groups; g += kBlock) *(V*)(out + j0 + g * kE) = __builtin_nontemporal_load((const V*)(in + j0 + g * kE));
     for (int64_t j = j0 + groups * kE + threadIdx.x; j < stop; j += kBlock) out[j] = in[j];
   }
@@ -153,6 +173,7 @@ template <typename E>
 __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ src, const int64_t* __restrict__ cu,
                                                           int64_t n_rows, int64_t n_cols, int left, E fill,
                                                           E* __restrict__ dst) {
+  constexpr int kCopyChunk = copy_chunk<E>();
   const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
   for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
     const int64_t chunk = w / n_rows, b = w - chunk * n_rows, t0 = chunk * kCopyChunk;
@@ -187,8 +208,9 @@ __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ 
   }
 }
 
-static inline unsigned copy_grid(int64_t n_rows, int64_t n_cols) {
-  const int64_t chunks = (n_cols + kCopyChunk - 1) / kCopyChunk;
+static inline unsigned copy_grid(int64_t n_rows, int64_t n_cols, int elem_bytes) {
+  const int64_t chunk = kCopyChunkBytes / elem_bytes;
+  const int64_t chunks = (n_cols + chunk - 1) / chunk;
   return slot_grid(row_slots(n_rows) * chunks, 262144);
 }
 
@@ -231,7 +253,9 @@ extern "C" int orlhf_pack_rows(const void* src, int elem_bytes, int64_t n_rows, 
   ORLHF_CHECK_ARG(n_rows >= 0 && n_cols >= 0, "pack_rows: n_rows=%lld n_cols=%lld", (long long)n_rows, (long long)n_cols);
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(src != nullptr && dst != nullptr && cu_seqlens != nullptr, "pack_rows: NULL argument");
-  const dim3 grid(copy_grid(n_rows, n_cols)), block(kBlock);
+  ORLHF_CHECK_ARG(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8,
+                  "row layout: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
+  const dim3 grid(copy_grid(n_rows, n_cols, elem_bytes)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
   switch (elem_bytes) {
     case 1: hipLaunchKernelGGL(pack_rows_kernel<uint8_t>, grid, block, 0, s, (const uint8_t*)src, n_rows, n_cols, first, cu_seqlens, (uint8_t*)dst); break;
@@ -249,7 +273,9 @@ extern "C" int orlhf_pad_rows(const void* src, int elem_bytes, const int64_t* cu
   ORLHF_CHECK_ARG(n_rows >= 0 && n_cols >= 0, "pad_rows: n_rows=%lld n_cols=%lld", (long long)n_rows, (long long)n_cols);
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(dst != nullptr && cu_seqlens != nullptr, "pad_rows: NULL argument");
-  const dim3 grid(copy_grid(n_rows, n_cols)), block(kBlock);
+  ORLHF_CHECK_ARG(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8,
+                  "row layout: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
+  const dim3 grid(copy_grid(n_rows, n_cols, elem_bytes)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
   const int left = left_side != 0;
   switch (elem_bytes) {
