@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 18
+#define ORLHF_ABI_VERSION 19
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -630,6 +630,15 @@ int orlhf_cu_seqlens(const int64_t* lengths, int64_t n_rows, int64_t* cu_seqlens
 int orlhf_pack_rows(const void* src, int elem_bytes, int64_t n_rows, int64_t n_cols,
                     const int64_t* first, const int64_t* cu_seqlens, void* dst,
                     orlhf_stream_t stream);
+
+/* dst[cu[b] + j] = src[src_start[b] + j] for j < cu[b+1] - cu[b]: rows picked out of a packed
+ * array into a new packed array, in any order and with repeats (a replay buffer handing out a
+ * micro-batch without going through the padded form of
+ * openrlhf/trainer/ppo_utils/experience.py:199-247). max_len bounds the row lengths (it sizes the
+ * launch; rows longer than it are cut). Elements are elem_bytes (1, 2, 4, 8) wide. */
+int orlhf_gather_rows(const void* src, int elem_bytes, int64_t n_rows, int64_t max_len,
+                      const int64_t* src_start, const int64_t* cu_seqlens, void* dst,
+                      orlhf_stream_t stream);
 
 /*
  * zero_pad_sequences(..., side, value, stack=True) (openrlhf/utils/utils.py:93-106) from the

@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 
 class Norm(Structure):
@@ -117,6 +117,7 @@ SIGNATURES = {
     "orlhf_row_extents": (c_int, [P, c_int, I64, I64, P, P, P, P]),
     "orlhf_cu_seqlens": (c_int, [P, I64, P, P]),
     "orlhf_pack_rows": (c_int, [P, c_int, I64, I64, P, P, P, P]),
+    "orlhf_gather_rows": (c_int, [P, c_int, I64, I64, P, P, P, P]),
     "orlhf_pad_rows": (c_int, [P, c_int, P, I64, I64, c_int, c_uint64, P, P]),
     "orlhf_sequence_logps_fwd": (c_int, [P, P, c_int, P, I64, I64, P, P, P, P]),
     "orlhf_sequence_logps_bwd": (c_int, [P, P, P, c_int, P, P, I64, I64, P, P]),

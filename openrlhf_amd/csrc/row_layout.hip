@@ -5,6 +5,7 @@
 //   row_extents   first / one-past-last non-zero column of every mask row
 //   cu_seqlens    exclusive prefix sum of row lengths (one workgroup, chained 256-wide scans)
 //   pack_rows     dst[cu[b] + j] = src[b, first[b] + j]
+//   gather_rows   dst[cu[b] + j] = src[start[b] + j]: rows picked out of another packed array
 //   pad_rows      dst[b, :] = fill, then the row's tokens on the left or on the right side
 #include "common.h"
 
@@ -142,7 +143,10 @@ struct Vec16 {
   static constexpr int kElems = 16 / sizeof(E);
 };
 
-template <typename E>
+// PITCHED: the source is a padded [n_rows, n_cols] grid and `first` (nullable) the first column of
+// each row. Otherwise the source is flat, `first[b]` is the element where output row b starts in
+// it, and n_cols only bounds the row lengths (it sizes the grid).
+template <typename E, bool PITCHED>
 __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__ src, int64_t n_rows, int64_t n_cols,
                                                            const int64_t* __restrict__ first,
                                                            const int64_t* __restrict__ cu, E* __restrict__ dst) {
@@ -157,8 +161,9 @@ __global__ __launch_bounds__(kBlock) void pack_rows_kernel(const E* __restrict__
     if (j0 >= len) continue;
     const int64_t f = first != nullptr ? first[b] : 0;
     int64_t stop = j0 + kCopyChunk < len ? j0 + kCopyChunk : len;
-    stop = stop < n_cols - f ? stop : n_cols - f;
-    const E* in = src + b * n_cols + f;
+    const int64_t bound = PITCHED ? n_cols - f : n_cols;  // the grid's columns / the stated longest row
+    stop = stop < bound ? stop : bound;
+    const E* in = PITCHED ? src + b * n_cols + f : src + f;
     E* out = dst + start;
     constexpr int kE = Vec16<E>::kElems;
     typedef typename Vec16<E>::type V;
@@ -258,13 +263,34 @@ extern "C" int orlhf_pack_rows(const void* src, int elem_bytes, int64_t n_rows, 
   const dim3 grid(copy_grid(n_rows, n_cols, elem_bytes)), block(kBlock);
   hipStream_t s = (hipStream_t)stream;
   switch (elem_bytes) {
-    case 1: hipLaunchKernelGGL(pack_rows_kernel<uint8_t>, grid, block, 0, s, (const uint8_t*)src, n_rows, n_cols, first, cu_seqlens, (uint8_t*)dst); break;
-    case 2: hipLaunchKernelGGL(pack_rows_kernel<uint16_t>, grid, block, 0, s, (const uint16_t*)src, n_rows, n_cols, first, cu_seqlens, (uint16_t*)dst); break;
-    case 4: hipLaunchKernelGGL(pack_rows_kernel<uint32_t>, grid, block, 0, s, (const uint32_t*)src, n_rows, n_cols, first, cu_seqlens, (uint32_t*)dst); break;
-    case 8: hipLaunchKernelGGL(pack_rows_kernel<uint64_t>, grid, block, 0, s, (const uint64_t*)src, n_rows, n_cols, first, cu_seqlens, (uint64_t*)dst); break;
+    case 1: hipLaunchKernelGGL((pack_rows_kernel<uint8_t, true>), grid, block, 0, s, (const uint8_t*)src, n_rows, n_cols, first, cu_seqlens, (uint8_t*)dst); break;
+    case 2: hipLaunchKernelGGL((pack_rows_kernel<uint16_t, true>), grid, block, 0, s, (const uint16_t*)src, n_rows, n_cols, first, cu_seqlens, (uint16_t*)dst); break;
+    case 4: hipLaunchKernelGGL((pack_rows_kernel<uint32_t, true>), grid, block, 0, s, (const uint32_t*)src, n_rows, n_cols, first, cu_seqlens, (uint32_t*)dst); break;
+    case 8: hipLaunchKernelGGL((pack_rows_kernel<uint64_t, true>), grid, block, 0, s, (const uint64_t*)src, n_rows, n_cols, first, cu_seqlens, (uint64_t*)dst); break;
     default: return fail(ORLHF_ERR_INVALID_ARG, "pack_rows: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
   }
   ORLHF_CHECK_LAUNCH("orlhf_pack_rows");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_gather_rows(const void* src, int elem_bytes, int64_t n_rows, int64_t max_len,
+                                 const int64_t* src_start, const int64_t* cu_seqlens, void* dst,
+                                 orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n_rows >= 0 && max_len >= 0, "gather_rows: n_rows=%lld max_len=%lld", (long long)n_rows, (long long)max_len);
+  if (n_rows * max_len == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(src != nullptr && dst != nullptr && cu_seqlens != nullptr && src_start != nullptr,
+                  "gather_rows: NULL argument");
+  ORLHF_CHECK_ARG(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8,
+                  "row layout: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
+  const dim3 grid(copy_grid(n_rows, max_len, elem_bytes)), block(kBlock);
+  hipStream_t s = (hipStream_t)stream;
+  switch (elem_bytes) {
+    case 1: hipLaunchKernelGGL((pack_rows_kernel<uint8_t, false>), grid, block, 0, s, (const uint8_t*)src, n_rows, max_len, src_start, cu_seqlens, (uint8_t*)dst); break;
+    case 2: hipLaunchKernelGGL((pack_rows_kernel<uint16_t, false>), grid, block, 0, s, (const uint16_t*)src, n_rows, max_len, src_start, cu_seqlens, (uint16_t*)dst); break;
+    case 4: hipLaunchKernelGGL((pack_rows_kernel<uint32_t, false>), grid, block, 0, s, (const uint32_t*)src, n_rows, max_len, src_start, cu_seqlens, (uint32_t*)dst); break;
+    default: hipLaunchKernelGGL((pack_rows_kernel<uint64_t, false>), grid, block, 0, s, (const uint64_t*)src, n_rows, max_len, src_start, cu_seqlens, (uint64_t*)dst); break;
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_gather_rows");
   return ORLHF_OK;
 }
 

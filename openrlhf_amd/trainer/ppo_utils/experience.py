@@ -348,6 +348,168 @@ def remove_padding_in_sequences(items: List[Experience]) -> List[Experience]:
     return items
 
 
+def gather_packed_rows(flat: torch.Tensor, src_start: torch.Tensor, cu_seqlens: torch.Tensor, max_len: int,
+                       total: int) -> torch.Tensor:
+    """Rows picked out of a packed array: output row b (``cu_seqlens[b] .. cu_seqlens[b+1]-1`` of
+    the result) holds the elements of ``flat`` from ``src_start[b]`` on. ``max_len`` bounds the row
+    lengths, ``total`` is ``cu_seqlens[-1]``."""
+    dev = require_gpu(flat, src_start, cu_seqlens)
+    if flat.element_size() not in _BITS:
+        raise ValueError(f"unsupported element size {flat.element_size()}")
+    src = flat.reshape(-1).contiguous()
+    out = torch.empty(int(total), dtype=flat.dtype, device=dev)
+    n_rows = cu_seqlens.numel() - 1
+    if total == 0 or n_rows == 0:
+        return out
+    with _lib.on_device(dev):
+        call("orlhf_gather_rows", ptr(src), src.element_size(), n_rows, int(max_len),
+             ptr(src_start.to(torch.int64).contiguous()), ptr(cu_seqlens.to(torch.int64).contiguous()), ptr(out),
+             stream_of(dev))
+    return out
+
+
+@dataclass
+class PackedExperience:
+    """A batch whose per-step fields stay packed between the rollout and the training step.
+
+    The reference moves a rollout batch to the trainer as ``split_experience_batch`` ->
+    ``remove_padding_in_sequences`` -> (replay buffer) -> ``make_experience_batch``
+    (openrlhf/trainer/ppo_utils/experience.py:164-247): every hop slices or pads each field of each
+    sample. Here the batch is packed once (``from_experience``): every per-step field is one flat
+    tensor holding, row after row, what ``remove_padding_in_sequences`` keeps of it (everything but
+    the columns behind the last attended token), with one ``cu_seqlens`` per field width (``T`` for
+    ``sequences`` / ``attention_mask``, ``A`` for the action fields). The per-token kernels take
+    these tensors as they are (``actions()`` is a ``PackedSteps``); ``select`` hands out any rows as
+    a new packed batch (a replay buffer's micro-batch) with one gather launch per field;
+    ``to_experience`` is the padded batch ``make_experience_batch`` would have built from the same
+    samples."""
+
+    steps: Dict[str, torch.Tensor]          # name -> flat tensor
+    widths: Dict[str, int]                  # name -> width of the padded field it came from
+    cu: Dict[int, torch.Tensor]             # width -> int64 [B+1] boundaries
+    totals: Dict[int, int]                  # width -> cu[width][-1]
+    episode: Dict[str, torch.Tensor] = field(default_factory=dict)   # [B] tensors
+    meta: Dict[str, Any] = field(default_factory=dict)               # index / prompts / labels / images / mm_train_inputs / info
+
+    def __len__(self) -> int:
+        return next(iter(self.cu.values())).numel() - 1 if self.cu else 0
+
+    @classmethod
+    def from_experience(cls, exp: "Experience") -> "PackedExperience":
+        att = exp.attention_mask
+        if att is None or att.dim() != 2:
+            raise ValueError("a batched Experience with an attention_mask [B, T] is needed")
+        t = att.shape[1]
+        _, end, _ = row_extents(att)
+        keep_t = torch.where(end > 0, end, torch.full_like(end, t))  # an all-zero mask keeps everything (argmax 0)
+        steps, widths, cu, totals = {}, {}, {}, {}
+        for name in STEP_FIELDS:
+            value = getattr(exp, name)
+            if value is None:
+                continue
+            if value.dim() != 2 or value.shape[0] != att.shape[0]:
+                raise ValueError(f"{name} must be [B, width], got {tuple(value.shape)}")
+            w = value.shape[1]
+            if w not in cu:
+                lengths = (keep_t - (t - w)).clamp_(min=0)  # the same number of trailing columns goes
+                cu[w] = cu_seqlens_of(lengths)
+                totals[w] = int(cu[w][-1])
+            steps[name] = pack_padded(value, cu[w], None, totals[w])
+            widths[name] = w
+        episode = {n: getattr(exp, n) for n in EPISODE_FIELDS if getattr(exp, n) is not None}
+        meta = {n: getattr(exp, n) for n in ("index", "prompts", "labels", "images", "mm_train_inputs", "info")}
+        return cls(steps, widths, cu, totals, episode, meta)
+
+    def actions(self, names=None) -> PackedSteps:
+        """The action-wide fields (the width of ``action_mask``) as a ``PackedSteps``: what the
+        per-token kernels take with ``cu_seqlens=``."""
+        w = self.widths["action_mask"]
+        names = [n for n, wn in self.widths.items() if wn == w] if names is None else names
+        first = torch.zeros(len(self), dtype=torch.int64, device=self.cu[w].device)
+        return PackedSteps(self.cu[w], first, w, self.totals[w], {n: self.steps[n] for n in names})
+
+    def set_step(self, name: str, flat: torch.Tensor, like: str = "action_mask") -> None:
+        """Adds or replaces a per-step field computed in the packed layout (advantages, returns, kl)."""
+        w = self.widths[like]
+        if flat.numel() != self.totals[w]:
+            raise ValueError(f"{name}: {flat.numel()} elements, the packed fields of width {w} hold {self.totals[w]}")
+        self.steps[name], self.widths[name] = flat.reshape(-1), w
+
+    def select(self, rows) -> "PackedExperience":
+        """The given rows (a list of ints; any order, repeats allowed) as a new packed batch."""
+        rows = [int(r) for r in rows]
+        n = len(self)
+        if any(r < -n or r >= n for r in rows):
+            raise IndexError(f"row index out of range for a batch of {n}")
+        rows = [r % n for r in rows]
+        dev = next(iter(self.cu.values())).device
+        idx = torch.tensor(rows, dtype=torch.int64, device=dev)
+        cu, totals, starts = {}, {}, {}
+        for w, old in self.cu.items():
+            starts[w] = old[idx]
+            cu[w] = cu_seqlens_of(old[idx + 1] - starts[w])
+            totals[w] = int(cu[w][-1])
+        steps = {name: gather_packed_rows(flat, starts[self.widths[name]], cu[self.widths[name]], self.widths[name],
+                                          totals[self.widths[name]])
+                 for name, flat in self.steps.items()}
+        episode = {n_: v[idx.to(v.device)] for n_, v in self.episode.items()}
+
+        def pick(value):
+            if isinstance(value, list):
+                return [value[r] for r in rows] if len(value) == n else value
+            if isinstance(value, torch.Tensor):
+                return value[idx.to(value.device)] if value.dim() > 0 and len(value) == n else value
+            if isinstance(value, dict):
+                return {k: pick(v) for k, v in value.items()}
+            return value
+
+        return PackedExperience(steps, dict(self.widths), cu, totals, episode, {k: pick(v) for k, v in self.meta.items()})
+
+    @staticmethod
+    def concat(batches: List["PackedExperience"]) -> "PackedExperience":
+        """Several packed batches as one (rows in the order given)."""
+        if not batches:
+            raise ValueError("Empty batch list")
+        head = batches[0]
+        if any(b.widths.keys() != head.widths.keys() for b in batches):
+            raise ValueError("batches hold different per-step fields")
+        # a field's width only bounds its rows: the joint batch takes the largest
+        cu, totals, width_of = {}, {}, {}
+        for name in head.widths:
+            width_of[name] = max(b.widths[name] for b in batches)
+        for name, w in width_of.items():
+            if w in cu:
+                continue
+            parts, offset = [head.cu[head.widths[name]][:1]], 0
+            for b in batches:
+                c = b.cu[b.widths[name]]
+                parts.append(c[1:] + offset)
+                offset += b.totals[b.widths[name]]
+            cu[w], totals[w] = torch.cat(parts), offset
+        steps = {name: torch.cat([b.steps[name] for b in batches]) for name in head.widths}
+        episode = {n_: torch.cat([b.episode[n_] for b in batches]) for n_ in head.episode}
+        meta = {k: Experience._merge_item([b.meta[k] for b in batches]) if head.meta.get(k) is not None else None
+                for k in head.meta}
+        return PackedExperience(steps, width_of, cu, totals, episode, meta)
+
+    def to_experience(self, widths: Optional[Dict[int, int]] = None) -> "Experience":
+        """The padded batch ``make_experience_batch`` builds from the un-padded samples: every
+        per-step field right-padded with 0 to its longest row. ``widths`` (packed width -> padded
+        width) saves reading the longest row back. Fields added with ``set_step`` under a name the
+        Experience does not have stay behind."""
+        out = {}
+        for name, flat in self.steps.items():
+            if name not in STEP_FIELDS:  # a working field of the packed batch, no Experience attribute
+                continue
+            w = self.widths[name]
+            c = self.cu[w]
+            n_cols = widths[w] if widths is not None and w in widths else (int((c[1:] - c[:-1]).max()) if len(self) else 0)
+            out[name] = pad_packed(flat, c, n_cols, "right", 0)
+        out.update(self.episode)
+        out.update({k: v for k, v in self.meta.items() if v is not None})
+        return Experience(**out)
+
+
 def balance_experiences(experiences, args):
     """Spreads long and short sequences evenly over the data-parallel ranks by pairing chunks of
     the length-sorted samples from both ends (experience.py:250-283)."""

@@ -129,3 +129,114 @@ def test_packed_fields_of_an_experience(cuda):
     packed = PolicyLoss()(ps["action_log_probs"], po["old"], po["adv"], action_mask=ps["action_mask"],
                           cu_seqlens=ps.cu_seqlens, max_seqlen=ps.max_seqlen)[0]
     assert abs(padded.item() - packed.item()) <= 1e-6
+
+
+def _ragged_batch(dev, seed=3, b=9, t=41):
+    """Right-padded rows of every length from 1 to t, one row without padding, one all-zero mask."""
+    from openrlhf_amd.trainer.ppo_utils.experience import Experience
+
+    g = torch.Generator().manual_seed(seed)
+    lens = torch.randint(1, t + 1, (b,), generator=g)
+    lens[0], lens[1] = t, 0
+    att = (torch.arange(t)[None, :] < lens[:, None]).long()
+    a = t - 1
+    amask = att[:, 1:].bool().clone()
+    amask[:, :2] = False
+    amask[3, 5:9] = False  # a hole inside a row stays inside its extent
+    mk = lambda: torch.randn(b, a, generator=g)
+    return Experience(
+        sequences=torch.randint(1, 1000, (b, t), generator=g).to(dev), attention_mask=att.to(dev),
+        action_mask=amask.to(dev), action_log_probs=mk().to(dev), base_action_log_probs=mk().to(dev),
+        values=mk().to(dev), kl=mk().to(torch.bfloat16).to(dev), rewards=torch.randn(b, generator=g).to(dev),
+        total_length=lens.to(dev), prompts=[f"p{i}" for i in range(b)], labels=[f"l{i}" for i in range(b)],
+        info={"tag": [f"t{i}" for i in range(b)], "score": torch.arange(b).float().to(dev)},
+    ), lens
+
+
+def _reference_hops(exp, rows=None):
+    """What the reference's hops build from the batch: split, cut the padding, re-batch (the
+    mirrors of experience.py:164-247, themselves checked against the layout oracle above)."""
+    import copy
+
+    from openrlhf_amd.trainer.ppo_utils.experience import (
+        make_experience_batch, remove_padding_in_sequences, split_experience_batch)
+
+    items = remove_padding_in_sequences(split_experience_batch(copy.copy(exp)))
+    if rows is not None:
+        items = [items[r] for r in rows]
+    return make_experience_batch(items), items
+
+
+def test_packed_experience_equals_the_reference_hops(cuda):
+    from openrlhf_amd.trainer.ppo_utils.experience import STEP_FIELDS, PackedExperience
+
+    exp, lens = _ragged_batch(cuda)
+    want, items = _reference_hops(exp)
+    pe = PackedExperience.from_experience(exp)
+    assert len(pe) == 9
+    # every flat field is the concatenation of what remove_padding_in_sequences keeps of each sample
+    for name in ("sequences", "attention_mask", "action_mask", "action_log_probs", "values", "kl"):
+        cat = torch.cat([getattr(it, name) for it in items])
+        assert pe.steps[name].dtype == cat.dtype and torch.equal(pe.steps[name], cat), name
+    keep = [olay.unpadded_length(exp.attention_mask[r].cpu()) for r in range(9)]
+    assert pe.cu[41].tolist() == [0] + torch.tensor(keep).cumsum(0).tolist()
+    got = pe.to_experience()
+    for name in STEP_FIELDS:
+        w, g_ = getattr(want, name), getattr(got, name)
+        assert (w is None) == (g_ is None), name
+        if w is not None:
+            assert w.shape == g_.shape and w.dtype == g_.dtype and torch.equal(w, g_), name
+    assert torch.equal(got.rewards, exp.rewards) and got.prompts == exp.prompts and got.info["tag"] == exp.info["tag"]
+    # a known padded width saves the read-back
+    assert torch.equal(pe.to_experience(widths={41: 41, 40: 40}).values, want.values)
+
+
+def test_packed_experience_select_and_concat(cuda):
+    from openrlhf_amd.trainer.ppo_utils.experience import PackedExperience
+
+    exp, _ = _ragged_batch(cuda, seed=5)
+    pe = PackedExperience.from_experience(exp)
+    rows = [4, 0, 4, 8, 1, -2]
+    sub = pe.select(rows)
+    want, _ = _reference_hops(exp, [r % 9 for r in rows])
+    got = sub.to_experience()
+    for name in ("sequences", "attention_mask", "action_mask", "action_log_probs", "base_action_log_probs", "values", "kl"):
+        assert torch.equal(getattr(got, name), getattr(want, name)), name
+    assert torch.equal(got.rewards, exp.rewards[[4, 0, 4, 8, 1, 7]]) and got.prompts == ["p4", "p0", "p4", "p8", "p1", "p7"]
+    assert got.info["tag"] == ["t4", "t0", "t4", "t8", "t1", "t7"] and torch.equal(got.info["score"], exp.info["score"][[4, 0, 4, 8, 1, 7]])
+    with pytest.raises(IndexError):
+        pe.select([9])
+    assert len(pe.select([])) == 0 and pe.select([]).steps["values"].numel() == 0
+    # two halves joined again are the whole
+    both = PackedExperience.concat([pe.select(range(0, 4)), pe.select(range(4, 9))])
+    for name, flat in pe.steps.items():
+        assert torch.equal(both.steps[name], flat), name
+    assert torch.equal(both.cu[40], pe.cu[40]) and both.meta["prompts"] == exp.prompts
+    assert torch.equal(both.episode["rewards"], exp.rewards)
+
+
+def test_packed_experience_feeds_the_per_token_kernels(cuda):
+    """Advantages computed on the packed fields and stored back equal the padded computation on the
+    columns the samples keep."""
+    from openrlhf_amd.trainer.ppo_utils.experience import PackedExperience
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import get_advantages_and_returns
+
+    exp, _ = _ragged_batch(cuda, seed=7)
+    exp.values = exp.values * exp.action_mask
+    rewards = exp.action_log_probs * exp.action_mask
+    adv_p, ret_p = get_advantages_and_returns(exp.values, rewards, exp.action_mask, 0.99, 0.95)
+    pe = PackedExperience.from_experience(exp)
+    pe.set_step("rewards_t", pe.steps["action_log_probs"] * pe.steps["action_mask"])
+    ps = pe.actions()
+    adv, ret = get_advantages_and_returns(ps["values"], ps["rewards_t"], ps["action_mask"], 0.99, 0.95,
+                                          cu_seqlens=ps.cu_seqlens, max_seqlen=ps.max_seqlen, row_order=ps.longest_first)
+    pe.set_step("advantages", adv)
+    pe.set_step("returns", ret)
+    got = pe.to_experience()
+    width = got.advantages.shape[1]
+    keep = (torch.arange(width, device=cuda)[None, :] < (pe.cu[40][1:] - pe.cu[40][:-1])[:, None])
+    # behind a row's last attended token the padded scan sees zeros only, so the kept columns agree
+    assert torch.allclose(got.advantages, adv_p[:, :width] * keep, rtol=1e-6, atol=1e-6)
+    assert torch.allclose(got.returns, ret_p[:, :width] * keep, rtol=1e-6, atol=1e-6)
+    with pytest.raises(ValueError):
+        pe.set_step("bad", adv[:-1])
