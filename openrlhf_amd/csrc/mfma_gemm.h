@@ -103,19 +103,28 @@ __device__ __forceinline__ void fetch_slab(u32x4 (&r)[8], const Operand& op, int
 // of the slab, so lane L fetches the chunk that the swizzle puts at position (L & 7) of row
 // (L >> 3) of those 8 rows. Rows past the operand arrive as zeros (resource bounds). The caller
 // waits for these loads (vmcnt) before the barrier that publishes the slab.
-__device__ __forceinline__ void dma_slab(const Operand& op, int64_t row0, int64_t k0, char* slab, uint32_t wave_u,
-                                         uint32_t lane) {
-  const __amdgpu_buffer_rsrc_t rs = slab_resource<false>(op, row0, k0);
-  const uint32_t ld2 = (uint32_t)op.ld * 2u;
-  const uint32_t lrow = lane >> 3, x = (lane & 7u) ^ lrow;
-  const uint32_t vbase = lrow * ld2;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    // rows (wave_u * 8 + i) * 8 .. + 7: swz(row) = (row & 7) ^ ((row >> 3) & 7) = lrow ^ i
+struct SlabDma {
+  __amdgpu_buffer_rsrc_t rs;
+  uint32_t ld2, vbase, x, wave_u;
+  char* slab;
+  __device__ __forceinline__ SlabDma(const Operand& op, int64_t row0, int64_t k0, char* slab_, uint32_t wave_u_, uint32_t lane)
+      : rs(slab_resource<false>(op, row0, k0)), ld2((uint32_t)op.ld * 2u), wave_u(wave_u_), slab(slab_) {
+    const uint32_t lrow = lane >> 3;
+    x = (lane & 7u) ^ lrow;
+    vbase = lrow * ld2;
+  }
+  // load i of this wave's 8: rows (wave_u * 8 + i) * 8 .. + 7, swz(row) = (row & 7) ^ ((row >> 3) & 7) = lrow ^ i
+  __device__ __forceinline__ void issue(int i) const {
     const uint32_t voff = vbase + ((x ^ (uint32_t)i) << 4);
     __builtin_amdgcn_raw_ptr_buffer_load_lds(rs, (__attribute__((address_space(3))) void*)(slab + (wave_u * 8u + i) * 1024u), 16,
                                              voff, (wave_u * 64u + (uint32_t)i * 8u) * ld2, 0, 0);
   }
+};
+__device__ __forceinline__ void dma_slab(const Operand& op, int64_t row0, int64_t k0, char* slab, uint32_t wave_u,
+                                         uint32_t lane) {
+  const SlabDma d(op, row0, k0, slab, wave_u, lane);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) d.issue(i);
 }
 
 // ---- registers -> LDS slab ([256][64] swizzled). K-major: chunks I0 .. I1-1 of this thread.
@@ -177,6 +186,22 @@ __device__ __forceinline__ void load_frags(Frags& f, const char* slab_a, const c
   }
 }
 
+// The same reads with the 8 loads of a slab's LDS-direct transfer between them, in program order:
+// the compiler keeps LDS-direct loads and LDS reads in order (both touch LDS), so this is what
+// spreads the loads under the MFMAs instead of leaving them as one block in front of the step.
+__device__ __forceinline__ void load_frags_between_dma(Frags& f, const char* slab_a, const char* slab_b, int ks, uint32_t wm,
+                                                       uint32_t wn, uint32_t lane, const SlabDma& d) {
+  const uint32_t lr = lane & 31u, lk = lane >> 5;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const uint32_t ra = wm * 128u + t * 32u + lr, rb = wn * 128u + t * 32u + lr;
+    d.issue(2 * t);
+    f.a[t] = *(const u32x4*)(slab_a + ra * 128u + (((ks * 2u + lk) ^ swz(ra)) << 4));
+    d.issue(2 * t + 1);
+    f.b[t] = *(const u32x4*)(slab_b + rb * 128u + (((ks * 2u + lk) ^ swz(rb)) << 4));
+  }
+}
+
 template <int DT>
 __device__ __forceinline__ void mfma_step(f32x16 (&acc)[4][4], const Frags& f) {
 #pragma unroll
@@ -186,12 +211,32 @@ __device__ __forceinline__ void mfma_step(f32x16 (&acc)[4][4], const Frags& f) {
   }
 }
 
+// Issue order of one k-step of the steady loop: the eight LDS reads of the next fragments, and
+// N_VMEM global loads into registers per read, go out under the first eight MFMAs; the other eight
+// MFMAs cover their latency. Left to itself the scheduler sinks the reads to the end of the step,
+// where the next step's first MFMA waits for them with the matrix pipe idle. (LDS-direct loads
+// match no group; they keep their program order among the LDS reads, which is what
+// load_frags_between_dma uses.)
+template <int N_VMEM>
+__device__ __forceinline__ void issue_order() {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // one LDS read
+    if (N_VMEM > 0) __builtin_amdgcn_sched_group_barrier(0x010, N_VMEM, 0);  // global loads into registers
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+  }
+  __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+}
+
 // ---- the whole product of one output tile: acc = A[row0_a.., :] * B[row0_b.., :]^T over k in [0, depth)
 // `lds` = kLdsBytes of dynamic shared memory.
 //
-// Iteration s multiplies slab s out of one LDS buffer while slab s + 1 arrives in the other:
-//  * a K-major operand's slab is loaded straight into LDS (dma_slab), issued at the top of the
-//    iteration; only a slab that crosses the end of the depth goes through registers (masking);
+// Iteration s multiplies slab s out of one LDS buffer while slab s + 1 is (or arrives) in the other:
+//  * a K-major operand's slab is loaded straight into LDS (SlabDma): slab s + 2 as soon as the
+//    barrier of iteration s has freed the buffer slab s was read from, a whole iteration before
+//    the barrier that publishes it, its loads placed between that k-step's LDS reads so that each
+//    goes out under an MFMA and the matrix pipe never waits for a burst of address arithmetic and
+//    load issue; only a slab that crosses the end of the depth goes through registers (masking);
 //  * an MN-major operand's slab s + 1 sits in registers (fetched during iteration s - 1), is
 //    transposed and written to LDS during the first k-steps, and the fetch of slab s + 2 is issued
 //    into the registers it leaves.
@@ -206,6 +251,9 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
   // Everything addressed below derives from the thread index: making it opaque keeps a caller's
   // loop over tiles from hoisting a hundred address registers out of the product and holding
   // them (spilled) across its epilogue; they are recomputed per tile instead.
+  // operands whose next slab is carried in registers (K-major ones through registers as well were
+  // 3-11 % slower than the LDS-direct loads)
+  constexpr bool A_REG = A_MN_MAJOR, B_REG = B_MN_MAJOR;
   uint32_t tid = threadIdx.x;
   asm volatile("" : "+v"(tid));
   const uint32_t lane = tid & 63u, wave = tid >> 6;
@@ -228,63 +276,88 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
   stage_slab<A_MN_MAJOR>(ra, lds, tid);
   stage_slab<B_MN_MAJOR>(rb, lds + kSlabBytes, tid);
   if (n_slabs > 1) {  // MN-major operands carry slab s + 1 in registers from one iteration to the next
-    if (A_MN_MAJOR) fetch_slab<true, true>(ra, a, row0_a, kSlab, tid);
-    if (B_MN_MAJOR) fetch_slab<true, true>(rb, b, row0_b, kSlab, tid);
+    if (A_REG) fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, kSlab, tid);
+    if (B_REG) fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, kSlab, tid);
   }
   __syncthreads();
+  if (full > 1) {  // slab 1 is whole: A's half starts towards the second buffer now, B's in the first iteration
+    if (!A_REG) dma_slab(a, row0_a, kSlab, lds + kStageBytes, wave_u, lane);
+  }
   Frags f0, f1;
   load_frags(f0, lds, lds + kSlabBytes, 0, wm, wn, lane);
   int64_t s = 0;
 
-  // One steady-state iteration: slab s in buffer PARITY, slab s + 1 arrives in the other.
+  // One steady-state iteration: slab `it` in buffer PARITY; slab it + 1 is whole and lands in (or
+  // is staged into) the other buffer. Needs it + 1 < full.
   auto steady = [&](auto parity, int64_t it) {
     constexpr int P = decltype(parity)::value;
-    const char* cur = lds + P * kStageBytes;
+    char* cur = lds + P * kStageBytes;
     char* nxt = lds + (1 - P) * kStageBytes;
     const int64_t k1 = (it + 1) * kSlab, k2 = (it + 2) * kSlab;
+    const SlabDma db(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);  // B's slab it + 1 (unused if B_REG)
     // k-step 0
-    if (!A_MN_MAJOR) dma_slab(a, row0_a, k1, nxt, wave_u, lane);
-    if (!B_MN_MAJOR) dma_slab(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);
-    load_frags(f1, cur, cur + kSlabBytes, 1, wm, wn, lane);
-    if (A_MN_MAJOR) stage_slab<true, 0, 4>(ra, nxt, tid);
-    if (B_MN_MAJOR) stage_slab<true, 0, 4>(rb, nxt + kSlabBytes, tid);
+    if (!B_REG) {
+      load_frags_between_dma(f1, cur, cur + kSlabBytes, 1, wm, wn, lane, db);
+    } else {
+      load_frags(f1, cur, cur + kSlabBytes, 1, wm, wn, lane);
+    }
+    if (A_REG) stage_slab<A_MN_MAJOR, 0, 4>(ra, nxt, tid);
+    if (B_REG) stage_slab<B_MN_MAJOR, 0, 4>(rb, nxt + kSlabBytes, tid);
     mfma_step<DT>(acc, f0);
+    issue_order<0>();
     __builtin_amdgcn_sched_barrier(0);
     // k-step 1
     load_frags(f0, cur, cur + kSlabBytes, 2, wm, wn, lane);
-    if (A_MN_MAJOR) stage_slab<true, 4, 8>(ra, nxt, tid);
-    if (B_MN_MAJOR) stage_slab<true, 4, 8>(rb, nxt + kSlabBytes, tid);
+    if (A_REG) stage_slab<A_MN_MAJOR, 4, 8>(ra, nxt, tid);
+    if (B_REG) stage_slab<B_MN_MAJOR, 4, 8>(rb, nxt + kSlabBytes, tid);
     mfma_step<DT>(acc, f1);
+    issue_order<0>();
     __builtin_amdgcn_sched_barrier(0);
     // k-step 2
     load_frags(f1, cur, cur + kSlabBytes, 3, wm, wn, lane);
-    if (A_MN_MAJOR) fetch_slab<true, false>(ra, a, row0_a, k2, tid);
-    if (B_MN_MAJOR) fetch_slab<true, false>(rb, b, row0_b, k2, tid);
+    if (A_REG) fetch_slab<A_MN_MAJOR, !A_MN_MAJOR>(ra, a, row0_a, k2, tid);
+    if (B_REG) fetch_slab<B_MN_MAJOR, !B_MN_MAJOR>(rb, b, row0_b, k2, tid);
     mfma_step<DT>(acc, f0);
-    // every wave holds its last fragments of `cur`; slab s + 1 is complete in `nxt`
+    issue_order<(A_REG ? 1 : 0) + (B_REG ? 1 : 0)>();
+    // every wave holds its last fragments of `cur`; slab it + 1 is complete in `nxt`
     __syncthreads();
+    // `cur` is free: slab it + 2 starts towards it now, its loads spread between the LDS reads
+    // under the first MFMAs, and has until the next iteration's barrier. In the last iteration
+    // there is no such slab: slab 0 is loaded again instead of branching (nobody reads it; whatever
+    // touches this buffer next waits for its own later loads, and loads return in order).
     // k-step 3, over the read of the next slab's first fragments
-    load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
+    if (!A_REG) {
+      const SlabDma da(a, row0_a, it + 2 < full ? k2 : 0, cur, wave_u, lane);
+      load_frags_between_dma(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane, da);
+    } else {
+      load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
+    }
     mfma_step<DT>(acc, f1);
+    issue_order<0>();
     __builtin_amdgcn_sched_barrier(0);
   };
-  for (; s + 3 < full; s += 2) {  // pairs of steady iterations: slabs up to s + 3 exist and are whole
+  for (; s + 2 < full; s += 2) {  // pairs of steady iterations: the buffers' addresses are constants
     steady(std::integral_constant<int, 0>{}, s);
     steady(std::integral_constant<int, 1>{}, s + 1);
   }
+  if (s + 1 < full) {  // s is even here
+    steady(std::integral_constant<int, 0>{}, s);
+    ++s;
+  }
+  // s == full - 1 (or 0): slab s is in its buffer, no load into LDS is outstanding
   for (; s < n_slabs; ++s) {  // the last slabs: a k tail may need masking, slabs run out
     const char* cur = lds + (s & 1) * kStageBytes;
     char* nxt = lds + ((s + 1) & 1) * kStageBytes;
     const bool has1 = s + 1 < n_slabs, has2 = s + 2 < n_slabs;
     if (has1) {
-      if (!A_MN_MAJOR) fetch_slab<false, true>(ra, a, row0_a, (s + 1) * kSlab, tid);
-      if (!B_MN_MAJOR) fetch_slab<false, true>(rb, b, row0_b, (s + 1) * kSlab, tid);
-      if (A_MN_MAJOR) stage_slab<true>(ra, nxt, tid);
-      if (B_MN_MAJOR) stage_slab<true>(rb, nxt + kSlabBytes, tid);
+      if (!A_REG) fetch_slab<false, true>(ra, a, row0_a, (s + 1) * kSlab, tid);
+      if (!B_REG) fetch_slab<false, true>(rb, b, row0_b, (s + 1) * kSlab, tid);
+      if (A_REG) stage_slab<A_MN_MAJOR>(ra, nxt, tid);
+      if (B_REG) stage_slab<B_MN_MAJOR>(rb, nxt + kSlabBytes, tid);
     }
     if (has2) {
-      if (A_MN_MAJOR) fetch_slab<true, true>(ra, a, row0_a, (s + 2) * kSlab, tid);
-      if (B_MN_MAJOR) fetch_slab<true, true>(rb, b, row0_b, (s + 2) * kSlab, tid);
+      if (A_REG) fetch_slab<A_MN_MAJOR, true>(ra, a, row0_a, (s + 2) * kSlab, tid);
+      if (B_REG) fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, (s + 2) * kSlab, tid);
     }
     load_frags(f1, cur, cur + kSlabBytes, 1, wm, wn, lane);
     mfma_step<DT>(acc, f0);
@@ -293,13 +366,16 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     load_frags(f1, cur, cur + kSlabBytes, 3, wm, wn, lane);
     mfma_step<DT>(acc, f0);
     if (has1) {
-      if (!A_MN_MAJOR) stage_slab<false>(ra, nxt, tid);
-      if (!B_MN_MAJOR) stage_slab<false>(rb, nxt + kSlabBytes, tid);
+      if (!A_REG) stage_slab<false>(ra, nxt, tid);
+      if (!B_REG) stage_slab<false>(rb, nxt + kSlabBytes, tid);
       __syncthreads();
       load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
     }
     mfma_step<DT>(acc, f1);
   }
+  // the reload that stood in for a missing slab may still be on its way into LDS: it is long
+  // done by now, the wait only makes that explicit for whoever touches the buffers next
+  if (!A_REG) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   // no closing barrier: after the barrier inside the last iteration no wave reads the slab
   // buffers any more, but a caller that reuses them as scratch must synchronise first
 }
