@@ -359,6 +359,27 @@ __global__ __launch_bounds__(kBlock) void lmhead_round_kernel(const float* __res
   }
 }
 
+// dst[c][r] = src[r][c] for 16-bit elements, 64 x 64 tiles through LDS: the hidden states as
+// [H][N] so that the weight gradient's second operand is K-major (straight into LDS) as well.
+__global__ __launch_bounds__(kBlock) void lmhead_transpose_kernel(const uint16_t* __restrict__ src, int64_t n_rows,
+                                                                  int64_t n_cols, int64_t ld_src, uint16_t* __restrict__ dst,
+                                                                  int64_t ld_dst) {
+  __shared__ uint16_t tile[64][65];
+  const int64_t r0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const int64_t r = r0 + ty + 4 * k, c = c0 + tx;
+    tile[ty + 4 * k][tx] = (r < n_rows && c < n_cols) ? src[r * ld_src + c] : (uint16_t)0;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 16; ++k) {
+    const int64_t c = c0 + ty + 4 * k, r = r0 + tx;
+    if (c < n_cols && r < n_rows) dst[c * ld_dst + r] = tile[tx][ty + 4 * k];
+  }
+}
+
 template <int DT>
 __global__ __launch_bounds__(kBlock) void lmhead_zero_kernel(uint16_t* __restrict__ dst, int64_t n_rows, int64_t n_cols, int64_t ld) {
   const int64_t n = n_rows * n_cols;
@@ -403,6 +424,10 @@ static int64_t records_bytes(int64_t n_rows, int64_t vocab) {
 }
 // fp32 accumulator of dHidden.
 static int64_t dhidden_bytes(int64_t n_rows, int64_t hidden_dim) { return round_up(n_rows * hidden_dim * 4, 256); }
+// the transposed hidden states [hidden_dim][ld]: rows padded off the powers of two (a 16 KiB row
+// pitch sends every row to the same L2 channels)
+static int64_t transposed_ld(int64_t n_rows) { return round_up(n_rows, 8) + 64; }
+static int64_t transposed_bytes(int64_t n_rows, int64_t hidden_dim) { return round_up(hidden_dim * transposed_ld(n_rows) * 2, 256); }
 
 template <int DT>
 static int launch_fwd(const void* hidden, const void* weight, int64_t n_rows, int64_t hidden_dim, int64_t vocab,
@@ -438,15 +463,22 @@ static int launch_bwd(const void* hidden, const void* weight, int64_t n_rows, in
   const Operand w{(const uint16_t*)weight, weight_stride, vocab, hidden_dim};
   const Operand h{(const uint16_t*)hidden, hidden_stride, n_rows, hidden_dim};
   float* dh_acc = (float*)workspace;
-  uint16_t* p_chunk = (uint16_t*)(workspace + dhidden_bytes(n_rows, hidden_dim));
+  uint16_t* h_t = (uint16_t*)(workspace + dhidden_bytes(n_rows, hidden_dim));
+  uint16_t* p_chunk = (uint16_t*)(workspace + dhidden_bytes(n_rows, hidden_dim) + transposed_bytes(n_rows, hidden_dim));
+  const int64_t ld_t = transposed_ld(n_rows);
   const int64_t n_tb = (n_rows + 255) / 256, tiles_h = (hidden_dim + 255) / 256;
   const bool both_t = temperature != 1.0;
   const dim3 block(mm::kThreads);
   if (allow_lds(lmhead_bwd_p_kernel<DT, true>) != hipSuccess || allow_lds(lmhead_bwd_p_kernel<DT, false>) != hipSuccess ||
       allow_lds(lmhead_gemm_f32_kernel<DT, false, true, false>) != hipSuccess ||
       allow_lds(lmhead_gemm_f32_kernel<DT, false, true, true>) != hipSuccess ||
-      allow_lds(lmhead_gemm_lowp_kernel<DT, true, true>) != hipSuccess)
+      allow_lds(lmhead_gemm_lowp_kernel<DT, true, false>) != hipSuccess)
     return fail(ORLHF_ERR_LAUNCH, "lmhead_bwd: cannot get %d bytes of LDS", mm::kLdsBytes);
+  if (grad_weight != nullptr) {
+    hipLaunchKernelGGL(lmhead_transpose_kernel, dim3((unsigned)((n_rows + 63) / 64), (unsigned)((hidden_dim + 63) / 64)),
+                       dim3(kBlock), 0, s, (const uint16_t*)hidden, n_rows, hidden_dim, hidden_stride, h_t, ld_t);
+    ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(transpose)");
+  }
   for (int64_t v0 = 0; v0 < vocab; v0 += chunk_cols) {
     const int64_t cols = vocab - v0 < chunk_cols ? vocab - v0 : chunk_cols;  // valid vocabulary entries of this chunk
     const int64_t ctiles = (cols + 255) / 256;
@@ -478,9 +510,9 @@ static int launch_bwd(const void* hidden, const void* weight, int64_t n_rows, in
     // (3) dW[v0 + v][h] = sum_n P[n][v] * hidden[n][h]
     if (grad_weight != nullptr) {
       const Operand a{p_chunk, ldp, cols, n_rows};
-      const Operand b{(const uint16_t*)hidden, hidden_stride, hidden_dim, n_rows};
+      const Operand b{h_t, ld_t, hidden_dim, n_rows};
       const dim3 grid(grid_for_items(ctiles * tiles_h));
-      hipLaunchKernelGGL((lmhead_gemm_lowp_kernel<DT, true, true>), grid, block, mm::kLdsBytes, s, a, b,
+      hipLaunchKernelGGL((lmhead_gemm_lowp_kernel<DT, true, false>), grid, block, mm::kLdsBytes, s, a, b,
                          (uint16_t*)grad_weight + v0 * grad_weight_stride, grad_weight_stride, ctiles, tiles_h);
       ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(dW)");
     }
@@ -501,12 +533,13 @@ using namespace orlhf;
 extern "C" int64_t orlhf_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab, int backward) {
   if (n_rows < 0 || hidden_dim <= 0 || vocab <= 0) return 0;
   if (!backward) return lm::records_bytes(n_rows, vocab);
-  // the fp32 dHidden accumulator plus a chunk of P of about 256 MiB (at least one tile column, at most the vocabulary)
+  // the fp32 dHidden accumulator, the transposed hidden states, and a chunk of P of about 256 MiB
+  // (at least one tile column, at most the vocabulary)
   const int64_t rows = n_rows > 0 ? n_rows : 1;
   int64_t cols = ((256ll << 20) / (2 * rows)) / 256 * 256;
   const int64_t vpad = lm::round_up(vocab, 256);
   cols = cols < 256 ? 256 : (cols > vpad ? vpad : cols);
-  return lm::dhidden_bytes(n_rows, hidden_dim) + rows * cols * 2;
+  return lm::dhidden_bytes(n_rows, hidden_dim) + lm::transposed_bytes(n_rows, hidden_dim) + rows * cols * 2;
 }
 
 extern "C" int orlhf_lmhead_logprob_entropy_fwd(const void* hidden, const void* weight, int dtype, int64_t n_rows,
@@ -561,7 +594,7 @@ extern "C" int orlhf_lmhead_logprob_entropy_bwd(const void* hidden, const void* 
   ORLHF_CHECK_ARG(row_stats != nullptr && (g_logprob != nullptr || g_entropy != nullptr),
                   "lmhead_logprob_entropy_bwd: row_stats and at least one upstream gradient are needed");
   ORLHF_CHECK_ARG(g_logprob == nullptr || labels != nullptr, "lmhead_logprob_entropy_bwd: labels is NULL");
-  const int64_t fixed = lm::dhidden_bytes(n_rows, hidden_dim);
+  const int64_t fixed = lm::dhidden_bytes(n_rows, hidden_dim) + lm::transposed_bytes(n_rows, hidden_dim);
   int64_t cols = workspace != nullptr && workspace_bytes > fixed ? ((workspace_bytes - fixed) / (2 * n_rows)) / 256 * 256 : 0;
   const int64_t vpad = lm::round_up(vocab, 256);
   if (cols > vpad) cols = vpad;
