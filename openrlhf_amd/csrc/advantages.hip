@@ -186,49 +186,63 @@ struct RowReward {
   double sum;
 };
 
-// `whole`: the tile lies inside the row (no lane needs to look at the row's end). Must be called by
-// all lanes of the workgroup (it exchanges the following value across lanes).
+// The fp32 arrays of one row as buffer resources that end where the row ends: a 16-byte access
+// that reaches past the row reads zeros there and stores nothing there (the range check is per
+// dword), so the lane that meets the row's end, and the lanes past it, run the same two or three
+// instructions as every other lane instead of an element-by-element branch.
+struct ScanRow {
+  __amdgpu_buffer_rsrc_t rewards, values, adv, ret;
+};
+template <bool GAE>
+__device__ __forceinline__ ScanRow scan_row(const RowWalk& rw, const float* values, const float* rewards, float* adv,
+                                            float* ret) {
+  // rows hold fewer than 2^30 tokens (host check on the row bound; a longer packed row is cut there)
+  const int bytes = (int)(uint32_t)((rw.len < (1ll << 30) - 1 ? rw.len : (1ll << 30) - 1) * 4);
+  ScanRow r;
+  r.rewards = __builtin_amdgcn_make_buffer_rsrc((void*)(rewards + rw.base), 0, bytes, 0x00020000);
+  r.ret = __builtin_amdgcn_make_buffer_rsrc((void*)(ret + rw.base), 0, bytes, 0x00020000);
+  r.values = __builtin_amdgcn_make_buffer_rsrc((void*)(GAE ? values + rw.base : rewards + rw.base), 0, bytes, 0x00020000);
+  r.adv = __builtin_amdgcn_make_buffer_rsrc((void*)(GAE ? adv + rw.base : ret + rw.base), 0, bytes, 0x00020000);
+  return r;
+}
+constexpr int kNonTemporal = 2;  // cache-policy bits of a buffer access: nt
+
+// Must be called by all lanes of the workgroup (it exchanges the following value across lanes).
+// n_total: tokens in the whole arrays (a mask load may read past the row, never past the array).
 template <int MASK_DT, bool GAE, bool REWARD, int ITEMS>
-__device__ __forceinline__ ScanTile<ITEMS> load_scan_tile(const RowWalk& rw, int64_t tile0, bool whole,
+__device__ __forceinline__ ScanTile<ITEMS> load_scan_tile(const RowWalk& rw, const ScanRow& row, int64_t tile0, int64_t n_total,
                                                    const float* __restrict__ values,
-                                                   const float* __restrict__ rewards,
                                                    const void* __restrict__ mask, RowReward& rr) {
   static_assert(ITEMS == 4 || ITEMS == 8, "a lane's tokens are one or two 16-byte loads");
   ScanTile<ITEMS> t;
   const int64_t p0 = tile0 + (int64_t)threadIdx.x * ITEMS;
+  const uint32_t off = (uint32_t)p0 * 4u;
   auto reward_of = [&](float raw, int64_t p) {
     if (!REWARD) return raw;
     const float tok = ((p == rr.eos) ? rr.seq : 0.0f) + rr.neg_coef * raw;
     rr.sum += (double)tok;
     return tok;
   };
-  if (whole || p0 + ITEMS <= rw.len) {  // this lane's four tokens lie in the row
 #pragma unroll
-    for (int q = 0; q < ITEMS / 4; ++q) {
-      float m[4];
-      // two groups per lane share their cache lines: cached loads then (non-temporal ones fetched
-      // 47 % more than the rewards and the mask hold)
+  for (int q = 0; q < ITEMS / 4; ++q) {
+    // two groups per lane share their cache lines: cached loads then (non-temporal ones fetched
+    // 47 % more than the rewards and the mask hold)
+    const f32x4 r4 = __builtin_bit_cast(
+        f32x4, __builtin_amdgcn_raw_buffer_load_b128(row.rewards, off + q * 16u, 0, ITEMS == 4 ? kNonTemporal : 0));
+    f32x4 v4 = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (GAE) v4 = __builtin_bit_cast(f32x4, __builtin_amdgcn_raw_buffer_load_b128(row.values, off + q * 16u, 0, 0));  // plain: the last lane re-reads across the wave's end
+    float m[4];
+    if (rw.base + p0 + q * 4 + 4 <= n_total) {  // past the row's end the mask of the next row is read; its tokens are zeros here
       load_mask4<MASK_DT, ITEMS == 4>(mask, rw.base + p0 + q * 4, m);
-      const f32x4 r4 = load_once<ITEMS == 4>((const f32x4e*)(rewards + rw.base + p0 + q * 4));
-      f32x4 v4 = {0.0f, 0.0f, 0.0f, 0.0f};
-      if (GAE) v4 = *(const f32x4e*)(values + rw.base + p0 + q * 4);  // plain: the last lane re-reads across the wave's end
+    } else {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        t.r[q * 4 + j] = m[j] * reward_of(r4[j], p0 + q * 4 + j);
-        t.v[q * 4 + j] = m[j] * v4[j];
-      }
+      for (int j = 0; j < 4; ++j) m[j] = (p0 + q * 4 + j < rw.len) ? load_mask<MASK_DT>(mask, rw.base + p0 + q * 4 + j) : 0.0f;
     }
-  } else {  // the lane that meets the row's end, and the lanes past it
 #pragma unroll
-    for (int j = 0; j < ITEMS; ++j) {
-      const int64_t p = p0 + j;
-      t.r[j] = 0.0f;
-      t.v[j] = 0.0f;
-      if (p < rw.len) {
-        const float m = load_mask<MASK_DT>(mask, rw.base + p);
-        t.r[j] = m * reward_of(rewards[rw.base + p], p);
-        if (GAE) t.v[j] = m * values[rw.base + p];
-      }
+    for (int j = 0; j < 4; ++j) {
+      const bool in_row = p0 + q * 4 + j < rw.len;
+      t.r[q * 4 + j] = in_row ? m[j] * reward_of(r4[j], p0 + q * 4 + j) : 0.0f;
+      t.v[q * 4 + j] = in_row ? m[j] * v4[j] : 0.0f;
     }
   }
   t.v[ITEMS] = 0.0f;
@@ -246,15 +260,14 @@ __device__ __forceinline__ ScanTile<ITEMS> load_scan_tile(const RowWalk& rw, int
 // Four consecutive outputs of a lane. GAE's two outputs leave with non-temporal stores (10 %
 // faster there; the single output of the returns is faster with plain stores).
 template <bool GAE>
-__device__ __forceinline__ void store_scan4(float* __restrict__ adv, float* __restrict__ ret, int64_t i0,
-                                            const float* a, const float* r) {
+__device__ __forceinline__ void store_scan4(const ScanRow& row, uint32_t off, const float* a, const float* r) {
   const f32x4 a4 = {a[0], a[1], a[2], a[3]};
   if (GAE) {
     const f32x4 r4 = {r[0], r[1], r[2], r[3]};
-    __builtin_nontemporal_store(a4, (f32x4e*)(adv + i0));
-    __builtin_nontemporal_store(r4, (f32x4e*)(ret + i0));
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, a4), row.adv, off, 0, kNonTemporal);
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, r4), row.ret, off, 0, kNonTemporal);
   } else {
-    *(f32x4e*)(ret + i0) = a4;
+    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, a4), row.ret, off, 0, 0);
   }
 }
 
@@ -291,6 +304,7 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
   for (int k = 1; k <= ITEMS; ++k) pw[k] = pw[k - 1] * coef;
 
   const int slot_b = slot_bits(rows.n_rows);
+  const int64_t n_total = rows.cu != nullptr ? rows.cu[rows.n_rows] : rows.n_rows * rows.n_cols;
   int buf = 0;
   // A caller that knows the row lengths hands the rows out longest first (rows.order): the last
   // workgroups to start then hold the shortest rows, instead of a long row's sequential walk
@@ -314,16 +328,14 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
     }
     const int64_t n_tiles = (rw.len + kScanTile - 1) / kScanTile;
     double tile_carry = 0.0;  // A at the first token of the previous (later) tile
-    auto whole = [&](int64_t tile) {
-      return (tile + 1) * kScanTile <= rw.len;
-    };
+    const ScanRow row = scan_row<GAE>(rw, values, rewards, adv, ret);
     ScanTile<ITEMS> cur =
-        load_scan_tile<MASK_DT, GAE, REWARD, ITEMS>(rw, (n_tiles - 1) * kScanTile, whole(n_tiles - 1), values, rewards, mask, rr);
+        load_scan_tile<MASK_DT, GAE, REWARD, ITEMS>(rw, row, (n_tiles - 1) * kScanTile, n_total, values, mask, rr);
     for (int64_t tile = n_tiles - 1; tile >= 0; --tile) {
       const int64_t tile0 = tile * kScanTile;
       ScanTile<ITEMS> nxt = cur;
       if (tile > 0)
-        nxt = load_scan_tile<MASK_DT, GAE, REWARD, ITEMS>(rw, tile0 - kScanTile, whole(tile - 1), values, rewards, mask, rr);
+        nxt = load_scan_tile<MASK_DT, GAE, REWARD, ITEMS>(rw, row, tile0 - kScanTile, n_total, values, mask, rr);
       // in-lane recurrence with zero carry-in
       double local[ITEMS];
       double run = 0.0;
@@ -370,23 +382,8 @@ __global__ __launch_bounds__(kBlock) void reverse_scan_kernel(Rows rows, const f
         out_a[j] = (float)a_t;
         out_r[j] = (float)(a_t + (double)cur.v[j]);
       }
-      if (whole(tile) || p0 + ITEMS <= rw.len) {
-        store_scan4<GAE>(adv, ret, rw.base + p0, out_a, out_r);
-        if (ITEMS == 8) store_scan4<GAE>(adv, ret, rw.base + p0 + 4, out_a + 4, out_r + 4);
-      } else {
-#pragma unroll
-        for (int j = 0; j < ITEMS; ++j) {
-          const int64_t p = p0 + j;
-          if (p < rw.len) {
-            if (GAE) {
-              adv[rw.base + p] = out_a[j];
-              ret[rw.base + p] = out_r[j];
-            } else {
-              ret[rw.base + p] = out_a[j];
-            }
-          }
-        }
-      }
+      store_scan4<GAE>(row, (uint32_t)p0 * 4u, out_a, out_r);
+      if (ITEMS == 8) store_scan4<GAE>(row, (uint32_t)p0 * 4u + 16u, out_a + 4, out_r + 4);
       cur = nxt;
     }
     if (REWARD && sr.reward_sum != nullptr) {  // uniform: reward_sum is a kernel argument
@@ -668,6 +665,7 @@ extern "C" int orlhf_gae_scan(const float* values, const float* rewards, const v
                               int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens, const int64_t* row_order,
                               float gamma, float lambd, float* advantages, float* returns, orlhf_stream_t stream) {
   if (int rc = check_rows("gae_scan", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(n_cols < (1ll << 30), "gae_scan: rows of %lld tokens (the limit is 2^30 - 1)", (long long)n_cols);
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(values && rewards && advantages && returns, "gae_scan: NULL pointer");
   const Rows rows{n_rows, n_cols, cu_seqlens, 0, row_order};
@@ -681,6 +679,7 @@ extern "C" int orlhf_discounted_returns(const float* rewards, const void* mask, 
                                         int64_t n_cols, const int64_t* cu_seqlens, const int64_t* row_order,
                                         float gamma, float* returns, orlhf_stream_t stream) {
   if (int rc = check_rows("discounted_returns", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(n_cols < (1ll << 30), "discounted_returns: rows of %lld tokens (the limit is 2^30 - 1)", (long long)n_cols);
   if (n_rows * n_cols == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(rewards && returns, "discounted_returns: NULL pointer");
   const Rows rows{n_rows, n_cols, cu_seqlens, 0, row_order};
@@ -696,6 +695,7 @@ extern "C" int orlhf_reward_scan(const float* r, float kl_coef, const float* kl,
                                  float clip_high, float gamma, float lambd, float* advantages, float* returns,
                                  float* reward_sum, orlhf_stream_t stream) {
   if (int rc = check_rows("reward_scan", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(n_cols < (1ll << 30), "reward_scan: rows of %lld tokens (the limit is 2^30 - 1)", (long long)n_cols);
   if (n_rows == 0) return ORLHF_OK;
   ORLHF_CHECK_ARG(r != nullptr && returns != nullptr && (kl != nullptr || n_cols == 0), "reward_scan: NULL pointer");
   ORLHF_CHECK_ARG((values == nullptr) == (advantages == nullptr),
