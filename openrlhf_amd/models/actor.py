@@ -9,7 +9,8 @@ Differences by construction: bf16 logits are consumed directly (no [N, V] fp32 c
 and entropy come from ONE pass over the logits, and with ``skip_masked=True`` (default) positions
 whose log-prob the reference multiplies by zero are not read at all, forward or backward; their
 entropy is returned as 0 (the trainer only ever aggregates entropy under the same mask,
-openrlhf/trainer/ray/ppo_actor.py:345-350).
+openrlhf/trainer/ray/ppo_actor.py:345-350). ``actor_forward_tail_from_hidden`` starts one step
+earlier, at the decoder's last hidden states, and never stores the logits.
 """
 from typing import Optional, Tuple, Union
 
@@ -80,6 +81,51 @@ def actor_forward_tail(
         lp = repad(lp_p)
         ent = None if ent_p is None else repad(ent_p)
 
+    lp = lp[:, :-1]
+    if action_mask is not None:
+        lp = lp[:, -action_mask.shape[1] :] * action_mask.float()
+    if return_entropy:
+        return lp, ent[:, :-1]
+    return lp
+
+
+def actor_forward_tail_from_hidden(
+    hidden_states: torch.Tensor,
+    lm_head_weight: torch.Tensor,
+    sequences: torch.Tensor,
+    action_mask: Optional[torch.Tensor] = None,
+    attention_mask: Optional[torch.Tensor] = None,
+    temperature: float = 1.0,
+    packed_indices: Optional[torch.Tensor] = None,
+    return_entropy: bool = False,
+) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
+    """The same tail with the lm-head projection in front and the logits never stored: what
+    openrlhf/models/actor.py:263-296 computes from ``self.model(...)["logits"]``, from the decoder's
+    last hidden states ``[B, T, H]`` (or ``[1, Ttot, H]`` / ``[Ttot, H]`` with ``packed_indices``)
+    and ``lm_head.weight [V, H]`` (bf16 or fp16). Positions whose log-prob the reference multiplies
+    by zero are left out of the projection altogether; gradients reach the hidden states and the
+    weight. Same outputs and shapes as ``actor_forward_tail``."""
+    from .utils import lm_head_logprobs_and_entropy
+
+    batch, seqlen = sequences.shape
+    rolled = torch.roll(sequences, shifts=-1, dims=1)
+    need = torch.zeros(batch, seqlen, dtype=torch.bool, device=sequences.device)
+    if action_mask is not None:
+        width = action_mask.shape[1]
+        need[:, seqlen - 1 - width : seqlen - 1] = action_mask != 0
+    else:
+        need[:, : seqlen - 1] = True if attention_mask is None else attention_mask[:, : seqlen - 1] != 0
+    if packed_indices is None:
+        lp, ent = lm_head_logprobs_and_entropy(hidden_states, lm_head_weight, rolled, temperature, row_mask=need)
+    else:
+        flat = hidden_states.reshape(-1, hidden_states.shape[-1])
+        lp_p, ent_p = lm_head_logprobs_and_entropy(flat, lm_head_weight, rolled.reshape(-1)[packed_indices], temperature,
+                                                   row_mask=need.reshape(-1)[packed_indices])
+
+        def repad(x):
+            return x.new_zeros(batch * seqlen).index_copy(0, packed_indices, x).view(batch, seqlen)
+
+        lp, ent = repad(lp_p), repad(ent_p)
     lp = lp[:, :-1]
     if action_mask is not None:
         lp = lp[:, -action_mask.shape[1] :] * action_mask.float()

@@ -109,3 +109,54 @@ def test_return_all_logprobs_for_sft(cuda):
     assert out.shape == ref.shape
     assert (out.cpu().double() - ref)[keep].abs().max().item() <= 1e-5
     assert out.cpu()[~keep].abs().max().item() == 0.0
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_tail_from_hidden_states(cuda, packed):
+    """The same tail from the decoder's last hidden states and lm_head.weight, logits never stored:
+    against the oracle on ``hidden @ W.T`` in fp64 (2e-3 abs for bf16 operands; gradients of the
+    hidden states and of the weight within the rounding of a bf16 logits gradient and result)."""
+    from openrlhf_amd.models.actor import actor_forward_tail_from_hidden, unpad_indices
+
+    b, t, a, hdim, vocab, temperature = 4, 36, 15, 96, 1234, 0.8
+    _, seqs, attn, amask = _batch(7, b=b, t=t, vocab=vocab, a=a)
+    g = torch.Generator().manual_seed(8)
+    hidden = torch.randn(b, t, hdim, generator=g).to(torch.bfloat16)
+    weight = (torch.randn(vocab, hdim, generator=g) * 0.3).to(torch.bfloat16)
+    flat_keep = attn.reshape(-1).bool()
+
+    h64 = hidden.double().requires_grad_(True)
+    w64 = weight.double().requires_grad_(True)
+    logits64 = h64 @ w64.T
+    ref_in = logits64.reshape(-1, vocab)[flat_keep].unsqueeze(0) if packed else logits64
+    ref_lp, ref_ent = _oracle_tail64(ref_in, seqs, attn, amask, temperature, packed)
+    w_lp = torch.randn(ref_lp.shape, generator=g)
+    w_ent = torch.randn(ref_ent.shape, generator=g)
+    ent_mask = torch.zeros_like(ref_ent)
+    ent_mask[:, -a:] = amask.double()
+    ((ref_lp * w_lp.double()).sum() + (ref_ent * w_ent.double() * ent_mask).sum()).backward()
+
+    hd = hidden.to(cuda)
+    if packed:
+        hd = hd.reshape(-1, hdim)[flat_keep.to(cuda)].unsqueeze(0).contiguous()
+    hd.requires_grad_(True)
+    wd = weight.to(cuda).requires_grad_(True)
+    lp, ent = actor_forward_tail_from_hidden(
+        hd, wd, seqs.to(cuda), amask.to(cuda), attn.to(cuda), temperature=temperature,
+        packed_indices=unpad_indices(attn.to(cuda)) if packed else None, return_entropy=True)
+    assert lp.shape == ref_lp.shape and ent.shape == ref_ent.shape
+    assert (lp.cpu().double() - ref_lp.detach()).abs().max().item() <= 2e-3
+    assert (ent.cpu().double() - ref_ent.detach())[ent_mask.bool()].abs().max().item() <= 2e-3
+    assert ent.cpu()[~ent_mask.bool()].abs().max().item() == 0.0
+    ((lp * w_lp.to(cuda)).sum() + (ent * w_ent.to(cuda) * ent_mask.float().to(cuda)).sum()).backward()
+    ref_gh = h64.grad.reshape(-1, hdim)[flat_keep].unsqueeze(0) if packed else h64.grad
+    for got, ref in ((hd.grad, ref_gh), (wd.grad, w64.grad)):
+        err = (got.cpu().double() - ref).abs()
+        scale = ref.abs().max().item()
+        assert err.max().item() <= 4 * 2.0 ** -8 * scale + 1e-9, (err.max().item(), scale)
+        assert (err.pow(2).sum() / ref.pow(2).sum()).sqrt().item() <= 2 * 2.0 ** -8
+    # positions outside the action mask are left out of the projection: no gradient reaches them
+    need = torch.zeros(b, t, dtype=torch.bool)
+    need[:, t - 1 - a : t - 1] = amask
+    dead = ~need.reshape(-1)[flat_keep] if packed else ~need.reshape(-1)
+    assert hd.grad.reshape(-1, hdim)[dead.to(cuda)].abs().max().item() == 0.0
