@@ -22,7 +22,7 @@ import torch
 
 from ... import _lib
 from ..._lib import call, ptr, require_gpu, stream_of
-from ...models.actor import actor_forward_tail
+from ...models.actor import actor_forward_tail, actor_forward_tail_from_hidden
 from ...models.loss import PolicyLoss, aggregate_loss
 from ...models.utils import _KL_CODES, _as_rows, _workspace, compute_approx_kl, masked_mean
 
@@ -31,14 +31,22 @@ def actor_loss_step(
     logits, sequences, attention_mask, action_mask, old_action_log_probs, advantages, policy_loss_fn: PolicyLoss,
     base_action_log_probs=None, kl_estimator="k1", kl_coef=0.0, entropy_coef=None, rollout_log_probs=None,
     temperature=1.0, packed_indices=None, dp_size=1, batch_num_tokens=None, global_batch_size=None,
-    inplace_backward=False,
+    inplace_backward=False, lm_head_weight=None,
 ):
-    """Reference-order composition (ppo_actor.py:294-352) on the separate kernels; differentiable."""
+    """Reference-order composition (ppo_actor.py:294-352) on the separate kernels; differentiable.
+    With ``lm_head_weight [V, H]`` the first argument holds the decoder's last hidden states instead
+    of logits and the projection is fused into the log-prob / entropy (the logits are never stored;
+    gradients reach the hidden states and the weight)."""
     info = dict(dp_size=dp_size, batch_num_tokens=batch_num_tokens, global_batch_size=global_batch_size)
     want_entropy = entropy_coef is not None
-    out = actor_forward_tail(logits, sequences, action_mask, attention_mask, temperature=temperature,
-                             packed_indices=packed_indices, return_entropy=want_entropy,
-                             inplace_backward=inplace_backward)
+    if lm_head_weight is not None:
+        out = actor_forward_tail_from_hidden(logits, lm_head_weight, sequences, action_mask, attention_mask,
+                                             temperature=temperature, packed_indices=packed_indices,
+                                             return_entropy=want_entropy)
+    else:
+        out = actor_forward_tail(logits, sequences, action_mask, attention_mask, temperature=temperature,
+                                 packed_indices=packed_indices, return_entropy=want_entropy,
+                                 inplace_backward=inplace_backward)
     action_log_probs, entropy = out if want_entropy else (out, None)
     actor_loss, clip_ratio, ppo_kl, vllm_kl = policy_loss_fn(
         action_log_probs, old_action_log_probs, advantages, action_mask=action_mask,

@@ -181,3 +181,50 @@ def test_fused_step_on_a_vocabulary_longer_than_the_registers(cuda):
         assert abs(out[key].item() - ref[key].item()) <= 2e-5 * max(1.0, abs(ref[key].item())), key
     ga, gb = xa.grad.float(), xb.grad.float()
     assert (ga - gb).abs().max().item() <= 2.0 ** -7 * ga.abs().max().item()
+
+
+@pytest.mark.parametrize("case", [CASES[1], CASES[2]])
+@pytest.mark.parametrize("packed", [False, True])
+def test_actor_step_from_hidden_states(cuda, case, packed):
+    """The composed step with the lm-head projection fused in (hidden states and lm_head.weight in
+    place of logits): the oracle's step on ``hidden @ W.T`` in fp64; values within 2e-3, gradients
+    of the hidden states and the weight within the rounding of a bf16 logits gradient."""
+    from openrlhf_amd.models.actor import unpad_indices
+    from openrlhf_amd.models.loss import PolicyLoss
+    from openrlhf_amd.trainer.ray.ppo_actor import actor_loss_step
+
+    b, t, a, hdim, vocab = 6, 48, 20, 128, 1500
+    _, seqs, attn, amask, old, adv, base, roll = _batch(13, b=b, t=t, vocab=vocab, a=a)
+    g = torch.Generator().manual_seed(14)
+    hidden = torch.randn(b, t, hdim, generator=g).to(torch.bfloat16)
+    weight = (torch.randn(vocab, hdim, generator=g) * 0.25).to(torch.bfloat16)
+    kl_est, kl_coef = case["kl"]
+    keep = attn.reshape(-1).bool()
+
+    h64 = hidden.double().requires_grad_(True)
+    w64 = weight.double().requires_grad_(True)
+    logits64 = h64 @ w64.T
+    ref_in = logits64.reshape(-1, vocab)[keep].unsqueeze(0) if packed else logits64
+    ref = _oracle_step(ref_in, seqs, attn, amask, old, adv, base, roll, 1.0, packed, case["pol"], kl_est, kl_coef,
+                       case["ent"], case["info"])
+    ref["loss"].backward()
+
+    d = cuda
+    hd = hidden.to(d)
+    if packed:
+        hd = hd.reshape(-1, hdim)[keep.to(d)].contiguous()
+    hd.requires_grad_(True)
+    wd = weight.to(d).requires_grad_(True)
+    out = actor_loss_step(hd, seqs.to(d), attn.to(d), amask.to(d), old.to(d), adv.to(d), PolicyLoss(**case["pol"]),
+                          base_action_log_probs=base.to(d), kl_estimator=kl_est, kl_coef=kl_coef, entropy_coef=case["ent"],
+                          rollout_log_probs=roll.to(d), temperature=1.0,
+                          packed_indices=unpad_indices(attn.to(d)) if packed else None, lm_head_weight=wd, **case["info"])
+    out["loss"].backward()
+    for key in ("loss", "actor_loss", "clip_ratio", "ppo_kl", "kl_loss", "entropy_loss", "logprobs_diff"):
+        want = ref[key].item()
+        assert abs(out[key].item() - want) <= 2e-3 * max(1.0, abs(want)), (key, out[key].item(), want)
+    ref_gh = h64.grad.reshape(-1, hdim)[keep] if packed else h64.grad
+    for got, want in ((hd.grad, ref_gh), (wd.grad, w64.grad)):
+        err = (got.cpu().double() - want).abs()
+        scale = want.abs().max().item()
+        assert err.max().item() <= 6 * 2.0 ** -8 * scale + 1e-9, (err.max().item(), scale)
