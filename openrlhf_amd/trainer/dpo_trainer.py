@@ -11,7 +11,7 @@ import torch
 
 from .. import _lib
 from .._lib import call, ptr, require_gpu, stream_of
-from ..models.actor import actor_forward_tail
+from ..models.actor import actor_forward_tail, actor_forward_tail_from_hidden
 from ..models.loss import DPOLoss
 from ..models.utils import _f32
 
@@ -95,26 +95,31 @@ def concatenated_inputs(chosen_ids, c_mask, reject_ids, r_mask, prompt_id_lens, 
 
 
 def concatenated_logps(logits, input_ids, att_masks, prompt_id_lens, n_chosen: int, temperature: float = 1.0,
-                       inplace_backward: bool = False):
+                       inplace_backward: bool = False, lm_head_weight=None):
     """What ``concatenated_forward`` returns after the model call (dpo_trainer.py:314-326):
     ``(chosen_logps, rejected_logps, nll_loss)`` from the logits of the stacked batch, where
     ``nll_loss = -mean(per-sequence mean log-prob of the chosen half)``. Only response positions
-    are read from the logits."""
+    are read from the logits. With ``lm_head_weight [V, H]`` the first argument holds the decoder's
+    last hidden states and the projection is fused in (logits never stored)."""
     need = response_mask(att_masks, prompt_id_lens)
-    lp = actor_forward_tail(logits, input_ids, action_mask=need, temperature=temperature,
-                            inplace_backward=inplace_backward)
+    if lm_head_weight is not None:
+        lp = actor_forward_tail_from_hidden(logits, lm_head_weight, input_ids, action_mask=need, temperature=temperature)
+    else:
+        lp = actor_forward_tail(logits, input_ids, action_mask=need, temperature=temperature,
+                                inplace_backward=inplace_backward)
     sums, means = get_batch_logps(lp, att_masks, prompt_id_lens)
     return sums[:n_chosen], sums[n_chosen:], -means[:n_chosen].mean()
 
 
 def dpo_loss_step(logits, input_ids, att_masks, prompt_id_lens, n_chosen: int, reference_chosen_logps,
                   reference_rejected_logps, loss_fn: DPOLoss, nll_loss_coef: float = 0.0,
-                  temperature: float = 1.0, inplace_backward: bool = False):
+                  temperature: float = 1.0, inplace_backward: bool = False, lm_head_weight=None):
     """Policy half of the DPO step (dpo_trainer.py:157-180) from the stacked batch's logits:
     returns a dict with ``loss = preference_loss + nll_loss * nll_loss_coef`` (the Mixtral
     auxiliary loss is the caller's), the preference loss, both reward estimates and the NLL."""
     chosen, rejected, nll = concatenated_logps(logits, input_ids, att_masks, prompt_id_lens, n_chosen,
-                                               temperature=temperature, inplace_backward=inplace_backward)
+                                               temperature=temperature, inplace_backward=inplace_backward,
+                                               lm_head_weight=lm_head_weight)
     preference_loss, chosen_reward, reject_reward = loss_fn(chosen, rejected, reference_chosen_logps,
                                                             reference_rejected_logps)
     loss = preference_loss + nll * nll_loss_coef if nll_loss_coef else preference_loss

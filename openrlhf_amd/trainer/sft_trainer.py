@@ -13,7 +13,7 @@ in either mode.
 """
 import torch
 
-from ..models.actor import actor_forward_tail
+from ..models.actor import actor_forward_tail, actor_forward_tail_from_hidden
 from ..models.loss import SFTLoss
 from ..models.utils import fused_logprob_entropy_fwd_bwd
 from .ray.ppo_actor import _HandOverGradient, _row_coef
@@ -21,15 +21,20 @@ from .ray.ppo_actor import _HandOverGradient, _row_coef
 
 def sft_loss_step(logits, inputs, attention_mask, loss_mask, loss_fn: SFTLoss = None, fused: bool = False,
                   dp_size=1, batch_num_tokens=None, global_batch_size=None, loss_scale: float = 1.0,
-                  inplace_backward: bool = False):
+                  inplace_backward: bool = False, lm_head_weight=None):
     """logits ``[B, T, V]``, inputs / attention_mask / loss_mask ``[B, T]``. Returns
     ``(gpt_loss, per_token_log_probs [B, T-1])``. With ``fused=True`` the logits are consumed (their
     storage holds ``loss_scale * d(gpt_loss)/d(logits)``) and ``(gpt_loss * loss_scale).backward()``
-    hands that gradient to the layer that produced them."""
+    hands that gradient to the layer that produced them. With ``lm_head_weight [V, H]`` the first
+    argument holds the decoder's last hidden states ``[B, T, H]`` and the projection is fused into
+    the log-probs (logits never stored; ``fused`` does not apply)."""
     loss_fn = loss_fn if loss_fn is not None else SFTLoss()
     info = dict(dp_size=dp_size, batch_num_tokens=batch_num_tokens, global_batch_size=global_batch_size)
     shifted = loss_mask[:, :-1]
     batch, seqlen = inputs.shape
+    if lm_head_weight is not None:
+        lp = actor_forward_tail_from_hidden(logits, lm_head_weight, inputs, action_mask=(shifted != 0), temperature=1.0)
+        return loss_fn(lp, shifted, **info), lp
     if not fused:
         # log-probs are needed where the loss mask is set; the attention mask only marks padding
         lp = actor_forward_tail(logits, inputs, action_mask=(shifted != 0), temperature=1.0,

@@ -308,3 +308,58 @@ def test_gpt_lm_loss_vs_torch_cross_entropy(cuda, dtype):
     assert torch.isnan(GPTLMLoss()(logits.to(cuda), everything_ignored.to(cuda)))
     with pytest.raises(NotImplementedError):
         GPTLMLoss(ring_attn_group=object())
+
+
+def test_sft_and_dpo_steps_from_hidden_states(cuda):
+    """Both steps with the lm-head projection fused in (hidden states and lm_head.weight in place of
+    logits): the oracle on ``hidden @ W.T`` in fp64, values within 2e-3 (sums of up to 40 log-probs:
+    40 x that), gradients within the rounding of a bf16 logits gradient and result."""
+    from openrlhf_amd.models.loss import DPOLoss, SFTLoss
+    from openrlhf_amd.trainer.dpo_trainer import concatenated_inputs, dpo_loss_step
+    from openrlhf_amd.trainer.sft_trainer import sft_loss_step
+
+    hdim, vocab = 96, 1201
+    c_ids, c_mask, r_ids, r_mask, prompt, g = _dpo_batch(6)
+    ids, att, lens = concatenated_inputs(c_ids, c_mask, r_ids, r_mask, prompt, pad_token_id=0)
+    ids = ids % vocab
+    hidden = torch.randn(6, 40, hdim, generator=g).to(torch.bfloat16)
+    weight = (torch.randn(vocab, hdim, generator=g) * 0.25).to(torch.bfloat16)
+    ref_c, ref_r, beta = -torch.rand(3, generator=g) * 60, -torch.rand(3, generator=g) * 60, 0.1
+
+    def grads_close(got, want):
+        err = (got.cpu().double() - want).abs()
+        assert err.max().item() <= 6 * 2.0 ** -8 * want.abs().max().item() + 1e-9, (err.max().item(), want.abs().max().item())
+
+    # DPO
+    h64, w64 = hidden.double().requires_grad_(True), weight.double().requires_grad_(True)
+    lp = otn.log_probs_from_logits(h64 @ w64.T, torch.roll(ids, -1, 1), 1.0)[:, :-1]
+    sums, means = ol.get_batch_logps(lp, att, lens)
+    ref_pref, _, _ = ol.dpo_loss(sums[:3], sums[3:], ref_c.double(), ref_r.double(), beta)
+    ref_loss = ref_pref + (-means[:3].mean()) * 0.3
+    ref_loss.backward()
+    hd, wd = hidden.to(cuda).requires_grad_(True), weight.to(cuda).requires_grad_(True)
+    out = dpo_loss_step(hd, ids.to(cuda), att.to(cuda), lens, 3, ref_c.to(cuda), ref_r.to(cuda), DPOLoss(beta),
+                        nll_loss_coef=0.3, lm_head_weight=wd)
+    _close(out["chosen_logps"], sums[:3].detach(), 2e-3 * 40)
+    _close(out["rejected_logps"], sums[3:].detach(), 2e-3 * 40)
+    _close(out["loss"], ref_loss.detach(), 2e-2)
+    out["loss"].backward()
+    grads_close(hd.grad, h64.grad)
+    grads_close(wd.grad, w64.grad)
+
+    # SFT
+    loss_mask = att.clone()
+    loss_mask[:, :5] = 0
+    loss_mask[4] = 0
+    shifted = loss_mask[:, :-1]
+    h64, w64 = hidden.double().requires_grad_(True), weight.double().requires_grad_(True)
+    lp_ref = otn.log_probs_from_logits(h64 @ w64.T, torch.roll(ids, -1, 1), 1.0)[:, :-1]
+    ref_loss = ol.aggregate_loss(-lp_ref, shifted.double(), token_level_loss=True)
+    ref_loss.backward()
+    hd, wd = hidden.to(cuda).requires_grad_(True), weight.to(cuda).requires_grad_(True)
+    loss, lp_d = sft_loss_step(hd, ids.to(cuda), att.to(cuda), loss_mask.to(cuda), SFTLoss(True), lm_head_weight=wd)
+    _close(loss, ref_loss.detach(), 2e-3 * max(1.0, abs(ref_loss.item())))
+    _close(lp_d, (lp_ref * shifted).detach(), 2e-3)
+    loss.backward()
+    grads_close(hd.grad, h64.grad)
+    grads_close(wd.grad, w64.grad)
