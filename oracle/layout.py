@@ -30,3 +30,18 @@ def unpad_boundaries(attention_mask):
     (openrlhf/models/ring_attn_utils.py:129-140): cumulative count of attended tokens per row."""
     lens = attention_mask.long().sum(dim=-1)
     return torch.cat([torch.zeros(1, dtype=torch.long), lens.cumsum(0)])
+
+
+def unpad_and_rebatch(field, attention_mask):
+    """One per-step field of a batch after the reference's hops split_experience_batch ->
+    remove_padding_in_sequences -> make_experience_batch
+    (openrlhf/trainer/ppo_utils/experience.py:164-247): every row loses as many trailing columns
+    as its attention-mask row has trailing zeros (none if the mask row is all zeros or ends in a
+    one: ``right_pad == 0 -> None``), then the rows are right-padded with 0 to the longest and
+    stacked. Returns (batch, kept lengths)."""
+    rows, kept = [], []
+    for value, mask_row in zip(field, attention_mask):
+        right_pad = int(mask_row.flip(0).argmax())
+        rows.append(value[: -right_pad] if right_pad else value)
+        kept.append(rows[-1].numel())
+    return zero_pad_sequences(rows, "right", 0, stack=True), kept

@@ -181,6 +181,12 @@ def test_packed_experience_equals_the_reference_hops(cuda):
     keep = [olay.unpadded_length(exp.attention_mask[r].cpu()) for r in range(9)]
     assert pe.cu[41].tolist() == [0] + torch.tensor(keep).cumsum(0).tolist()
     got = pe.to_experience()
+    # straight against the layout oracle's restatement of the three hops
+    for name in ("sequences", "attention_mask", "action_mask", "action_log_probs", "base_action_log_probs", "values", "kl"):
+        ref, kept = olay.unpad_and_rebatch(getattr(exp, name).cpu(), exp.attention_mask.cpu())
+        assert torch.equal(getattr(got, name).cpu(), ref), name
+        w_ = getattr(exp, name).shape[1]
+        assert (pe.cu[w_][1:] - pe.cu[w_][:-1]).tolist() == kept, name
     for name in STEP_FIELDS:
         w, g_ = getattr(want, name), getattr(got, name)
         assert (w is None) == (g_ is None), name

@@ -381,3 +381,22 @@ def test_masked_normalize_kl_rows_and_token_sum_golden():
     close(ol.aggregate_seq_token_sum(adv, mask, dp_size=2, global_batch_size=5.0), agg["seq_token_sum_global"], 1e-12)
     # every sequence of the same length L: token-sum mode = L * the reference's seq-mean mode
     close(ol.aggregate_seq_token_sum(adv, full), 16 * ol.aggregate_loss(adv, full, token_level_loss=False), 1e-9)
+
+
+def test_layout_unpad_and_rebatch_known_answer():
+    """The three hops on a literal batch (openrlhf/trainer/ppo_utils/experience.py:164-247): trailing
+    zeros of the attention mask go, an all-zero mask row and a row ending in a one keep everything,
+    the A = T - 1 wide field loses the same number of columns, rows are right-padded with zeros."""
+    import torch
+
+    from oracle import layout as olay
+
+    att = torch.tensor([[1, 1, 1, 0, 0], [0, 0, 0, 0, 0], [1, 1, 0, 1, 1], [1, 0, 0, 0, 0]])
+    seq = torch.arange(20).view(4, 5) + 1
+    out, kept = olay.unpad_and_rebatch(seq, att)
+    assert kept == [3, 5, 5, 1]
+    assert out.tolist() == [[1, 2, 3, 0, 0], [6, 7, 8, 9, 10], [11, 12, 13, 14, 15], [16, 0, 0, 0, 0]]
+    act = torch.arange(16).view(4, 4) + 1.0
+    out, kept = olay.unpad_and_rebatch(act, att)
+    assert kept == [2, 4, 4, 0]
+    assert out.tolist() == [[1, 2, 0, 0], [5, 6, 7, 8], [9, 10, 11, 12], [0, 0, 0, 0]]
