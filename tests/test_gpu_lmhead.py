@@ -162,3 +162,19 @@ def test_lmhead_full_size(cuda):
     ref_ent = otn.compute_entropy(x64.double())
     assert (lp[pick.to(cuda)].detach().cpu().double() - ref_lp).abs().max().item() <= 2e-3
     assert (ent[pick.to(cuda)].detach().cpu().double() - ref_ent).abs().max().item() <= 2e-3
+
+
+def test_lmhead_every_row_masked(cuda):
+    """A row mask that leaves nothing: zeros out, zero gradients, nothing launched on an empty batch."""
+    from openrlhf_amd.models.utils import lm_head_logprobs_and_entropy
+
+    h = torch.randn(5, 64, device=cuda).bfloat16().requires_grad_(True)
+    w = torch.randn(100, 64, device=cuda).bfloat16().requires_grad_(True)
+    labels = torch.randint(0, 100, (5,), device=cuda)
+    lp, ent = lm_head_logprobs_and_entropy(h, w, labels, 1.0, row_mask=torch.zeros(5, dtype=torch.bool, device=cuda))
+    assert lp.shape == (5,) and lp.abs().max().item() == 0.0 and ent.abs().max().item() == 0.0
+    (lp.sum() + ent.sum()).backward()
+    assert h.grad.abs().max().item() == 0.0 and w.grad.abs().max().item() == 0.0
+    # and an empty batch
+    lp0, ent0 = lm_head_logprobs_and_entropy(h[:0], w, labels[:0], 1.0)
+    assert lp0.shape == (0,) and ent0.shape == (0,)
