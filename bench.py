@@ -343,6 +343,50 @@ def bench_few_rows(dev, n=64, vocab=VOCAB, copies=32):
     }
 
 
+def bench_matrix_tile(dev, m=8192, n=8192, k=8192, reps=10):
+    """--workload matrix_tile: the matrix-core tile of the lm-head path as a plain bf16 product
+    (orlhf_matrix_tile_probe), with its slab loads and with the operands resident in LDS (the same
+    LDS reads, MFMAs and barriers, nothing loaded: what the tile is bounded by on this GPU and
+    clock), on random operands and on operands whose rows are all equal (less switching in the
+    multipliers, higher clock), beside torch.matmul (hipBLASLt) on the same shapes."""
+    from openrlhf_amd import _lib
+    from openrlhf_amd._lib import call, ptr, stream_of
+
+    tiles = ((m + 255) // 256) * ((n + 255) // 256)
+    sums = torch.empty(tiles * 256, device=dev, dtype=torch.float32)
+    st = stream_of(dev)
+    flops = 2.0 * m * n * k
+
+    def timed(fn):
+        fn(); fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+
+    out = {}
+    for name, make in (("random", lambda r, c: torch.randn(r, c, device=dev)),
+                       ("equal_rows", lambda r, c: torch.randn(1, c, device=dev).expand(r, c).contiguous())):
+        a, b = make(m, k).to(torch.bfloat16), make(n, k).to(torch.bfloat16)
+        entry = {}
+        for label, resident in (("tile", 0), ("tile_operands_resident", 1)):
+            ms = timed(lambda: call("orlhf_matrix_tile_probe", ptr(a), ptr(b), _lib.BF16, m, n, k, k, k, resident, ptr(sums), st))
+            entry[label] = {"ms": ms, "tflops": flops / ms / 1e9}
+        call("orlhf_matrix_tile_probe", ptr(a), ptr(b), _lib.BF16, m, n, k, k, k, 0, ptr(sums), st)
+        got = sums.view(-1, 256).sum(1)[:4].double()
+        want = torch.stack([(a[:256].double().sum(0) * b[j * 256:(j + 1) * 256].double().sum(0)).sum() for j in range(4)])
+        entry["checked"] = bool(((got - want).abs() <= 1e-3 * want.abs().clamp_min(1e3)).all())
+        ms = timed(lambda: torch.matmul(a, b.t()))
+        entry["torch_matmul"] = {"ms": ms, "tflops": flops / ms / 1e9}
+        out[name] = entry
+    return {"workload": f"plain bf16 product [{m}, {k}] x [{n}, {k}]^T through the lm-head path's matrix-core tile", "n_gpus": 1,
+            "peak_tflops": MFMA_PEAK_TFLOPS, "entries": out}
+
+
 def bench_kernels(args, dev):
     """--workload kernels: the three vocabulary-row kernels launched back to back on ONE resident
     buffer of --rows x 151936 bf16 logits (forward, in-place backward, one-pass forward+backward,
@@ -688,7 +732,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--ring", type=int, default=6, help="distinct logits buffers per timed segment")
     ap.add_argument("--cpu-rows", type=int, default=4096, help="rows of the CPU-baseline sample")
-    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token", "kernels", "torch_eager", "ceilings", "lmhead", "few_rows"],
+    ap.add_argument("--workload", default="logprob", choices=["logprob", "per_token", "kernels", "torch_eager", "ceilings", "lmhead", "few_rows", "matrix_tile"],
                     help="logprob: the headline step (default); per_token: the small kernels of configs 3/4; "
                          "torch_eager: the reference's eager torch op sequence on this GPU beside the HIP path; "
                          "ceilings: plain read / read+write / copy / fill streams on the headline buffers; "
@@ -725,6 +769,9 @@ def main():
     if args.workload == "lmhead":
         print(json.dumps({"workload": "lm-head + log-prob + entropy, logits never stored", "n_gpus": 1,
                           **bench_lmhead(dev, n=args.rows if args.rows != 8192 else 4096)}), flush=True)
+        return
+    if args.workload == "matrix_tile":
+        print(json.dumps(bench_matrix_tile(dev)), flush=True)
         return
     if args.workload == "few_rows":
         print(json.dumps({"n_gpus": 1, **bench_few_rows(dev, n=args.rows if args.rows != 8192 else 64)}), flush=True)

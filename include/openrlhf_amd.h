@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 19
+#define ORLHF_ABI_VERSION 20
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -210,6 +210,22 @@ int orlhf_lmhead_logprob_entropy_bwd(const void* hidden, const void* weight, int
                                      int64_t grad_hidden_stride, void* grad_weight,
                                      int64_t grad_weight_stride, void* workspace,
                                      int64_t workspace_bytes, orlhf_stream_t stream);
+
+/*
+ * Measurement aid, no counterpart in the reference: the plain product of two K-major operands,
+ * a [m, k] (row stride lda) and b [n, k] (row stride ldb), bf16 or fp16, through the matrix-core
+ * tile the lm-head entry points above are built on, one 256 x 256 tile per workgroup. Nothing but
+ * the product is done: thread t of tile (i, j) leaves the sum of its 256 accumulators in
+ * tile_sums[(i * ceil(n / 256) + j) * 256 + t] (float, ceil(m / 256) * ceil(n / 256) * 256
+ * entries), so the 256 sums of a tile add up to the sum of that block of a * b^T. With
+ * resident_operands != 0 the steady loop loads nothing (every slab is multiplied out of what the
+ * LDS buffers hold after the first two slabs; the sums are meaningless): the time of that run is
+ * what the same LDS reads, MFMAs and barriers take on their own, the ceiling the tile can be read
+ * against on a given GPU and clock. Operands need 4-byte aligned bases and even row strides.
+ */
+int orlhf_matrix_tile_probe(const void* a, const void* b, int dtype, int64_t m, int64_t n, int64_t k,
+                            int64_t lda, int64_t ldb, int resident_operands, float* tile_sums,
+                            orlhf_stream_t stream);
 
 /*
  * The loss assembly of the PPO actor step (openrlhf/trainer/ray/ppo_actor.py:305-352) folded into

@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 
 class Norm(Structure):
@@ -81,6 +81,7 @@ SIGNATURES = {
     "orlhf_lmhead_logprob_entropy_fwd": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, P, c_double, P, P, P, P, I64, P]),
     "orlhf_lmhead_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, P, c_double, P, P, P, P, I64, P,
                                                  I64, P, I64, P]),
+    "orlhf_matrix_tile_probe": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, c_int, P, P]),
     "orlhf_policy_step_fwd_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, POINTER(StepTerms), P, P, P, P]),
     "orlhf_actor_step_gather": (c_int, [P, P, c_int, P, I64, I64, I64, I64, P, P, P, P, P, P, c_float, P, P, P, P, P, P, P, P,
                                         P, P]),

@@ -359,6 +359,33 @@ __global__ __launch_bounds__(kBlock) void lmhead_round_kernel(const float* __res
   }
 }
 
+// Measurement: the plain product A * B^T of two K-major operands through the tile core, one tile per
+// workgroup in the same order as the kernels above; every thread leaves the sum of its 256
+// accumulators (tile_sums[tile * 256 + thread]), so nothing but the product is timed and the
+// result can still be checked (a tile's sums add up to the sum of its block of A * B^T).
+template <int DT, bool RESIDENT_OPERANDS>
+__global__ __launch_bounds__(mm::kThreads, 1) void matrix_tile_probe_kernel(Operand a, Operand b, float* __restrict__ tile_sums,
+                                                                            int64_t tiles_m, int64_t tiles_n) {
+  extern __shared__ __align__(16) char lds[];
+  const int64_t n_items = tiles_m * tiles_n;
+  const int64_t item = mm::xcd_contiguous(blockIdx.x, n_items);
+  if (item >= n_items) return;
+  int64_t tm, tn;
+  mm::grouped_tile(item, tiles_m, tiles_n, tm, tn);
+  f32x16 acc[4][4];
+  mm::tile_product<DT, false, false, RESIDENT_OPERANDS>(acc, a, b, tm * 256, tn * 256, lds);
+  float sum = 0.0f;
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sum += acc[mt][nt][r];
+    }
+  }
+  tile_sums[(tm * tiles_n + tn) * mm::kThreads + threadIdx.x] = sum;
+}
+
 // dst[c][r] = src[r][c] for 16-bit elements, 64 x 64 tiles through LDS: the hidden states as
 // [H][N] so that the weight gradient's second operand is K-major (straight into LDS) as well.
 __global__ __launch_bounds__(kBlock) void lmhead_transpose_kernel(const uint16_t* __restrict__ src, int64_t n_rows,
@@ -608,4 +635,33 @@ extern "C" int orlhf_lmhead_logprob_entropy_bwd(const void* hidden, const void* 
   return lm::launch_bwd<ORLHF_F16>(hidden, weight, n_rows, hidden_dim, vocab, hidden_stride, weight_stride, labels,
                                    temperature, g_logprob, g_entropy, row_stats, grad_hidden, grad_hidden_stride,
                                    grad_weight, grad_weight_stride, (char*)workspace, cols, s);
+}
+
+extern "C" int orlhf_matrix_tile_probe(const void* a, const void* b, int dtype, int64_t m, int64_t n, int64_t k,
+                                       int64_t lda, int64_t ldb, int resident_operands, float* tile_sums,
+                                       orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(dtype == ORLHF_BF16 || dtype == ORLHF_F16, "matrix_tile_probe: dtype %d (bf16 or fp16)", dtype);
+  ORLHF_CHECK_ARG(m > 0 && n > 0 && k > 0 && lda >= k && ldb >= k, "matrix_tile_probe: m=%lld n=%lld k=%lld lda=%lld ldb=%lld",
+                  (long long)m, (long long)n, (long long)k, (long long)lda, (long long)ldb);
+  ORLHF_CHECK_ARG(a != nullptr && b != nullptr && tile_sums != nullptr, "matrix_tile_probe: NULL argument");
+  ORLHF_CHECK_ARG((((uintptr_t)a | (uintptr_t)b) & 3u) == 0 && ((lda | ldb) & 1) == 0,
+                  "matrix_tile_probe: operands need 4-byte aligned bases and even row strides");
+  const lm::Operand oa{(const uint16_t*)a, lda, m, k}, ob{(const uint16_t*)b, ldb, n, k};
+  const int64_t tiles_m = (m + 255) / 256, tiles_n = (n + 255) / 256;
+  const dim3 grid(lm::grid_for_items(tiles_m * tiles_n)), block(mm::kThreads);
+  hipStream_t s = (hipStream_t)stream;
+#define ORLHF_PROBE(DT, RES)                                                                                   \
+  {                                                                                                            \
+    if (lm::allow_lds(lm::matrix_tile_probe_kernel<DT, RES>) != hipSuccess)                                    \
+      return fail(ORLHF_ERR_LAUNCH, "matrix_tile_probe: cannot get %d bytes of LDS", mm::kLdsBytes);           \
+    hipLaunchKernelGGL((lm::matrix_tile_probe_kernel<DT, RES>), grid, block, mm::kLdsBytes, s, oa, ob, tile_sums, tiles_m, tiles_n); \
+  }
+  if (dtype == ORLHF_BF16) {
+    if (resident_operands) ORLHF_PROBE(ORLHF_BF16, true) else ORLHF_PROBE(ORLHF_BF16, false)
+  } else {
+    if (resident_operands) ORLHF_PROBE(ORLHF_F16, true) else ORLHF_PROBE(ORLHF_F16, false)
+  }
+#undef ORLHF_PROBE
+  ORLHF_CHECK_LAUNCH("orlhf_matrix_tile_probe");
+  return ORLHF_OK;
 }

@@ -245,7 +245,10 @@ __device__ __forceinline__ void issue_order() {
 // next slab's first fragments: the matrix pipe does not drain at a slab boundary.
 // (Touching slab s + 2 an iteration early to warm the L2 changed nothing: the counters put the
 // average L2 read latency of these loads at ~270 cycles, far below an iteration.)
-template <int DT, bool A_MN_MAJOR, bool B_MN_MAJOR>
+// RESIDENT_OPERANDS (measurement only): the steady loop issues no slab loads, every slab is
+// multiplied out of whatever the LDS buffers hold. The result is meaningless; the time is what the
+// same LDS reads, MFMAs and barriers take when nothing else uses the LDS and the load path.
+template <int DT, bool A_MN_MAJOR, bool B_MN_MAJOR, bool RESIDENT_OPERANDS = false>
 __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand& a, const Operand& b, int64_t row0_a,
                                              int64_t row0_b, char* lds) {
   // Everything addressed below derives from the thread index: making it opaque keeps a caller's
@@ -296,7 +299,7 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     const int64_t k1 = (it + 1) * kSlab, k2 = (it + 2) * kSlab;
     const SlabDma db(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);  // B's slab it + 1 (unused if B_REG)
     // k-step 0
-    if (!B_REG) {
+    if (!B_REG && !RESIDENT_OPERANDS) {
       load_frags_between_dma(f1, cur, cur + kSlabBytes, 1, wm, wn, lane, db);
     } else {
       load_frags(f1, cur, cur + kSlabBytes, 1, wm, wn, lane);
@@ -326,7 +329,7 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     // there is no such slab: slab 0 is loaded again instead of branching (nobody reads it; whatever
     // touches this buffer next waits for its own later loads, and loads return in order).
     // k-step 3, over the read of the next slab's first fragments
-    if (!A_REG) {
+    if (!A_REG && !RESIDENT_OPERANDS) {
       const SlabDma da(a, row0_a, it + 2 < full ? k2 : 0, cur, wave_u, lane);
       load_frags_between_dma(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane, da);
     } else {

@@ -178,3 +178,27 @@ def test_lmhead_every_row_masked(cuda):
     # and an empty batch
     lp0, ent0 = lm_head_logprobs_and_entropy(h[:0], w, labels[:0], 1.0)
     assert lp0.shape == (0,) and ent0.shape == (0,)
+
+
+@pytest.mark.parametrize("m,n,k", [(256, 256, 64), (300, 515, 204), (1000, 259, 4102), (64, 700, 130)])
+def test_matrix_tile_probe_sums(cuda, m, n, k):
+    """The measurement entry computes the product it times: the 256 thread sums of every tile add up
+    to the sum of that 256 x 256 block of a @ b.T (fp32 reference on the same bf16 operands)."""
+    from openrlhf_amd import _lib
+    from openrlhf_amd._lib import call, ptr, stream_of
+
+    g = torch.Generator().manual_seed(m + n + k)
+    a = torch.randn(m, k, generator=g).to(torch.bfloat16).to(cuda)
+    b = torch.randn(n, k, generator=g).to(torch.bfloat16).to(cuda)
+    tm, tn = (m + 255) // 256, (n + 255) // 256
+    sums = torch.full((tm * tn * 256,), float("nan"), device=cuda)
+    call("orlhf_matrix_tile_probe", ptr(a), ptr(b), _lib.BF16, m, n, k, k, k, 0, ptr(sums), stream_of(cuda))
+    c = a.float() @ b.float().T
+    scale = c.abs().sum().item() / (tm * tn)
+    for i in range(tm):
+        for j in range(tn):
+            want = c[i * 256:(i + 1) * 256, j * 256:(j + 1) * 256].double().sum().item()
+            got = sums[(i * tn + j) * 256:(i * tn + j + 1) * 256].double().sum().item()
+            assert abs(got - want) <= 1e-5 * scale + 1e-3, (i, j, got, want)
+    with pytest.raises(_lib.KernelError):
+        call("orlhf_matrix_tile_probe", ptr(a), ptr(b), _lib.F32, m, n, k, k, k, 0, ptr(sums), stream_of(cuda))
