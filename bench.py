@@ -347,7 +347,8 @@ def bench_matrix_tile(dev, m=8192, n=8192, k=8192, reps=10):
     """--workload matrix_tile: the matrix-core tile of the lm-head path as a plain bf16 product
     (orlhf_matrix_tile_probe), with its slab loads and with the operands resident in LDS (the same
     LDS reads, MFMAs and barriers, nothing loaded: what the tile is bounded by on this GPU and
-    clock), on random operands and on operands whose rows are all equal (less switching in the
+    clock) and with all loads hitting the L1 (row stride 0: the cost of issuing the loads and
+    writing LDS without the cost of fetching), on random operands and on operands whose rows are all equal (less switching in the
     multipliers, higher clock), beside torch.matmul (hipBLASLt) on the same shapes."""
     from openrlhf_amd import _lib
     from openrlhf_amd._lib import call, ptr, stream_of
@@ -368,13 +369,22 @@ def bench_matrix_tile(dev, m=8192, n=8192, k=8192, reps=10):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / reps
 
+    # the first few dozen milliseconds of matrix work after idling run at a lower clock: bring the
+    # GPU to its sustained state before anything is timed
+    wa, wb = torch.randn(m, k, device=dev).to(torch.bfloat16), torch.randn(n, k, device=dev).to(torch.bfloat16)
+    for _ in range(60):
+        call("orlhf_matrix_tile_probe", ptr(wa), ptr(wb), _lib.BF16, m, n, k, k, k, 0, ptr(sums), st)
+    torch.cuda.synchronize()
+    del wa, wb
+
     out = {}
     for name, make in (("random", lambda r, c: torch.randn(r, c, device=dev)),
                        ("equal_rows", lambda r, c: torch.randn(1, c, device=dev).expand(r, c).contiguous())):
         a, b = make(m, k).to(torch.bfloat16), make(n, k).to(torch.bfloat16)
         entry = {}
-        for label, resident in (("tile", 0), ("tile_operands_resident", 1)):
-            ms = timed(lambda: call("orlhf_matrix_tile_probe", ptr(a), ptr(b), _lib.BF16, m, n, k, k, k, resident, ptr(sums), st))
+        # "one row": row stride 0, every row of an operand is its first row, so all loads hit the L1
+        for label, resident, ld in (("tile", 0, k), ("tile_loads_hit_l1", 0, 0), ("tile_operands_resident", 1, k)):
+            ms = timed(lambda: call("orlhf_matrix_tile_probe", ptr(a), ptr(b), _lib.BF16, m, n, k, ld, ld, resident, ptr(sums), st))
             entry[label] = {"ms": ms, "tflops": flops / ms / 1e9}
         call("orlhf_matrix_tile_probe", ptr(a), ptr(b), _lib.BF16, m, n, k, k, k, 0, ptr(sums), st)
         got = sums.view(-1, 256).sum(1)[:4].double()

@@ -221,7 +221,9 @@ int orlhf_lmhead_logprob_entropy_bwd(const void* hidden, const void* weight, int
  * resident_operands != 0 the steady loop loads nothing (every slab is multiplied out of what the
  * LDS buffers hold after the first two slabs; the sums are meaningless): the time of that run is
  * what the same LDS reads, MFMAs and barriers take on their own, the ceiling the tile can be read
- * against on a given GPU and clock. Operands need 4-byte aligned bases and even row strides.
+ * against on a given GPU and clock. A row stride of 0 makes every row of that operand its first
+ * row (all loads of the steady loop then hit the L1: the cost of issuing them and writing LDS,
+ * without the cost of fetching). Operands need 4-byte aligned bases and even row strides.
  */
 int orlhf_matrix_tile_probe(const void* a, const void* b, int dtype, int64_t m, int64_t n, int64_t k,
                             int64_t lda, int64_t ldb, int resident_operands, float* tile_sums,

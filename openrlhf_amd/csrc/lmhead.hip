@@ -641,7 +641,9 @@ extern "C" int orlhf_matrix_tile_probe(const void* a, const void* b, int dtype, 
                                        int64_t lda, int64_t ldb, int resident_operands, float* tile_sums,
                                        orlhf_stream_t stream) {
   ORLHF_CHECK_ARG(dtype == ORLHF_BF16 || dtype == ORLHF_F16, "matrix_tile_probe: dtype %d (bf16 or fp16)", dtype);
-  ORLHF_CHECK_ARG(m > 0 && n > 0 && k > 0 && lda >= k && ldb >= k, "matrix_tile_probe: m=%lld n=%lld k=%lld lda=%lld ldb=%lld",
+  // a leading dimension of 0 makes every row of that operand the same row: all its loads hit the L1
+  ORLHF_CHECK_ARG(m > 0 && n > 0 && k > 0 && (lda >= k || lda == 0) && (ldb >= k || ldb == 0),
+                  "matrix_tile_probe: m=%lld n=%lld k=%lld lda=%lld ldb=%lld",
                   (long long)m, (long long)n, (long long)k, (long long)lda, (long long)ldb);
   ORLHF_CHECK_ARG(a != nullptr && b != nullptr && tile_sums != nullptr, "matrix_tile_probe: NULL argument");
   ORLHF_CHECK_ARG((((uintptr_t)a | (uintptr_t)b) & 3u) == 0 && ((lda | ldb) & 1) == 0,

@@ -27,6 +27,7 @@
 // (l >> 5) * 8; result register r of lane l is C[8 * (r / 4) + 4 * (l >> 5) + (r & 3)][l & 31].
 #pragma once
 #include <type_traits>
+#include <utility>
 
 #include "common.h"
 
@@ -228,6 +229,72 @@ __device__ __forceinline__ void issue_order() {
   __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
 }
 
+// One k-step with every instruction's place pinned: slot I = [LDS read I of the next fragments (I < 8)],
+// MFMA I, [whatever `loads` issues at slot I]; nothing moves across a slot's end.
+template <int DT, int I, class Reads, class Loads>
+__device__ __forceinline__ void pinned_slot(f32x16 (&acc)[4][4], const Frags& use, Reads& reads, Loads& loads) {
+  reads(std::integral_constant<int, I>{});
+  acc[I >> 2][I & 3] = Mfma<DT>::run(use.a[I >> 2], use.b[I & 3], acc[I >> 2][I & 3]);
+  loads(std::integral_constant<int, I>{});
+  __builtin_amdgcn_sched_barrier(0);
+}
+template <int DT, class Reads, class Loads, int... I>
+__device__ __forceinline__ void pinned_step(f32x16 (&acc)[4][4], const Frags& use, Reads& reads, Loads& loads,
+                                            std::integer_sequence<int, I...>) {
+  (pinned_slot<DT, I>(acc, use, reads, loads), ...);
+}
+constexpr int bits_below(uint32_t mask, int i) { return __builtin_popcount(mask & ((1u << i) - 1u)); }
+
+// reads(I): LDS read I (a0 b0 a1 b1 ...) of the fragments of k-step `ks2 / 2` of a slab
+struct FragReads {
+  Frags& f;
+  const char* slab_a;
+  const char* slab_b;
+  uint32_t ks2, wm, wn, lr, lk;
+  template <int I>
+  __device__ __forceinline__ void operator()(std::integral_constant<int, I>) const {
+    if constexpr (I < 8) {
+      constexpr int t = I >> 1;
+      if constexpr ((I & 1) == 0) {
+        const uint32_t ra = wm * 128u + t * 32u + lr;
+        f.a[t] = *(const u32x4*)(slab_a + ra * 128u + (((ks2 + lk) ^ swz(ra)) << 4));
+      } else {
+        const uint32_t rb = wn * 128u + t * 32u + lr;
+        f.b[t] = *(const u32x4*)(slab_b + rb * 128u + (((ks2 + lk) ^ swz(rb)) << 4));
+      }
+    }
+  }
+};
+// loads(I): the slab pair's load number BASE + (set bits of MASK below I), if bit I of MASK is set
+template <uint32_t MASK, int BASE>
+struct SlabLoads {
+  const SlabDma& da;
+  const SlabDma& db;
+  template <int I>
+  __device__ __forceinline__ void operator()(std::integral_constant<int, I>) const {
+    if constexpr (((MASK >> I) & 1u) != 0) {
+      constexpr int n = BASE + bits_below(MASK, I);
+      if constexpr (n < 8) da.issue(n); else db.issue(n - 8);
+    }
+  }
+};
+struct NoLoads {
+  template <int I>
+  __device__ __forceinline__ void operator()(std::integral_constant<int, I>) const {}
+};
+
+// Slots at which the 16 LDS-direct loads of a slab pair (8 of A, then 8 of B; per wave) are issued:
+// every other slot of k-step 3 (right after the barrier that frees the buffer) and of k-step 0 of
+// the next iteration, which leaves k-steps 1 and 2 for them to land. Measured against the
+// alternatives at 8192^3: one load per MFMA in those two k-steps (between the LDS reads) 2-4 %
+// slower; one per three MFMAs over k-steps 3, 0, 1, or any set that reaches into k-step 1, 1-4 %
+// slower (the barrier then waits for the last ones); all 16 in k-step 3 3-5 % slower. Cache-policy
+// bits on the loads change nothing (non-temporal: 7-20 % slower).
+constexpr uint32_t kDmaSlots3 = 0x5555u;
+constexpr uint32_t kDmaSlots0 = 0x5555u;
+constexpr uint32_t kDmaSlots1 = 0x0u;
+static_assert(__builtin_popcount(kDmaSlots3) + __builtin_popcount(kDmaSlots0) + __builtin_popcount(kDmaSlots1) == 16, "16 loads per slab pair");
+
 // ---- the whole product of one output tile: acc = A[row0_a.., :] * B[row0_b.., :]^T over k in [0, depth)
 // `lds` = kLdsBytes of dynamic shared memory.
 //
@@ -236,7 +303,9 @@ __device__ __forceinline__ void issue_order() {
 //    barrier of iteration s has freed the buffer slab s was read from, a whole iteration before
 //    the barrier that publishes it, its loads placed between that k-step's LDS reads so that each
 //    goes out under an MFMA and the matrix pipe never waits for a burst of address arithmetic and
-//    load issue; only a slab that crosses the end of the depth goes through registers (masking);
+//    load issue (when both operands are K-major every instruction of the iteration has a fixed
+//    slot instead: steady_kk below); only a slab that crosses the end of the depth goes through
+//    registers (masking);
 //  * an MN-major operand's slab s + 1 sits in registers (fetched during iteration s - 1), is
 //    transposed and written to LDS during the first k-steps, and the fetch of slab s + 2 is issued
 //    into the registers it leaves.
@@ -283,8 +352,22 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     if (B_REG) fetch_slab<B_MN_MAJOR, true>(rb, b, row0_b, kSlab, tid);
   }
   __syncthreads();
-  if (full > 1) {  // slab 1 is whole: A's half starts towards the second buffer now, B's in the first iteration
-    if (!A_REG) dma_slab(a, row0_a, kSlab, lds + kStageBytes, wave_u, lane);
+  constexpr bool KK = !A_REG && !B_REG;  // both slabs by LDS-direct loads: the pinned schedule
+  constexpr int n3 = __builtin_popcount(kDmaSlots3), n0 = __builtin_popcount(kDmaSlots0);
+  using Slots16 = std::make_integer_sequence<int, 16>;
+  if (full > 1) {  // slab 1 is whole: its first loads start towards the second buffer now
+    if (KK) {
+      if (!RESIDENT_OPERANDS) {
+        const SlabDma da(a, row0_a, kSlab, lds + kStageBytes, wave_u, lane);
+        const SlabDma db(b, row0_b, kSlab, lds + kStageBytes + kSlabBytes, wave_u, lane);
+#pragma unroll
+        for (int n = 0; n < n3; ++n) {
+          if (n < 8) da.issue(n); else db.issue(n - 8);
+        }
+      }
+    } else if (!A_REG) {
+      dma_slab(a, row0_a, kSlab, lds + kStageBytes, wave_u, lane);
+    }
   }
   Frags f0, f1;
   load_frags(f0, lds, lds + kSlabBytes, 0, wm, wn, lane);
@@ -339,12 +422,50 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     issue_order<0>();
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The same iteration when both operands arrive by LDS-direct loads: slab it + 1 has had its first
+  // loads since k-step 3 of the previous iteration and gets the rest in k-steps 0 and 1; after the
+  // barrier slab it + 2 starts towards `cur` (in the last iteration slab 0 again instead of a branch:
+  // nobody reads it, and whatever touches this buffer next waits for its own later loads).
+  auto steady_kk = [&](auto parity, int64_t it) {
+    constexpr int P = decltype(parity)::value;
+    char* cur = lds + P * kStageBytes;
+    char* nxt = lds + (1 - P) * kStageBytes;
+    const int64_t k1 = (it + 1) * kSlab, k2 = it + 2 < full ? (it + 2) * kSlab : 0;
+    const uint32_t lr = lane & 31u, lk = lane >> 5;
+    const SlabDma da1(a, row0_a, k1, nxt, wave_u, lane), db1(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);
+    NoLoads none;
+    {
+      FragReads rd{f1, cur, cur + kSlabBytes, 2, wm, wn, lr, lk};
+      SlabLoads<kDmaSlots0, n3> ld{da1, db1};
+      if (RESIDENT_OPERANDS) pinned_step<DT>(acc, f0, rd, none, Slots16{}); else pinned_step<DT>(acc, f0, rd, ld, Slots16{});
+    }
+    {
+      FragReads rd{f0, cur, cur + kSlabBytes, 4, wm, wn, lr, lk};
+      SlabLoads<kDmaSlots1, n3 + n0> ld{da1, db1};
+      if (RESIDENT_OPERANDS) pinned_step<DT>(acc, f1, rd, none, Slots16{}); else pinned_step<DT>(acc, f1, rd, ld, Slots16{});
+    }
+    {
+      FragReads rd{f1, cur, cur + kSlabBytes, 6, wm, wn, lr, lk};
+      pinned_step<DT>(acc, f0, rd, none, Slots16{});
+    }
+    // every wave holds its last fragments of `cur`; slab it + 1 is complete in `nxt`
+    __syncthreads();
+    const SlabDma da2(a, row0_a, k2, cur, wave_u, lane), db2(b, row0_b, k2, cur + kSlabBytes, wave_u, lane);
+    {
+      FragReads rd{f0, nxt, nxt + kSlabBytes, 0, wm, wn, lr, lk};
+      SlabLoads<kDmaSlots3, 0> ld{da2, db2};
+      if (RESIDENT_OPERANDS) pinned_step<DT>(acc, f1, rd, none, Slots16{}); else pinned_step<DT>(acc, f1, rd, ld, Slots16{});
+    }
+  };
+  auto iteration = [&](auto parity, int64_t it) {
+    if constexpr (KK) steady_kk(parity, it); else steady(parity, it);
+  };
   for (; s + 2 < full; s += 2) {  // pairs of steady iterations: the buffers' addresses are constants
-    steady(std::integral_constant<int, 0>{}, s);
-    steady(std::integral_constant<int, 1>{}, s + 1);
+    iteration(std::integral_constant<int, 0>{}, s);
+    iteration(std::integral_constant<int, 1>{}, s + 1);
   }
   if (s + 1 < full) {  // s is even here
-    steady(std::integral_constant<int, 0>{}, s);
+    iteration(std::integral_constant<int, 0>{}, s);
     ++s;
   }
   // s == full - 1 (or 0): slab s is in its buffer, no load into LDS is outstanding
