@@ -611,6 +611,21 @@ def bench_per_token(args, dev, emit=True):
     att = [torch.cat([m_[:, :1], m_], dim=1) for m_ in mask]
     prompt_lens = torch.randint(1, 64, (b,), generator=g).to(dev)
     record("config4.dpo_sequence_logps", timed(rot(lambda k: get_batch_logps(lp[k], att[k], prompt_lens))), padded, 5)
+    # the unpadding in front of the packed forward and the re-padding behind it
+    # (openrlhf/models/ring_attn_utils.py:103-182): mask read twice (counts, ranks), per attended token
+    # its id read and four int64 written; back: zeros, then value and index read, value written
+    from openrlhf_amd.models.ring_attn_utils import gather_and_pad_tensor, unpad_and_slice_tensor
+    seqs = torch.randint(0, 151936, (b, a + 1), generator=g).to(dev)
+    n_att = [int(m_.sum()) for m_ in att]
+    mb = att[0].element_size()
+    record("config4.unpad_and_slice_tensor",
+           timed(rot(lambda k: unpad_and_slice_tensor(seqs, att[k], None, total_tokens=n_att[k]))), b * (a + 1),
+           2 * mb + (8 + 32) * n_att[0] / (b * (a + 1)))
+    up = [unpad_and_slice_tensor(seqs, att[k], None) for k in range(RING)]
+    vals = [torch.randn(1, n_att[k], device=dev) for k in range(RING)]
+    record("config4.gather_and_pad_tensor",
+           timed(rot(lambda k: gather_and_pad_tensor(vals[k], None, 0, up[k][4], b, a + 1))), b * (a + 1),
+           4 + (4 + 8 + 4) * n_att[0] / (b * (a + 1)))
     if emit:
         print(json.dumps({"workload": "per-token kernels at BASELINE config 3 / config 4 sizes (padded [B, A] fp32)",
                           "n_gpus": 1, "unit": "GB/s", "peak": HBM_PEAK_GBS, "entries": res}), flush=True)

@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 20
+#define ORLHF_ABI_VERSION 21
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -667,6 +667,42 @@ int orlhf_gather_rows(const void* src, int elem_bytes, int64_t n_rows, int64_t m
 int orlhf_pad_rows(const void* src, int elem_bytes, const int64_t* cu_seqlens, int64_t n_rows,
                    int64_t n_cols, int left_side, uint64_t fill_bits, void* dst,
                    orlhf_stream_t stream);
+
+/*
+ * The unpadding in front of the packed model forward, unpad_and_slice_tensor on one GPU
+ * (openrlhf/models/ring_attn_utils.py:129-140), which calls unpad_input / index_first_axis of
+ * flash-attn 2.8.3 (flash_attn/bert_padding.py, not in the reference tree; its published
+ * algorithm: indices = nonzero(mask.flatten()), seqlens = mask.sum(-1), cu_seqlens =
+ * pad(cumsum(seqlens), (1, 0)), gathers by indices), for masks of zeros and ones with the ones
+ * anywhere in a row (left padding, right padding, holes).
+ *
+ * orlhf_mask_row_counts: counts[b] = number of non-zero columns of mask row b (seqlens_in_batch;
+ *   orlhf_cu_seqlens turns them into cu_seqlens).
+ * orlhf_unpad_sequences: for the r-th non-zero column t of row b, at slot cu_seqlens[b] + r of each
+ *   output that is not NULL:
+ *     indices          b * n_cols + t                      (unpad_input's indices)
+ *     packed_sequences sequences[b, t]                     (:130-131)
+ *     rolled_sequences sequences[b, (t + 1) mod n_cols]    (torch.roll(sequences, -1, 1), :129,132-136)
+ *     position_ids     r                                   (clip(cumsum(mask, -1) - 1, min=0), :137-140)
+ *   sequences may be NULL when neither sequence output is asked for. capacity is the number of
+ *   slots each output holds (cu_seqlens[n_rows] when they are sized exactly); slots past it are
+ *   not written.
+ */
+int orlhf_mask_row_counts(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                          int64_t* counts, orlhf_stream_t stream);
+int orlhf_unpad_sequences(const int64_t* sequences, const void* mask, int mask_dtype,
+                          int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
+                          int64_t capacity, int64_t* indices, int64_t* packed_sequences,
+                          int64_t* rolled_sequences, int64_t* position_ids, orlhf_stream_t stream);
+
+/*
+ * The way back, gather_and_pad_tensor on one GPU (openrlhf/models/ring_attn_utils.py:181, which is
+ * flash-attn's pad_input: zeros, then output[indices] = input): dst holds n_dst rows of `inner`
+ * elements of elem_bytes (1, 2, 4, 8) bytes, all set to zero, then row indices[i] receives row i
+ * of src (n rows). dst must be 16-byte aligned; an index outside [0, n_dst) is skipped.
+ */
+int orlhf_pad_by_indices(const void* src, int elem_bytes, int64_t n, int64_t inner,
+                         const int64_t* indices, int64_t n_dst, void* dst, orlhf_stream_t stream);
 
 #ifdef __cplusplus
 }

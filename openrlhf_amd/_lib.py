@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 20
+ABI_VERSION = 21
 
 
 class Norm(Structure):
@@ -120,6 +120,9 @@ SIGNATURES = {
     "orlhf_pack_rows": (c_int, [P, c_int, I64, I64, P, P, P, P]),
     "orlhf_gather_rows": (c_int, [P, c_int, I64, I64, P, P, P, P]),
     "orlhf_pad_rows": (c_int, [P, c_int, P, I64, I64, c_int, c_uint64, P, P]),
+    "orlhf_mask_row_counts": (c_int, [P, c_int, I64, I64, P, P]),
+    "orlhf_unpad_sequences": (c_int, [P, P, c_int, I64, I64, P, I64, P, P, P, P, P]),
+    "orlhf_pad_by_indices": (c_int, [P, c_int, I64, I64, P, I64, P, P]),
     "orlhf_sequence_logps_fwd": (c_int, [P, P, c_int, P, I64, I64, P, P, P, P]),
     "orlhf_sequence_logps_bwd": (c_int, [P, P, P, c_int, P, P, I64, I64, P, P]),
     "orlhf_pair_loss_fwd": (c_int, [P, P, P, P, I64, c_int, c_double, c_double, P, P, P, P]),

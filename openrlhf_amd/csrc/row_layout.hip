@@ -7,6 +7,9 @@
 //   pack_rows     dst[cu[b] + j] = src[b, first[b] + j]
 //   gather_rows   dst[cu[b] + j] = src[start[b] + j]: rows picked out of another packed array
 //   pad_rows      dst[b, :] = fill, then the row's tokens on the left or on the right side
+//   unpad         the non-zero positions of a [B, T] mask in row-major order (masks with holes too): their
+//                 count per row, and per position its flat index, token, next token and rank in its row
+//   pad_by_indices  the way back: zeros, then dst[indices[i]] = src[i]
 #include "common.h"
 
 namespace orlhf {
@@ -213,6 +216,140 @@ __global__ __launch_bounds__(kBlock) void pad_rows_kernel(const E* __restrict__ 
   }
 }
 
+// Non-zero columns of mask row b in rising order. A workgroup walks its row in tiles of
+// kUnpadCols * kBlock columns, kUnpadCols consecutive columns per lane; a lane's rank among the
+// row's non-zero columns is (non-zeros of earlier tiles) + (those of earlier waves) + (wave scan).
+// COUNT_ONLY leaves the row's count; otherwise position r of row b goes to slot cu[b] + r of every
+// output that is asked for: its flat index b * n_cols + t, sequences[b, t],
+// sequences[b, (t + 1) mod n_cols] and r. A lane whose columns are all non-zero (the inside of an
+// attended span: almost every lane that writes at all) moves its tokens with 16-byte loads and
+// stores.
+constexpr int kUnpadCols = 8;
+
+template <int MASK_DT, bool COUNT_ONLY>
+__global__ __launch_bounds__(kBlock) void unpad_rows_kernel(const int64_t* __restrict__ sequences,
+                                                            const void* __restrict__ mask, int64_t n_rows, int64_t n_cols,
+                                                            const int64_t* __restrict__ cu, int64_t capacity,
+                                                            int64_t* __restrict__ counts,
+                                                            int64_t* __restrict__ indices, int64_t* __restrict__ packed,
+                                                            int64_t* __restrict__ rolled, int64_t* __restrict__ position) {
+  __shared__ int wave_tot[2][kWavesPerBlock];  // alternating slots: one barrier per tile
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  int par = 0;
+  for (int64_t b = blockIdx.x; b < n_rows; b += gridDim.x) {
+    const int64_t out0 = COUNT_ONLY ? 0 : cu[b];
+    int64_t run = 0;  // non-zero columns of the row before this tile
+    for (int64_t t0 = 0; t0 < n_cols; t0 += kUnpadCols * kBlock, par ^= 1) {
+      const int64_t t = t0 + kUnpadCols * (int64_t)threadIdx.x;
+      uint32_t nz = 0;  // bit k: column t + k is inside the row and non-zero
+      if (t + kUnpadCols <= n_cols) {  // whole group inside the row
+        float m[kUnpadCols];
+#pragma unroll
+        for (int q = 0; q < kUnpadCols / 4; ++q) load_mask4<MASK_DT, false>(mask, b * n_cols + t + 4 * q, m + 4 * q);
+#pragma unroll
+        for (int k = 0; k < kUnpadCols; ++k) nz |= m[k] != 0.0f ? 1u << k : 0u;
+      } else {
+#pragma unroll
+        for (int k = 0; k < kUnpadCols; ++k)
+          nz |= (t + k < n_cols && load_mask<MASK_DT>(mask, b * n_cols + t + k) != 0.0f) ? 1u << k : 0u;
+      }
+      const int c = __builtin_popcount(nz);
+      int incl = c;
+#pragma unroll
+      for (int o = 1; o < kWave; o <<= 1) {
+        const int up = __shfl_up(incl, o, kWave);
+        if (lane >= o) incl += up;
+      }
+      if (lane == kWave - 1) wave_tot[par][wave] = incl;
+      __syncthreads();
+      int before = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < kWavesPerBlock; ++w) {
+        const int v = wave_tot[par][w];
+        before += w < wave ? v : 0;
+        total += v;
+      }
+      constexpr int kWaveCols = kUnpadCols * kWave;
+      const bool wave_dense = !COUNT_ONLY && __all(nz == (1u << kUnpadCols) - 1u) &&
+                              out0 + run + before + kWaveCols <= capacity;
+      if (wave_dense) {
+        // the wave's 512 columns are 512 consecutive slots: lanes take them two at a time, interleaved,
+        // so that every load and store of the wave covers 1 KiB of consecutive memory
+        const int64_t col0 = t0 + (int64_t)wave * kWaveCols, at0 = b * n_cols + col0, dst0 = out0 + run + before;
+#pragma unroll
+        for (int j = 0; j < kWaveCols / (2 * kWave); ++j) {
+          const int64_t off = 2 * kWave * j + 2 * lane;
+          if (indices != nullptr) *(i64x2e*)(indices + dst0 + off) = i64x2{at0 + off, at0 + off + 1};
+          if (position != nullptr) *(i64x2e*)(position + dst0 + off) = i64x2{run + before + off, run + before + off + 1};
+          if (packed != nullptr || rolled != nullptr) {
+            const i64x2 v = *(const i64x2e*)(sequences + at0 + off);
+            if (packed != nullptr) *(i64x2e*)(packed + dst0 + off) = v;
+            if (rolled != nullptr) {
+              const int64_t after = sequences[col0 + off + 2 == n_cols ? b * n_cols : at0 + off + 2];
+              *(i64x2e*)(rolled + dst0 + off) = i64x2{v[1], after};
+            }
+          }
+        }
+      } else if (!COUNT_ONLY && c > 0) {
+        int64_t r = run + before + incl - c;
+        const int64_t at0 = b * n_cols + t, dst0 = out0 + r;
+        if (nz == (1u << kUnpadCols) - 1u && dst0 + kUnpadCols <= capacity) {
+          int64_t tok[kUnpadCols + 1];
+          if (packed != nullptr || rolled != nullptr) {
+#pragma unroll
+            for (int q = 0; q < kUnpadCols / 2; ++q) {
+              const i64x2 v = *(const i64x2e*)(sequences + at0 + 2 * q);
+              tok[2 * q] = v[0];
+              tok[2 * q + 1] = v[1];
+            }
+            tok[kUnpadCols] = rolled != nullptr ? sequences[t + kUnpadCols == n_cols ? b * n_cols : at0 + kUnpadCols] : 0;
+          }
+#pragma unroll
+          for (int q = 0; q < kUnpadCols / 2; ++q) {
+            if (indices != nullptr) *(i64x2e*)(indices + dst0 + 2 * q) = i64x2{at0 + 2 * q, at0 + 2 * q + 1};
+            if (packed != nullptr) *(i64x2e*)(packed + dst0 + 2 * q) = i64x2{tok[2 * q], tok[2 * q + 1]};
+            if (rolled != nullptr) *(i64x2e*)(rolled + dst0 + 2 * q) = i64x2{tok[2 * q + 1], tok[2 * q + 2]};
+            if (position != nullptr) *(i64x2e*)(position + dst0 + 2 * q) = i64x2{r + 2 * q, r + 2 * q + 1};
+          }
+        } else {
+#pragma unroll
+          for (int k = 0; k < kUnpadCols; ++k) {
+            const bool on = (nz >> k) & 1u;
+            if (on && out0 + r < capacity) {  // slots past the outputs' stated size are dropped
+              const int64_t at = at0 + k, dst = out0 + r;
+              if (indices != nullptr) indices[dst] = at;
+              if (packed != nullptr) packed[dst] = sequences[at];
+              if (rolled != nullptr) rolled[dst] = sequences[t + k + 1 == n_cols ? b * n_cols : at + 1];
+              if (position != nullptr) position[dst] = r;
+            }
+            r += on ? 1 : 0;
+          }
+        }
+      }
+      run += total;
+    }
+    if (COUNT_ONLY && threadIdx.x == 0) counts[b] = run;
+  }
+}
+
+// dst[indices[i] * inner + j] = src[i * inner + j]; an index outside [0, n_dst) is skipped.
+template <typename E>
+__global__ __launch_bounds__(kBlock) void scatter_index_kernel(const E* __restrict__ src, const int64_t* __restrict__ indices,
+                                                               int64_t n, int64_t inner, int64_t n_dst, E* __restrict__ dst) {
+  const int64_t total = n * inner;
+  for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < total; e += (int64_t)gridDim.x * kBlock) {
+    const int64_t i = e / inner, j = e - i * inner, to = indices[i];
+    if ((uint64_t)to < (uint64_t)n_dst) dst[to * inner + j] = src[e];
+  }
+}
+
+__global__ __launch_bounds__(kBlock) void zero_bytes_kernel(char* __restrict__ dst, int64_t bytes) {
+  const int64_t groups = bytes / 16;  // dst is 16-byte aligned (checked by the caller)
+  for (int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x; g < groups; g += (int64_t)gridDim.x * kBlock)
+    *(u32x4*)(dst + g * 16) = u32x4{0u, 0u, 0u, 0u};
+  for (int64_t i = groups * 16 + (int64_t)blockIdx.x * kBlock + threadIdx.x; i < bytes; i += (int64_t)gridDim.x * kBlock) dst[i] = 0;
+}
+
 static inline unsigned copy_grid(int64_t n_rows, int64_t n_cols, int elem_bytes) {
   const int64_t chunk = kCopyChunkBytes / elem_bytes;
   const int64_t chunks = (n_cols + chunk - 1) / chunk;
@@ -312,5 +449,80 @@ extern "C" int orlhf_pad_rows(const void* src, int elem_bytes, const int64_t* cu
     default: return fail(ORLHF_ERR_INVALID_ARG, "pad_rows: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
   }
   ORLHF_CHECK_LAUNCH("orlhf_pad_rows");
+  return ORLHF_OK;
+}
+
+template <bool COUNT_ONLY>
+static int launch_unpad(const int64_t* sequences, const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
+                        const int64_t* cu, int64_t capacity, int64_t* counts, int64_t* indices, int64_t* packed,
+                        int64_t* rolled, int64_t* position, hipStream_t s) {
+  const dim3 grid(slot_grid(n_rows, 65536)), block(kBlock);
+  switch (mask_dtype) {
+    case ORLHF_MASK_U8:
+      hipLaunchKernelGGL((unpad_rows_kernel<ORLHF_MASK_U8, COUNT_ONLY>), grid, block, 0, s, sequences, mask, n_rows, n_cols, cu, capacity, counts, indices, packed, rolled, position);
+      break;
+    case ORLHF_MASK_F32:
+      hipLaunchKernelGGL((unpad_rows_kernel<ORLHF_MASK_F32, COUNT_ONLY>), grid, block, 0, s, sequences, mask, n_rows, n_cols, cu, capacity, counts, indices, packed, rolled, position);
+      break;
+    default:
+      hipLaunchKernelGGL((unpad_rows_kernel<ORLHF_MASK_I64, COUNT_ONLY>), grid, block, 0, s, sequences, mask, n_rows, n_cols, cu, capacity, counts, indices, packed, rolled, position);
+      break;
+  }
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_mask_row_counts(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols, int64_t* counts,
+                                     orlhf_stream_t stream) {
+  if (int rc = check_rows("mask_row_counts", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(mask_dtype != ORLHF_MASK_NONE, "mask_row_counts: needs a mask");
+  if (n_rows == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(counts != nullptr, "mask_row_counts: counts is NULL");
+  launch_unpad<true>(nullptr, mask, mask_dtype, n_rows, n_cols, nullptr, 0, counts, nullptr, nullptr, nullptr, nullptr,
+                     (hipStream_t)stream);
+  ORLHF_CHECK_LAUNCH("orlhf_mask_row_counts");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_unpad_sequences(const int64_t* sequences, const void* mask, int mask_dtype, int64_t n_rows,
+                                     int64_t n_cols, const int64_t* cu_seqlens, int64_t capacity, int64_t* indices,
+                                     int64_t* packed_sequences, int64_t* rolled_sequences, int64_t* position_ids,
+                                     orlhf_stream_t stream) {
+  if (int rc = check_rows("unpad_sequences", n_rows, n_cols, mask, mask_dtype)) return rc;
+  ORLHF_CHECK_ARG(mask_dtype != ORLHF_MASK_NONE, "unpad_sequences: needs a mask");
+  ORLHF_CHECK_ARG(capacity >= 0, "unpad_sequences: capacity=%lld", (long long)capacity);
+  if (n_rows * n_cols == 0 || capacity == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(cu_seqlens != nullptr, "unpad_sequences: cu_seqlens is NULL");
+  ORLHF_CHECK_ARG(indices != nullptr || packed_sequences != nullptr || rolled_sequences != nullptr || position_ids != nullptr,
+                  "unpad_sequences: nothing to compute");
+  ORLHF_CHECK_ARG(sequences != nullptr || (packed_sequences == nullptr && rolled_sequences == nullptr),
+                  "unpad_sequences: sequences is NULL");
+  launch_unpad<false>(sequences, mask, mask_dtype, n_rows, n_cols, cu_seqlens, capacity, nullptr, indices, packed_sequences,
+                      rolled_sequences, position_ids, (hipStream_t)stream);
+  ORLHF_CHECK_LAUNCH("orlhf_unpad_sequences");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_pad_by_indices(const void* src, int elem_bytes, int64_t n, int64_t inner, const int64_t* indices,
+                                    int64_t n_dst, void* dst, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n >= 0 && inner >= 1 && n_dst >= 0, "pad_by_indices: n=%lld inner=%lld n_dst=%lld", (long long)n,
+                  (long long)inner, (long long)n_dst);
+  ORLHF_CHECK_ARG(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8,
+                  "row layout: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
+  if (n_dst == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(dst != nullptr && ((uintptr_t)dst & 15u) == 0, "pad_by_indices: dst must be non-NULL and 16-byte aligned");
+  ORLHF_CHECK_ARG(n == 0 || (src != nullptr && indices != nullptr), "pad_by_indices: NULL argument");
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t bytes = n_dst * inner * elem_bytes;
+  hipLaunchKernelGGL(zero_bytes_kernel, dim3(flat_grid(bytes / 16 + 1)), dim3(kBlock), 0, s, (char*)dst, bytes);
+  ORLHF_CHECK_LAUNCH("orlhf_pad_by_indices(zero)");
+  if (n == 0) return ORLHF_OK;
+  const dim3 grid(flat_grid(n * inner)), block(kBlock);
+  switch (elem_bytes) {
+    case 1: hipLaunchKernelGGL(scatter_index_kernel<uint8_t>, grid, block, 0, s, (const uint8_t*)src, indices, n, inner, n_dst, (uint8_t*)dst); break;
+    case 2: hipLaunchKernelGGL(scatter_index_kernel<uint16_t>, grid, block, 0, s, (const uint16_t*)src, indices, n, inner, n_dst, (uint16_t*)dst); break;
+    case 4: hipLaunchKernelGGL(scatter_index_kernel<uint32_t>, grid, block, 0, s, (const uint32_t*)src, indices, n, inner, n_dst, (uint32_t*)dst); break;
+    default: hipLaunchKernelGGL(scatter_index_kernel<uint64_t>, grid, block, 0, s, (const uint64_t*)src, indices, n, inner, n_dst, (uint64_t*)dst); break;
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_pad_by_indices");
   return ORLHF_OK;
 }

@@ -19,10 +19,7 @@ import torch
 from .utils import logprobs_and_entropy_from_logits
 
 
-def unpad_indices(attention_mask: torch.Tensor) -> torch.Tensor:
-    """Flat positions of the attended tokens in row-major order: the ``indices`` flash-attn's
-    unpad_input returns (openrlhf/models/ring_attn_utils.py:130)."""
-    return torch.nonzero(attention_mask.reshape(-1), as_tuple=False).squeeze(-1)
+from .ring_attn_utils import gather_and_pad_tensor, unpad_indices  # noqa: F401  (unpad_indices is part of this module's API)
 
 
 def actor_forward_tail(

@@ -45,3 +45,35 @@ def unpad_and_rebatch(field, attention_mask):
         rows.append(value[: -right_pad] if right_pad else value)
         kept.append(rows[-1].numel())
     return zero_pad_sequences(rows, "right", 0, stack=True), kept
+
+
+def unpad_and_slice_tensor(sequences, attention_mask):
+    """unpad_and_slice_tensor with ring_attn_group=None (openrlhf/models/ring_attn_utils.py:103-148).
+
+    It calls unpad_input / index_first_axis of flash-attn 2.8.3 (flash_attn/bert_padding.py, a
+    dependency that is not in the reference tree); restated from its published definition:
+    ``indices = nonzero(attention_mask.flatten())``, ``seqlens = attention_mask.sum(-1)``,
+    ``cu_seqlens = pad(cumsum(seqlens), (1, 0))``, ``index_first_axis(x, indices) = x[indices]``
+    on the flattened ``(b s)`` axis. Returns what the reference returns, plus cu_seqlens:
+    (sequences [1, Ttot], position_ids [1, Ttot], rolled_sequences [1, Ttot], 0, indices, cu_seqlens).
+    Pins: the reference's own docstring example (:112-118) and a cell-by-cell loop, in
+    tests/test_oracle_pins.py."""
+    rolled = torch.roll(sequences, shifts=-1, dims=1)  # :129
+    indices = torch.nonzero(attention_mask.flatten(), as_tuple=False).flatten()
+    seqlens = attention_mask.sum(dim=-1, dtype=torch.int32)
+    cu_seqlens = F.pad(torch.cumsum(seqlens, dim=0, dtype=torch.int32), (1, 0))
+    packed = sequences.reshape(-1)[indices].unsqueeze(0)  # :130-131
+    rolled = rolled.reshape(-1)[indices].unsqueeze(0)  # :132-136
+    position_ids = torch.clip(torch.cumsum(attention_mask, dim=-1) - 1, min=0, max=None)  # :137
+    position_ids = position_ids.reshape(-1)[indices].unsqueeze(0)  # :138-140
+    return packed, position_ids, rolled, 0, indices, cu_seqlens
+
+
+def gather_and_pad_tensor(tensor, indices, batch, seqlen):
+    """gather_and_pad_tensor with ring_attn_group=None (openrlhf/models/ring_attn_utils.py:151-182):
+    flash-attn's pad_input on the transposed [Ttot, 1] tensor, i.e. zeros of batch * seqlen rows
+    with ``output[indices] = input``, reshaped to [batch, seqlen]."""
+    values = tensor.transpose(0, 1)  # [Ttot, 1] or [Ttot, ...]
+    out = torch.zeros(batch * seqlen, *values.shape[1:], dtype=values.dtype)
+    out[indices] = values
+    return out.view(batch, seqlen, *values.shape[1:]).squeeze(-1)

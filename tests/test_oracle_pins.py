@@ -400,3 +400,44 @@ def test_layout_unpad_and_rebatch_known_answer():
     out, kept = olay.unpad_and_rebatch(act, att)
     assert kept == [2, 4, 4, 0]
     assert out.tolist() == [[1, 2, 0, 0], [5, 6, 7, 8], [9, 10, 11, 12], [0, 0, 0, 0]]
+
+
+def test_layout_unpad_and_slice_known_answers():
+    """unpad_and_slice_tensor / gather_and_pad_tensor restatements: the example in the reference's
+    docstrings (openrlhf/models/ring_attn_utils.py:112-118, :155-164) and a cell-by-cell walk of a
+    mask with left padding, right padding and holes."""
+    from oracle import layout as olay
+
+    seq = torch.tensor([[1, 2, 3, 0], [4, 5, 0, 0]])
+    att = torch.tensor([[1, 1, 1, 0], [1, 1, 0, 0]])
+    packed, pos, rolled, pad_len, indices, cu = olay.unpad_and_slice_tensor(seq, att)
+    assert packed.tolist() == [[1, 2, 3, 4, 5]] and pad_len == 0
+    assert indices.tolist() == [0, 1, 2, 4, 5] and cu.tolist() == [0, 3, 5]
+    assert pos.tolist() == [[0, 1, 2, 0, 1]] and rolled.tolist() == [[2, 3, 0, 5, 0]]
+    assert olay.gather_and_pad_tensor(packed, indices, 2, 4).tolist() == [[1, 2, 3, 0], [4, 5, 0, 0]]
+
+    g = torch.Generator().manual_seed(0)
+    att = (torch.rand(5, 13, generator=g) < 0.5).long()
+    att[0] = 0
+    att[1, :4] = 0
+    att[2, 9:] = 0
+    seq = torch.randint(0, 100, (5, 13), generator=g)
+    packed, pos, rolled, _, indices, cu = olay.unpad_and_slice_tensor(seq, att)
+    want_i, want_p, want_r, want_pos, want_cu = [], [], [], [], [0]
+    for b in range(5):
+        rank = 0
+        for t in range(13):
+            if att[b, t]:
+                want_i.append(b * 13 + t)
+                want_p.append(int(seq[b, t]))
+                want_r.append(int(seq[b, (t + 1) % 13]))
+                want_pos.append(rank)
+                rank += 1
+        want_cu.append(want_cu[-1] + rank)
+    assert indices.tolist() == want_i and packed[0].tolist() == want_p and rolled[0].tolist() == want_r
+    assert pos[0].tolist() == want_pos and cu.tolist() == want_cu
+    vals = torch.arange(1.0, len(want_i) + 1).unsqueeze(0)
+    padded = olay.gather_and_pad_tensor(vals, indices, 5, 13)
+    for b in range(5):
+        for t in range(13):
+            assert padded[b, t] == (vals[0, want_i.index(b * 13 + t)] if att[b, t] else 0)
