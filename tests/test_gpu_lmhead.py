@@ -110,6 +110,30 @@ def test_lmhead_batch_shape_row_mask_and_strides(cuda):
     assert torch.equal(lp2.reshape(-1)[2:], lm_head_logprobs_and_entropy(hidden.to(cuda), wd.detach(), labels.to(cuda), 0.9)[0].reshape(-1)[2:])
 
 
+@pytest.mark.parametrize("chunk_mib", [1, 3, 4096])
+def test_lmhead_backward_chunk_sizes(cuda, chunk_mib):
+    """The backward holds as much of the logits gradient at a time as its workspace offers: many
+    small chunks, a last chunk that is not a whole tile column, one chunk for everything. The
+    weight gradient does not depend on the cut (each entry is summed over tokens only); the hidden
+    states' gradient is summed over the vocabulary chunk by chunk in fp32."""
+    from openrlhf_amd.models.utils import lm_head_logprobs_and_entropy
+
+    n, hdim, vocab, temperature = 1500, 256, 20011, 0.8
+    hidden, weight, labels, g_lp, g_ent = _case(n, hdim, vocab, torch.bfloat16, seed=77)
+    _, _, ref_gh, ref_gw = _oracle(hidden, weight, labels, temperature, g_lp, g_ent)
+    grads = []
+    for mib in (None, chunk_mib):
+        hd = hidden.to(cuda).requires_grad_(True)
+        wd = weight.to(cuda).requires_grad_(True)
+        lp, ent = lm_head_logprobs_and_entropy(hd, wd, labels.to(cuda), temperature, backward_chunk_mib=mib)
+        torch.autograd.backward([lp, ent], [g_lp.to(cuda), g_ent.to(cuda)])
+        grads.append((hd.grad, wd.grad))
+    _grad_close(grads[1][0], ref_gh, torch.bfloat16)
+    _grad_close(grads[1][1], ref_gw, torch.bfloat16)
+    assert torch.equal(grads[0][1], grads[1][1])
+    assert (grads[0][0].float() - grads[1][0].float()).abs().max().item() <= 2.0 ** -7 * ref_gh.abs().max().item()
+
+
 def test_lmhead_rejects_what_it_cannot_run(cuda):
     from openrlhf_amd.models.utils import lm_head_logprobs_and_entropy
 
