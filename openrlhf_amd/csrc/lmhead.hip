@@ -56,7 +56,6 @@ __device__ __forceinline__ void fold_tile(const f32x16 (&acc)[4][4], Running (&r
     const float m_new = fmaxf(run[nt].m, mx);
     const float n1 = -m_new * c1, nT = -m_new * cT;
     float s1[2] = {0.0f, 0.0f}, t1[2] = {0.0f, 0.0f}, sT[2] = {0.0f, 0.0f};
-    float xl = run[nt].xl;
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
@@ -69,8 +68,18 @@ __device__ __forceinline__ void fold_tile(const f32x16 (&acc)[4][4], Running (&r
         s1[r & 1] += e;
         t1[r & 1] = fmaf(e, x, t1[r & 1]);
         if (BOTH_T) sT[r & 1] += real ? fast_exp2(fmaf(x, cT, nT)) : 0.0f;
-        xl = (lab_rel[nt] == reg_off(mt, r)) ? x : xl;
       }
+    }
+    // the label's logit: per token one lane of one tile of the vocabulary holds it, so the 64-way
+    // selection sits behind a branch that almost every wave skips
+    if (lab_rel[nt] >= 0) {
+      float xl = run[nt].xl;
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) xl = (lab_rel[nt] == reg_off(mt, r)) ? acc[mt][nt][r] : xl;
+      }
+      run[nt].xl = xl;
     }
     const float d = run[nt].m - m_new;  // <= 0
     const float q1 = fast_exp2(d * c1);
@@ -78,7 +87,6 @@ __device__ __forceinline__ void fold_tile(const f32x16 (&acc)[4][4], Running (&r
     run[nt].t1 = fmaf(run[nt].t1, q1, t1[0] + t1[1]);
     if (BOTH_T) run[nt].sT = fmaf(run[nt].sT, fast_exp2(d * cT), sT[0] + sT[1]);
     run[nt].m = m_new;
-    run[nt].xl = xl;
   }
 }
 
