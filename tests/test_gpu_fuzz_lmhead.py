@@ -12,7 +12,7 @@ from oracle import token_numerics as otn
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", list(range(16)) + [5024, 5025, 5028, 5044, 5051, 5054])  # the last six: a vocabulary of one entry
 def test_random_case(cuda, seed):
     from openrlhf_amd.models.utils import lm_head_logprobs_and_entropy
 
@@ -60,6 +60,8 @@ def test_random_case(cuda, seed):
         err = (got.cpu().double() - ref).abs()
         scale = ref.abs().max().item()
         assert torch.isfinite(got).all(), info
-        assert err.max().item() <= 4 * eps * scale + 1e-7, (info, err.max().item(), scale)
+        # the floor: softmax weights come from an fp32 exponent, so a weight that is exactly 1 (a
+        # vocabulary of one entry, where every gradient is exactly 0) comes out as 1 - 2e-7
+        assert err.max().item() <= 4 * eps * scale + 2e-6, (info, err.max().item(), scale)
     if mask is not None:
         assert gh[~mask.to(cuda)].abs().max().item() == 0.0 if bool((~mask).any()) else True
