@@ -508,6 +508,31 @@ def bench_per_token(args, dev, emit=True):
 
     chain_bytes = 10 + 17 + 14 + 13 + 13
     record("config3.chain_eager", timed(chain), padded, chain_bytes)
+    if emit and not getattr(args, "no_cpu_baseline", False):
+        # the same chain as the reference runs it, on the host: the CPU restatement of its op sequence
+        # (reward shaping, GAE as a loop over the columns, whitening, both losses' forward)
+        from oracle import advantages as oadv, losses as olos, token_numerics as otn
+        c_r, c_kl, c_mask, c_val = r.cpu(), kl.cpu(), mask.cpu().float(), values.cpu()
+        c_lp, c_old = lp3.cpu(), old3.cpu()
+
+        def cpu_chain():
+            rew_ = otn.compute_reward(c_r, 0.01, c_kl, c_mask)
+            adv_, ret_ = oadv.get_advantages_and_returns(c_val, rew_, c_mask, 1.0, 0.95)
+            adv_w = oadv.whiten_advantages([adv_], [c_mask])[0][0]
+            return (olos.policy_loss(c_lp, c_old, adv_w, action_mask=c_mask)[0],
+                    olos.value_loss(c_val + 0.1, c_val, ret_, action_mask=c_mask, clip_eps=0.2))
+
+        cpu_chain()
+        times = []
+        for _ in range(3):
+            t0 = time.perf_counter()
+            cpu_chain()
+            times.append(time.perf_counter() - t0)
+        med = sorted(times)[1]
+        res["config3.chain_cpu_baseline"] = {
+            "ms": med * 1e3, "tokens": padded, "tokens_per_s": padded / med, "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"the whole config 3 batch ({b} x {a} padded fp32): the oracle's restatement of the reference's op "
+                      f"sequence on torch CPU, median of 3 runs after a warm-up; {cpu_model()}"}
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side), torch.no_grad():
