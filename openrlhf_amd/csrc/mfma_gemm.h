@@ -289,7 +289,8 @@ struct NoLoads {
 // alternatives at 8192^3: one load per MFMA in those two k-steps (between the LDS reads) 2-4 %
 // slower; one per three MFMAs over k-steps 3, 0, 1, or any set that reaches into k-step 1, 1-4 %
 // slower (the barrier then waits for the last ones); all 16 in k-step 3 3-5 % slower. Cache-policy
-// bits on the loads change nothing (non-temporal: 7-20 % slower).
+// bits on the loads change nothing (non-temporal: 7-20 % slower), and neither does issuing them one
+// slot later in two of the four waves, so that at most two waves' loads meet at the CU's load path.
 constexpr uint32_t kDmaSlots3 = 0x5555u;
 constexpr uint32_t kDmaSlots0 = 0x5555u;
 constexpr uint32_t kDmaSlots1 = 0x0u;
