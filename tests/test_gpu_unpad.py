@@ -67,6 +67,22 @@ def test_unpad_mask_dtypes(mask_dtype):
     assert torch.equal(got[4].cpu(), want[4])
 
 
+def test_unpad_int32_and_strided_inputs():
+    from openrlhf_amd.models.ring_attn_utils import unpad_and_slice_tensor
+
+    g = torch.Generator().manual_seed(9)
+    mask = _mask("both", 11, 700, g)
+    seq = torch.randint(0, 1000, (11, 700), generator=g)
+    want = olay.unpad_and_slice_tensor(seq, mask)
+    seq_d = seq.to(torch.int32).t().contiguous().t().to(_dev())     # int32, column-major storage
+    mask_d = mask.t().contiguous().t().to(_dev())
+    got = unpad_and_slice_tensor(seq_d, mask_d, None)
+    assert got[0].dtype == torch.int32 and got[2].dtype == torch.int32
+    for w, gt in zip(want[:3], got[:3]):
+        assert torch.equal(gt.cpu().long(), w)
+    assert torch.equal(got[4].cpu(), want[4])
+
+
 def test_unpad_reference_docstring_example():
     """The example in the reference's docstring (ring_attn_utils.py:112-118)."""
     from openrlhf_amd.models.ring_attn_utils import unpad_and_slice_tensor
