@@ -229,6 +229,18 @@ __device__ __forceinline__ void issue_order() {
   __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
 }
 
+// Before the barrier that publishes a slab, its LDS-direct loads must have landed. The compiler's
+// own bookkeeping of these loads is not relied on (it left the wait out at one of the two barriers
+// of an unrolled iteration pair): loads retire in order, so allowing the YOUNGER loads that were
+// issued since (the 8 register loads of an operand carried in registers) to be outstanding waits
+// exactly for the slab.
+template <int YOUNGER>
+__device__ __forceinline__ void wait_slab_loads() {
+  static_assert(YOUNGER == 0 || YOUNGER == 8 || YOUNGER == 16, "8 register loads per operand and slab");
+  if (YOUNGER == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (YOUNGER == 8) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+}
+
 // One k-step with every instruction's place pinned: slot I = [LDS read I of the next fragments (I < 8)],
 // MFMA I, [whatever `loads` issues at slot I]; nothing moves across a slot's end.
 template <int DT, int I, class Reads, class Loads>
@@ -407,6 +419,7 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     mfma_step<DT>(acc, f0);
     issue_order<(A_REG ? 1 : 0) + (B_REG ? 1 : 0)>();
     // every wave holds its last fragments of `cur`; slab it + 1 is complete in `nxt`
+    if (!(A_REG && B_REG)) wait_slab_loads<(A_REG ? 8 : 0) + (B_REG ? 8 : 0)>();
     __syncthreads();
     // `cur` is free: slab it + 2 starts towards it now, its loads spread between the LDS reads
     // under the first MFMAs, and has until the next iteration's barrier. In the last iteration
@@ -450,6 +463,7 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
       pinned_step<DT>(acc, f0, rd, none, Slots16{});
     }
     // every wave holds its last fragments of `cur`; slab it + 1 is complete in `nxt`
+    wait_slab_loads<0>();
     __syncthreads();
     const SlabDma da2(a, row0_a, k2, cur, wave_u, lane), db2(b, row0_b, k2, cur + kSlabBytes, wave_u, lane);
     {
@@ -458,8 +472,71 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
       if (RESIDENT_OPERANDS) pinned_step<DT>(acc, f1, rd, none, Slots16{}); else pinned_step<DT>(acc, f1, rd, ld, Slots16{});
     }
   };
+  // The same iteration with one operand carried in registers, every instruction in a fixed slot:
+  // the register operand's slab it + 1 is written to LDS on the odd slots behind the LDS reads of
+  // k-steps 0 and 1 (four rows each), its slab it + 2 is fetched on the odd slots of k-step 2;
+  // the other operand's LDS-direct loads take the even slots of k-step 0 (B) or k-step 3 (A).
+  auto steady_mixed = [&](auto parity, int64_t it) {
+    constexpr int P = decltype(parity)::value;
+    char* cur = lds + P * kStageBytes;
+    char* nxt = lds + (1 - P) * kStageBytes;
+    const int64_t k1 = (it + 1) * kSlab, k2 = (it + 2) * kSlab;
+    const uint32_t lr = lane & 31u, lk = lane >> 5;
+    const SlabDma db(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);  // B's slab it + 1 (unused if B_REG)
+    auto stage_rows = [&](auto first) {  // rows FIRST .. FIRST + 3 on slots 9, 11, 13, 15
+      return [&, first](auto ic) {
+        constexpr int I = decltype(ic)::value, F = decltype(first)::value;
+        if constexpr (I >= 9 && (I & 1) == 1) {
+          constexpr int e = F + (I - 9) / 2;
+          if (A_REG) stage_slab<A_MN_MAJOR, e, e + 1>(ra, nxt, tid);
+          if (B_REG) stage_slab<B_MN_MAJOR, e, e + 1>(rb, nxt + kSlabBytes, tid);
+        }
+      };
+    };
+    {
+      FragReads rd{f1, cur, cur + kSlabBytes, 2, wm, wn, lr, lk};
+      auto stage = stage_rows(std::integral_constant<int, 0>{});
+      auto extra = [&](auto ic) {
+        constexpr int I = decltype(ic)::value;
+        if constexpr (!B_REG && (I & 1) == 0) db.issue(I / 2);
+        stage(ic);
+      };
+      pinned_step<DT>(acc, f0, rd, extra, Slots16{});
+    }
+    {
+      FragReads rd{f0, cur, cur + kSlabBytes, 4, wm, wn, lr, lk};
+      auto stage = stage_rows(std::integral_constant<int, 4>{});
+      pinned_step<DT>(acc, f1, rd, stage, Slots16{});
+    }
+    {
+      FragReads rd{f1, cur, cur + kSlabBytes, 6, wm, wn, lr, lk};
+      auto fetch = [&](auto ic) {
+        constexpr int I = decltype(ic)::value;
+        if constexpr ((I & 1) == 1) {
+          constexpr int i = I / 2;
+          if (A_REG) fetch_slab<A_MN_MAJOR, !A_MN_MAJOR, i, i + 1>(ra, a, row0_a, k2, tid);
+          if (B_REG) fetch_slab<B_MN_MAJOR, !B_MN_MAJOR, i, i + 1>(rb, b, row0_b, k2, tid);
+        }
+      };
+      pinned_step<DT>(acc, f0, rd, fetch, Slots16{});
+    }
+    // every wave holds its last fragments of `cur`; slab it + 1 is complete in `nxt`
+    wait_slab_loads<8>();
+    __syncthreads();
+    const SlabDma da(a, row0_a, it + 2 < full ? k2 : 0, cur, wave_u, lane);  // A's slab it + 2 (unused if A_REG)
+    {
+      FragReads rd{f0, nxt, nxt + kSlabBytes, 0, wm, wn, lr, lk};
+      auto extra = [&](auto ic) {
+        constexpr int I = decltype(ic)::value;
+        if constexpr (!A_REG && (I & 1) == 0) da.issue(I / 2);
+      };
+      pinned_step<DT>(acc, f1, rd, extra, Slots16{});
+    }
+  };
   auto iteration = [&](auto parity, int64_t it) {
-    if constexpr (KK) steady_kk(parity, it); else steady(parity, it);
+    if constexpr (KK) steady_kk(parity, it);
+    else if constexpr (A_REG != B_REG) steady_mixed(parity, it);
+    else steady(parity, it);
   };
   for (; s + 2 < full; s += 2) {  // pairs of steady iterations: the buffers' addresses are constants
     iteration(std::integral_constant<int, 0>{}, s);

@@ -188,6 +188,30 @@ def test_lmhead_full_size(cuda):
     assert (ent[pick.to(cuda)].detach().cpu().double() - ref_ent).abs().max().item() <= 2e-3
 
 
+def test_lmhead_backward_repeats_bit_for_bit(cuda):
+    """The three products of the backward at full size, with every CU busy and the slab loads at
+    their longest latencies, give the same bits every time (a slab published before its loads had
+    landed would show up as a run that differs), and so does a product deep enough for 2374 slabs."""
+    from openrlhf_amd.models.utils import lm_head_logprobs_and_entropy
+
+    n, hdim, vocab = 4096, 4096, 151936
+    g = torch.Generator(device=cuda).manual_seed(23)
+    hidden = torch.randn(n, hdim, generator=g, device=cuda).to(torch.bfloat16)
+    weight = (torch.randn(vocab, hdim, generator=g, device=cuda) * (3.0 / hdim ** 0.5)).to(torch.bfloat16)
+    labels = torch.randint(0, vocab, (n,), generator=g, device=cuda)
+    g_lp, g_ent = torch.randn(n, generator=g, device=cuda), torch.randn(n, generator=g, device=cuda)
+    for chunk_mib in (None, 2048):  # five chunks of the logits gradient; one chunk (the deepest dHidden product)
+        runs = []
+        for _ in range(3):
+            hd, wd = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
+            lp, ent = lm_head_logprobs_and_entropy(hd, wd, labels, 1.0, backward_chunk_mib=chunk_mib)
+            torch.autograd.backward([lp, ent], [g_lp, g_ent])
+            runs.append((lp.detach(), ent.detach(), hd.grad, wd.grad))
+        for other in runs[1:]:
+            for a, b in zip(runs[0], other):
+                assert torch.equal(a, b)
+
+
 def test_lmhead_every_row_masked(cuda):
     """A row mask that leaves nothing: zeros out, zero gradients, nothing launched on an empty batch."""
     from openrlhf_amd.models.utils import lm_head_logprobs_and_entropy
