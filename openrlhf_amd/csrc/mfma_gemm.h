@@ -187,22 +187,6 @@ __device__ __forceinline__ void load_frags(Frags& f, const char* slab_a, const c
   }
 }
 
-// The same reads with the 8 loads of a slab's LDS-direct transfer between them, in program order:
-// the compiler keeps LDS-direct loads and LDS reads in order (both touch LDS), so this is what
-// spreads the loads under the MFMAs instead of leaving them as one block in front of the step.
-__device__ __forceinline__ void load_frags_between_dma(Frags& f, const char* slab_a, const char* slab_b, int ks, uint32_t wm,
-                                                       uint32_t wn, uint32_t lane, const SlabDma& d) {
-  const uint32_t lr = lane & 31u, lk = lane >> 5;
-#pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const uint32_t ra = wm * 128u + t * 32u + lr, rb = wn * 128u + t * 32u + lr;
-    d.issue(2 * t);
-    f.a[t] = *(const u32x4*)(slab_a + ra * 128u + (((ks * 2u + lk) ^ swz(ra)) << 4));
-    d.issue(2 * t + 1);
-    f.b[t] = *(const u32x4*)(slab_b + rb * 128u + (((ks * 2u + lk) ^ swz(rb)) << 4));
-  }
-}
-
 template <int DT>
 __device__ __forceinline__ void mfma_step(f32x16 (&acc)[4][4], const Frags& f) {
 #pragma unroll
@@ -215,9 +199,8 @@ __device__ __forceinline__ void mfma_step(f32x16 (&acc)[4][4], const Frags& f) {
 // Issue order of one k-step of the steady loop: the eight LDS reads of the next fragments, and
 // N_VMEM global loads into registers per read, go out under the first eight MFMAs; the other eight
 // MFMAs cover their latency. Left to itself the scheduler sinks the reads to the end of the step,
-// where the next step's first MFMA waits for them with the matrix pipe idle. (LDS-direct loads
-// match no group; they keep their program order among the LDS reads, which is what
-// load_frags_between_dma uses.)
+// where the next step's first MFMA waits for them with the matrix pipe idle. (Used by the
+// iteration with two register operands only; the others pin every slot.)
 template <int N_VMEM>
 __device__ __forceinline__ void issue_order() {
 #pragma unroll
@@ -314,11 +297,9 @@ static_assert(__builtin_popcount(kDmaSlots3) + __builtin_popcount(kDmaSlots0) + 
 // Iteration s multiplies slab s out of one LDS buffer while slab s + 1 is (or arrives) in the other:
 //  * a K-major operand's slab is loaded straight into LDS (SlabDma): slab s + 2 as soon as the
 //    barrier of iteration s has freed the buffer slab s was read from, a whole iteration before
-//    the barrier that publishes it, its loads placed between that k-step's LDS reads so that each
-//    goes out under an MFMA and the matrix pipe never waits for a burst of address arithmetic and
-//    load issue (when both operands are K-major every instruction of the iteration has a fixed
-//    slot instead: steady_kk below); only a slab that crosses the end of the depth goes through
-//    registers (masking);
+//    the barrier that publishes it, its loads on fixed slots between the MFMAs (steady_kk,
+//    steady_mixed below) so that the matrix pipe never waits for a burst of address arithmetic
+//    and load issue; only a slab that crosses the end of the depth goes through registers (masking);
 //  * an MN-major operand's slab s + 1 sits in registers (fetched during iteration s - 1), is
 //    transposed and written to LDS during the first k-steps, and the fetch of slab s + 2 is issued
 //    into the registers it leaves.
@@ -387,51 +368,38 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
   int64_t s = 0;
 
   // One steady-state iteration: slab `it` in buffer PARITY; slab it + 1 is whole and lands in (or
-  // is staged into) the other buffer. Needs it + 1 < full.
+  // is staged into) the other buffer. Needs it + 1 < full. This version is for two operands
+  // carried in registers (no caller of the library has two MN-major operands): the issue order
+  // is left to the scheduler groups of issue_order.
   auto steady = [&](auto parity, int64_t it) {
     constexpr int P = decltype(parity)::value;
     char* cur = lds + P * kStageBytes;
     char* nxt = lds + (1 - P) * kStageBytes;
-    const int64_t k1 = (it + 1) * kSlab, k2 = (it + 2) * kSlab;
-    const SlabDma db(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);  // B's slab it + 1 (unused if B_REG)
+    const int64_t k2 = (it + 2) * kSlab;
     // k-step 0
-    if (!B_REG && !RESIDENT_OPERANDS) {
-      load_frags_between_dma(f1, cur, cur + kSlabBytes, 1, wm, wn, lane, db);
-    } else {
-      load_frags(f1, cur, cur + kSlabBytes, 1, wm, wn, lane);
-    }
-    if (A_REG) stage_slab<A_MN_MAJOR, 0, 4>(ra, nxt, tid);
-    if (B_REG) stage_slab<B_MN_MAJOR, 0, 4>(rb, nxt + kSlabBytes, tid);
+    load_frags(f1, cur, cur + kSlabBytes, 1, wm, wn, lane);
+    stage_slab<A_MN_MAJOR, 0, 4>(ra, nxt, tid);
+    stage_slab<B_MN_MAJOR, 0, 4>(rb, nxt + kSlabBytes, tid);
     mfma_step<DT>(acc, f0);
     issue_order<0>();
     __builtin_amdgcn_sched_barrier(0);
     // k-step 1
     load_frags(f0, cur, cur + kSlabBytes, 2, wm, wn, lane);
-    if (A_REG) stage_slab<A_MN_MAJOR, 4, 8>(ra, nxt, tid);
-    if (B_REG) stage_slab<B_MN_MAJOR, 4, 8>(rb, nxt + kSlabBytes, tid);
+    stage_slab<A_MN_MAJOR, 4, 8>(ra, nxt, tid);
+    stage_slab<B_MN_MAJOR, 4, 8>(rb, nxt + kSlabBytes, tid);
     mfma_step<DT>(acc, f1);
     issue_order<0>();
     __builtin_amdgcn_sched_barrier(0);
     // k-step 2
     load_frags(f1, cur, cur + kSlabBytes, 3, wm, wn, lane);
-    if (A_REG) fetch_slab<A_MN_MAJOR, !A_MN_MAJOR>(ra, a, row0_a, k2, tid);
-    if (B_REG) fetch_slab<B_MN_MAJOR, !B_MN_MAJOR>(rb, b, row0_b, k2, tid);
+    fetch_slab<A_MN_MAJOR, !A_MN_MAJOR>(ra, a, row0_a, k2, tid);
+    fetch_slab<B_MN_MAJOR, !B_MN_MAJOR>(rb, b, row0_b, k2, tid);
     mfma_step<DT>(acc, f0);
-    issue_order<(A_REG ? 1 : 0) + (B_REG ? 1 : 0)>();
+    issue_order<2>();
     // every wave holds its last fragments of `cur`; slab it + 1 is complete in `nxt`
-    if (!(A_REG && B_REG)) wait_slab_loads<(A_REG ? 8 : 0) + (B_REG ? 8 : 0)>();
     __syncthreads();
-    // `cur` is free: slab it + 2 starts towards it now, its loads spread between the LDS reads
-    // under the first MFMAs, and has until the next iteration's barrier. In the last iteration
-    // there is no such slab: slab 0 is loaded again instead of branching (nobody reads it; whatever
-    // touches this buffer next waits for its own later loads, and loads return in order).
     // k-step 3, over the read of the next slab's first fragments
-    if (!A_REG && !RESIDENT_OPERANDS) {
-      const SlabDma da(a, row0_a, it + 2 < full ? k2 : 0, cur, wave_u, lane);
-      load_frags_between_dma(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane, da);
-    } else {
-      load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
-    }
+    load_frags(f0, nxt, nxt + kSlabBytes, 0, wm, wn, lane);
     mfma_step<DT>(acc, f1);
     issue_order<0>();
     __builtin_amdgcn_sched_barrier(0);
