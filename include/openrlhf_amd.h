@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 21
+#define ORLHF_ABI_VERSION 22
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -169,65 +169,59 @@ int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logits, int dty
                                   const uint8_t* row_mask, orlhf_stream_t stream);
 
 /*
- * lm-head + log-prob + entropy with the logits never in memory: what Actor.forward does between
- * the last hidden states and the action log-probs (openrlhf/models/actor.py:263-285: the model's
- * lm_head projection, output["logits"].to(float32), compute_entropy, log_probs_from_logits) as
- * matrix-core tiles whose logits are folded into per-token statistics in registers.
- *   logits[i, v] = sum_h hidden[i, h] * weight[v, h]        (fp32 accumulation, never stored)
+ * lm-head + log-prob + entropy without the [n_rows, vocab] logits (or with as much of them as the
+ * caller has room for): what Actor.forward does between the last hidden states and the action
+ * log-probs (openrlhf/models/actor.py:263-285: the model's lm_head projection,
+ * output["logits"].to(float32), compute_entropy, log_probs_from_logits) as matrix-core tiles whose
+ * logits are folded into per-token statistics in registers.
+ *   logits[i, v] = round_to_dtype(sum_h hidden[i, h] * weight[v, h])   (fp32 accumulation; the 16-bit
+ *                  rounding is the one the reference's lm_head output has before its fp32 up-cast)
  *   logprob / entropy / row_stats as orlhf_logprob_entropy_fwd on those logits
  *   hidden  [n_rows, hidden_dim] and weight [vocab, hidden_dim] (the nn.Linear layout), bf16 or
- *           fp16 (`dtype`), element stride 1, row strides in elements; both 4-byte aligned with
- *           even strides and an even hidden_dim (else ORLHF_ERR_UNSUPPORTED)
+ *           fp16 (`dtype`), element stride 1, row strides in elements below 2^23; both 4-byte
+ *           aligned with even strides and an even hidden_dim (else ORLHF_ERR_UNSUPPORTED)
  *   labels  int64 [n_rows] (-100: logprob 0; any other label outside [0, vocab): NaN)
- *   workspace: orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, 0) bytes, 256-byte aligned
- * The reference rounds the logits to the 16-bit dtype before the fp32 up-cast; here they stay fp32,
- * which is the value-preserving side (the same decision as for 16-bit logits above).
+ *   kept_logits [n_rows, kept_stride] of `dtype`, or NULL with kept_cols = 0: the logits of the
+ *           first kept_cols vocabulary columns are stored there (the tiles produce them anyway), so
+ *           that the backward need not recompute them. kept_cols is a multiple of 256, at most the
+ *           vocabulary rounded up to 256 (then all logits are kept; columns past the vocabulary hold
+ *           zeros); kept_stride >= kept_cols, a multiple of 8; 16-byte aligned. Results do not
+ *           depend on kept_cols.
+ *   workspace: orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, kept_cols, 0) bytes, 256-byte aligned
  */
-int64_t orlhf_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab, int backward);
+int64_t orlhf_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab, int64_t kept_cols,
+                                     int backward);
 int orlhf_lmhead_logprob_entropy_fwd(const void* hidden, const void* weight, int dtype, int64_t n_rows,
                                      int64_t hidden_dim, int64_t vocab, int64_t hidden_stride,
                                      int64_t weight_stride, const int64_t* labels, double temperature,
-                                     float* logprob, float* entropy, float* row_stats, void* workspace,
+                                     float* logprob, float* entropy, float* row_stats, void* kept_logits,
+                                     int64_t kept_cols, int64_t kept_stride, void* workspace,
                                      int64_t workspace_bytes, orlhf_stream_t stream);
 /*
  * Backward of the above down to the hidden states and the lm_head weight (torch autograd through
  * openrlhf/models/actor.py:263-285 and the projection): with P = d(loss)/d(logits) as in
  * orlhf_logprob_entropy_bwd, rounded to `dtype` (the dtype the reference's logits gradient has),
  *   grad_hidden[i, h] = sum_v P[i, v] * weight[v, h]         grad_weight[v, h] = sum_i P[i, v] * hidden[i, h]
- * both accumulated in fp32 and rounded once to `dtype`. The vocabulary is processed in chunks: per
- * chunk the logits tiles are recomputed, P is written to the workspace and multiplied twice on the
- * matrix cores. grad_hidden [n_rows, hidden_dim] / grad_weight [vocab, hidden_dim]: either may be
- * NULL; row strides in elements. row_stats: from the forward. Rows whose upstream gradients are
- * both 0 contribute exact zeros.
- *   workspace: orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, 1) bytes or more (a larger
- *   workspace means wider chunks), 256-byte aligned.
+ * both accumulated in fp32 and rounded once to `dtype`. Over the kept columns P is written OVER
+ * kept_logits (the logits are gone afterwards); the rest of the vocabulary is processed in chunks:
+ * per chunk the logits tiles are recomputed, P is written to the workspace and multiplied twice on
+ * the matrix cores. The gradients are the same bits for every kept_cols and every chunk width (the
+ * kept logits are what the recompute rounds to, and grad_hidden's sum over the vocabulary is
+ * continued in the accumulators in one fixed order). kept_logits / kept_cols / kept_stride: as
+ * passed to the forward of the same inputs. grad_hidden [n_rows, hidden_dim] / grad_weight
+ * [vocab, hidden_dim]: either may be NULL; row strides in elements. row_stats: from the forward.
+ * Rows whose upstream gradients are both 0 contribute exact zeros.
+ *   workspace: orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, kept_cols, 1) bytes or more
+ *   (a larger workspace means wider chunks), 256-byte aligned.
  */
 int orlhf_lmhead_logprob_entropy_bwd(const void* hidden, const void* weight, int dtype, int64_t n_rows,
                                      int64_t hidden_dim, int64_t vocab, int64_t hidden_stride,
                                      int64_t weight_stride, const int64_t* labels, double temperature,
                                      const float* g_logprob, const float* g_entropy,
-                                     const float* row_stats, void* grad_hidden,
-                                     int64_t grad_hidden_stride, void* grad_weight,
-                                     int64_t grad_weight_stride, void* workspace,
+                                     const float* row_stats, void* kept_logits, int64_t kept_cols,
+                                     int64_t kept_stride, void* grad_hidden, int64_t grad_hidden_stride,
+                                     void* grad_weight, int64_t grad_weight_stride, void* workspace,
                                      int64_t workspace_bytes, orlhf_stream_t stream);
-
-/*
- * Measurement aid, no counterpart in the reference: the plain product of two K-major operands,
- * a [m, k] (row stride lda) and b [n, k] (row stride ldb), bf16 or fp16, through the matrix-core
- * tile the lm-head entry points above are built on, one 256 x 256 tile per workgroup. Nothing but
- * the product is done: thread t of tile (i, j) leaves the sum of its 256 accumulators in
- * tile_sums[(i * ceil(n / 256) + j) * 256 + t] (float, ceil(m / 256) * ceil(n / 256) * 256
- * entries), so the 256 sums of a tile add up to the sum of that block of a * b^T. With
- * resident_operands != 0 the steady loop loads nothing (every slab is multiplied out of what the
- * LDS buffers hold after the first two slabs; the sums are meaningless): the time of that run is
- * what the same LDS reads, MFMAs and barriers take on their own, the ceiling the tile can be read
- * against on a given GPU and clock. A row stride of 0 makes every row of that operand its first
- * row (all loads of the steady loop then hit the L1: the cost of issuing them and writing LDS,
- * without the cost of fetching). Operands need 4-byte aligned bases and even row strides.
- */
-int orlhf_matrix_tile_probe(const void* a, const void* b, int dtype, int64_t m, int64_t n, int64_t k,
-                            int64_t lda, int64_t ldb, int resident_operands, float* tile_sums,
-                            orlhf_stream_t stream);
 
 /*
  * The loss assembly of the PPO actor step (openrlhf/trainer/ray/ppo_actor.py:305-352) folded into
@@ -703,6 +697,50 @@ int orlhf_unpad_sequences(const int64_t* sequences, const void* mask, int mask_d
  */
 int orlhf_pad_by_indices(const void* src, int elem_bytes, int64_t n, int64_t inner,
                          const int64_t* indices, int64_t n_dst, void* dst, orlhf_stream_t stream);
+
+/*
+ * The inverse, flash-attn's index_first_axis (what unpad_input applies to every per-token tensor,
+ * openrlhf/models/ring_attn_utils.py:130-140, and the gradient of pad_input): row i of dst (n rows
+ * of `inner` elements) = row indices[i] of src (n_src rows); an index outside [0, n_src) gives a
+ * row of zeros.
+ */
+int orlhf_gather_by_indices(const void* src, int elem_bytes, int64_t n_src, int64_t inner,
+                            const int64_t* indices, int64_t n, void* dst, orlhf_stream_t stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Diagnostics. Not part of the reference-citing interface above: nothing of the reference maps to
+ * these two; they exist so that the matrix-core tile the lm-head entry points are built on can be
+ * tested and timed on its own (bench.py --workload matrix_tile, tests/test_gpu_matrix_tile.py).
+ * ------------------------------------------------------------------------------------------ */
+
+/*
+ * c [m, n] (fp32, row stride ldc) = or += a * b^T through that tile, one 256 x 256 tile per
+ * workgroup: a is [m, k] with row stride lda (a_mn_major = 0) or stored as [k, m] with row stride
+ * lda (a_mn_major = 1); b likewise with n. accumulate != 0 continues the sums found in c inside the
+ * accumulators (the same bits as one product over the concatenated depth). bf16 or fp16 operands,
+ * 4-byte aligned bases, even row strides below 2^23.
+ */
+int orlhf_matrix_tile_product(const void* a, const void* b, int dtype, int64_t m, int64_t n, int64_t k,
+                              int64_t lda, int64_t ldb, int a_mn_major, int b_mn_major, int accumulate,
+                              float* c, int64_t ldc, orlhf_stream_t stream);
+
+/*
+ * The plain product of two K-major operands,
+ * a [m, k] (row stride lda) and b [n, k] (row stride ldb), bf16 or fp16, through the matrix-core
+ * tile the lm-head entry points above are built on, one 256 x 256 tile per workgroup. Nothing but
+ * the product is done: thread t of tile (i, j) leaves the sum of its 256 accumulators in
+ * tile_sums[(i * ceil(n / 256) + j) * 256 + t] (float, ceil(m / 256) * ceil(n / 256) * 256
+ * entries), so the 256 sums of a tile add up to the sum of that block of a * b^T. With
+ * resident_operands != 0 the steady loop loads nothing (every slab is multiplied out of what the
+ * LDS buffers hold after the first two slabs; the sums are meaningless): the time of that run is
+ * what the same LDS reads, MFMAs and barriers take on their own, the ceiling the tile can be read
+ * against on a given GPU and clock. A row stride of 0 makes every row of that operand its first
+ * row (all loads of the steady loop then hit the L1: the cost of issuing them and writing LDS,
+ * without the cost of fetching). Operands need 4-byte aligned bases and even row strides.
+ */
+int orlhf_matrix_tile_probe(const void* a, const void* b, int dtype, int64_t m, int64_t n, int64_t k,
+                            int64_t lda, int64_t ldb, int resident_operands, float* tile_sums,
+                            orlhf_stream_t stream);
 
 #ifdef __cplusplus
 }

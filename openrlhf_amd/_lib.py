@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 21
+ABI_VERSION = 22
 
 
 class Norm(Structure):
@@ -77,10 +77,12 @@ SIGNATURES = {
     "orlhf_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P]),
     "orlhf_logprob_entropy_fwd_bwd_max_vocab": (I64, [c_int]),
     "orlhf_logprob_entropy_fwd_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P, P]),
-    "orlhf_lmhead_workspace_bytes": (I64, [I64, I64, I64, c_int]),
-    "orlhf_lmhead_logprob_entropy_fwd": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, P, c_double, P, P, P, P, I64, P]),
-    "orlhf_lmhead_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, P, c_double, P, P, P, P, I64, P,
-                                                 I64, P, I64, P]),
+    "orlhf_lmhead_workspace_bytes": (I64, [I64, I64, I64, I64, c_int]),
+    "orlhf_lmhead_logprob_entropy_fwd": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, P, c_double, P, P, P, P, I64, I64,
+                                                 P, I64, P]),
+    "orlhf_lmhead_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, P, c_double, P, P, P, P, I64, I64,
+                                                 P, I64, P, I64, P, I64, P]),
+    "orlhf_matrix_tile_product": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, c_int, c_int, c_int, P, I64, P]),
     "orlhf_matrix_tile_probe": (c_int, [P, P, c_int, I64, I64, I64, I64, I64, c_int, P, P]),
     "orlhf_policy_step_fwd_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, POINTER(StepTerms), P, P, P, P]),
     "orlhf_actor_step_gather": (c_int, [P, P, c_int, P, I64, I64, I64, I64, P, P, P, P, P, P, c_float, P, P, P, P, P, P, P, P,
@@ -123,6 +125,7 @@ SIGNATURES = {
     "orlhf_mask_row_counts": (c_int, [P, c_int, I64, I64, P, P]),
     "orlhf_unpad_sequences": (c_int, [P, P, c_int, I64, I64, P, I64, P, P, P, P, P]),
     "orlhf_pad_by_indices": (c_int, [P, c_int, I64, I64, P, I64, P, P]),
+    "orlhf_gather_by_indices": (c_int, [P, c_int, I64, I64, P, I64, P, P]),
     "orlhf_sequence_logps_fwd": (c_int, [P, P, c_int, P, I64, I64, P, P, P, P]),
     "orlhf_sequence_logps_bwd": (c_int, [P, P, P, c_int, P, P, I64, I64, P, P]),
     "orlhf_pair_loss_fwd": (c_int, [P, P, P, P, I64, c_int, c_double, c_double, P, P, P, P]),

@@ -343,6 +343,21 @@ __global__ __launch_bounds__(kBlock) void scatter_index_kernel(const E* __restri
   }
 }
 
+// dst[i * inner + j] = src[indices[i] * inner + j] (flash-attn's index_first_axis): V = the widest
+// unit (1 to 16 bytes) that divides a row and both bases, `units` of them per row; an index outside
+// [0, n_src) gives zeros.
+template <typename V>
+__global__ __launch_bounds__(kBlock) void gather_index_kernel(const V* __restrict__ src, const int64_t* __restrict__ indices,
+                                                              int64_t n, int64_t units, int64_t n_src, V* __restrict__ dst) {
+  const int64_t total = n * units;
+  for (int64_t e = (int64_t)blockIdx.x * kBlock + threadIdx.x; e < total; e += (int64_t)gridDim.x * kBlock) {
+    const int64_t i = e / units, j = e - i * units, from = indices[i];
+    V v{};
+    if ((uint64_t)from < (uint64_t)n_src) v = src[from * units + j];
+    dst[e] = v;
+  }
+}
+
 __global__ __launch_bounds__(kBlock) void zero_bytes_kernel(char* __restrict__ dst, int64_t bytes) {
   const int64_t groups = bytes / 16;  // dst is 16-byte aligned (checked by the caller)
   for (int64_t g = (int64_t)blockIdx.x * kBlock + threadIdx.x; g < groups; g += (int64_t)gridDim.x * kBlock)
@@ -524,5 +539,37 @@ extern "C" int orlhf_pad_by_indices(const void* src, int elem_bytes, int64_t n, 
     default: hipLaunchKernelGGL(scatter_index_kernel<uint64_t>, grid, block, 0, s, (const uint64_t*)src, indices, n, inner, n_dst, (uint64_t*)dst); break;
   }
   ORLHF_CHECK_LAUNCH("orlhf_pad_by_indices");
+  return ORLHF_OK;
+}
+
+extern "C" int orlhf_gather_by_indices(const void* src, int elem_bytes, int64_t n_src, int64_t inner, const int64_t* indices,
+                                       int64_t n, void* dst, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(n >= 0 && inner >= 1 && n_src >= 0, "gather_by_indices: n=%lld inner=%lld n_src=%lld", (long long)n,
+                  (long long)inner, (long long)n_src);
+  ORLHF_CHECK_ARG(elem_bytes == 1 || elem_bytes == 2 || elem_bytes == 4 || elem_bytes == 8,
+                  "row layout: element size %d (1, 2, 4 or 8 bytes)", elem_bytes);
+  if (n == 0) return ORLHF_OK;
+  ORLHF_CHECK_ARG(dst != nullptr && indices != nullptr && (src != nullptr || n_src == 0), "gather_by_indices: NULL argument");
+  hipStream_t s = (hipStream_t)stream;
+  const int64_t row_bytes = inner * elem_bytes;
+  const uintptr_t both = (uintptr_t)src | (uintptr_t)dst | (uintptr_t)row_bytes;
+  const dim3 block(kBlock);
+  if ((both & 15u) == 0) {
+    hipLaunchKernelGGL(gather_index_kernel<u32x4>, dim3(flat_grid(n * (row_bytes / 16))), block, 0, s, (const u32x4*)src, indices,
+                       n, row_bytes / 16, n_src, (u32x4*)dst);
+  } else if ((both & 7u) == 0) {
+    hipLaunchKernelGGL(gather_index_kernel<uint64_t>, dim3(flat_grid(n * (row_bytes / 8))), block, 0, s, (const uint64_t*)src,
+                       indices, n, row_bytes / 8, n_src, (uint64_t*)dst);
+  } else if ((both & 3u) == 0) {
+    hipLaunchKernelGGL(gather_index_kernel<uint32_t>, dim3(flat_grid(n * (row_bytes / 4))), block, 0, s, (const uint32_t*)src,
+                       indices, n, row_bytes / 4, n_src, (uint32_t*)dst);
+  } else if ((both & 1u) == 0) {
+    hipLaunchKernelGGL(gather_index_kernel<uint16_t>, dim3(flat_grid(n * (row_bytes / 2))), block, 0, s, (const uint16_t*)src,
+                       indices, n, row_bytes / 2, n_src, (uint16_t*)dst);
+  } else {
+    hipLaunchKernelGGL(gather_index_kernel<uint8_t>, dim3(flat_grid(n * row_bytes)), block, 0, s, (const uint8_t*)src, indices, n,
+                       row_bytes, n_src, (uint8_t*)dst);
+  }
+  ORLHF_CHECK_LAUNCH("orlhf_gather_by_indices");
   return ORLHF_OK;
 }

@@ -97,14 +97,24 @@ class _PadByIndices(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g):
         (indices,) = ctx.saved_tensors
-        return g.index_select(0, indices), None, None
+        g = g.contiguous()
+        inner = 1
+        for d in g.shape[1:]:
+            inner *= d
+        out = torch.empty((indices.numel(),) + tuple(g.shape[1:]), dtype=g.dtype, device=g.device)
+        with _lib.on_device(g.device):
+            call("orlhf_gather_by_indices", ptr(g), g.element_size(), g.shape[0], max(inner, 1), ptr(indices),
+                 indices.numel(), ptr(out), stream_of(g.device))
+        return out, None, None
 
 
 def gather_and_pad_tensor(tensor: torch.Tensor, ring_attn_group, ring_attn_pad_len, indices: torch.Tensor,
                           batch: int, seqlen: int) -> torch.Tensor:
-    """``[1, Ttot, ...]`` per-token values back on the ``[batch, seqlen, ...]`` grid: zeros, then
+    """``[1, Ttot, ...]`` per-token values back on the ``[batch, seqlen]`` grid: zeros, then
     position ``indices[i]`` receives token i (flash-attn's pad_input, as
-    openrlhf/models/ring_attn_utils.py:181 applies it). Differentiable in ``tensor``."""
+    openrlhf/models/ring_attn_utils.py:181 applies it to the transposed ``[Ttot, 1, ...]`` tensor,
+    followed by ``.squeeze(-1)``: ``[1, Ttot]`` gives ``[batch, seqlen]``, ``[1, Ttot, V]`` gives
+    ``[batch, seqlen, 1, V]`` as in the reference). Differentiable in ``tensor``."""
     _no_ring(ring_attn_group)
     if ring_attn_pad_len:
         raise NotImplementedError("one GPU: ring_attn_pad_len must be 0")
@@ -117,4 +127,4 @@ def gather_and_pad_tensor(tensor: torch.Tensor, ring_attn_group, ring_attn_pad_l
     if values.element_size() not in (1, 2, 4, 8):
         raise TypeError(f"unsupported dtype {values.dtype}")
     out = _PadByIndices.apply(values, indices.to(torch.int64).contiguous(), batch * seqlen)
-    return out.view(batch, seqlen, *values.shape[1:])
+    return out.view(batch, seqlen, 1, *values.shape[1:]).squeeze(-1)

@@ -195,13 +195,47 @@ def compute_entropy(logits: torch.Tensor, inplace_backward: bool = False) -> tor
     return _LogprobEntropy.apply(logits, None, 1.0, False, True, inplace_backward)[1]
 
 
-# ------------------------------------------------------------------ lm-head + log-prob, logits never stored
+# ------------------------------------------------------------------ lm-head + log-prob, logits not stored
+def _index_rows(src: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
+    """src[indices] along the first axis (rows of any width) with the library's gather kernel."""
+    src = src.contiguous()
+    inner = src[0].numel() if src.shape[0] > 0 else 1
+    out = torch.empty((indices.numel(),) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
+    with _lib.on_device(src.device):
+        call("orlhf_gather_by_indices", ptr(src), src.element_size(), src.shape[0], max(inner, 1), ptr(indices),
+             indices.numel(), ptr(out), stream_of(src.device))
+    return out
+
+
+def _scatter_rows(values: torch.Tensor, indices: torch.Tensor, n_dst: int) -> torch.Tensor:
+    """zeros(n_dst, ...) with rows ``indices`` set to ``values`` (the library's pad_by_indices)."""
+    values = values.contiguous()
+    inner = values[0].numel() if values.shape[0] > 0 else 1
+    out = torch.empty((n_dst,) + tuple(values.shape[1:]), dtype=values.dtype, device=values.device)
+    with _lib.on_device(values.device):
+        call("orlhf_pad_by_indices", ptr(values), values.element_size(), values.shape[0], max(inner, 1), ptr(indices),
+             n_dst, ptr(out), stream_of(values.device))
+    return out
+
+
+def _kept_columns(n_rows: int, vocab: int, keep_logits_mib) -> int:
+    """How many vocabulary columns of 16-bit logits (whole tiles of 256, row pitch columns + 64) a
+    budget in MiB holds for n_rows tokens; None keeps nothing."""
+    if not keep_logits_mib or n_rows == 0:
+        return 0
+    vpad = (vocab + 255) // 256 * 256
+    cols = int(keep_logits_mib * (1 << 20)) // (2 * n_rows) - 64
+    return max(0, min(vpad, cols // 256 * 256))
+
+
 class _LmHeadLogprobEntropy(torch.autograd.Function):
-    """(hidden states, lm_head weight) -> (log-prob of label, entropy) on matrix-core tiles."""
+    """(hidden states, lm_head weight) -> (log-prob of label, entropy) on matrix-core tiles.
+    ``keep`` (int64 row indices or None): only those rows of hidden / labels take part; the outputs
+    of the others are 0 and they get zero gradient."""
 
     @staticmethod
-    def forward(ctx, hidden, weight, labels, temperature, backward_chunk_mib=None):
-        dev = require_gpu(hidden, weight, labels)
+    def forward(ctx, hidden, weight, labels, temperature, backward_chunk_mib=None, keep_logits_mib=None, keep=None):
+        dev = require_gpu(hidden, weight, labels, keep)
         ctx.backward_chunk_mib = backward_chunk_mib
         if hidden.dtype != weight.dtype or hidden.dtype not in (torch.bfloat16, torch.float16):
             raise TypeError(f"hidden ({hidden.dtype}) and weight ({weight.dtype}) must both be bfloat16 or float16")
@@ -211,50 +245,74 @@ class _LmHeadLogprobEntropy(torch.autograd.Function):
             raise ValueError(f"labels shape {tuple(labels.shape)} != ({hidden.shape[0]},)")
         h = hidden.detach()
         w = weight.detach()
+        lab = labels.to(torch.int64).contiguous()
+        n_all = h.shape[0]
+        if keep is not None:
+            h, lab = _index_rows(h, keep), _index_rows(lab, keep)
         h = h if h.stride(1) == 1 and h.stride(0) % 2 == 0 and h.data_ptr() % 4 == 0 else h.contiguous()
         w = w if w.stride(1) == 1 and w.stride(0) % 2 == 0 and w.data_ptr() % 4 == 0 else w.contiguous()
         n, hdim = h.shape
         vocab = w.shape[0]
-        lab = labels.to(torch.int64).contiguous()
         code = _lib.dtype_code(h)
         opts = dict(device=dev, dtype=torch.float32)
         logprob, entropy, stats = torch.empty(n, **opts), torch.empty(n, **opts), torch.empty(n, 4, **opts)
         lib = _lib.load()
-        ws = torch.empty(lib.orlhf_lmhead_workspace_bytes(n, hdim, vocab, 0), dtype=torch.uint8, device=dev)
+        want_grad = ctx.needs_input_grad[0] or ctx.needs_input_grad[1]
+        kept_cols = _kept_columns(n, vocab, keep_logits_mib) if want_grad else 0
+        kept = torch.empty((n, kept_cols + 64), dtype=h.dtype, device=dev) if kept_cols > 0 else None
+        kept_ld = kept_cols + 64 if kept_cols > 0 else 0
+        ws = torch.empty(lib.orlhf_lmhead_workspace_bytes(n, hdim, vocab, kept_cols, 0), dtype=torch.uint8, device=dev)
         with _lib.on_device(dev):
             call("orlhf_lmhead_logprob_entropy_fwd", ptr(h), ptr(w), code, n, hdim, vocab, h.stride(0), w.stride(0),
-                 ptr(lab), float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(ws), ws.numel(), stream_of(dev))
+                 ptr(lab), float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(kept), kept_cols, kept_ld,
+                 ptr(ws), ws.numel(), stream_of(dev))
         ctx.temperature = float(temperature)
+        ctx.kept, ctx.kept_cols, ctx.kept_ld = kept, kept_cols, kept_ld
+        ctx.n_all = n_all
         ctx.set_materialize_grads(False)
-        ctx.save_for_backward(h, w, lab, stats)
+        ctx.save_for_backward(h, w, lab, stats, keep)
+        if keep is not None:
+            logprob, entropy = _scatter_rows(logprob, keep, n_all), _scatter_rows(entropy, keep, n_all)
         return logprob, entropy
 
     @staticmethod
     def backward(ctx, g_logprob, g_entropy):
-        h, w, lab, stats = ctx.saved_tensors
+        h, w, lab, stats, keep = ctx.saved_tensors
         need_h, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
         if (g_logprob is None and g_entropy is None) or not (need_h or need_w):
-            return None, None, None, None, None
+            return None, None, None, None, None, None, None
+        if ctx.kept_cols > 0 and ctx.kept is None:
+            raise RuntimeError("the stored logits of this lm-head call were turned into their gradient by an earlier "
+                               "backward; call it again (or use keep_logits_mib=None) to differentiate twice")
         dev = h.device
         n, hdim = h.shape
         vocab = w.shape[0]
-        glp = None if g_logprob is None else g_logprob.reshape(-1).to(torch.float32).contiguous()
-        gent = None if g_entropy is None else g_entropy.reshape(-1).to(torch.float32).contiguous()
+
+        def rows(g):
+            if g is None:
+                return None
+            g = g.reshape(-1).to(torch.float32).contiguous()
+            return g if keep is None else _index_rows(g, keep)
+
+        glp, gent = rows(g_logprob), rows(g_entropy)
         grad_h = torch.empty((n, hdim), device=dev, dtype=h.dtype) if need_h else None
         grad_w = torch.empty((vocab, hdim), device=dev, dtype=w.dtype) if need_w else None
         lib = _lib.load()
-        ws_bytes = lib.orlhf_lmhead_workspace_bytes(n, hdim, vocab, 1)
-        if ctx.backward_chunk_mib is not None:
+        ws_bytes = lib.orlhf_lmhead_workspace_bytes(n, hdim, vocab, ctx.kept_cols, 1)
+        if ctx.backward_chunk_mib is not None and ctx.kept_cols < (vocab + 255) // 256 * 256:
             # the library's default holds 256 MiB of the logits gradient at a time; the entry point
-            # takes whatever the workspace offers (whole vocabulary tiles, at most the vocabulary)
-            ws_bytes += (int(ctx.backward_chunk_mib) - 256) * (1 << 20)
-            ws_bytes = max(ws_bytes, lib.orlhf_lmhead_workspace_bytes(n, hdim, 256, 1))
+            # takes whatever the workspace offers (whole vocabulary tiles, at most what is not kept)
+            floor = lib.orlhf_lmhead_workspace_bytes(n, hdim, 256, 0, 1)
+            ws_bytes = max(floor, n * hdim * 4 + 256 + int(ctx.backward_chunk_mib) * (1 << 20))
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        kept, ctx.kept = ctx.kept, None
         with _lib.on_device(dev):
             call("orlhf_lmhead_logprob_entropy_bwd", ptr(h), ptr(w), _lib.dtype_code(h), n, hdim, vocab, h.stride(0),
-                 w.stride(0), ptr(lab), ctx.temperature, ptr(glp), ptr(gent), ptr(stats), ptr(grad_h), hdim,
-                 ptr(grad_w), hdim, ptr(ws), ws.numel(), stream_of(dev))
-        return grad_h, grad_w, None, None, None
+                 w.stride(0), ptr(lab), ctx.temperature, ptr(glp), ptr(gent), ptr(stats), ptr(kept), ctx.kept_cols,
+                 ctx.kept_ld, ptr(grad_h), hdim, ptr(grad_w), hdim, ptr(ws), ws.numel(), stream_of(dev))
+        if keep is not None and grad_h is not None:
+            grad_h = _scatter_rows(grad_h, keep, ctx.n_all)
+        return grad_h, grad_w, None, None, None, None, None
 
 
 def lm_head_logprobs_and_entropy(
@@ -264,34 +322,38 @@ def lm_head_logprobs_and_entropy(
     temperature: float = 1.0,
     row_mask: Optional[torch.Tensor] = None,
     backward_chunk_mib: Optional[int] = None,
+    keep_logits_mib: Optional[float] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """``logits = hidden_states @ lm_head_weight.T`` followed by ``log_probs_from_logits(logits,
     labels, temperature)`` and ``compute_entropy(logits)`` (openrlhf/models/actor.py:263-285 with
-    the projection that produces ``output["logits"]``), without the ``[..., V]`` logits ever being
-    stored: matrix-core tiles of the projection are folded into per-token statistics on chip, and
+    the projection that produces ``output["logits"]``), without the ``[..., V]`` logits being
+    stored: matrix-core tiles of the projection are rounded to the 16-bit dtype (as the reference's
+    lm_head output is before its fp32 up-cast) and folded into per-token statistics on chip, and
     the backward recomputes them chunk by chunk to produce the gradients of the hidden states and
-    of the weight. The logits stay in fp32 between the projection and the softmax (the reference
-    rounds them to the 16-bit dtype first). fp32 results.
+    of the weight. fp32 results.
 
     hidden_states ``[..., H]`` and lm_head_weight ``[V, H]`` in bfloat16 or float16; labels
     ``[...]``. ``row_mask`` (same shape as labels): positions with 0 are left out of the projection
-    altogether; their outputs are 0 and they receive zero gradient. ``backward_chunk_mib``: how
-    much of the logits gradient the backward holds at a time (default 256 MiB; at N = 4096,
-    V = 151 936 the whole of it, 1.2 GiB, makes the backward 4 % faster: fewer, longer launches)."""
+    altogether; their outputs are 0 and they receive zero gradient. ``keep_logits_mib``: the forward
+    stores the 16-bit logits of as many vocabulary columns as this budget holds (it produces them
+    anyway) and the backward recomputes only the others: with everything kept the backward is two
+    products instead of three. Results and gradients are the same bits for every budget.
+    ``backward_chunk_mib``: how much of the logits gradient of the columns that are NOT kept the
+    backward holds at a time (default 256 MiB)."""
     batch_shape = hidden_states.shape[:-1]
     if labels.shape != batch_shape:
         raise ValueError(f"labels shape {tuple(labels.shape)} != hidden batch shape {tuple(batch_shape)}")
     rows = hidden_states.reshape(-1, hidden_states.shape[-1])
     lab = labels.reshape(-1)
-    if row_mask is None:
-        lp, ent = _LmHeadLogprobEntropy.apply(rows, lm_head_weight, lab, temperature, backward_chunk_mib)
-        return lp.view(batch_shape), ent.view(batch_shape)
-    if row_mask.shape != batch_shape:
-        raise ValueError(f"row_mask shape {tuple(row_mask.shape)} != hidden batch shape {tuple(batch_shape)}")
-    keep = torch.nonzero(row_mask.reshape(-1) != 0, as_tuple=False).squeeze(-1)
-    lp_k, ent_k = _LmHeadLogprobEntropy.apply(rows[keep], lm_head_weight, lab[keep], temperature, backward_chunk_mib)
-    lp = torch.zeros(rows.shape[0], dtype=torch.float32, device=rows.device).index_copy(0, keep, lp_k)
-    ent = torch.zeros(rows.shape[0], dtype=torch.float32, device=rows.device).index_copy(0, keep, ent_k)
+    keep = None
+    if row_mask is not None:
+        if row_mask.shape != batch_shape:
+            raise ValueError(f"row_mask shape {tuple(row_mask.shape)} != hidden batch shape {tuple(batch_shape)}")
+        from .ring_attn_utils import unpad_indices
+
+        flat = row_mask.reshape(1, -1)
+        keep = unpad_indices(flat if flat.dtype in (torch.bool, torch.uint8) else flat != 0)
+    lp, ent = _LmHeadLogprobEntropy.apply(rows, lm_head_weight, lab, temperature, backward_chunk_mib, keep_logits_mib, keep)
     return lp.view(batch_shape), ent.view(batch_shape)
 
 
