@@ -95,34 +95,43 @@ def actor_forward_tail_from_hidden(
     temperature: float = 1.0,
     packed_indices: Optional[torch.Tensor] = None,
     return_entropy: bool = False,
+    skip_masked: bool = True,
+    keep_logits_mib: Optional[float] = None,
 ) -> Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]]:
     """The same tail with the lm-head projection in front and the logits never stored: what
     openrlhf/models/actor.py:263-296 computes from ``self.model(...)["logits"]``, from the decoder's
     last hidden states ``[B, T, H]`` (or ``[1, Ttot, H]`` / ``[Ttot, H]`` with ``packed_indices``)
-    and ``lm_head.weight [V, H]`` (bf16 or fp16). Positions whose log-prob the reference multiplies
-    by zero are left out of the projection altogether; gradients reach the hidden states and the
-    weight. Same outputs and shapes as ``actor_forward_tail``."""
-    from .utils import lm_head_logprobs_and_entropy
+    and ``lm_head.weight [V, H]`` (bf16 or fp16). With ``skip_masked=True`` (default) positions
+    whose log-prob the reference multiplies by zero (outside the action mask; with
+    ``action_mask=None`` the last column and the positions outside the attention mask) are left out
+    of the projection altogether: their log-prob and entropy are returned as 0 and they get no
+    gradient. ``skip_masked=False`` projects every row, which is what reproduces the reference's
+    values at padded positions when ``action_mask`` is None. Gradients reach the hidden states and
+    the weight. Same outputs and shapes as ``actor_forward_tail``."""
+    from .utils import _index_rows, lm_head_logprobs_and_entropy
 
     batch, seqlen = sequences.shape
     rolled = torch.roll(sequences, shifts=-1, dims=1)
-    need = torch.zeros(batch, seqlen, dtype=torch.bool, device=sequences.device)
-    if action_mask is not None:
-        width = action_mask.shape[1]
-        need[:, seqlen - 1 - width : seqlen - 1] = action_mask != 0
-    else:
-        need[:, : seqlen - 1] = True if attention_mask is None else attention_mask[:, : seqlen - 1] != 0
+    need = None
+    if skip_masked:
+        need = torch.zeros(batch, seqlen, dtype=torch.bool, device=sequences.device)
+        if action_mask is not None:
+            width = action_mask.shape[1]
+            need[:, seqlen - 1 - width : seqlen - 1] = action_mask != 0
+        else:
+            need[:, : seqlen - 1] = True if attention_mask is None else attention_mask[:, : seqlen - 1] != 0
     if packed_indices is None:
-        lp, ent = lm_head_logprobs_and_entropy(hidden_states, lm_head_weight, rolled, temperature, row_mask=need)
+        lp, ent = lm_head_logprobs_and_entropy(hidden_states, lm_head_weight, rolled, temperature, row_mask=need,
+                                               keep_logits_mib=keep_logits_mib)
     else:
         flat = hidden_states.reshape(-1, hidden_states.shape[-1])
-        lp_p, ent_p = lm_head_logprobs_and_entropy(flat, lm_head_weight, rolled.reshape(-1)[packed_indices], temperature,
-                                                   row_mask=need.reshape(-1)[packed_indices])
-
-        def repad(x):
-            return x.new_zeros(batch * seqlen).index_copy(0, packed_indices, x).view(batch, seqlen)
-
-        lp, ent = repad(lp_p), repad(ent_p)
+        idx = packed_indices.to(torch.int64).contiguous()
+        labels = _index_rows(rolled.reshape(-1).to(torch.int64), idx)
+        row_mask = None if need is None else _index_rows(need.reshape(-1).to(torch.uint8), idx)
+        lp_p, ent_p = lm_head_logprobs_and_entropy(flat, lm_head_weight, labels, temperature, row_mask=row_mask,
+                                                   keep_logits_mib=keep_logits_mib)
+        lp = gather_and_pad_tensor(lp_p.unsqueeze(0), None, 0, idx, batch, seqlen)
+        ent = gather_and_pad_tensor(ent_p.unsqueeze(0), None, 0, idx, batch, seqlen)
     lp = lp[:, :-1]
     if action_mask is not None:
         lp = lp[:, -action_mask.shape[1] :] * action_mask.float()

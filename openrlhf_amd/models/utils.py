@@ -199,7 +199,9 @@ def compute_entropy(logits: torch.Tensor, inplace_backward: bool = False) -> tor
 def _index_rows(src: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
     """src[indices] along the first axis (rows of any width) with the library's gather kernel."""
     src = src.contiguous()
-    inner = src[0].numel() if src.shape[0] > 0 else 1
+    inner = 1
+    for d in src.shape[1:]:
+        inner *= d
     out = torch.empty((indices.numel(),) + tuple(src.shape[1:]), dtype=src.dtype, device=src.device)
     with _lib.on_device(src.device):
         call("orlhf_gather_by_indices", ptr(src), src.element_size(), src.shape[0], max(inner, 1), ptr(indices),
@@ -210,7 +212,9 @@ def _index_rows(src: torch.Tensor, indices: torch.Tensor) -> torch.Tensor:
 def _scatter_rows(values: torch.Tensor, indices: torch.Tensor, n_dst: int) -> torch.Tensor:
     """zeros(n_dst, ...) with rows ``indices`` set to ``values`` (the library's pad_by_indices)."""
     values = values.contiguous()
-    inner = values[0].numel() if values.shape[0] > 0 else 1
+    inner = 1
+    for d in values.shape[1:]:
+        inner *= d
     out = torch.empty((n_dst,) + tuple(values.shape[1:]), dtype=values.dtype, device=values.device)
     with _lib.on_device(values.device):
         call("orlhf_pad_by_indices", ptr(values), values.element_size(), values.shape[0], max(inner, 1), ptr(indices),

@@ -31,18 +31,19 @@ def actor_loss_step(
     logits, sequences, attention_mask, action_mask, old_action_log_probs, advantages, policy_loss_fn: PolicyLoss,
     base_action_log_probs=None, kl_estimator="k1", kl_coef=0.0, entropy_coef=None, rollout_log_probs=None,
     temperature=1.0, packed_indices=None, dp_size=1, batch_num_tokens=None, global_batch_size=None,
-    inplace_backward=False, lm_head_weight=None,
+    inplace_backward=False, lm_head_weight=None, keep_logits_mib=None,
 ):
     """Reference-order composition (ppo_actor.py:294-352) on the separate kernels; differentiable.
     With ``lm_head_weight [V, H]`` the first argument holds the decoder's last hidden states instead
-    of logits and the projection is fused into the log-prob / entropy (the logits are never stored;
-    gradients reach the hidden states and the weight)."""
+    of logits and the projection is fused into the log-prob / entropy (the logits are not stored,
+    or only as many 16-bit columns of them as ``keep_logits_mib`` holds; gradients reach the hidden
+    states and the weight)."""
     info = dict(dp_size=dp_size, batch_num_tokens=batch_num_tokens, global_batch_size=global_batch_size)
     want_entropy = entropy_coef is not None
     if lm_head_weight is not None:
         out = actor_forward_tail_from_hidden(logits, lm_head_weight, sequences, action_mask, attention_mask,
                                              temperature=temperature, packed_indices=packed_indices,
-                                             return_entropy=want_entropy)
+                                             return_entropy=want_entropy, keep_logits_mib=keep_logits_mib)
     else:
         out = actor_forward_tail(logits, sequences, action_mask, attention_mask, temperature=temperature,
                                  packed_indices=packed_indices, return_entropy=want_entropy,

@@ -87,6 +87,68 @@ def test_entry_points_reject_bad_arguments_without_a_gpu(lib):
     assert lib.orlhf_whiten_workspace_bytes(10) > 0
 
 
+def test_matrix_core_entries_refuse_strides_their_offsets_cannot_address(lib):
+    """Row strides of 2^23 elements and more would wrap the 32-bit byte offsets inside a slab (up to
+    255 rows): refused before anything is launched. Odd strides and misaligned bases as well."""
+    from openrlhf_amd import _lib
+
+    def err():
+        return lib.orlhf_last_error().decode()
+
+    big = 1 << 23
+    fwd = lambda hs, ws, h=256, w=256: lib.orlhf_lmhead_logprob_entropy_fwd(  # noqa: E731
+        h, w, _lib.BF16, 4, 64, 100, hs, ws, None, 1.0, None, None, None, None, 0, 0, None, 0, None)
+    assert fwd(big, 64) == -3 and "2^23" in err() and "hidden" in err()
+    assert fwd(64, big) == -3 and "2^23" in err() and "weight" in err()
+    assert fwd(65, 64) == -3 and "even" in err()
+    assert fwd(64, 64, h=258) == -3 and "aligned" in err()
+    assert fwd(32, 64) == -1 and "stride" in err()
+    bwd = lib.orlhf_lmhead_logprob_entropy_bwd(256, 256, _lib.BF16, 4, 64, 100, 64, big, None, 1.0, None, None, None, None, 0, 0,
+                                               256, 64, None, 64, None, 0, None)
+    assert bwd == -3 and "2^23" in err()
+    # the stored logits: whole tiles, at most the padded vocabulary, rows on 16 bytes
+    kept = lambda cols, ld, ptr=256: lib.orlhf_lmhead_logprob_entropy_fwd(  # noqa: E731
+        256, 256, _lib.BF16, 4, 64, 1000, 64, 64, None, 1.0, None, None, None, ptr, cols, ld, None, 0, None)
+    assert kept(100, 1088) == -1 and "multiple of 256" in err()
+    assert kept(1280, 1344) == -1 and "padded vocabulary" in err()
+    assert kept(1024, 1028) == -3 and "multiple of 8" in err()
+    assert kept(1024, 512) == -1 and "kept_logits" in err()
+    assert kept(1024, 1088, ptr=None) == -1 and "NULL" in err()
+    prod = lambda lda, ldb: lib.orlhf_matrix_tile_product(256, 256, _lib.BF16, 8, 8, 64, lda, ldb, 0, 0, 0, 256, 8, None)  # noqa: E731
+    assert prod(big, 64) == -3 and "2^23" in err()
+    assert lib.orlhf_matrix_tile_probe(256, 256, _lib.BF16, 8, 8, 64, 64, big, 0, 256, None) == -3 and "2^23" in err()
+
+
+def test_matrix_core_kernels_do_not_spill():
+    """The compiler's own resource report for the matrix-core kernels: with 256 accumulator registers
+    per lane a few live values too many end up in scratch memory (and a spill inside the product
+    loop would cost far more than it looks). Compiles csrc/lmhead.hip for gfx950 with the library's
+    flags and reads the remarks: no kernel may spill a vector register or use scratch."""
+    import subprocess
+
+    from openrlhf_amd.csrc import build as b
+
+    src = os.path.join(b.CSRC, "lmhead.hip")
+    cmd = [b.find_hipcc(), *b.HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "--cuda-device-only", "-c", src, "-o", os.devnull,
+           "-Rpass-analysis=kernel-resource-usage"]
+    out = subprocess.run(cmd, capture_output=True, text=True)
+    assert out.returncode == 0, out.stderr[-2000:]
+    kernels, name = {}, None
+    for line in out.stderr.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", line)
+        if m:
+            name = m.group(1)
+            kernels[name] = {}
+            continue
+        m = re.search(r"remark:\s+(VGPRs Spill|ScratchSize \[bytes/lane\]|AGPRs|VGPRs): (\d+)", line)
+        if m and name:
+            kernels[name][m.group(1)] = int(m.group(2))
+    tiles = {k: v for k, v in kernels.items() if v.get("AGPRs", 0) == 256}  # the kernels built on the 256 x 256 tile
+    assert len(tiles) >= 20, sorted(kernels)
+    for k, v in kernels.items():
+        assert v["VGPRs Spill"] == 0 and v["ScratchSize [bytes/lane]"] == 0, (k, v)
+
+
 def test_python_mirrors_raise_like_the_reference(lib):
     from openrlhf_amd.models.loss import PolicyLoss, ValueLoss
     from openrlhf_amd.models.utils import compute_approx_kl, log_probs_from_logits

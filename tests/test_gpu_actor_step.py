@@ -187,8 +187,11 @@ def test_fused_step_on_a_vocabulary_longer_than_the_registers(cuda):
 @pytest.mark.parametrize("packed", [False, True])
 def test_actor_step_from_hidden_states(cuda, case, packed):
     """The composed step with the lm-head projection fused in (hidden states and lm_head.weight in
-    place of logits): the oracle's step on ``hidden @ W.T`` in fp64; values within 2e-3, gradients
-    of the hidden states and the weight within the rounding of a bf16 logits gradient."""
+    place of logits): the oracle's step on ``hidden @ W.T`` rounded to bf16 as the lm_head output is
+    (tests/lmhead_util.py), in fp64; values within 2e-3, gradients of the hidden states and the
+    weight within the rounding of a bf16 logits gradient."""
+    from tests.lmhead_util import straight_through_logits
+
     from openrlhf_amd.models.actor import unpad_indices
     from openrlhf_amd.models.loss import PolicyLoss
     from openrlhf_amd.trainer.ray.ppo_actor import actor_loss_step
@@ -203,7 +206,7 @@ def test_actor_step_from_hidden_states(cuda, case, packed):
 
     h64 = hidden.double().requires_grad_(True)
     w64 = weight.double().requires_grad_(True)
-    logits64 = h64 @ w64.T
+    logits64 = straight_through_logits(hidden, weight, h64, w64, cuda)
     ref_in = logits64.reshape(-1, vocab)[keep].unsqueeze(0) if packed else logits64
     ref = _oracle_step(ref_in, seqs, attn, amask, old, adv, base, roll, 1.0, packed, case["pol"], kl_est, kl_coef,
                        case["ent"], case["info"])

@@ -114,9 +114,11 @@ def test_return_all_logprobs_for_sft(cuda):
 @pytest.mark.parametrize("packed", [False, True])
 def test_tail_from_hidden_states(cuda, packed):
     """The same tail from the decoder's last hidden states and lm_head.weight, logits never stored:
-    against the oracle on ``hidden @ W.T`` in fp64 (2e-3 abs for bf16 operands; gradients of the
-    hidden states and of the weight within the rounding of a bf16 logits gradient and result)."""
+    against the oracle on ``hidden @ W.T`` rounded to bf16 as the lm_head output is
+    (tests/lmhead_util.py), in fp64 (2e-3 abs; gradients of the hidden states and of the weight
+    within the rounding of a bf16 logits gradient and result)."""
     from openrlhf_amd.models.actor import actor_forward_tail_from_hidden, unpad_indices
+    from tests.lmhead_util import straight_through_logits
 
     b, t, a, hdim, vocab, temperature = 4, 36, 15, 96, 1234, 0.8
     _, seqs, attn, amask = _batch(7, b=b, t=t, vocab=vocab, a=a)
@@ -127,7 +129,7 @@ def test_tail_from_hidden_states(cuda, packed):
 
     h64 = hidden.double().requires_grad_(True)
     w64 = weight.double().requires_grad_(True)
-    logits64 = h64 @ w64.T
+    logits64 = straight_through_logits(hidden, weight, h64, w64, cuda)
     ref_in = logits64.reshape(-1, vocab)[flat_keep].unsqueeze(0) if packed else logits64
     ref_lp, ref_ent = _oracle_tail64(ref_in, seqs, attn, amask, temperature, packed)
     w_lp = torch.randn(ref_lp.shape, generator=g)

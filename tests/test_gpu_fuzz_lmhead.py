@@ -1,13 +1,15 @@
 """Seeded random sweep over the lm-head + log-prob / entropy path: token counts, hidden sizes (any
 even number), vocabularies, dtypes, temperatures, padded row strides and row masks drawn at random,
-every case against the fp64 oracle applied to ``hidden @ W.T`` (values 2e-3 abs; gradients within
-the rounding of a 16-bit logits gradient and a 16-bit result)."""
+every case against the fp64 oracle applied to ``hidden @ W.T`` rounded to the 16-bit dtype as the
+lm_head output is (tests/lmhead_util.py; values 2e-3 abs; gradients within the rounding of a
+16-bit logits gradient and a 16-bit result)."""
 import random
 
 import pytest
 import torch
 
 from oracle import token_numerics as otn
+from tests.lmhead_util import straight_through_logits
 
 pytestmark = pytest.mark.gpu
 
@@ -35,7 +37,7 @@ def test_random_case(cuda, seed):
 
     h64 = hidden.double().requires_grad_(True)
     w64 = weight.double().requires_grad_(True)
-    logits = h64 @ w64.T
+    logits = straight_through_logits(hidden, weight, h64, w64, cuda)
     km = torch.ones(n, dtype=torch.float64) if mask is None else mask.double()
     ref_lp = otn.log_probs_from_logits(logits, labels, temperature) * km
     ref_ent = otn.compute_entropy(logits) * km

@@ -312,8 +312,10 @@ def test_gpt_lm_loss_vs_torch_cross_entropy(cuda, dtype):
 
 def test_sft_and_dpo_steps_from_hidden_states(cuda):
     """Both steps with the lm-head projection fused in (hidden states and lm_head.weight in place of
-    logits): the oracle on ``hidden @ W.T`` in fp64, values within 2e-3 (sums of up to 40 log-probs:
-    40 x that), gradients within the rounding of a bf16 logits gradient and result."""
+    logits): the oracle on ``hidden @ W.T`` rounded to bf16 as the lm_head output is
+    (tests/lmhead_util.py), in fp64, values within 2e-3 (sums of up to 40 log-probs: 40 x that),
+    gradients within the rounding of a bf16 logits gradient and result."""
+    from tests.lmhead_util import straight_through_logits
     from openrlhf_amd.models.loss import DPOLoss, SFTLoss
     from openrlhf_amd.trainer.dpo_trainer import concatenated_inputs, dpo_loss_step
     from openrlhf_amd.trainer.sft_trainer import sft_loss_step
@@ -332,7 +334,7 @@ def test_sft_and_dpo_steps_from_hidden_states(cuda):
 
     # DPO
     h64, w64 = hidden.double().requires_grad_(True), weight.double().requires_grad_(True)
-    lp = otn.log_probs_from_logits(h64 @ w64.T, torch.roll(ids, -1, 1), 1.0)[:, :-1]
+    lp = otn.log_probs_from_logits(straight_through_logits(hidden, weight, h64, w64, cuda), torch.roll(ids, -1, 1), 1.0)[:, :-1]
     sums, means = ol.get_batch_logps(lp, att, lens)
     ref_pref, _, _ = ol.dpo_loss(sums[:3], sums[3:], ref_c.double(), ref_r.double(), beta)
     ref_loss = ref_pref + (-means[:3].mean()) * 0.3
@@ -353,7 +355,7 @@ def test_sft_and_dpo_steps_from_hidden_states(cuda):
     loss_mask[4] = 0
     shifted = loss_mask[:, :-1]
     h64, w64 = hidden.double().requires_grad_(True), weight.double().requires_grad_(True)
-    lp_ref = otn.log_probs_from_logits(h64 @ w64.T, torch.roll(ids, -1, 1), 1.0)[:, :-1]
+    lp_ref = otn.log_probs_from_logits(straight_through_logits(hidden, weight, h64, w64, cuda), torch.roll(ids, -1, 1), 1.0)[:, :-1]
     ref_loss = ol.aggregate_loss(-lp_ref, shifted.double(), token_level_loss=True)
     ref_loss.backward()
     hd, wd = hidden.to(cuda).requires_grad_(True), weight.to(cuda).requires_grad_(True)

@@ -97,7 +97,7 @@ def test_unpad_reference_docstring_example():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.int64, torch.uint8])
-@pytest.mark.parametrize("trailing", [(), (3,), (2, 5)])
+@pytest.mark.parametrize("trailing", [(), (3,), (2, 5), (1,)])
 def test_gather_and_pad_matches_oracle(dtype, trailing):
     from openrlhf_amd.models.ring_attn_utils import gather_and_pad_tensor
 
@@ -109,8 +109,11 @@ def test_gather_and_pad_matches_oracle(dtype, trailing):
     vals = (torch.randn(1, n, *trailing, generator=g) * 50).to(dtype)
     want = olay.gather_and_pad_tensor(vals, indices, batch, seqlen)
     got = gather_and_pad_tensor(vals.to(_dev()), None, 0, indices.to(_dev()), batch, seqlen)
-    assert tuple(got.shape) == (batch, seqlen) + trailing
-    assert torch.equal(got.cpu().reshape(want.shape), want)
+    # the reference pads the transposed [Ttot, 1, ...] tensor and squeezes the last axis
+    # (ring_attn_utils.py:181): [1, Ttot] -> [B, T], [1, Ttot, 3] -> [B, T, 1, 3], [1, Ttot, 1] -> [B, T, 1]
+    expect = {(): (batch, seqlen), (3,): (batch, seqlen, 1, 3), (2, 5): (batch, seqlen, 1, 2, 5), (1,): (batch, seqlen, 1)}
+    assert tuple(got.shape) == tuple(want.shape) == expect[trailing]
+    assert torch.equal(got.cpu(), want)
 
 
 def test_gather_and_pad_round_trip_and_gradient():
