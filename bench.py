@@ -224,29 +224,59 @@ def bench_ceilings(pristine, bufs, labels, dev):
     return out
 
 
-def bench_lmhead(dev, n=4096, hdim=4096, vocab=VOCAB, reps=4):
-    """The lm-head + log-prob + entropy path with the logits never stored, at N tokens x H hidden x
-    V vocabulary in bf16: forward, and forward + backward down to d(hidden) and d(weight). Priced
-    against the dense bf16 matrix-core peak (2.5 PFLOP/s): 2 N H V flops forward, 8 N H V for
-    forward + backward (the backward recomputes the logits tiles, then two products)."""
-    from openrlhf_amd.models.utils import lm_head_logprobs_and_entropy
+def lmhead_traffic(n, hdim, vocab):
+    """HBM bytes per forward launch from the committed rocprofv3 --pmc summary of this shape
+    (FETCH_SIZE + WRITE_SIZE scaled by a copy of known size); None if it covers another shape or
+    another version of the kernels."""
+    path = os.path.join(ROOT, "profiles", f"lmhead_logprob_entropy_n{n}_h{hdim}_v{vocab}_hbm_traffic.txt")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    from openrlhf_amd import _lib
+    if f"abi_version = {_lib.ABI_VERSION}" not in text:
+        return None
+    for line in text.splitlines():
+        parts = line.split()
+        if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == "lmhead_fwd_kernel":
+            return float(parts[2])
+    return None
+
+
+def bench_lmhead(dev, n=4096, hdim=4096, vocab=VOCAB, reps=4, roofline=True):
+    """The lm-head + log-prob + entropy path at N tokens x H hidden x V vocabulary in bf16, forward and
+    forward + backward down to d(hidden) and d(weight), three ways on the same inputs:
+      * fused, nothing kept: the backward recomputes the logits tiles (8 N H V flops in all);
+      * fused, every logit kept (keep_logits_mib): forward + two products (6 N H V), the logits
+        stored once by the forward's tiles and turned into their gradient in place;
+      * materialised: torch.matmul (hipBLASLt) -> bf16 logits -> the one-pass vocabulary-row kernel
+        (log-prob, entropy and the logits gradient in place) -> two torch.matmul products,
+    each with the device memory it holds beyond the inputs at its peak. The roofline prices the
+    forward kernel against the dense bf16 matrix-core peak (2.5 PFLOP/s) with 2 N H V flops."""
+    from openrlhf_amd.models.utils import fused_logprob_entropy_fwd_bwd, lm_head_logprobs_and_entropy
 
     g = torch.Generator(device=dev).manual_seed(3)
     hidden = torch.randn(n, hdim, generator=g, device=dev).to(torch.bfloat16)
     weight = (torch.randn(vocab, hdim, generator=g, device=dev) * (3.0 / hdim ** 0.5)).to(torch.bfloat16)
     labels = torch.randint(0, vocab, (n,), generator=g, device=dev)
     g_lp, g_ent = torch.randn(n, generator=g, device=dev), torch.randn(n, generator=g, device=dev)
+    all_mib = (n * ((vocab + 255) // 256 * 256 + 64) * 2 >> 20) + 1
 
     def ev(fn):
-        fn()
+        """(ms per call, peak bytes allocated beyond what was there before)"""
+        out = fn()
+        del out
         torch.cuda.synchronize()
+        base = torch.cuda.memory_allocated(dev)
+        torch.cuda.reset_peak_memory_stats(dev)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(reps):
-            fn()
+            out = fn()
+            del out
         e1.record()
         torch.cuda.synchronize()
-        return e0.elapsed_time(e1) / reps
+        return e0.elapsed_time(e1) / reps, torch.cuda.max_memory_allocated(dev) - base
 
     def fwd():
         with torch.no_grad():
@@ -254,32 +284,75 @@ def bench_lmhead(dev, n=4096, hdim=4096, vocab=VOCAB, reps=4):
 
     hd, wd = hidden.clone().requires_grad_(True), weight.clone().requires_grad_(True)
 
-    def fwd_bwd():
-        lp, ent = lm_head_logprobs_and_entropy(hd, wd, labels, 1.0)
-        torch.autograd.backward([lp, ent], [g_lp, g_ent])
-        hd.grad = None
-        wd.grad = None
+    def fused(keep_mib):
+        def run():
+            lp, ent = lm_head_logprobs_and_entropy(hd, wd, labels, 1.0, keep_logits_mib=keep_mib)
+            torch.autograd.backward([lp, ent], [g_lp, g_ent])
+            gh, gw = hd.grad, wd.grad
+            hd.grad = wd.grad = None
+            return lp.detach(), ent.detach(), gh, gw
+        return run
 
-    ms_f, ms_fb = ev(fwd), ev(fwd_bwd)
+    def materialised():
+        with torch.no_grad():
+            logits = torch.matmul(hidden, weight.t())
+            lp, ent, p = fused_logprob_entropy_fwd_bwd(logits, labels, g_lp, g_ent, 1.0, inplace=True)
+            return lp, ent, torch.matmul(p, weight), torch.matmul(p.t(), hidden)
+
+    def materialised_fwd():
+        with torch.no_grad():
+            from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
+            return logprobs_and_entropy_from_logits(torch.matmul(hidden, weight.t()), labels, 1.0)
+
+    ms_f, mem_f = ev(fwd)
+    ms_fb, mem_fb = ev(fused(None))
+    ms_fk, mem_fk = ev(fused(all_mib))
+    ms_half, mem_half = ev(fused(all_mib // 2))
+    ms_m, mem_m = ev(materialised)
+    ms_mf, mem_mf = ev(materialised_fwd)
     flops = 2.0 * n * hdim * vocab
-    # check (outside the timed region): a row sample against the vocabulary-row kernels on the fp32 projection
-    from openrlhf_amd.models.utils import logprobs_and_entropy_from_logits
-    pick = torch.arange(0, n, max(1, n // 64), device=dev)[:64]
-    lp, ent = fwd()
-    lp2, ent2 = logprobs_and_entropy_from_logits(hidden[pick].float() @ weight.float().T, labels[pick], 1.0)
-    ok = (lp[pick] - lp2).abs().max().item() <= 1e-3 and (ent[pick] - ent2).abs().max().item() <= 1e-3
-    return {
-        "entry": "openrlhf_amd.models.utils.lm_head_logprobs_and_entropy (logits never stored)",
-        "config": {"tokens": n, "hidden": hdim, "vocab": vocab, "dtype": "bf16"},
-        "forward_ms": ms_f, "forward_tokens_per_s": n / (ms_f * 1e-3),
-        "forward_backward_ms": ms_fb, "forward_backward_tokens_per_s": n / (ms_fb * 1e-3),
-        "checked": ok,
-        "roofline": {"bound": "mfma", "kernel": "lmhead_fwd_kernel<bf16> (256x256 MFMA 32x32x16 tiles + per-token statistics)",
-                     "achieved": flops / (ms_f * 1e-3) / 1e12, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": flops / (ms_f * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, "flops_per_launch": flops,
-                     "forward_backward_achieved": 4 * flops / (ms_fb * 1e-3) / 1e12,
-                     "forward_backward_frac": 4 * flops / (ms_fb * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS},
+    # checks (outside the timed region): values and both gradients of the fused routes against the
+    # materialised route (its logits differ from the tiles' by the rounding of the accumulation order:
+    # a few entries per thousand tokens move by one 16-bit step), and the budgets against each other
+    a, b, c = fused(None)(), fused(all_mib)(), materialised()
+    same_bits = all(torch.equal(x, y) for x, y in zip(a, b))
+    med = lambda x: x.abs().float().flatten()[:: max(1, x.numel() // 1000003)].median().item()  # noqa: E731
+    check = {
+        "budgets_bit_identical": same_bits,
+        "logprob_median_abs_diff_vs_materialised": med(a[0] - c[0]),
+        "entropy_median_abs_diff_vs_materialised": med(a[1] - c[1]),
+        "grad_hidden_rel_fro_vs_materialised": ((a[2].float() - c[2].float()).norm() / c[2].float().norm()).item(),
+        "grad_weight_rel_fro_vs_materialised": ((a[3].float() - c[3].float()).norm() / c[3].float().norm()).item(),
     }
+    ok = (same_bits and check["logprob_median_abs_diff_vs_materialised"] <= 1e-3
+          and check["grad_hidden_rel_fro_vs_materialised"] <= 2.0 ** -6 and check["grad_weight_rel_fro_vs_materialised"] <= 2.0 ** -6)
+    del a, b, c
+    out = {
+        "entry": "openrlhf_amd.models.utils.lm_head_logprobs_and_entropy",
+        "config": {"tokens": n, "hidden": hdim, "vocab": vocab, "dtype": "bf16"},
+        "forward_ms": ms_f, "forward_tokens_per_s": n / (ms_f * 1e-3), "forward_extra_bytes": mem_f,
+        "forward_backward_ms": ms_fb, "forward_backward_tokens_per_s": n / (ms_fb * 1e-3),
+        "routes": {
+            "fused_nothing_kept": {"forward_backward_ms": ms_fb, "peak_extra_bytes": mem_fb},
+            "fused_half_of_the_logits_kept": {"forward_backward_ms": ms_half, "peak_extra_bytes": mem_half},
+            "fused_all_logits_kept": {"forward_backward_ms": ms_fk, "peak_extra_bytes": mem_fk},
+            "materialised_torch_matmul": {"forward_ms": ms_mf, "forward_extra_bytes": mem_mf, "forward_backward_ms": ms_m,
+                                          "peak_extra_bytes": mem_m},
+            "note": "peak_extra_bytes: device memory beyond the inputs at the route's peak, outputs and gradients "
+                    "(0.034 + 1.245 GB at N = 4096) included",
+        },
+        "checked": ok, "check": check,
+    }
+    if roofline:
+        out["roofline"] = {"bound": "mfma", "kernel": "lmhead_fwd_kernel<bf16> (256x256 MFMA 32x32x16 tiles + per-token statistics)",
+                           "achieved": flops / (ms_f * 1e-3) / 1e12, "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                           "frac": flops / (ms_f * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS, "flops_per_launch": flops,
+                           "traffic": lmhead_traffic(n, hdim, vocab),
+                           "forward_backward_all_kept_achieved": 3 * flops / (ms_fk * 1e-3) / 1e12,
+                           "forward_backward_all_kept_frac": 3 * flops / (ms_fk * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS,
+                           "forward_backward_nothing_kept_achieved": 4 * flops / (ms_fb * 1e-3) / 1e12,
+                           "forward_backward_nothing_kept_frac": 4 * flops / (ms_fb * 1e-3) / 1e12 / MFMA_PEAK_TFLOPS}
+    return out
 
 
 def bench_few_rows(dev, n=64, vocab=VOCAB, copies=32):
@@ -817,7 +890,7 @@ def main():
         bench_torch_eager(args, dev)
         return
     if args.workload == "lmhead":
-        print(json.dumps({"workload": "lm-head + log-prob + entropy, logits never stored", "n_gpus": 1,
+        print(json.dumps({"workload": "lm-head + log-prob + entropy, fused against materialised logits", "n_gpus": 1,
                           **bench_lmhead(dev, n=args.rows if args.rows != 8192 else 4096)}), flush=True)
         return
     if args.workload == "matrix_tile":
@@ -1004,6 +1077,9 @@ def main():
         del bufs[1:]  # the ring is no longer needed
         torch.cuda.empty_cache()
         out["lmhead_logprob_entropy"] = bench_lmhead(dev)
+        # the same at the token count of the headline workload (config 2's packed batch)
+        big = bench_lmhead(dev, n=n_tok, reps=2, roofline=False)
+        out["lmhead_logprob_entropy"]["at_config2_tokens"] = {k: big[k] for k in ("config", "forward_ms", "routes", "checked", "check")}
     if not args.no_per_token:
         out["few_rows_n64"] = bench_few_rows(dev)
         entries = bench_per_token(args, dev, emit=False)

@@ -668,12 +668,15 @@ static int launch_bwd(const void* hidden, const void* weight, int64_t n_rows, in
 
 using namespace orlhf;
 
-// Columns of P the backward's workspace holds at a time when nothing else is said: about 256 MiB,
-// at least one tile column, at most what is not kept.
+// Columns of P the backward's workspace holds at a time when nothing else is said: about 256 MiB but
+// no fewer than 8192 columns (every chunk re-reads and re-writes the fp32 sum of the hidden-state
+// gradient, 8 bytes per token and hidden column: with many tokens narrow chunks would spend more
+// time on that than on their products), at most what is not kept.
 static int64_t default_chunk_cols(int64_t n_rows, int64_t open_cols) {
   const int64_t rows = n_rows > 0 ? n_rows : 1;
   int64_t cols = ((256ll << 20) / (2 * rows)) / 256 * 256;
-  return cols < 256 ? 256 : (cols > open_cols ? open_cols : cols);
+  cols = cols < 8192 ? 8192 : cols;
+  return cols > open_cols ? open_cols : cols;
 }
 
 extern "C" int64_t orlhf_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_dim, int64_t vocab, int64_t kept_cols,
@@ -682,9 +685,8 @@ extern "C" int64_t orlhf_lmhead_workspace_bytes(int64_t n_rows, int64_t hidden_d
   if (!backward) return lm::records_bytes(n_rows, vocab);
   const int64_t rows = n_rows > 0 ? n_rows : 1;
   const int64_t open_cols = lm::round_up(vocab, 256) - kept_cols;
-  int64_t bytes = lm::dhidden_bytes(n_rows, hidden_dim);
-  if (open_cols > 0) bytes += rows * lm::p_chunk_ld(default_chunk_cols(n_rows, open_cols)) * 2;
-  return bytes;
+  if (open_cols <= 0) return 256;  // everything kept: one product per gradient, nothing to carry between launches
+  return lm::dhidden_bytes(n_rows, hidden_dim) + rows * lm::p_chunk_ld(default_chunk_cols(n_rows, open_cols)) * 2;
 }
 
 extern "C" int orlhf_lmhead_logprob_entropy_fwd(const void* hidden, const void* weight, int dtype, int64_t n_rows,
@@ -758,10 +760,6 @@ extern "C" int orlhf_lmhead_logprob_entropy_bwd(const void* hidden, const void* 
     ORLHF_CHECK_ARG(cols >= 256, "lmhead_logprob_entropy_bwd: workspace of %lld bytes is too small (orlhf_lmhead_workspace_bytes gives %lld)",
                     (long long)workspace_bytes, (long long)orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, kept_cols, 1));
     if (lm::p_chunk_ld(cols) >= mm::kMaxLd) cols = (mm::kMaxLd - 1 - lm::p_chunk_ld(0)) / 256 * 256;
-  } else {
-    ORLHF_CHECK_ARG(workspace != nullptr && workspace_bytes >= fixed,
-                    "lmhead_logprob_entropy_bwd: workspace of %lld bytes is too small (orlhf_lmhead_workspace_bytes gives %lld)",
-                    (long long)workspace_bytes, (long long)fixed);
   }
   ORLHF_CHECK_ARG(((uintptr_t)workspace & 255u) == 0, "lmhead_logprob_entropy_bwd: workspace must be 256-byte aligned");
   if (dtype == ORLHF_BF16)

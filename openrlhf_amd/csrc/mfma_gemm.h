@@ -163,10 +163,17 @@ struct Mfma<ORLHF_F16> {
   }
 };
 
-// ---- fragments of one k-step (16 k) of a slab: 4 row-tiles of A and 4 of B for this wave
+// ---- fragments of one k-step (16 k) of a slab: 4 row-tiles of A and 4 of B for this wave, each as
+// two halves of 4 k (a transpose read delivers one half; the halves are joined only after the wait
+// for such reads, so that no register copy can run ahead of the data)
 struct Frags {
-  u32x4 a[4], b[4];
+  u32x2 a[4][2], b[4][2];
 };
+__device__ __forceinline__ u32x4 whole(const u32x2 (&h)[2]) { return u32x4{h[0][0], h[0][1], h[1][0], h[1][1]}; }
+__device__ __forceinline__ void halves(u32x2 (&h)[2], const u32x4& v) {
+  h[0] = u32x2{v[0], v[1]};
+  h[1] = u32x2{v[2], v[3]};
+}
 
 // The lane's coordinates in a wave's 128-row quadrant `wq` of an operand.
 struct LanePos {
@@ -174,18 +181,34 @@ struct LanePos {
 };
 
 // Row-tile t (32 rows) of k-step ks: the whole fragment of a K-major slab (one 16-byte read) ...
-__device__ __forceinline__ u32x4 read_frag_k(const char* slab, int ks, int t, const LanePos& p) {
+__device__ __forceinline__ u32x4 read_frag_k(const char* slab, int ks, int t, const LanePos& p) {  // ks, t: constants after inlining
   const uint32_t row = p.wq * 128u + (uint32_t)t * 32u + (p.lane & 31u);
   return *(const u32x4*)(slab + row * 128u + ((((uint32_t)ks * 2u + (p.lane >> 5)) ^ swz(row)) << 4));
 }
-// ... and half h (k 4 h .. 4 h + 3 of the lane's 8) of the fragment of an MN-major slab: lane r of a
+// ... and half H (k 4 H .. 4 H + 3 of the lane's 8) of the fragment of an MN-major slab: lane r of a
 // 16-lane group addresses k-row (r >> 2) of the group's four and rows 4 (r & 3) .. + 3 of its sixteen.
-__device__ __forceinline__ u32x2 read_frag_mn(const char* slab, int ks, int t, int h, const LanePos& p) {
+// The read is written as inline assembly: for the builtin the compiler cannot tell which LDS buffer
+// is read and makes every such read wait (vmcnt(0)) for the LDS-direct loads that are in flight
+// into the OTHER buffer, which serialises the whole pipeline (a third of the rate). The price is
+// that the compiler does not wait for these reads either: wait_frags() below does, once per k-step.
+template <int KS, int T, int H>
+__device__ __forceinline__ u32x2 read_frag_mn(const char* slab, const LanePos& p) {
   const uint32_t r = p.lane & 15u, g = p.lane >> 4, q = r >> 2;
-  const uint32_t k = (uint32_t)ks * 16u + 8u * (g >> 1) + 4u * (uint32_t)h + q;
-  const uint32_t c = p.wq * 16u + 4u * (uint32_t)t + 2u * (g & 1u) + ((r & 3u) >> 1);
-  const char* at = slab + k * 512u + ((c ^ (q << 2)) << 4) + (r & 1u) * 8u;
-  return __builtin_bit_cast(u32x2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)at));
+  const uint32_t k = 8u * (g >> 1) + q;                                 // + 16 KS + 4 H: in the immediate offset
+  const uint32_t c = p.wq * 16u + 4u * (uint32_t)T + 2u * (g & 1u) + ((r & 3u) >> 1);
+  typedef const __attribute__((address_space(3))) char* lds_bytes;
+  const uint32_t at = (uint32_t)(uintptr_t)(lds_bytes)slab + k * 512u + ((c ^ (q << 2)) << 4) + (r & 1u) * 8u;
+  u32x2 v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(at), "n"(KS * 8192 + H * 2048));
+  return v;
+}
+// Everything read from LDS so far has arrived; the fragments are tied to the wait, so that nothing
+// that uses them is scheduled ahead of it.
+__device__ __forceinline__ void wait_frags(Frags& f) {
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(f.a[0][0]), "+v"(f.a[0][1]), "+v"(f.a[1][0]), "+v"(f.a[1][1]), "+v"(f.a[2][0]), "+v"(f.a[2][1]),
+                 "+v"(f.a[3][0]), "+v"(f.a[3][1]), "+v"(f.b[0][0]), "+v"(f.b[0][1]), "+v"(f.b[1][0]), "+v"(f.b[1][1]),
+                 "+v"(f.b[2][0]), "+v"(f.b[2][1]), "+v"(f.b[3][0]), "+v"(f.b[3][1]));
 }
 
 // Read number I of a k-step's fragments, in the order a0 b0 a1 b1 ... (an MN-major operand has two
@@ -193,39 +216,51 @@ __device__ __forceinline__ u32x2 read_frag_mn(const char* slab, int ks, int t, i
 template <bool A_MN, bool B_MN>
 struct FragPlan {
   static constexpr int kA = A_MN ? 2 : 1, kB = B_MN ? 2 : 1, kPerTile = kA + kB, kReads = 4 * kPerTile;
-  template <int I>
-  static __device__ __forceinline__ void read(Frags& f, const char* slab_a, const char* slab_b, int ks, const LanePos& pa,
+  static constexpr bool kAsmReads = A_MN || B_MN;  // reads the compiler does not wait for: wait_frags()
+  // With transpose reads in the mix all reads of a k-step go out in its first 12 slots, so that the
+  // last one has four MFMAs to land before the wait at the step's end.
+  static constexpr int kReadsPerSlot = kReads > 12 ? 2 : 1;
+  template <int KS, int I>
+  static __device__ __forceinline__ void read(Frags& f, const char* slab_a, const char* slab_b, const LanePos& pa,
                                               const LanePos& pb) {
     if constexpr (I < kReads) {
       constexpr int t = I / kPerTile, j = I % kPerTile;
       if constexpr (j < kA) {
         if constexpr (A_MN) {
-          const u32x2 v = read_frag_mn(slab_a, ks, t, j, pa);
-          f.a[t][2 * j] = v[0];
-          f.a[t][2 * j + 1] = v[1];
+          f.a[t][j] = read_frag_mn<KS, t, j>(slab_a, pa);
         } else {
-          f.a[t] = read_frag_k(slab_a, ks, t, pa);
+          halves(f.a[t], read_frag_k(slab_a, KS, t, pa));
         }
       } else {
         constexpr int h = j - kA;
         if constexpr (B_MN) {
-          const u32x2 v = read_frag_mn(slab_b, ks, t, h, pb);
-          f.b[t][2 * h] = v[0];
-          f.b[t][2 * h + 1] = v[1];
+          f.b[t][h] = read_frag_mn<KS, t, h>(slab_b, pb);
         } else {
-          f.b[t] = read_frag_k(slab_b, ks, t, pb);
+          halves(f.b[t], read_frag_k(slab_b, KS, t, pb));
         }
       }
     }
   }
-  template <int... I>
-  static __device__ __forceinline__ void read_all(Frags& f, const char* slab_a, const char* slab_b, int ks, const LanePos& pa,
-                                                  const LanePos& pb, std::integer_sequence<int, I...>) {
-    (read<I>(f, slab_a, slab_b, ks, pa, pb), ...);
+  // the reads of pinned slot S
+  template <int KS, int S>
+  static __device__ __forceinline__ void read_slot(Frags& f, const char* slab_a, const char* slab_b, const LanePos& pa,
+                                                   const LanePos& pb) {
+    if constexpr (kReadsPerSlot == 1) {
+      read<KS, S>(f, slab_a, slab_b, pa, pb);
+    } else if constexpr (S < 8) {
+      read<KS, 2 * S>(f, slab_a, slab_b, pa, pb);
+      read<KS, 2 * S + 1>(f, slab_a, slab_b, pa, pb);
+    }
   }
-  static __device__ __forceinline__ void read_all(Frags& f, const char* slab_a, const char* slab_b, int ks, const LanePos& pa,
+  template <int KS, int... I>
+  static __device__ __forceinline__ void read_all(Frags& f, const char* slab_a, const char* slab_b, const LanePos& pa,
+                                                  const LanePos& pb, std::integer_sequence<int, I...>) {
+    (read<KS, I>(f, slab_a, slab_b, pa, pb), ...);
+  }
+  template <int KS>
+  static __device__ __forceinline__ void read_all(Frags& f, const char* slab_a, const char* slab_b, const LanePos& pa,
                                                   const LanePos& pb) {
-    read_all(f, slab_a, slab_b, ks, pa, pb, std::make_integer_sequence<int, kReads>{});
+    read_all<KS>(f, slab_a, slab_b, pa, pb, std::make_integer_sequence<int, kReads>{});
   }
 };
 
@@ -234,7 +269,7 @@ __device__ __forceinline__ void mfma_step(f32x16 (&acc)[4][4], const Frags& f) {
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
-    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = Mfma<DT>::run(f.a[mt], f.b[nt], acc[mt][nt]);
+    for (int nt = 0; nt < 4; ++nt) acc[mt][nt] = Mfma<DT>::run(whole(f.a[mt]), whole(f.b[nt]), acc[mt][nt]);
   }
 }
 
@@ -246,7 +281,7 @@ __device__ __forceinline__ void mfma_step(f32x16 (&acc)[4][4], const Frags& f) {
 template <int DT, int I, class Reads, class Loads>
 __device__ __forceinline__ void pinned_slot(f32x16 (&acc)[4][4], const Frags& use, Reads& reads, Loads& loads) {
   reads(std::integral_constant<int, I>{});
-  acc[I >> 2][I & 3] = Mfma<DT>::run(use.a[I >> 2], use.b[I & 3], acc[I >> 2][I & 3]);
+  acc[I >> 2][I & 3] = Mfma<DT>::run(whole(use.a[I >> 2]), whole(use.b[I & 3]), acc[I >> 2][I & 3]);
   loads(std::integral_constant<int, I>{});
   __builtin_amdgcn_sched_barrier(0);
 }
@@ -257,18 +292,17 @@ __device__ __forceinline__ void pinned_step(f32x16 (&acc)[4][4], const Frags& us
 }
 constexpr int bits_below(uint32_t mask, int i) { return __builtin_popcount(mask & ((1u << i) - 1u)); }
 
-// reads(I): LDS read I of the fragments of k-step KS of a slab pair
-template <bool A_MN, bool B_MN>
+// reads(S): the LDS reads of slot S for the fragments of k-step KS of a slab pair
+template <bool A_MN, bool B_MN, int KS>
 struct FragReads {
   Frags& f;
   const char* slab_a;
   const char* slab_b;
-  int ks;
   const LanePos& pa;
   const LanePos& pb;
-  template <int I>
-  __device__ __forceinline__ void operator()(std::integral_constant<int, I>) const {
-    FragPlan<A_MN, B_MN>::template read<I>(f, slab_a, slab_b, ks, pa, pb);
+  template <int S>
+  __device__ __forceinline__ void operator()(std::integral_constant<int, S>) const {
+    FragPlan<A_MN, B_MN>::template read_slot<KS, S>(f, slab_a, slab_b, pa, pb);
   }
 };
 // loads(I): the slab pair's load number BASE + (set bits of MASK below I), if bit I of MASK is set
@@ -377,7 +411,7 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     }
   }
   Frags f0, f1;
-  Plan::read_all(f0, lds, lds + kSlabBytes, 0, pa, pb);
+  Plan::template read_all<0>(f0, lds, lds + kSlabBytes, pa, pb);
   int64_t s = 0;
 
   // One steady-state iteration: slab `it` in buffer PARITY; slab it + 1 (whole) has had its first
@@ -394,25 +428,29 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     const SlabDma<B_MN> db1(b, row0_b, k1, nxt + kSlabBytes, wave_u, lane);
     NoLoads none;
     {
-      FragReads<A_MN, B_MN> rd{f1, cur, cur + kSlabBytes, 1, pa, pb};
+      FragReads<A_MN, B_MN, 1> rd{f1, cur, cur + kSlabBytes, pa, pb};
       SlabLoads<kDmaSlots0, n3, A_MN, B_MN> ld{da1, db1};
+      if (Plan::kAsmReads) wait_frags(f0);
       if (RESIDENT_OPERANDS) pinned_step<DT>(acc, f0, rd, none, Slots16{}); else pinned_step<DT>(acc, f0, rd, ld, Slots16{});
     }
     {
-      FragReads<A_MN, B_MN> rd{f0, cur, cur + kSlabBytes, 2, pa, pb};
+      FragReads<A_MN, B_MN, 2> rd{f0, cur, cur + kSlabBytes, pa, pb};
+      if (Plan::kAsmReads) wait_frags(f1);
       pinned_step<DT>(acc, f1, rd, none, Slots16{});
     }
     {
-      FragReads<A_MN, B_MN> rd{f1, cur, cur + kSlabBytes, 3, pa, pb};
+      FragReads<A_MN, B_MN, 3> rd{f1, cur, cur + kSlabBytes, pa, pb};
+      if (Plan::kAsmReads) wait_frags(f0);
       pinned_step<DT>(acc, f0, rd, none, Slots16{});
     }
     // every wave holds its last fragments of `cur`; slab it + 1 is complete in `nxt`
+    if (Plan::kAsmReads) wait_frags(f1);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     const SlabDma<A_MN> da2(a, row0_a, k2, cur, wave_u, lane);
     const SlabDma<B_MN> db2(b, row0_b, k2, cur + kSlabBytes, wave_u, lane);
     {
-      FragReads<A_MN, B_MN> rd{f0, nxt, nxt + kSlabBytes, 0, pa, pb};
+      FragReads<A_MN, B_MN, 0> rd{f0, nxt, nxt + kSlabBytes, pa, pb};
       SlabLoads<kDmaSlots3, 0, A_MN, B_MN> ld{da2, db2};
       if (RESIDENT_OPERANDS) pinned_step<DT>(acc, f1, rd, none, Slots16{}); else pinned_step<DT>(acc, f1, rd, ld, Slots16{});
     }
@@ -431,19 +469,23 @@ __device__ __forceinline__ void tile_product(f32x16 (&acc)[4][4], const Operand&
     const char* cur = lds + (s & 1) * kStageBytes;
     char* nxt = lds + ((s + 1) & 1) * kStageBytes;
     const bool has1 = s + 1 < n_slabs;
-    Plan::read_all(f1, cur, cur + kSlabBytes, 1, pa, pb);
+    if (Plan::kAsmReads) wait_frags(f0);
+    Plan::template read_all<1>(f1, cur, cur + kSlabBytes, pa, pb);
     mfma_step<DT>(acc, f0);
-    Plan::read_all(f0, cur, cur + kSlabBytes, 2, pa, pb);
+    if (Plan::kAsmReads) wait_frags(f1);
+    Plan::template read_all<2>(f0, cur, cur + kSlabBytes, pa, pb);
     mfma_step<DT>(acc, f1);
-    Plan::read_all(f1, cur, cur + kSlabBytes, 3, pa, pb);
+    if (Plan::kAsmReads) wait_frags(f0);
+    Plan::template read_all<3>(f1, cur, cur + kSlabBytes, pa, pb);
     mfma_step<DT>(acc, f0);
+    if (Plan::kAsmReads) wait_frags(f1);
     if (has1) {
       // `nxt` was last read in iteration s - 1, whose barrier every wave has passed; the loads
       // below are younger than any load still on its way there and complete after it
       load_slab(s + 1, nxt);
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
-      Plan::read_all(f0, nxt, nxt + kSlabBytes, 0, pa, pb);
+      Plan::template read_all<0>(f0, nxt, nxt + kSlabBytes, pa, pb);
     }
     mfma_step<DT>(acc, f1);
   }
