@@ -643,6 +643,18 @@ int orlhf_pack_rows(const void* src, int elem_bytes, int64_t n_rows, int64_t n_c
                     const int64_t* first, const int64_t* cu_seqlens, void* dst,
                     orlhf_stream_t stream);
 
+/* orlhf_pack_rows for several fields that share n_rows, n_cols, first and cu_seqlens, in one launch
+ * per eight fields (a rollout batch packs four to ten per-token tensors over the same mask:
+ * openrlhf/trainer/ppo_utils/experience.py:199-247 slices every field of every sample). `fields` is a
+ * HOST array of n_fields entries; the pointers inside are device pointers. */
+typedef struct orlhf_pack_field {
+  const void* src; /* [n_rows, n_cols] elements of elem_bytes */
+  void* dst;       /* cu_seqlens[n_rows] elements */
+  int elem_bytes;  /* 1, 2, 4 or 8 */
+} orlhf_pack_field;
+int orlhf_pack_rows_multi(const orlhf_pack_field* fields, int n_fields, int64_t n_rows, int64_t n_cols,
+                          const int64_t* first, const int64_t* cu_seqlens, orlhf_stream_t stream);
+
 /* dst[cu[b] + j] = src[src_start[b] + j] for j < cu[b+1] - cu[b]: rows picked out of a packed
  * array into a new packed array, in any order and with repeats (a replay buffer handing out a
  * micro-batch without going through the padded form of
@@ -671,7 +683,8 @@ int orlhf_pad_rows(const void* src, int elem_bytes, const int64_t* cu_seqlens, i
  * anywhere in a row (left padding, right padding, holes).
  *
  * orlhf_mask_row_counts: counts[b] = number of non-zero columns of mask row b (seqlens_in_batch;
- *   orlhf_cu_seqlens turns them into cu_seqlens).
+ *   orlhf_cu_seqlens turns them into cu_seqlens). tile_counts (int32 [n_rows, ceil(n_cols /
+ *   ORLHF_UNPAD_TILE)], nullable): the same per tile of ORLHF_UNPAD_TILE columns, from the same pass.
  * orlhf_unpad_sequences: for the r-th non-zero column t of row b, at slot cu_seqlens[b] + r of each
  *   output that is not NULL:
  *     indices          b * n_cols + t                      (unpad_input's indices)
@@ -680,14 +693,19 @@ int orlhf_pad_rows(const void* src, int elem_bytes, const int64_t* cu_seqlens, i
  *     position_ids     r                                   (clip(cumsum(mask, -1) - 1, min=0), :137-140)
  *   sequences may be NULL when neither sequence output is asked for. capacity is the number of
  *   slots each output holds (cu_seqlens[n_rows] when they are sized exactly); slots past it are
- *   not written.
+ *   not written. tile_counts: what orlhf_mask_row_counts wrote for the same mask, or NULL. With it
+ *   every (row, tile) is a work item of its own that knows its first slot (tiles without attended
+ *   columns cost nothing and fully attended ones do not read the mask); without it a workgroup
+ *   walks a whole row, tile after tile. Same outputs either way.
  */
+#define ORLHF_UNPAD_TILE 2048
 int orlhf_mask_row_counts(const void* mask, int mask_dtype, int64_t n_rows, int64_t n_cols,
-                          int64_t* counts, orlhf_stream_t stream);
+                          int64_t* counts, int32_t* tile_counts, orlhf_stream_t stream);
 int orlhf_unpad_sequences(const int64_t* sequences, const void* mask, int mask_dtype,
                           int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,
-                          int64_t capacity, int64_t* indices, int64_t* packed_sequences,
-                          int64_t* rolled_sequences, int64_t* position_ids, orlhf_stream_t stream);
+                          const int32_t* tile_counts, int64_t capacity, int64_t* indices,
+                          int64_t* packed_sequences, int64_t* rolled_sequences, int64_t* position_ids,
+                          orlhf_stream_t stream);
 
 /*
  * The way back, gather_and_pad_tensor on one GPU (openrlhf/models/ring_attn_utils.py:181, which is

@@ -23,6 +23,7 @@ GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
 ABI_VERSION = 22
+UNPAD_TILE = 2048  # ORLHF_UNPAD_TILE
 
 
 class Norm(Structure):
@@ -41,6 +42,10 @@ class PolicyParams(Structure):
         ("token_level", c_int),
         ("norm", Norm),
     ]
+
+
+class PackField(Structure):
+    _fields_ = [("src", c_void_p), ("dst", c_void_p), ("elem_bytes", c_int)]
 
 
 class StepTerms(Structure):
@@ -120,10 +125,11 @@ SIGNATURES = {
     "orlhf_row_extents": (c_int, [P, c_int, I64, I64, P, P, P, P]),
     "orlhf_cu_seqlens": (c_int, [P, I64, P, P]),
     "orlhf_pack_rows": (c_int, [P, c_int, I64, I64, P, P, P, P]),
+    "orlhf_pack_rows_multi": (c_int, [POINTER(PackField), c_int, I64, I64, P, P, P]),
     "orlhf_gather_rows": (c_int, [P, c_int, I64, I64, P, P, P, P]),
     "orlhf_pad_rows": (c_int, [P, c_int, P, I64, I64, c_int, c_uint64, P, P]),
-    "orlhf_mask_row_counts": (c_int, [P, c_int, I64, I64, P, P]),
-    "orlhf_unpad_sequences": (c_int, [P, P, c_int, I64, I64, P, I64, P, P, P, P, P]),
+    "orlhf_mask_row_counts": (c_int, [P, c_int, I64, I64, P, P, P]),
+    "orlhf_unpad_sequences": (c_int, [P, P, c_int, I64, I64, P, P, I64, P, P, P, P, P]),
     "orlhf_pad_by_indices": (c_int, [P, c_int, I64, I64, P, I64, P, P]),
     "orlhf_gather_by_indices": (c_int, [P, c_int, I64, I64, P, I64, P, P]),
     "orlhf_sequence_logps_fwd": (c_int, [P, P, c_int, P, I64, I64, P, P, P, P]),

@@ -21,6 +21,19 @@ def _no_ring(ring_attn_group):
         raise NotImplementedError("one GPU: ring_attn_group must be None")
 
 
+def _count(mptr, mcode, batch, seqlen, dev):
+    """One pass over the mask: cu_seqlens [B + 1] and the attended columns of every (row, tile)."""
+    cu = torch.empty(batch + 1, dtype=torch.int64, device=dev)
+    counts = torch.empty(max(batch, 1), dtype=torch.int64, device=dev)
+    n_tiles = (seqlen + _lib.UNPAD_TILE - 1) // _lib.UNPAD_TILE
+    tiles = torch.empty(max(batch * n_tiles, 1), dtype=torch.int32, device=dev)
+    with _lib.on_device(dev):
+        st = stream_of(dev)
+        call("orlhf_mask_row_counts", mptr, mcode, batch, seqlen, ptr(counts), ptr(tiles), st)
+        call("orlhf_cu_seqlens", ptr(counts), batch, ptr(cu), st)
+    return cu, tiles
+
+
 def unpad_and_slice_tensor(sequences: torch.Tensor, attention_mask: torch.Tensor, ring_attn_group=None,
                            total_tokens: Optional[int] = None, return_cu_seqlens: bool = False):
     """``(sequences [1, Ttot], position_ids [1, Ttot], rolled_sequences [1, Ttot], 0, indices [Ttot])``
@@ -34,18 +47,13 @@ def unpad_and_slice_tensor(sequences: torch.Tensor, attention_mask: torch.Tensor
     batch, seqlen = sequences.shape
     seqs = sequences.to(torch.int64).contiguous()
     mkeep, mptr, mcode = _lib.mask_arg(attention_mask)
-    cu = torch.empty(batch + 1, dtype=torch.int64, device=dev)
-    counts = torch.empty(max(batch, 1), dtype=torch.int64, device=dev)
-    with _lib.on_device(dev):
-        st = stream_of(dev)
-        call("orlhf_mask_row_counts", mptr, mcode, batch, seqlen, ptr(counts), st)
-        call("orlhf_cu_seqlens", ptr(counts), batch, ptr(cu), st)
+    cu, tiles = _count(mptr, mcode, batch, seqlen, dev)
     total = int(cu[-1]) if total_tokens is None else int(total_tokens)
     out = torch.empty(4, max(total, 1), dtype=torch.int64, device=dev)
     if total > 0:
         with _lib.on_device(dev):
-            call("orlhf_unpad_sequences", ptr(seqs), mptr, mcode, batch, seqlen, ptr(cu), total, ptr(out[0]), ptr(out[1]),
-                 ptr(out[2]), ptr(out[3]), stream_of(dev))
+            call("orlhf_unpad_sequences", ptr(seqs), mptr, mcode, batch, seqlen, ptr(cu), ptr(tiles), total, ptr(out[0]),
+                 ptr(out[1]), ptr(out[2]), ptr(out[3]), stream_of(dev))
     indices, packed, rolled, position_ids = (out[i, :total] for i in range(4))
     packed = packed.to(sequences.dtype).unsqueeze(0)
     rolled = rolled.to(sequences.dtype).unsqueeze(0)
@@ -61,18 +69,13 @@ def unpad_indices(attention_mask: torch.Tensor, total_tokens: Optional[int] = No
         raise ValueError(f"attention_mask must be [B, T], got {tuple(attention_mask.shape)}")
     batch, seqlen = attention_mask.shape
     mkeep, mptr, mcode = _lib.mask_arg(attention_mask)
-    cu = torch.empty(batch + 1, dtype=torch.int64, device=dev)
-    counts = torch.empty(max(batch, 1), dtype=torch.int64, device=dev)
-    with _lib.on_device(dev):
-        st = stream_of(dev)
-        call("orlhf_mask_row_counts", mptr, mcode, batch, seqlen, ptr(counts), st)
-        call("orlhf_cu_seqlens", ptr(counts), batch, ptr(cu), st)
+    cu, tiles = _count(mptr, mcode, batch, seqlen, dev)
     total = int(cu[-1]) if total_tokens is None else int(total_tokens)
     indices = torch.empty(max(total, 1), dtype=torch.int64, device=dev)
     if total > 0:
         with _lib.on_device(dev):
-            call("orlhf_unpad_sequences", None, mptr, mcode, batch, seqlen, ptr(cu), total, ptr(indices), None, None, None,
-                 stream_of(dev))
+            call("orlhf_unpad_sequences", None, mptr, mcode, batch, seqlen, ptr(cu), ptr(tiles), total, ptr(indices), None,
+                 None, None, stream_of(dev))
     return indices[:total]
 
 

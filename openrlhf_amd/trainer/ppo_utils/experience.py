@@ -77,6 +77,36 @@ def pack_padded(x: torch.Tensor, cu_seqlens: torch.Tensor, first: Optional[torch
     return out
 
 
+def pack_padded_fields(fields: Dict[str, Optional[torch.Tensor]], cu_seqlens: torch.Tensor,
+                       first: Optional[torch.Tensor], total: int) -> Dict[str, Optional[torch.Tensor]]:
+    """``pack_padded`` of every ``[B, A]`` tensor in ``fields`` (``None`` entries are carried through)
+    with one launch per eight fields instead of one per field."""
+    live = {k: v for k, v in fields.items() if v is not None}
+    out: Dict[str, Optional[torch.Tensor]] = {k: None for k in fields}
+    if not live:
+        return out
+    dev = require_gpu(cu_seqlens, first, *live.values())
+    shape = next(iter(live.values())).shape
+    for k, v in live.items():
+        if v.dim() != 2 or v.shape != shape or cu_seqlens.numel() != shape[0] + 1:
+            raise ValueError(f"field {k}: {tuple(v.shape)} against {tuple(shape)} and {cu_seqlens.numel()} boundaries")
+        if v.element_size() not in _BITS:
+            raise ValueError(f"unsupported element size {v.element_size()}")
+    srcs = {k: v.contiguous() for k, v in live.items()}
+    for k, v in srcs.items():
+        out[k] = torch.empty(total, dtype=v.dtype, device=dev)
+    if total == 0:
+        return out
+    cu = cu_seqlens.to(torch.int64).contiguous()
+    f = None if first is None else first.to(torch.int64).contiguous()
+    arr = (_lib.PackField * len(srcs))()
+    for i, (k, v) in enumerate(srcs.items()):
+        arr[i].src, arr[i].dst, arr[i].elem_bytes = v.data_ptr(), out[k].data_ptr(), v.element_size()
+    with _lib.on_device(dev):
+        call("orlhf_pack_rows_multi", arr, len(srcs), shape[0], shape[1], ptr(f), ptr(cu), stream_of(dev))
+    return out
+
+
 def pad_packed(flat: torch.Tensor, cu_seqlens: torch.Tensor, n_cols: int, side: str = "right", value=0) -> torch.Tensor:
     """``[B, n_cols]`` tensor whose row b holds tokens ``cu[b] .. cu[b+1]-1`` of ``flat`` with
     ``value`` as padding on ``side`` — ``zero_pad_sequences(rows, side, value, stack=True)``
@@ -117,7 +147,7 @@ class PackedSteps:
         first, _, length = row_extents(mask)
         cu = cu_seqlens_of(length)
         total = int(cu[-1]) if total is None else int(total)
-        packed = {k: (None if v is None else pack_padded(v, cu, first, total)) for k, v in fields.items()}
+        packed = pack_padded_fields(fields, cu, first, total)
         return cls(cu, first, mask.shape[1], total, packed)
 
     @property

@@ -144,3 +144,54 @@ def test_unpad_empty_and_errors():
         unpad_and_slice_tensor(seq, torch.ones_like(seq), object())
     with pytest.raises(ValueError):
         unpad_and_slice_tensor(seq, torch.ones(3, 7, dtype=torch.long, device=_dev()), None)
+
+
+@pytest.mark.parametrize("kind", ["right", "left", "both", "holes", "full", "empty_rows"])
+def test_tile_and_row_walks_agree(kind):
+    """The C entry point with the per-tile counts (one workgroup per tile) and without them (one
+    workgroup walks a row): the same outputs, bit for bit, on rows that span several tiles of
+    ORLHF_UNPAD_TILE columns, and both equal the oracle."""
+    from openrlhf_amd import _lib
+    from openrlhf_amd._lib import call, ptr, stream_of
+
+    g = torch.Generator().manual_seed(21)
+    batch, seqlen = 7, 3 * _lib.UNPAD_TILE + 777
+    if kind == "full":
+        mask = torch.ones(batch, seqlen, dtype=torch.long)
+    elif kind == "empty_rows":
+        mask = _mask("holes", batch, seqlen, g)
+        mask[1] = 0
+        mask[5] = 0
+    else:
+        mask = _mask(kind, batch, seqlen, g)
+    seq = torch.randint(0, 50000, (batch, seqlen), generator=g)
+    want = olay.unpad_and_slice_tensor(seq, mask)
+    d = _dev()
+    seq_d, mask_d = seq.to(d), mask.to(torch.uint8).to(d)
+    counts = torch.empty(batch, dtype=torch.int64, device=d)
+    n_tiles = (seqlen + _lib.UNPAD_TILE - 1) // _lib.UNPAD_TILE
+    tiles = torch.full((batch, n_tiles), -1, dtype=torch.int32, device=d)
+    cu = torch.empty(batch + 1, dtype=torch.int64, device=d)
+    st = stream_of(d)
+    call("orlhf_mask_row_counts", ptr(mask_d), _lib.MASK_U8, batch, seqlen, ptr(counts), ptr(tiles), st)
+    call("orlhf_cu_seqlens", ptr(counts), batch, ptr(cu), st)
+    assert torch.equal(counts.cpu(), mask.sum(1))
+    assert torch.equal(tiles.cpu().long(), torch.stack([mask[:, i * _lib.UNPAD_TILE:(i + 1) * _lib.UNPAD_TILE].sum(1) for i in range(n_tiles)], 1))
+    total = int(cu[-1])
+    outs = []
+    for tile_counts in (tiles, None):
+        out = torch.full((4, max(total, 1)), -7, dtype=torch.int64, device=d)
+        call("orlhf_unpad_sequences", ptr(seq_d), ptr(mask_d), _lib.MASK_U8, batch, seqlen, ptr(cu), ptr(tile_counts), total,
+             ptr(out[0]), ptr(out[1]), ptr(out[2]), ptr(out[3]), st)
+        outs.append(out[:, :total].cpu())
+    assert torch.equal(outs[0], outs[1])
+    indices, packed, rolled, position = outs[0]
+    assert torch.equal(packed, want[0][0]) and torch.equal(position, want[1][0]) and torch.equal(rolled, want[2][0])
+    assert torch.equal(indices, want[4])
+    # a capacity below the total: the slots past it are dropped, the others are unchanged
+    if total > 100:
+        cap = total - 37
+        out = torch.full((4, total), -7, dtype=torch.int64, device=d)
+        call("orlhf_unpad_sequences", ptr(seq_d), ptr(mask_d), _lib.MASK_U8, batch, seqlen, ptr(cu), ptr(tiles), cap,
+             ptr(out[0]), ptr(out[1]), ptr(out[2]), ptr(out[3]), st)
+        assert torch.equal(out[:, :cap].cpu(), outs[0][:, :cap]) and bool((out[:, cap:] == -7).all())
