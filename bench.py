@@ -374,9 +374,15 @@ def bench_few_rows(dev, n=64, vocab=VOCAB, copies=32):
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=dev)
     st = stream_of(dev)
 
-    def cut(x):
+    tickets = torch.zeros(n, dtype=torch.int32, device=dev)
+
+    def cut(x):  # one launch: the workgroup that finishes a row's last segment merges the row
         call("orlhf_logprob_entropy_fwd_split", ptr(x), _lib.BF16, n, vocab, vocab, ptr(labels), 1.0, ptr(lp), ptr(ent),
-             ptr(stats), None, ptr(ws), ws_bytes, st)
+             ptr(stats), None, ptr(ws), ws_bytes, ptr(tickets), st)
+
+    def cut_two_launches(x):  # no tickets: a second kernel merges
+        call("orlhf_logprob_entropy_fwd_split", ptr(x), _lib.BF16, n, vocab, vocab, ptr(labels), 1.0, ptr(lp), ptr(ent),
+             ptr(stats), None, ptr(ws), ws_bytes, None, st)
 
     def whole(x):
         call("orlhf_logprob_entropy_fwd", ptr(x), _lib.BF16, n, vocab, vocab, ptr(labels), 1.0, ptr(lp), ptr(ent),
@@ -398,7 +404,9 @@ def bench_few_rows(dev, n=64, vocab=VOCAB, copies=32):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / len(xs)
 
-    whole_ms, cut_ms = timed(whole), timed(cut)
+    whole_ms, cut_ms, cut2_ms = timed(whole), timed(cut), timed(cut_two_launches)
+    cut_two_launches(xs[0])
+    lp_cut2 = lp.clone()
     cut(xs[0])
     lp_cut = lp.clone()
     whole(xs[0])
@@ -409,6 +417,8 @@ def bench_few_rows(dev, n=64, vocab=VOCAB, copies=32):
         "segments_per_row": ws_bytes // (n * 32) if ws_bytes else 1,
         "forward_whole_rows_us": whole_ms * 1e3, "forward_whole_rows_gbs": n * row_bytes / whole_ms / 1e6,
         "forward_cut_rows_us": cut_ms * 1e3, "forward_cut_rows_gbs": n * row_bytes / cut_ms / 1e6,
+        "forward_cut_rows_merge_kernel_us": cut2_ms * 1e3,
+        "cut_rows_one_launch_equals_two_launches": bool(torch.equal(lp_cut, lp_cut2)),
         "backward_cut_rows_us": bwd_ms * 1e3, "backward_cut_rows_gbs": 2 * n * row_bytes / bwd_ms / 1e6,
         "max_abs_diff_cut_vs_whole": (lp_cut - lp).abs().max().item(),
         "note": "a launch this small is a few microseconds: the times include the launch itself and the ramp of the "

@@ -34,7 +34,7 @@
 extern "C" {
 #endif
 
-#define ORLHF_ABI_VERSION 22
+#define ORLHF_ABI_VERSION 23
 
 #define ORLHF_OK 0
 #define ORLHF_ERR_INVALID_ARG (-1) /* null pointer, bad size / dtype / enum                     */
@@ -113,21 +113,29 @@ int orlhf_divide_rows_inplace(void* logits, int dtype, int64_t n_rows, int64_t v
 /*
  * The same forward for launches with fewer rows than the GPU has compute units (short rollouts,
  * a 64-token micro-batch): every row is cut into segments, one workgroup per (row, segment)
- * writes a partial record (running maxima and sums) into `workspace`, and a second small kernel
- * merges a row's records in segment order and finishes the row as the whole-row kernel does. Same
+ * writes a partial record (running maxima and sums) into `workspace`, and the records of a row are
+ * merged in segment order, in fp64, and the row finished as the whole-row kernel does. Same
  * arguments, outputs and conventions as orlhf_logprob_entropy_fwd (same reference lines:
  * openrlhf/models/utils.py:139-163,182-186); results agree with it to the rounding of the fp32
  * partial sums. orlhf_logprob_entropy_split_workspace_bytes returns the bytes this shape needs, 0
  * when the rows would not be cut (256 rows or more, or rows shorter than 64 KiB); then the call is
  * orlhf_logprob_entropy_fwd itself and `workspace` may be NULL. The cut depends on the shape
  * only. orlhf_logprob_entropy_bwd needs no workspace and cuts its rows by the same rule itself.
+ *
+ * Who merges: with `tickets` NULL a second small kernel does. With `tickets` (n_rows int32, ALL
+ * ZERO on entry) the forward kernel does it itself: every segment draws a ticket of its row when
+ * its record is written, and the workgroup that draws the last one merges the row and puts the
+ * ticket back to zero, so one launch is all and the same array serves the next call unchanged.
+ * Nothing waits for anything. Both ways merge the same records in the same order: the outputs are
+ * bit-identical. Calls that may overlap on the GPU need ticket arrays of their own, and an array
+ * whose call was aborted midway has to be zeroed again.
  */
 int64_t orlhf_logprob_entropy_split_workspace_bytes(int dtype, int64_t n_rows, int64_t vocab);
 int orlhf_logprob_entropy_fwd_split(const void* logits, int dtype, int64_t n_rows, int64_t vocab,
                                     int64_t row_stride, const int64_t* labels, double temperature,
                                     float* logprob, float* entropy, float* row_stats,
                                     const uint8_t* row_mask, void* workspace, int64_t workspace_bytes,
-                                    orlhf_stream_t stream);
+                                    int32_t* tickets, orlhf_stream_t stream);
 
 /*
  * Backward of the above in one streaming pass, written in the logits dtype:

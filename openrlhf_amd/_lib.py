@@ -22,7 +22,7 @@ IS_NONE, IS_TIS, IS_ICEPOP, IS_SEQ_MASK_TIS = 0, 1, 2, 3
 GROUP_IDENTITY, GROUP_RLOO, GROUP_BASELINE, GROUP_NORM = 0, 1, 2, 3
 PAIR_DPO_SIGMOID, PAIR_DPO_IPO, PAIR_LOGSIGMOID, PAIR_LOGEXP = 0, 1, 2, 3
 
-ABI_VERSION = 22
+ABI_VERSION = 23
 UNPAD_TILE = 2048  # ORLHF_UNPAD_TILE
 
 
@@ -77,7 +77,7 @@ SIGNATURES = {
     "orlhf_last_error": (c_char_p, []),
     "orlhf_logprob_entropy_fwd": (c_int, [P, c_int, I64, I64, I64, P, c_double, P, P, P, P, c_int, P]),
     "orlhf_logprob_entropy_split_workspace_bytes": (I64, [c_int, I64, I64]),
-    "orlhf_logprob_entropy_fwd_split": (c_int, [P, c_int, I64, I64, I64, P, c_double, P, P, P, P, P, I64, P]),
+    "orlhf_logprob_entropy_fwd_split": (c_int, [P, c_int, I64, I64, I64, P, c_double, P, P, P, P, P, I64, P, P]),
     "orlhf_divide_rows_inplace": (c_int, [P, c_int, I64, I64, I64, c_double, P]),
     "orlhf_logprob_entropy_bwd": (c_int, [P, P, c_int, I64, I64, I64, I64, P, c_double, P, P, P, P, P]),
     "orlhf_logprob_entropy_fwd_bwd_max_vocab": (I64, [c_int]),

@@ -192,6 +192,7 @@ struct RowSplit {
   int n;
   uint32_t seg_elems;
   float* partials;
+  int* tickets = nullptr;  // one per row, zero between launches: the segment that arrives last merges its row
 };
 
 struct WorkItem {
@@ -208,6 +209,83 @@ __device__ __forceinline__ WorkItem work_item(int64_t w, const RowSplit& split, 
 }
 
 __device__ __forceinline__ bool sums_usable(float s) { return s > 0.0f && s < INFINITY; }
+
+// Merges the segment records of one row and finishes the row exactly as the whole-row epilogue
+// does: ONE WAVE calls it, lane k holds segment k (at most 64), maxima and sums go through the
+// fixed butterfly of the wave reductions in fp64, so the result does not depend on which segment was
+// written when. FRESH: the records were written by other workgroups of the same launch; they are
+// read past the L1, which may hold a line from before a neighbouring record was written.
+template <bool FRESH>
+__device__ __forceinline__ void merge_row(int64_t row_i, int64_t vocab, const int64_t* __restrict__ labels, double temperature,
+                                          float* __restrict__ logprob, float* __restrict__ entropy,
+                                          float* __restrict__ row_stats, bool scaled_set, bool plain_set, bool want_lp,
+                                          const RowSplit& split) {
+  const double c_plain = 1.4426950408889634, c_scaled = 1.4426950408889634 / temperature;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t label = want_lp ? labels[row_i] : -1;
+  // maxima in log2 units: a fast-pass record holds them so, a safe-pass record holds the segment
+  // maximum in logit units in both fields. Lanes past the last segment hold the neutral record.
+  double mt = -INFINITY, m1 = -INFINITY, sT = 0.0, s1 = 0.0, t1 = 0.0;
+  float x_label = 0.0f;  // the segment that holds the label has read its logit
+  if (lane < split.n) {
+    const float* rec = split.partials + (row_i * split.n + lane) * kPartial;
+    float r[kPartial];
+    if (FRESH) {
+#pragma unroll
+      for (int k = 0; k < kPartial; k += 2) {
+        const uint64_t two = __hip_atomic_load((const uint64_t*)rec + k / 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        r[k] = as_float((uint32_t)two);
+        r[k + 1] = as_float((uint32_t)(two >> 32));
+      }
+    } else {
+      const f32x4 a = *(const f32x4*)rec, b = *(const f32x4*)(rec + 4);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) r[k] = a[k], r[4 + k] = b[k];
+    }
+    const bool fast = r[5] != 0.0f;
+    mt = (double)r[0] * (fast ? 1.0 : c_scaled);
+    m1 = (double)r[2] * (fast ? 1.0 : c_plain);
+    sT = (double)r[1];
+    s1 = (double)r[3];
+    t1 = (double)r[4];
+    if (label >= 0 && label < vocab && (uint32_t)lane == (uint32_t)label / split.seg_elems) x_label = r[6];
+  }
+  x_label = wave_sum(x_label);  // one lane holds it, the others 0
+  double MT = mt, M1 = m1;
+#pragma unroll
+  for (int o = kWave / 2; o > 0; o >>= 1) {
+    const double ot = __shfl_xor(MT, o, kWave), o1 = __shfl_xor(M1, o, kWave);
+    MT = ot > MT ? ot : MT;
+    M1 = o1 > M1 ? o1 : M1;
+  }
+  // a segment at the row maximum (or one that saw nothing finite) keeps its sums as they are:
+  // 0, or the NaN markers of the safe pass
+  const double rT = (mt != -INFINITY && mt != MT) ? exp2(mt - MT) : 1.0;
+  const double r1 = (m1 != -INFINITY && m1 != M1) ? exp2(m1 - M1) : 1.0;
+  sT = wave_sum(sT * rT);
+  s1 = wave_sum(s1 * r1);
+  t1 = wave_sum(t1 * r1);
+  if (lane != 0) return;
+  double lse_t = 0.0, lse_1 = 0.0, ex = 0.0;
+  if (scaled_set) lse_t = MT * kLn2d + log(sT);
+  if (plain_set) {
+    lse_1 = M1 * kLn2d + log(s1);
+    ex = t1 / s1;
+    if (!scaled_set) lse_t = lse_1;
+  }
+  if (want_lp) {
+    float lp;
+    if (label >= 0 && label < vocab) {
+      lp = (float)((double)x_label / temperature - lse_t);
+    } else {
+      lp = (label == -100) ? 0.0f : NAN;
+    }
+    logprob[row_i] = lp;
+  }
+  if (plain_set && entropy != nullptr) entropy[row_i] = (float)(lse_1 - ex);
+  if (row_stats != nullptr)
+    *(f32x4*)(row_stats + row_i * 4) = f32x4{(float)lse_t, (float)(plain_set ? lse_1 : lse_t), (float)ex, 0.0f};
+}
 
 // ---------------------------------------------------------------- forward kernel
 template <int DT, int MODE>
@@ -231,7 +309,8 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
     const WorkItem item = work_item(work, split, vocab);
     const int64_t row_i = item.row;
     if (row_mask != nullptr && row_mask[row_i] == 0) {  // row not wanted: outputs 0, logits not read
-      if (split.n > 1) continue;                        // (the merging kernel writes the zeros)
+      // cut rows: the merging kernel writes the zeros, or the row's first segment where nothing merges
+      if (split.n > 1 && (split.tickets == nullptr || item.first != 0u)) continue;
       if (tid == 0) {
         if (MODE != kEntOnly && logprob != nullptr) logprob[row_i] = 0.0f;
         if (MT::kPlainSet && entropy != nullptr) entropy[row_i] = 0.0f;
@@ -242,6 +321,16 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
     const char* row = logits + row_i * row_stride_bytes + (int64_t)item.first * E::kSize;
     const int64_t seg_len = item.len;
     const RowGeom g = row_geom<DT>(row, seg_len, scalar_only != 0);
+
+    // the label and its logit, asked for now: the row's last instructions do not wait on two
+    // dependent loads then (on a launch of a few microseconds that wait is a tenth of the whole)
+    int64_t label = -1;
+    float x_label = 0.0f;
+    if (MODE != kEntOnly && logprob != nullptr && tid == 0) {
+      label = labels[row_i];
+      const int64_t at = label - (int64_t)item.first;
+      if (at >= 0 && at < seg_len) x_label = E::load1(row + at * E::kSize);
+    }
 
     // ---- reference maximum of this wave: first vector (or first scalar) of each lane
     float m_ref = -INFINITY;
@@ -347,15 +436,37 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
     }
 
     if (split.n > 1) {  // a segment: its sums go to the merging kernel as they are
+      int drawn = 0;
       if (tid == 0) {
-        float x_label = 0.0f;
-        if (MODE != kEntOnly && logprob != nullptr) {
-          const int64_t at = labels[row_i] - (int64_t)item.first;
-          if (at >= 0 && at < seg_len) x_label = E::load1(row + at * E::kSize);
-        }
         float* rec = split.partials + work * kPartial;
-        *(f32x4*)rec = f32x4{sums.MT, sums.sT, sums.M1, sums.s1};
-        *(f32x4*)(rec + 4) = f32x4{sums.t1, ok ? 1.0f : 0.0f, x_label, 0.0f};
+        const float r[kPartial] = {sums.MT, sums.sT, sums.M1, sums.s1, sums.t1, ok ? 1.0f : 0.0f, x_label, 0.0f};
+        if (split.tickets == nullptr) {
+          *(f32x4*)rec = f32x4{r[0], r[1], r[2], r[3]};
+          *(f32x4*)(rec + 4) = f32x4{r[4], r[5], r[6], r[7]};
+        } else {
+          // The segment that takes the row's last ticket finds every record of the row written and
+          // merges them, in segment order whoever came when. Nobody waits for anybody; the ticket
+          // goes back to zero for the next launch. Records and tickets go to and come from device
+          // memory as device-scope accesses, which pass the caches that the compute dies do not
+          // share; a writer has its stores acknowledged before it draws. (A device-scope fence
+          // would do as well, at the price of walking a die's whole L2 per workgroup: several
+          // microseconds on a launch that takes ten.)
+#pragma unroll
+          for (int k = 0; k < kPartial; k += 2) {
+            const uint64_t two = (uint64_t)__builtin_bit_cast(uint32_t, r[k]) | (uint64_t)__builtin_bit_cast(uint32_t, r[k + 1]) << 32;
+            __hip_atomic_store((uint64_t*)rec + k / 2, two, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+          __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+          __builtin_amdgcn_s_waitcnt(0);  // vmcnt(0): this thread's stores have been acknowledged
+          drawn = __hip_atomic_fetch_add(split.tickets + row_i, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      if (split.tickets != nullptr && wave == 0) {  // the other waves go on to their next segment
+        if (__shfl(drawn, 0, kWave) == split.n - 1) {
+          merge_row<true>(row_i, vocab, labels, temperature, logprob, entropy, row_stats, MT::kScaledSet, MT::kPlainSet,
+                          MODE != kEntOnly && logprob != nullptr, split);
+          if (lane == 0) __hip_atomic_store(split.tickets + row_i, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
       }
       continue;
     }
@@ -374,11 +485,9 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
         if (!MT::kScaledSet) lse_t = lse_1;  // T == 1 (or entropy only)
       }
       if (MODE != kEntOnly && logprob != nullptr) {
-        const int64_t label = labels[row_i];
         float lp;
         if (label >= 0 && label < vocab) {
-          const double xl = (double)E::load1(row + label * E::kSize);
-          lp = (float)(xl / temperature - lse_t);
+          lp = (float)((double)x_label / temperature - lse_t);
         } else {
           lp = (label == -100) ? 0.0f : NAN;
         }
@@ -393,18 +502,13 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_fwd_kernel(
   }
 }
 
-// Merges the segment records of every row and finishes the row exactly as the whole-row epilogue
-// does: one wave per row, lane k holds segment k (at most 64), maxima and sums go through the
-// fixed butterfly of the wave reductions in fp64, so the result does not depend on scheduling.
+// The merge as a launch of its own (callers that pass no tickets): one wave per row.
 template <int DT>
 __global__ __launch_bounds__(kBlock) void logprob_entropy_merge_kernel(
-    const char* __restrict__ logits, int64_t n_rows, int64_t vocab, int64_t row_stride_bytes,
-    const int64_t* __restrict__ labels, double temperature, float* __restrict__ logprob,
+    int64_t n_rows, int64_t vocab, const int64_t* __restrict__ labels, double temperature, float* __restrict__ logprob,
     float* __restrict__ entropy, float* __restrict__ row_stats, const uint8_t* __restrict__ row_mask,
     int mode, RowSplit split) {
-  using E = Elt<DT>;
   const bool scaled_set = (mode == kLpOnly || mode == kBothT), plain_set = (mode != kLpOnly);
-  const double c_plain = 1.4426950408889634, c_scaled = 1.4426950408889634 / temperature;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t row_i = (int64_t)blockIdx.x * kWavesPerBlock + threadIdx.x / kWave;
   if (row_i >= n_rows) return;
@@ -417,57 +521,7 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_merge_kernel(
     }
     return;
   }
-  const int64_t label = want_lp ? labels[row_i] : -1;
-  // maxima in log2 units: a fast-pass record holds them so, a safe-pass record holds the segment
-  // maximum in logit units in both fields. Lanes past the last segment hold the neutral record.
-  double mt = -INFINITY, m1 = -INFINITY, sT = 0.0, s1 = 0.0, t1 = 0.0;
-  float x_label = 0.0f;  // the segment that holds the label has read its logit
-  if (lane < split.n) {
-    const float* rec = split.partials + (row_i * split.n + lane) * kPartial;
-    const f32x4 a = *(const f32x4*)rec, b = *(const f32x4*)(rec + 4);
-    const bool fast = b[1] != 0.0f;
-    mt = (double)a[0] * (fast ? 1.0 : c_scaled);
-    m1 = (double)a[2] * (fast ? 1.0 : c_plain);
-    sT = (double)a[1];
-    s1 = (double)a[3];
-    t1 = (double)b[0];
-    if (label >= 0 && label < vocab && (uint32_t)lane == (uint32_t)label / split.seg_elems) x_label = b[2];
-  }
-  x_label = wave_sum(x_label);  // one lane holds it, the others 0
-  double MT = mt, M1 = m1;
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    const double ot = __shfl_xor(MT, o, kWave), o1 = __shfl_xor(M1, o, kWave);
-    MT = ot > MT ? ot : MT;
-    M1 = o1 > M1 ? o1 : M1;
-  }
-  // a segment at the row maximum (or one that saw nothing finite) keeps its sums as they are:
-  // 0, or the NaN markers of the safe pass
-  const double rT = (mt != -INFINITY && mt != MT) ? exp2(mt - MT) : 1.0;
-  const double r1 = (m1 != -INFINITY && m1 != M1) ? exp2(m1 - M1) : 1.0;
-  sT = wave_sum(sT * rT);
-  s1 = wave_sum(s1 * r1);
-  t1 = wave_sum(t1 * r1);
-  if (lane != 0) return;
-  double lse_t = 0.0, lse_1 = 0.0, ex = 0.0;
-  if (scaled_set) lse_t = MT * kLn2d + log(sT);
-  if (plain_set) {
-    lse_1 = M1 * kLn2d + log(s1);
-    ex = t1 / s1;
-    if (!scaled_set) lse_t = lse_1;
-  }
-  if (want_lp) {
-    float lp;
-    if (label >= 0 && label < vocab) {
-      lp = (float)((double)x_label / temperature - lse_t);
-    } else {
-      lp = (label == -100) ? 0.0f : NAN;
-    }
-    logprob[row_i] = lp;
-  }
-  if (plain_set && entropy != nullptr) entropy[row_i] = (float)(lse_1 - ex);
-  if (row_stats != nullptr)
-    *(f32x4*)(row_stats + row_i * 4) = f32x4{(float)lse_t, (float)(plain_set ? lse_1 : lse_t), (float)ex, 0.0f};
+  merge_row<false>(row_i, vocab, labels, temperature, logprob, entropy, row_stats, scaled_set, plain_set, want_lp, split);
 }
 
 // ---------------------------------------------------------------- backward kernel
@@ -559,7 +613,7 @@ static RowSplit row_split(int64_t n_rows, int64_t vocab, int esize) {
 template <int DT>
 static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t row_stride,
                       const int64_t* labels, double temperature, float* logprob, float* entropy,
-                      float* row_stats, const uint8_t* row_mask, void* workspace, int64_t workspace_bytes,
+                      float* row_stats, const uint8_t* row_mask, void* workspace, int64_t workspace_bytes, int* tickets,
                       hipStream_t stream) {
   using E = Elt<DT>;
   const bool want_lp = logprob != nullptr;
@@ -578,6 +632,7 @@ static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
                       "logprob_entropy_fwd_split: workspace of %lld bytes too small or not 16-byte aligned",
                       (long long)workspace_bytes);
       split.partials = (float*)workspace;
+      split.tickets = tickets;
     }
   }
   const dim3 grid(grid_for_rows(n_rows * split.n)), block(kBlock);
@@ -593,10 +648,9 @@ static int launch_fwd(const void* logits, int64_t n_rows, int64_t vocab, int64_t
   }
 #undef ORLHF_FWD
   ORLHF_CHECK_LAUNCH("orlhf_logprob_entropy_fwd");
-  if (split.n > 1) {
+  if (split.n > 1 && split.tickets == nullptr) {
     hipLaunchKernelGGL((logprob_entropy_merge_kernel<DT>), dim3((unsigned)((n_rows + kWavesPerBlock - 1) / kWavesPerBlock)), block, 0,
-                       stream, p, n_rows, vocab, stride_bytes, labels, temperature, logprob, entropy, row_stats,
-                       row_mask, mode, split);
+                       stream, n_rows, vocab, labels, temperature, logprob, entropy, row_stats, row_mask, mode, split);
     ORLHF_CHECK_LAUNCH("orlhf_logprob_entropy_fwd_split(merge)");
   }
   return ORLHF_OK;
@@ -688,7 +742,7 @@ extern "C" int orlhf_divide_rows_inplace(void* logits, int dtype, int64_t n_rows
 static int forward_entry(const void* logits, int dtype, int64_t n_rows, int64_t vocab, int64_t row_stride,
                          const int64_t* labels, double temperature, float* logprob, float* entropy,
                          float* row_stats, const uint8_t* row_mask, int flags, void* workspace,
-                         int64_t workspace_bytes, orlhf_stream_t stream) {
+                         int64_t workspace_bytes, int32_t* tickets, orlhf_stream_t stream) {
   ORLHF_CHECK_ARG(n_rows >= 0 && vocab > 0, "logprob_entropy_fwd: n_rows=%lld vocab=%lld",
                   (long long)n_rows, (long long)vocab);
   ORLHF_CHECK_ARG(row_stride >= vocab, "logprob_entropy_fwd: row_stride %lld < vocab %lld",
@@ -708,15 +762,15 @@ static int forward_entry(const void* logits, int dtype, int64_t n_rows, int64_t 
     case ORLHF_F32:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 3u) == 0, "logprob_entropy_fwd: logits not 4-byte aligned");
       return launch_fwd<ORLHF_F32>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                   entropy, row_stats, row_mask, workspace, workspace_bytes, s);
+                                   entropy, row_stats, row_mask, workspace, workspace_bytes, tickets, s);
     case ORLHF_BF16:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 1u) == 0, "logprob_entropy_fwd: logits not 2-byte aligned");
       return launch_fwd<ORLHF_BF16>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                    entropy, row_stats, row_mask, workspace, workspace_bytes, s);
+                                    entropy, row_stats, row_mask, workspace, workspace_bytes, tickets, s);
     case ORLHF_F16:
       ORLHF_CHECK_ARG(((uintptr_t)logits & 1u) == 0, "logprob_entropy_fwd: logits not 2-byte aligned");
       return launch_fwd<ORLHF_F16>(logits, n_rows, vocab, row_stride, labels, temperature, logprob,
-                                   entropy, row_stats, row_mask, workspace, workspace_bytes, s);
+                                   entropy, row_stats, row_mask, workspace, workspace_bytes, tickets, s);
     default:
       return fail(ORLHF_ERR_INVALID_ARG, "logprob_entropy_fwd: unknown dtype %d", dtype);
   }
@@ -728,7 +782,7 @@ extern "C" int orlhf_logprob_entropy_fwd(const void* logits, int dtype, int64_t 
                                          float* row_stats, const uint8_t* row_mask, int flags,
                                          orlhf_stream_t stream) {
   return forward_entry(logits, dtype, n_rows, vocab, row_stride, labels, temperature, logprob, entropy, row_stats,
-                       row_mask, flags, nullptr, 0, stream);
+                       row_mask, flags, nullptr, 0, nullptr, stream);
 }
 
 extern "C" int64_t orlhf_logprob_entropy_split_workspace_bytes(int dtype, int64_t n_rows, int64_t vocab) {
@@ -741,11 +795,12 @@ extern "C" int orlhf_logprob_entropy_fwd_split(const void* logits, int dtype, in
                                                int64_t row_stride, const int64_t* labels, double temperature,
                                                float* logprob, float* entropy, float* row_stats,
                                                const uint8_t* row_mask, void* workspace, int64_t workspace_bytes,
-                                               orlhf_stream_t stream) {
+                                               int32_t* tickets, orlhf_stream_t stream) {
+  ORLHF_CHECK_ARG(((uintptr_t)tickets & 3u) == 0, "logprob_entropy_fwd_split: tickets not 4-byte aligned");
   ORLHF_CHECK_ARG(workspace != nullptr || orlhf_logprob_entropy_split_workspace_bytes(dtype, n_rows, vocab) == 0,
                   "logprob_entropy_fwd_split: this shape needs a workspace (orlhf_logprob_entropy_split_workspace_bytes)");
   return forward_entry(logits, dtype, n_rows, vocab, row_stride, labels, temperature, logprob, entropy, row_stats,
-                       row_mask, 0, workspace, workspace_bytes, stream);
+                       row_mask, 0, workspace, workspace_bytes, tickets, stream);
 }
 
 extern "C" int orlhf_logprob_entropy_bwd(const void* logits, void* grad_logits, int dtype,

@@ -45,14 +45,32 @@ def _as_rows(logits: torch.Tensor):
 
 
 
+_TICKETS = {}  # (device index, stream handle) -> int32 tickets, all zero whenever no forward is in flight
+
+
+def _row_tickets(dev, n_rows):
+    """The tickets of the few-row forward: zero on entry, put back to zero by the kernel itself, so one
+    array per (device, stream) serves every call (calls on one stream do not overlap). Allocated and
+    zeroed outside any graph capture: the few-row launch is at most 255 rows, so 256 always do."""
+    key = (dev.index if dev.index is not None else torch.cuda.current_device(), stream_of(dev))
+    t = _TICKETS.get(key)
+    if t is None or t.numel() < n_rows:
+        if torch.cuda.is_current_stream_capturing():
+            return None  # first use of this stream is under capture: the two-launch form needs no state
+        t = _TICKETS[key] = torch.zeros(max(256, n_rows), dtype=torch.int32, device=dev)
+    return t
+
+
 def _forward_rows(rows, code, n_rows, vocab, row_stride, lab, temperature, logprob, entropy, stats, rmask, dev):
     """One forward launch over vocabulary rows. With fewer rows than the GPU has compute units the
-    rows are cut into segments (one workgroup each) whose partial sums a second kernel merges."""
+    rows are cut into segments (one workgroup each); the workgroup that finishes a row's last segment
+    merges the row's partial sums."""
     ws_bytes = _lib.load().orlhf_logprob_entropy_split_workspace_bytes(code, n_rows, vocab)
     if ws_bytes > 0:
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
         call("orlhf_logprob_entropy_fwd_split", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
-             float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), ptr(ws), ws_bytes, stream_of(dev))
+             float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), ptr(ws), ws_bytes,
+             ptr(_row_tickets(dev, n_rows)), stream_of(dev))
     else:
         call("orlhf_logprob_entropy_fwd", ptr(rows), code, n_rows, vocab, row_stride, ptr(lab),
              float(temperature), ptr(logprob), ptr(entropy), ptr(stats), ptr(rmask), 0, stream_of(dev))

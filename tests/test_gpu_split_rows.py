@@ -191,11 +191,81 @@ def test_split_entry_contract(cuda):
     ws = torch.empty(need, dtype=torch.uint8, device=cuda)
     args = (ptr(xd), 1, 64, 151936, 151936, ptr(ld), 1.0, ptr(lp), ptr(ent), None, None)
     with pytest.raises(_lib.KernelError, match="workspace"):
-        call("orlhf_logprob_entropy_fwd_split", *args, None, 0, stream_of(cuda))
+        call("orlhf_logprob_entropy_fwd_split", *args, None, 0, None, stream_of(cuda))
     with pytest.raises(_lib.KernelError, match="workspace"):
-        call("orlhf_logprob_entropy_fwd_split", *args, ptr(ws), need - 1, stream_of(cuda))
-    call("orlhf_logprob_entropy_fwd_split", *args, ptr(ws), need, stream_of(cuda))
+        call("orlhf_logprob_entropy_fwd_split", *args, ptr(ws), need - 1, None, stream_of(cuda))
+    call("orlhf_logprob_entropy_fwd_split", *args, ptr(ws), need, None, stream_of(cuda))
     lp2, ent2 = torch.empty(64, device=cuda), torch.empty(64, device=cuda)
     call("orlhf_logprob_entropy_fwd", ptr(xd), 1, 64, 151936, 151936, ptr(ld), 1.0, ptr(lp2), ptr(ent2), None, None, 0,
          stream_of(cuda))
     assert (lp - lp2).abs().max().item() <= 4e-6 and (ent - ent2).abs().max().item() <= 4e-6
+
+
+@pytest.mark.parametrize("rows", [1, 7, 64, 255])
+@pytest.mark.parametrize(
+    "vocab,dtype,temperature,want",
+    [
+        (151936, torch.bfloat16, 1.0, "both"),
+        (151936, torch.bfloat16, 0.6, "both"),
+        (151936, torch.bfloat16, 0.6, "logprob"),
+        (50257, torch.float32, 0.7, "entropy"),
+        (65536, torch.float16, 1.0, "both"),
+    ],
+)
+def test_merge_by_last_segment_is_bit_identical(cuda, rows, vocab, dtype, temperature, want):
+    """With tickets the forward kernel merges a row in the workgroup that finishes its last segment;
+    without, a second kernel does. Same records, same order: the same bits, whichever workgroup
+    came last, launch after launch on the same ticket array (the kernel leaves it zero), with rows
+    masked out, extreme rows (the safe pass) and labels outside the vocabulary among them."""
+    from openrlhf_amd import _lib
+    from openrlhf_amd._lib import call, ptr, stream_of
+
+    lib = _lib.load()
+    x, labels, _, _ = _case(rows, vocab, dtype, 3.0, seed=rows + vocab)
+    x[0, 5] = 30000.0 if dtype == torch.float16 else 3e38   # the fast pass overflows on this row
+    if rows > 2:
+        labels[1] = -100
+        x[2, vocab // 2:] = -float("inf")
+    mask = torch.ones(rows, dtype=torch.uint8)
+    if rows > 4:
+        mask[3] = 0
+    xd, ld, md = x.to(cuda), labels.to(cuda), mask.to(cuda)
+    need = lib.orlhf_logprob_entropy_split_workspace_bytes(_lib.dtype_code(xd), rows, vocab)
+    assert need > 0
+    tickets = torch.zeros(rows, dtype=torch.int32, device=cuda)
+
+    def run(t):
+        ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=cuda)
+        lp = torch.full((rows,), 7.0, device=cuda) if want != "entropy" else None
+        ent = torch.full((rows,), 7.0, device=cuda) if want != "logprob" else None
+        stats = torch.full((rows, 4), 7.0, device=cuda)
+        call("orlhf_logprob_entropy_fwd_split", ptr(xd), _lib.dtype_code(xd), rows, vocab, vocab, ptr(ld), temperature,
+             ptr(lp), ptr(ent), ptr(stats), ptr(md), ptr(ws), need, ptr(t), stream_of(cuda))
+        return [o for o in (lp, ent, stats) if o is not None]
+
+    two_launches = run(None)
+    for _ in range(3):
+        one_launch = run(tickets)
+        assert int(tickets.abs().sum().item()) == 0
+        for a, b in zip(two_launches, one_launch):
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    if rows > 4:
+        assert all(float(o[3].abs().sum().item()) == 0.0 for o in two_launches)
+
+
+def test_mirror_keeps_one_ticket_array_per_stream(cuda):
+    """The Python mirror's ticket array: one per (device, stream), zero between calls, reused."""
+    from openrlhf_amd.models import utils
+
+    x, labels, _, _ = _case(64, 151936, torch.bfloat16, 3.0, seed=11)
+    xd, ld = x.to(cuda), labels.to(cuda)
+    lp0, ent0 = utils.logprobs_and_entropy_from_logits(xd, ld, 1.0)
+    side = torch.cuda.Stream(device=cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    with torch.cuda.stream(side):
+        lp1, ent1 = utils.logprobs_and_entropy_from_logits(xd, ld, 1.0)
+    side.synchronize()
+    torch.cuda.synchronize()
+    assert torch.equal(lp0, lp1) and torch.equal(ent0, ent1)
+    mine = [t for (d, _), t in utils._TICKETS.items() if d == cuda.index]
+    assert len(mine) >= 2 and all(int(t.abs().sum().item()) == 0 for t in mine)
