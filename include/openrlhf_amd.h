@@ -438,6 +438,9 @@ int orlhf_policy_loss_fwd_grad(const float* log_probs, const float* old_log_prob
  * routine. No counterpart in the reference. Problems whose orlhf_token_workspace_bytes(n_rows,
  * n_cols) exceeds the scratch return ORLHF_ERR_UNSUPPORTED. All calls on one GPU share that GPU's
  * scratch: calls that overlap on one GPU (different streams or host threads) race; serialise them.
+ * `stream` has to belong to the current device (ORLHF_ERR_INVALID_ARG otherwise: the scratch is
+ * the current device's). The first call on a device looks the scratch up (hipGetSymbolAddress) and
+ * has to come outside stream capture; every later call on that device may be captured.
  */
 #define ORLHF_NOALLOC_SCRATCH_BYTES (8 << 20)
 int orlhf_policy_loss_fwd_noalloc(const float* log_probs, const float* old_log_probs,
@@ -500,7 +503,11 @@ int orlhf_compute_reward(const float* r, float kl_coef, const float* kl, const v
  * row_order (int64 [n_rows], nullable; also in the two scans below): a permutation of the rows;
  * workgroup slot s walks row row_order[s]. Results do not depend on it; a caller that knows the
  * row lengths of a ragged packed batch passes the rows longest first, so that no long row's
- * sequential walk is left running alone at the end of the launch.
+ * sequential walk is left running alone at the end of the launch. The kernels trust it to be a
+ * permutation: an entry outside [0, n_rows) is skipped, a row named twice is computed twice (to the
+ * same values), and a row that no entry names keeps whatever its outputs held. A caller that
+ * cannot vouch for it (the library's own Python wrappers build it with a sort of the lengths)
+ * passes NULL.
  */
 int orlhf_gae_scan(const float* values, const float* rewards, const void* mask, int mask_dtype,
                    int64_t n_rows, int64_t n_cols, const int64_t* cu_seqlens,

@@ -876,13 +876,24 @@ namespace orlhf {
 constexpr int kMaxDevices = 64;
 static std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
-// Address of `scratch` on the current device (looked up on the first call per device).
-static int scratch_on_current_device(void** out) {
+// Address of `scratch` on the current device (looked up on the first call per device). The kernels
+// run on `stream`'s device: a stream of another device than the current one would be handed the
+// current device's address, so that is refused.
+static int scratch_on_current_device(hipStream_t stream, void** out) {
   int device = -1;
   hipError_t e = hipGetDevice(&device);
   if (e != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "policy_loss_fwd_noalloc: hipGetDevice: %s", hipGetErrorString(e));
   if (device < 0 || device >= kMaxDevices)
     return fail(ORLHF_ERR_UNSUPPORTED, "policy_loss_fwd_noalloc: device index %d outside [0, %d)", device, kMaxDevices);
+  if (stream != nullptr) {
+    int stream_device = -1;
+    e = hipStreamGetDevice(stream, &stream_device);
+    if (e != hipSuccess)
+      return fail(ORLHF_ERR_LAUNCH, "policy_loss_fwd_noalloc: hipStreamGetDevice: %s", hipGetErrorString(e));
+    if (stream_device != device)
+      return fail(ORLHF_ERR_INVALID_ARG, "policy_loss_fwd_noalloc: the stream belongs to device %d, the current device is %d",
+                  stream_device, device);
+  }
   void* p = g_scratch_ptr[device].load(std::memory_order_acquire);
   if (p == nullptr) {
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
@@ -910,7 +921,7 @@ extern "C" int orlhf_policy_loss_fwd_noalloc(const float* log_probs, const float
                 "scratch holds %lld; use orlhf_policy_loss_fwd with a workspace",
                 (long long)n_rows, (long long)n_cols, (long long)need, (long long)ORLHF_NOALLOC_SCRATCH_BYTES);
   void* ws = nullptr;
-  if (int rc = scratch_on_current_device(&ws)) return rc;
+  if (int rc = scratch_on_current_device((hipStream_t)stream, &ws)) return rc;
   // every (row, chunk) partial the later stages read is written by the first stage of this call:
   // nothing in the scratch has to start at zero
   return policy_loss_fwd_impl(log_probs, old_log_probs, advantages, mask, mask_dtype, rollout_log_probs, n_rows,

@@ -80,3 +80,40 @@ def test_no_alloc_entry_rejects_what_the_scratch_cannot_hold(lib, cuda):
         _lib.call("orlhf_policy_loss_fwd_noalloc", dummy.data_ptr(), dummy.data_ptr(), dummy.data_ptr(), None,
                   _lib.MASK_NONE, None, rows, cols, None, ctypes.byref(params), dummy.data_ptr(), dummy.data_ptr(),
                   dummy.data_ptr(), _lib.stream_of(cuda))
+
+
+def test_no_alloc_entry_replays_from_a_captured_graph(lib, cuda):
+    """After one eager call on the device (which looks the scratch up) the entry may be captured: every
+    replay, with eager calls on other shapes in between that leave their partial sums in the same
+    scratch, gives the bits of the workspace entry on the inputs then in the captured buffers."""
+    from openrlhf_amd import _lib
+
+    rows, cols = 96, 4100
+    _both(lib, _lib, cuda, 16, 900, 3, True, None)                   # the device's first call, eager
+    (lp, old, adv, roll), mask = _inputs(cuda, rows, cols, 4)
+    params = _params(_lib, True, 3.0)
+    out, coef, aux = torch.zeros(4, device=cuda), torch.zeros(rows, device=cuda), torch.zeros(rows, 2, device=cuda)
+    side = torch.cuda.Stream(device=cuda)
+    side.wait_stream(torch.cuda.current_stream(cuda))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            _lib.call("orlhf_policy_loss_fwd_noalloc", lp.data_ptr(), old.data_ptr(), adv.data_ptr(), mask.data_ptr(),
+                      _lib.MASK_U8, roll.data_ptr(), rows, cols, None, ctypes.byref(params), out.data_ptr(),
+                      coef.data_ptr(), aux.data_ptr(), _lib.stream_of(cuda))
+    torch.cuda.current_stream(cuda).wait_stream(side)
+    ws = torch.empty(lib.orlhf_token_workspace_bytes(rows, cols), dtype=torch.uint8, device=cuda)
+    for replay in range(3):
+        (lp2, old2, adv2, roll2), _ = _inputs(cuda, rows, cols, 10 + replay)
+        for dst, src in ((lp, lp2), (old, old2), (adv, adv2), (roll, roll2)):
+            dst.copy_(src)
+        out.fill_(-7.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        ref, rcoef, raux = torch.zeros(4, device=cuda), torch.zeros(rows, device=cuda), torch.zeros(rows, 2, device=cuda)
+        _lib.call("orlhf_policy_loss_fwd", lp.data_ptr(), old.data_ptr(), adv.data_ptr(), mask.data_ptr(), _lib.MASK_U8,
+                  roll.data_ptr(), rows, cols, None, ctypes.byref(params), ws.data_ptr(), ref.data_ptr(),
+                  rcoef.data_ptr(), raux.data_ptr(), _lib.stream_of(cuda))
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref) and torch.equal(coef, rcoef) and torch.equal(aux, raux), replay
+        _both(lib, _lib, cuda, 300, 5000, replay, True, None)         # eager work through the same scratch
