@@ -193,7 +193,7 @@ int orlhf_logprob_entropy_fwd_bwd(const void* logits, void* grad_logits, int dty
  *           first kept_cols vocabulary columns are stored there (the tiles produce them anyway), so
  *           that the backward need not recompute them. kept_cols is a multiple of 256, at most the
  *           vocabulary rounded up to 256 (then all logits are kept; columns past the vocabulary hold
- *           zeros); kept_stride >= kept_cols, a multiple of 8; 16-byte aligned. Results do not
+ *           a large negative filler, which the backward overwrites with zeros); kept_stride >= kept_cols, a multiple of 8; 16-byte aligned. Results do not
  *           depend on kept_cols.
  *   workspace: orlhf_lmhead_workspace_bytes(n_rows, hidden_dim, vocab, kept_cols, 0) bytes, 256-byte aligned
  */

@@ -64,21 +64,24 @@ struct Running {
   float m, s1, t1, sT, xl;
 };
 
-// Folds one rounded column into the running statistics of its token. bias[mt][r] is 0 for a
-// vocabulary entry and kLow for a register past the vocabulary (last vocabulary tile only), whose
-// logit is exactly 0 (its weight rows read as zeros): x + bias is then so low that the entry
-// contributes exact zeros, also when the lane has seen no real entry yet and m_new is still kLow.
-// One code path for every tile: the sum costs what unpacking the column a second time would.
+// Filler of accumulators past the vocabulary in the last vocabulary tile (their weight rows read
+// as zeros, so the product leaves what they start with): kLow for bf16, the most negative finite
+// number for fp16. e^(filler - m) is exactly 0 for any real m and filler * 0 is 0: such an entry
+// contributes nothing, also when the lane has seen no real entry and its maximum is the filler.
+template <int DT>
+__device__ __forceinline__ constexpr float filler() { return DT == ORLHF_BF16 ? kLow : -65504.0f; }
+
+// Folds one rounded column into the running statistics of its token. One code path for every tile:
+// registers past the vocabulary hold the filler.
 template <int DT, bool BOTH_T>
-__device__ __forceinline__ void fold_column(const uint32_t (&pk)[4][8], const float (&bias)[4][16], Running& run, int lab_rel,
-                                            float c1, float cT) {
+__device__ __forceinline__ void fold_column(const uint32_t (&pk)[4][8], Running& run, int lab_rel, float c1, float cT) {
   float x[4][16];
   float mx = kLow;
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      x[mt][r] = unpack_half<DT>(pk[mt][r >> 1], r & 1) + bias[mt][r];
+      x[mt][r] = unpack_half<DT>(pk[mt][r >> 1], r & 1);
       mx = fmaxf(mx, x[mt][r]);
     }
   }
@@ -153,23 +156,28 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, 
   const int64_t n_tokens = h.rows, vocab = w.rows;
 
   f32x16 acc[4][4];
-  mm::tile_product<DT, false, false>(acc, w, h, (int64_t)vt * 256, (int64_t)tb * 256, lds);
+  {
+    uint32_t t0 = threadIdx.x;
+    asm volatile("" : "+v"(t0));  // opaque: nothing computed for the start values is kept for the epilogue
+    const int64_t left = vocab - ((int64_t)vt * 256 + ((t0 >> 6) & 1u) * 128 + 4 * ((t0 & 63u) >> 5));
+    // registers past the vocabulary (last vocabulary tile only) start, and stay, at the filler
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float start = reg_off(mt, r) < left ? 0.0f : filler<DT>();
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt) acc[mt][nt][r] = start;
+      }
+    }
+  }
+  mm::tile_product<DT, false, false, false>(acc, w, h, (int64_t)vt * 256, (int64_t)tb * 256, lds);
 
   const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, wm = wave & 1u, wn = wave >> 1;
   const int64_t vbase = (int64_t)vt * 256 + wm * 128 + 4 * (lane >> 5);  // vocabulary index of this lane's register offset 0
   const bool keep = vt < kept_tiles;
   __syncthreads();  // every wave is done with the slab buffers: they serve as the exchange area now
   float* ex = (float*)lds;  // [2 wm][2 wn][4 tokens][32 lanes][4 fields]
-  // 0 for the lane's vocabulary entries, kLow for registers past the vocabulary (last tile only)
-  float bias[4][16];
-  {
-    const int64_t left = vocab - vbase;
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) bias[mt][r] = reg_off(mt, r) < left ? 0.0f : kLow;
-    }
-  }
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
     const int64_t tok = (int64_t)tb * 256 + mm::acc_col(wn, nt, lane);
@@ -179,7 +187,7 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, 
     round_column<DT>(acc, nt, pk);
     if (keep && tok < n_tokens) store_column(kept + tok * kept_ld + vbase, pk);
     Running run{kLow, 0.0f, 0.0f, 0.0f, kLow};
-    fold_column<DT, BOTH_T>(pk, bias, run, lab_rel, c1, cT);
+    fold_column<DT, BOTH_T>(pk, run, lab_rel, c1, cT);
     if (run.xl != kLow && tok < n_tokens) x_label[tok] = run.xl;  // exactly one lane of the grid holds a token's label
     // the two lane halves and the two waves along the vocabulary hold parts of the same tokens
     Running o;
