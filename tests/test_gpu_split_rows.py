@@ -269,3 +269,39 @@ def test_mirror_keeps_one_ticket_array_per_stream(cuda):
     assert torch.equal(lp0, lp1) and torch.equal(ent0, ent1)
     mine = [t for (d, _), t in utils._TICKETS.items() if d == cuda.index]
     assert len(mine) >= 2 and all(int(t.abs().sum().item()) == 0 for t in mine)
+
+
+def test_merge_by_last_segment_over_many_launches(cuda):
+    """The same ticket array through 600 launches back to back (three shapes in rotation, no
+    synchronisation between launches): every launch's outputs are the two-launch form's bits and the
+    tickets are back at zero at the end. Which workgroup draws a row's last ticket changes from launch
+    to launch; the records it reads must be complete whoever it is."""
+    from openrlhf_amd import _lib
+    from openrlhf_amd._lib import call, ptr, stream_of
+
+    lib = _lib.load()
+    shapes = [(64, 151936, torch.bfloat16), (255, 65536, torch.float16), (7, 50257, torch.float32)]
+    tickets = torch.zeros(256, dtype=torch.int32, device=cuda)
+    cases = []
+    for k, (rows, vocab, dtype) in enumerate(shapes):
+        x, labels, _, _ = _case(rows, vocab, dtype, 3.0, seed=100 + k)
+        xd, ld = x.to(cuda), labels.to(cuda)
+        need = lib.orlhf_logprob_entropy_split_workspace_bytes(_lib.dtype_code(xd), rows, vocab)
+        ws = torch.empty(need, dtype=torch.uint8, device=cuda)
+        want = [torch.empty(rows, device=cuda), torch.empty(rows, device=cuda), torch.empty(rows, 4, device=cuda)]
+        args = (ptr(xd), _lib.dtype_code(xd), rows, vocab, vocab, ptr(ld), 0.8)
+        call("orlhf_logprob_entropy_fwd_split", *args, *(ptr(o) for o in want), None, ptr(ws), need, None, stream_of(cuda))
+        cases.append((args, ws, need, want, xd, ld))
+    torch.cuda.synchronize()
+    rounds = 200
+    outs = [[torch.full_like(w, 7.0) for w in want] for (_, _, _, want, _, _) in cases]
+    bad = torch.zeros((), dtype=torch.int64, device=cuda)
+    for r in range(rounds):
+        for (args, ws, need, want, _, _), got in zip(cases, outs):
+            call("orlhf_logprob_entropy_fwd_split", *args, *(ptr(o) for o in got), None, ptr(ws), need, ptr(tickets),
+                 stream_of(cuda))
+            for a, b in zip(want, got):
+                bad += (a.view(torch.int32) != b.view(torch.int32)).sum()
+                b.fill_(7.0)
+    assert int(bad.item()) == 0
+    assert int(tickets.abs().sum().item()) == 0
