@@ -49,8 +49,10 @@ def check_rounded_logits(kept, hidden, weight, rows=None):
     x = hidden[sel].double() @ weight.double().T
     got = kept[sel][:, :vocab].double()
     u = unit_roundoff(kept.dtype)
-    # half an ulp is at most u/2 * 2|x| relative to the binade's lower end; the fp32 accumulation adds ~1e-6 * |h||w|
-    slack = 2e-6 * (hidden[sel].double().abs() @ weight.double().abs().T)
+    # half an ulp is at most u/2 * 2|x| relative to the binade's lower end (for fp16 never less than half
+    # the spacing of its subnormals, 2^-25); the fp32 accumulation adds ~1e-6 * |h||w|
+    floor = 2.0 ** -25 if kept.dtype == torch.float16 else 0.0
+    slack = 2e-6 * (hidden[sel].double().abs() @ weight.double().abs().T) + floor
     excess = ((got - x).abs() - (u * x.abs() + slack)).max().item()
     assert excess <= 0, excess
     return x

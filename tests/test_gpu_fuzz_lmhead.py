@@ -1,8 +1,9 @@
 """Seeded random sweep over the lm-head + log-prob / entropy path: token counts, hidden sizes (any
 even number), vocabularies, dtypes, temperatures, padded row strides and row masks drawn at random,
-every case against the fp64 oracle applied to ``hidden @ W.T`` rounded to the 16-bit dtype as the
-lm_head output is (tests/lmhead_util.py; values 2e-3 abs; gradients within the rounding of a
-16-bit logits gradient and a 16-bit result)."""
+and the memory budget for kept logits (none, a sliver, everything), every case against the fp64
+oracle applied to ``hidden @ W.T`` rounded to the 16-bit dtype as the lm_head output is
+(tests/lmhead_util.py; values 2e-3 abs; gradients within the rounding of a 16-bit logits gradient
+and a 16-bit result)."""
 import random
 
 import pytest
@@ -14,7 +15,7 @@ from tests.lmhead_util import straight_through_logits
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("seed", list(range(16)) + [5024, 5025, 5028, 5044, 5051, 5054])  # the last six: a vocabulary of one entry
+@pytest.mark.parametrize("seed", list(range(40)) + [42, 229, 255, 5024, 5025, 5028, 5044, 5051, 5054])  # the last six: a vocabulary of one entry
 def test_random_case(cuda, seed):
     from openrlhf_amd.models.utils import lm_head_logprobs_and_entropy
 
@@ -26,7 +27,8 @@ def test_random_case(cuda, seed):
     temperature = rng.choice([1.0, 1.0, 0.6, 1.5])
     pad_h, pad_w = 2 * rng.choice([0, 0, 1, 4]), 2 * rng.choice([0, 0, 3])
     use_mask = rng.random() < 0.5
-    info = (seed, dtype, n, hdim, vocab, temperature, pad_h, pad_w, use_mask)
+    keep_mib = rng.choice([None, None, 0.3, 1e6])       # drawn last: the earlier draws of a seed stay what they were
+    info = (seed, dtype, n, hdim, vocab, temperature, pad_h, pad_w, use_mask, keep_mib)
 
     g = torch.Generator().manual_seed(seed)
     hidden = torch.randn(n, hdim, generator=g).to(dtype)
@@ -51,7 +53,7 @@ def test_random_case(cuda, seed):
     hd = hbuf[:, :hdim].requires_grad_(True)
     wd = wbuf[:, :hdim].requires_grad_(True)
     lp, ent = lm_head_logprobs_and_entropy(hd, wd, labels.to(cuda), temperature,
-                                           row_mask=None if mask is None else mask.to(cuda))
+                                           row_mask=None if mask is None else mask.to(cuda), keep_logits_mib=keep_mib)
     assert (lp.detach().cpu().double() - ref_lp.detach()).abs().max().item() <= 2e-3, info
     assert (ent.detach().cpu().double() - ref_ent.detach()).abs().max().item() <= 2e-3, info
     if mask is not None and not bool(mask.any()):
