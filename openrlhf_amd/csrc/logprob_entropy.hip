@@ -14,7 +14,8 @@
 //   * a launch with fewer rows than the chip has compute units cuts every row into segments, one
 //     workgroup per (row, segment): the backward needs nothing else (an element's gradient depends
 //     on the row only through its saved statistics), the forward writes one partial record per
-//     segment and a small second kernel merges a row's records in a fixed order.
+//     segment, and a row's records are merged in a fixed order by the workgroup that finishes the
+//     row's last segment (given a ticket per row) or by a small second kernel.
 #include <stdlib.h>
 
 #include "vocab_rows.h"
@@ -585,10 +586,7 @@ __global__ __launch_bounds__(kBlock) void logprob_entropy_bwd_kernel(
 // ---------------------------------------------------------------- host side
 static int grid_for_rows(int64_t n_rows) {
   // one workgroup per row; cap the grid and stride over rows beyond it
-  int64_t cap = 1 << 20;
-#ifdef ORLHF_TUNING
-  if (const char* e = getenv("ORLHF_GRID_CAP")) cap = atoll(e);
-#endif
+  const int64_t cap = 1 << 20;
   return (int)(n_rows < cap ? n_rows : cap);
 }
 

@@ -205,18 +205,12 @@ __global__ __launch_bounds__(kBlock) void pack_rows_multi_kernel(PackFields f, i
                                                                  const int64_t* __restrict__ first,
                                                                  const int64_t* __restrict__ cu) {
   const int64_t chunks = (n_cols + kMultiCols - 1) / kMultiCols;
-#ifdef ORLHF_PACK_ROW_MAJOR
-  for (int64_t w = blockIdx.x; w < n_rows * chunks; w += gridDim.x) {
-    const int64_t b = w / chunks;
-    int64_t chunk = (w - b * chunks) + b % chunks;
-    chunk = chunk >= chunks ? chunk - chunks : chunk;
-#else
+  // rows fastest, as in the one-field kernel (row-major numbering of the items measured 6 % slower here)
   const int64_t slots = row_slots(n_rows);
   const int slot_b = slot_bits(n_rows);
   for (int64_t w = blockIdx.x; w < slots * chunks; w += gridDim.x) {
     const int64_t chunk = w / slots, b = row_of_slot(w - chunk * slots, w, slot_b);
     if (b >= n_rows) continue;
-#endif
     const int64_t j0 = chunk * kMultiCols;
     const int64_t start = cu[b], len = cu[b + 1] - start;
     if (j0 >= len) continue;
@@ -398,12 +392,8 @@ __global__ __launch_bounds__(kBlock) void unpad_rows_kernel(const int64_t* __res
 // waiting for the tiles before it, a tile without non-zero columns costs one load of its count, and
 // a tile whose columns are all non-zero (the inside of an attended span: all but one or two tiles
 // of a row) does not read the mask at all.
-// Consecutive tiles of a row per workgroup. Measured on 4096 x 16385 cells, half attended, all four
-// outputs: 1 tile 0.272 ms, 2 0.277, 3 0.291, 4 0.299 (the two computed outputs alone are fastest at 3-4).
-#ifndef ORLHF_UNPAD_TILES_PER_ITEM
-#define ORLHF_UNPAD_TILES_PER_ITEM 1
-#endif
-constexpr int kUnpadTilesPerItem = ORLHF_UNPAD_TILES_PER_ITEM;
+// One tile per workgroup: with 2, 3 or 4 consecutive tiles of a row per workgroup the same launch
+// (4096 x 16385 cells, half attended, all four outputs) took 0.277, 0.291 and 0.299 ms against 0.272.
 
 template <int MASK_DT>
 __global__ __launch_bounds__(kBlock) void unpad_tiles_kernel(const int64_t* __restrict__ sequences,
@@ -416,24 +406,21 @@ __global__ __launch_bounds__(kBlock) void unpad_tiles_kernel(const int64_t* __re
   __shared__ int wave_tot[kWavesPerBlock];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int64_t n_chunks = (n_cols + kTileCols - 1) / kTileCols;
-  const int64_t groups = (n_chunks + kUnpadTilesPerItem - 1) / kUnpadTilesPerItem;
-  for (int64_t w = blockIdx.x; w < n_rows * groups; w += gridDim.x) {
+  for (int64_t w = blockIdx.x; w < n_rows * n_chunks; w += gridDim.x) {
     // row-major: the workgroups that run at the same time write neighbouring stretches of every
-    // output (DRAM pages stay open); the tile groups of a row are taken in an order rotated by the
-    // row number, so that the groups past the ends of short rows do not all fall on the same XCDs
-    const int64_t b = w / groups;
-    int64_t grp = (w - b * groups) + b % groups;
-    grp = grp >= groups ? grp - groups : grp;
+    // output (DRAM pages stay open); the tiles of a row are taken in an order rotated by the row
+    // number, so that the tiles past the ends of short rows do not all fall on the same XCDs
+    const int64_t b = w / n_chunks;
+    int64_t ch = (w - b * n_chunks) + b % n_chunks;
+    ch = ch >= n_chunks ? ch - n_chunks : ch;
     const int32_t* cc = chunk_counts + b * n_chunks;
-    const int64_t ch0 = grp * kUnpadTilesPerItem;
-    int64_t run = 0;  // non-zero columns of the row before this group (every wave sums them for itself)
-    for (int64_t j = lane; j < ch0; j += kWave) run += cc[j];
+    const int c_tile = cc[ch];
+    if (c_tile == 0) continue;
+    int64_t run = 0;  // non-zero columns of the row before this tile (every wave sums them for itself)
+    for (int64_t j = lane; j < ch; j += kWave) run += cc[j];
 #pragma unroll
     for (int o = kWave / 2; o > 0; o >>= 1) run += __shfl_xor(run, o, kWave);
     const int64_t out0 = cu[b];
-   for (int64_t ch = ch0; ch < ch0 + kUnpadTilesPerItem && ch < n_chunks; ++ch) {
-    const int c_tile = cc[ch];
-    if (c_tile == 0) continue;
     const int64_t t0 = ch * kTileCols;
     // the wave's 512 columns as 512 consecutive slots: lanes take them two at a time, interleaved,
     // so that every load and store of the wave covers 1 KiB of consecutive memory
@@ -465,7 +452,6 @@ __global__ __launch_bounds__(kBlock) void unpad_tiles_kernel(const int64_t* __re
     };
     if (c_tile == kTileCols && out0 + run + kTileCols <= capacity) {  // all columns attended: the mask is not read
       dense_wave((int64_t)wave * kWaveCols);
-      run += c_tile;
       continue;
     }
     const int64_t t = t0 + kUnpadCols * (int64_t)threadIdx.x;
@@ -532,8 +518,6 @@ __global__ __launch_bounds__(kBlock) void unpad_tiles_kernel(const int64_t* __re
         }
       }
     }
-    run += c_tile;
-   }
   }
 }
 
@@ -720,7 +704,7 @@ static void launch_unpad_tiles(const int64_t* sequences, const void* mask, int m
                                const int64_t* cu, const int32_t* chunk_counts, int64_t capacity, int64_t* indices,
                                int64_t* packed, int64_t* rolled, int64_t* position, hipStream_t s) {
   const int64_t n_chunks = (n_cols + ORLHF_UNPAD_TILE - 1) / ORLHF_UNPAD_TILE;
-  const dim3 grid(slot_grid(n_rows * ((n_chunks + kUnpadTilesPerItem - 1) / kUnpadTilesPerItem), 1 << 20)), block(kBlock);
+  const dim3 grid(slot_grid(n_rows * n_chunks, 1 << 20)), block(kBlock);
   switch (mask_dtype) {
     case ORLHF_MASK_U8:
       hipLaunchKernelGGL(unpad_tiles_kernel<ORLHF_MASK_U8>, grid, block, 0, s, sequences, mask, n_rows, n_cols, cu, chunk_counts, capacity, indices, packed, rolled, position);
