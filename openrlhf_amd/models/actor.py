@@ -61,22 +61,20 @@ def actor_forward_tail(
             logits, labels, temperature, inplace_backward=inplace_backward, row_mask=row_mask
         ) if return_entropy else (_lp_only(logits, labels, temperature, inplace_backward, row_mask), None)
     else:
+        from .utils import _index_rows
+
         flat_logits = logits.reshape(-1, logits.shape[-1])
-        labels = rolled.reshape(-1)[packed_indices]
-        row_mask = None if need is None else need.reshape(-1)[packed_indices]
+        idx = packed_indices.to(torch.int64).contiguous()
+        labels = _index_rows(rolled.reshape(-1).to(torch.int64), idx)
+        row_mask = None if need is None else _index_rows(need.reshape(-1).to(torch.uint8), idx)
         if return_entropy:
             lp_p, ent_p = logprobs_and_entropy_from_logits(
                 flat_logits, labels, temperature, inplace_backward=inplace_backward, row_mask=row_mask
             )
         else:
             lp_p, ent_p = _lp_only(flat_logits, labels, temperature, inplace_backward, row_mask), None
-
-        def repad(flat):
-            full = flat.new_zeros(batch * seqlen)
-            return full.index_copy(0, packed_indices, flat).view(batch, seqlen)
-
-        lp = repad(lp_p)
-        ent = None if ent_p is None else repad(ent_p)
+        lp = gather_and_pad_tensor(lp_p.unsqueeze(0), None, 0, idx, batch, seqlen)
+        ent = None if ent_p is None else gather_and_pad_tensor(ent_p.unsqueeze(0), None, 0, idx, batch, seqlen)
 
     lp = lp[:, :-1]
     if action_mask is not None:
