@@ -104,11 +104,17 @@ def experience_kl(
 
 
 def _order_arg(row_order, n_rows, dev):
-    """A row permutation as the kernels take it (int64 on the device), or None."""
+    """A row permutation as the kernels take it (int64 on the device), or None. The kernels trust it:
+    a row that it does not name keeps whatever its outputs held. An order that arrives on the host
+    is checked here (sorting it must give 0 .. n_rows - 1); one that is already on the device
+    (``PackedSteps.longest_first`` builds it there with a sort) is not read back."""
     if row_order is None:
         return None
     if row_order.numel() != n_rows:
         raise ValueError(f"row_order has {row_order.numel()} entries for {n_rows} rows")
+    if row_order.device.type == "cpu":
+        if not torch.equal(torch.sort(row_order.reshape(-1).to(torch.int64)).values, torch.arange(n_rows, dtype=torch.int64)):
+            raise ValueError("row_order is not a permutation of the rows")
     return row_order.to(device=dev, dtype=torch.int64).contiguous()
 
 

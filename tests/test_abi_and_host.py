@@ -306,3 +306,20 @@ def test_every_intra_package_import_resolves():
                 except ImportError:
                     missing.append((rel, mod, alias.name))
     assert not missing, missing
+
+
+def test_row_order_from_the_host_must_be_a_permutation():
+    """A row order handed over as a CPU tensor is checked before it reaches the kernels (which trust
+    it: a row that no entry names would keep whatever its outputs held)."""
+    import torch
+
+    from openrlhf_amd.trainer.ppo_utils.experience_maker import _order_arg
+
+    cpu = torch.device("cpu")
+    assert _order_arg(None, 4, cpu) is None
+    assert _order_arg(torch.tensor([2, 0, 3, 1]), 4, cpu).tolist() == [2, 0, 3, 1]
+    for bad in ([0, 0, 1, 2], [0, 1, 2, 4], [-1, 0, 1, 2]):
+        with pytest.raises(ValueError, match="permutation"):
+            _order_arg(torch.tensor(bad), 4, cpu)
+    with pytest.raises(ValueError, match="entries"):
+        _order_arg(torch.tensor([0, 1, 2]), 4, cpu)

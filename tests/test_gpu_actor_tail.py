@@ -162,3 +162,30 @@ def test_tail_from_hidden_states(cuda, packed):
     need[:, t - 1 - a : t - 1] = amask
     dead = ~need.reshape(-1)[flat_keep] if packed else ~need.reshape(-1)
     assert hd.grad.reshape(-1, hdim)[dead.to(cuda)].abs().max().item() == 0.0
+
+
+def test_tail_from_hidden_states_every_position(cuda):
+    """``action_mask=None`` on a padded batch: the reference returns real log-probs and entropies at
+    padded positions too (actor.py:283-290 multiply by no mask); ``skip_masked=False`` projects
+    every row and reproduces them, the default leaves the positions outside the attention mask at 0."""
+    from openrlhf_amd.models.actor import actor_forward_tail_from_hidden
+    from tests.lmhead_util import straight_through_logits
+
+    b, t, hdim, vocab, temperature = 3, 20, 64, 777, 0.9
+    _, seqs, attn, _ = _batch(21, b=b, t=t, vocab=vocab, a=7)
+    g = torch.Generator().manual_seed(22)
+    hidden = torch.randn(b, t, hdim, generator=g).to(torch.bfloat16)
+    weight = (torch.randn(vocab, hdim, generator=g) * 0.3).to(torch.bfloat16)
+    logits64 = straight_through_logits(hidden, weight, hidden.double(), weight.double(), cuda)
+    ref_lp = otn.log_probs_from_logits(logits64, torch.roll(seqs, -1, 1), temperature)[:, :-1]
+    ref_ent = otn.compute_entropy(logits64)[:, :-1]
+    args = (hidden.to(cuda), weight.to(cuda), seqs.to(cuda), None, attn.to(cuda))
+    lp, ent = actor_forward_tail_from_hidden(*args, temperature=temperature, return_entropy=True, skip_masked=False)
+    assert lp.shape == ref_lp.shape and ent.shape == ref_ent.shape
+    assert (lp.cpu().double() - ref_lp).abs().max().item() <= 2e-3
+    assert (ent.cpu().double() - ref_ent).abs().max().item() <= 2e-3
+    keep = attn[:, :-1].bool()
+    assert bool((~keep).any())
+    lp_s, ent_s = actor_forward_tail_from_hidden(*args, temperature=temperature, return_entropy=True)
+    assert (lp_s.cpu().double() - ref_lp)[keep].abs().max().item() <= 2e-3
+    assert lp_s.cpu()[~keep].abs().max().item() == 0.0 and ent_s.cpu()[~keep].abs().max().item() == 0.0
