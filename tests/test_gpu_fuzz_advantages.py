@@ -13,12 +13,14 @@ from oracle import token_numerics as otn
 pytestmark = pytest.mark.gpu
 
 
-def _rel(got, ref, rtol, tag):
+def _rel(got, ref, rtol, tag, at_least=1e-30):
+    """Within rtol of the largest reference entry, or of `at_least` (the size of the inputs, where
+    the outputs are differences of them and may all be small)."""
     got, ref = got.detach().cpu().double(), ref.detach().double()
     assert got.shape == ref.shape, tag
     if ref.numel() == 0:
         return
-    scale = max(ref.abs().max().item(), 1e-30)
+    scale = max(ref.abs().max().item(), at_least)
     assert (got - ref).abs().max().item() <= rtol * scale, (tag, (got - ref).abs().max().item(), scale)
 
 
@@ -43,7 +45,7 @@ def _offset(t, off, dev):
     return view
 
 
-@pytest.mark.parametrize("seed", range(36))
+@pytest.mark.parametrize("seed", list(range(36)) + [2325, 2648, 3639])
 def test_random_rows(cuda, seed):
     from openrlhf_amd.models.utils import compute_reward, masked_normalize
     from openrlhf_amd.trainer.ppo_utils.experience_maker import (
@@ -100,8 +102,16 @@ def test_random_rows(cuda, seed):
     _rel(n_ret, o_g, 1e-5, tag)
 
     # masked_normalize
+    # masked_normalize: the reference forms x - mean in fp32, and a row whose kept values nearly
+    # coincide divides that rounding (2^-24 |x|) by its tiny standard deviation
     if mask_dtype is not None:
-        _rel(masked_normalize(put(values), dm), otn.masked_normalize(values.double(), m64), 2e-5, tag)
+        want = otn.masked_normalize(values.double(), m64)
+        cnt = m64.sum(1, keepdim=True).clamp(min=1)
+        mean = (values.double() * m64).sum(1, keepdim=True) / cnt
+        var = ((((values.double() - mean) * m64) ** 2).sum(1, keepdim=True) / cnt).clamp(min=1e-8)
+        slack = 2.0 ** -22 * values.abs().amax(1, keepdim=True).double() * var.rsqrt()
+        err = (masked_normalize(put(values), dm).cpu().double() - want).abs()
+        assert bool((err <= 2e-5 * max(want.abs().max().item(), 1e-30) + slack).all()), (tag, err.max().item())
 
     # packed layout: each row from its first to its last kept column, holes included
     if mask.any(1).all():
@@ -120,6 +130,7 @@ def test_random_rows(cuda, seed):
             row_rew = otn.compute_reward(r[i:i + 1].double(), kl_coef, o_kl[i:i + 1, f:e], row_m, clip)
             ra, rr = oa.get_advantages_and_returns(values[i:i + 1, f:e].double(), row_rew, row_m, gamma, lambd)
             lo, hi = int(cu[i]), int(cu[i + 1])
-            _rel(p_adv[lo:hi], ra[0], 1e-5, tag)
-            _rel(p_ret[lo:hi], rr[0], 1e-5, tag)
+            size = max(values[i, f:e].abs().max().item(), row_rew.abs().max().item())
+            _rel(p_adv[lo:hi], ra[0], 1e-5, tag, at_least=size)
+            _rel(p_ret[lo:hi], rr[0], 1e-5, tag, at_least=size)
             assert abs(p_sum[i].item() - row_rew.sum().item()) <= 1e-5 * max(1.0, row_rew.abs().sum().item()), tag

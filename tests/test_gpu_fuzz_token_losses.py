@@ -24,7 +24,38 @@ def _mask(rng, g, b, a):
     return m
 
 
-@pytest.mark.parametrize("seed", range(40))
+def _on_an_edge(lp, old, roll, mask, cfg, kind, margin=2e-6):
+    """Entries that sit on a step: the clipped surrogate, the dual clip and the importance filters
+    are step functions of a ratio, so an entry whose ratio lies within `margin` (relative) of a
+    threshold may take one branch in fp32 and the other in the fp64 oracle (among 300 000 entries
+    one does now and then), which moves its gradient and the loss by that entry's whole term.
+    Token-level ratios mark their entry, sequence-level ones (GSPO, seq-mask-tis) their whole row."""
+    m = mask.double()
+    cnt = m.sum(-1, keepdim=True).clamp(min=1)
+
+    def near(x, *edges):
+        hit = torch.zeros_like(x, dtype=torch.bool)
+        for e in edges:
+            if e is not None:
+                hit |= (x - e).abs() <= margin * abs(e)
+        return hit
+
+    if kind.startswith("gspo"):
+        log_ratio = (lp.double() - roll.double()) if kind == "gspo-is" else (lp.double() - old.double())
+        ratio = ((log_ratio * m).sum(-1, keepdim=True) / cnt).exp().expand_as(m)
+    else:
+        ratio = (lp.double() - old.double()).clamp(-20.0, 20.0).exp()
+    edge = near(ratio, 1 - cfg["clip_eps_low"], 1 + cfg["clip_eps_high"], cfg["dual_clip"])
+    if kind in ("tis", "icepop", "seq-mask-tis"):
+        lo, hi = cfg["vllm_is_truncated_threshold"]
+        log_is = old.double() - roll.double()
+        edge |= near(log_is.exp(), lo, hi)
+        if kind == "seq-mask-tis":
+            edge |= near(((log_is * m).sum(-1, keepdim=True) / cnt).exp().expand_as(m), lo, hi)
+    return edge
+
+
+@pytest.mark.parametrize("seed", list(range(40)) + [1760, 1934, 2972])
 def test_random_policy_and_value_loss(cuda, seed):
     from openrlhf_amd.models.loss import PolicyLoss, ValueLoss
 
@@ -46,6 +77,12 @@ def test_random_policy_and_value_loss(cuda, seed):
         cfg.update(policy_loss_type="gspo")
         if kind == "gspo-is":
             cfg.update(enable_vllm_is_correction=True, vllm_is_truncated_threshold=[0.5, 2.0])
+    for _ in range(4):  # entries drawn onto a step are moved off it: the comparison is about arithmetic, not about ties
+        edge = _on_an_edge(lp, old, roll, mask, {"dual_clip": None, **cfg}, kind)
+        if not edge.any():
+            break
+        lp, roll = torch.where(edge, lp + 1e-3, lp), torch.where(edge, roll - 2e-3, roll)
+    assert not _on_an_edge(lp, old, roll, mask, {"dual_clip": None, **cfg}, kind).any()
     info = rng.choice([{}, dict(dp_size=2, batch_num_tokens=float(mask.sum()) * 1.7, global_batch_size=float(b) * 1.3)])
     mask_dtype = rng.choice([torch.bool, torch.float32, torch.int64])
     use_roll = cfg.get("enable_vllm_is_correction", False)
