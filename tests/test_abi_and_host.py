@@ -119,18 +119,15 @@ def test_matrix_core_entries_refuse_strides_their_offsets_cannot_address(lib):
     assert lib.orlhf_matrix_tile_probe(256, 256, _lib.BF16, 8, 8, 64, 64, big, 0, 256, None) == -3 and "2^23" in err()
 
 
-def test_matrix_core_kernels_do_not_spill():
-    """The compiler's own resource report for the matrix-core kernels: with 256 accumulator registers
-    per lane a few live values too many end up in scratch memory (and a spill inside the product
-    loop would cost far more than it looks). Compiles csrc/lmhead.hip for gfx950 with the library's
-    flags and reads the remarks: no kernel may spill a vector register or use scratch."""
+def _resource_report(source):
+    """The compiler's own per-kernel resource remarks for one source file of the library, compiled
+    for gfx950 with the library's flags: {mangled kernel name: {"VGPRs": n, "VGPRs Spill": n, ...}}."""
     import subprocess
 
     from openrlhf_amd.csrc import build as b
 
-    src = os.path.join(b.CSRC, "lmhead.hip")
-    cmd = [b.find_hipcc(), *b.HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "--cuda-device-only", "-c", src, "-o", os.devnull,
-           "-Rpass-analysis=kernel-resource-usage"]
+    cmd = [b.find_hipcc(), *b.HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "--cuda-device-only", "-c",
+           os.path.join(b.CSRC, source), "-o", os.devnull, "-Rpass-analysis=kernel-resource-usage"]
     out = subprocess.run(cmd, capture_output=True, text=True)
     assert out.returncode == 0, out.stderr[-2000:]
     kernels, name = {}, None
@@ -143,9 +140,28 @@ def test_matrix_core_kernels_do_not_spill():
         m = re.search(r"remark:\s+(VGPRs Spill|ScratchSize \[bytes/lane\]|AGPRs|VGPRs): (\d+)", line)
         if m and name:
             kernels[name][m.group(1)] = int(m.group(2))
+    return kernels
+
+
+def test_matrix_core_kernels_do_not_spill():
+    """With 256 accumulator registers per lane a few live values too many end up in scratch memory
+    (and a spill inside the product loop would cost far more than it looks): no kernel of
+    csrc/lmhead.hip may spill a vector register or use scratch."""
+    kernels = _resource_report("lmhead.hip")
     tiles = {k: v for k, v in kernels.items() if v.get("AGPRs", 0) == 256}  # the kernels built on the 256 x 256 tile
     assert len(tiles) >= 20, sorted(kernels)
     for k, v in kernels.items():
+        assert v["VGPRs Spill"] == 0 and v["ScratchSize [bytes/lane]"] == 0, (k, v)
+
+
+def test_one_pass_kernel_of_the_benchmark_does_not_spill():
+    """The one-pass forward + backward kernel holds a whole vocabulary row in registers (254-256 of
+    them): its bf16, temperature-1 bodies with 38 chunks per lane, which the benchmark and the PPO
+    step run, must stay free of spills (template arguments: dtype 1 = bf16, modes 0-2, 38 chunks)."""
+    kernels = _resource_report("logprob_entropy_fused.hip")
+    bodies = {k: v for k, v in kernels.items() if re.search(r"fused_pipe_kernelILi1ELi[012]ELi38E", k)}
+    assert len(bodies) >= 6, sorted(kernels)
+    for k, v in bodies.items():
         assert v["VGPRs Spill"] == 0 and v["ScratchSize [bytes/lane]"] == 0, (k, v)
 
 
