@@ -127,13 +127,47 @@ __device__ __forceinline__ void merge(Running& a, const Running& b, float c1, fl
   a.m = m;
 }
 
-// The 8-byte pieces of one rounded column, 4 consecutive vocabulary entries each, to row `out`
-// (= the token's row, at the tile's first column + this wave's 128 + this lane half's 4).
-__device__ __forceinline__ void store_column(uint16_t* out, const uint32_t (&pk)[4][8]) {
+// ---------------------------------------------------------------- a tile of 16-bit results leaves in whole rows
+// A lane of the tile holds single columns of 32 rows (or, formed transposed, 8-byte pieces of 32
+// rows): stored from the registers, every store instruction touches 32-64 rows, and a CU issues a
+// few hundred of them per tile at one per 16 cycles. The tile goes through LDS instead (the slab
+// buffers are free once the product is done): each lane deposits its 8-byte pieces, and after a
+// barrier every 32 lanes pick up one whole 512-byte row of the tile and store it with 16 bytes per
+// lane. Rows lie kOutPitch bytes apart: 512 + 8, so that the 32 rows a wave's deposit touches fall
+// on 32 different pairs of LDS banks.
+constexpr int kOutPitch = 520;
+constexpr int kOutBytes = 256 * kOutPitch;  // 133 120: more than the slab buffers (131 072)
+constexpr int kExchangeBytes = 8192;        // the forward's per-token statistics of the four waves, behind the tile
+constexpr int kLaunchLds = kOutBytes + kExchangeBytes;
+static_assert(kOutBytes >= mm::kLdsBytes && kLaunchLds <= 160 * 1024, "dynamic LDS of every matrix-core launch");
+
+// Four consecutive 16-bit results (lo = the first two) of tile row `row` at tile column `col` (a multiple of 4).
+__device__ __forceinline__ void deposit4(char* lds, uint32_t row, uint32_t col, uint32_t lo, uint32_t hi) {
+  *(u32x2*)(lds + row * kOutPitch + col * 2) = u32x2{lo, hi};
+}
+
+// After a barrier: the deposited tile to out[r * ld + c] for r < rows_valid, c < cols_valid (out points
+// at the tile's first element). Whole 16-byte pieces where out and ld allow 16-byte stores.
+__device__ __forceinline__ void flush_rows(const char* lds, uint16_t* __restrict__ out, int64_t ld, int64_t rows_valid,
+                                           int64_t cols_valid) {
+  const uint32_t tid = threadIdx.x, piece = tid & 31u, sub = tid >> 5;  // 32 pieces of 8 columns per row, 8 rows per step
+  const bool vec = (((uintptr_t)out & 15u) == 0) && ((ld & 7) == 0);
+  const int64_t c0 = (int64_t)piece * 8;
+#pragma unroll 4
+  for (uint32_t step = 0; step < 32; ++step) {
+    const uint32_t row = step * 8 + sub;
+    if ((int64_t)row >= rows_valid || c0 >= cols_valid) continue;
+    const char* src = lds + row * kOutPitch + piece * 16;
+    const u32x2 lo = *(const u32x2*)src, hi = *(const u32x2*)(src + 8);
+    uint16_t* dst = out + (int64_t)row * ld + c0;
+    if (vec && c0 + 8 <= cols_valid) {
+      *(u32x4*)dst = u32x4{lo[0], lo[1], hi[0], hi[1]};
+    } else {
+      const uint32_t w[4] = {lo[0], lo[1], hi[0], hi[1]};
 #pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-#pragma unroll
-    for (int g = 0; g < 4; ++g) *(u32x2*)(out + mt * 32 + g * 8) = u32x2{pk[mt][2 * g], pk[mt][2 * g + 1]};
+      for (int e = 0; e < 8; ++e)
+        if (c0 + e < cols_valid) dst[e] = (uint16_t)(e & 1 ? w[e >> 1] >> 16 : w[e >> 1] & 0xffffu);
+    }
   }
 }
 
@@ -177,7 +211,7 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, 
   const int64_t vbase = (int64_t)vt * 256 + wm * 128 + 4 * (lane >> 5);  // vocabulary index of this lane's register offset 0
   const bool keep = vt < kept_tiles;
   __syncthreads();  // every wave is done with the slab buffers: they serve as the exchange area now
-  float* ex = (float*)lds;  // [2 wm][2 wn][4 tokens][32 lanes][4 fields]
+  float* ex = (float*)(lds + kOutBytes);  // [2 wm][2 wn][4 tokens][32 lanes][4 fields], behind the tile of kept logits
 #pragma unroll
   for (int nt = 0; nt < 4; ++nt) {
     const int64_t tok = (int64_t)tb * 256 + mm::acc_col(wn, nt, lane);
@@ -185,7 +219,14 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, 
     const int lab_rel = (d >= 0 && d < 128) ? (int)d : -1;
     uint32_t pk[4][8];
     round_column<DT>(acc, nt, pk);
-    if (keep && tok < n_tokens) store_column(kept + tok * kept_ld + vbase, pk);
+    if (keep) {  // the rounded logits of this token (tile row), 4 consecutive vocabulary entries per piece
+      const uint32_t row = mm::acc_col(wn, nt, lane);
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) deposit4(lds, row, mm::acc_row(wm, mt, 4 * g, lane), pk[mt][2 * g], pk[mt][2 * g + 1]);
+      }
+    }
     Running run{kLow, 0.0f, 0.0f, 0.0f, kLow};
     fold_column<DT, BOTH_T>(pk, run, lab_rel, c1, cT);
     if (run.xl != kLow && tok < n_tokens) x_label[tok] = run.xl;  // exactly one lane of the grid holds a token's label
@@ -200,6 +241,8 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_fwd_kernel(Operand w, 
     if (lane < 32) *(f32x4*)(ex + (((wm * 2 + wn) * 4 + nt) * 32 + lane) * 4) = f32x4{run.m, run.s1, run.t1, run.sT};
   }
   __syncthreads();
+  // the kept tile leaves in whole token rows of 256 vocabulary entries (the kept array is whole tiles wide)
+  if (keep) flush_rows(lds, kept + (int64_t)tb * 256 * kept_ld + (int64_t)vt * 256, kept_ld, n_tokens - (int64_t)tb * 256, 256);
   if (wm == 0 && lane < 32) {
 #pragma unroll
     for (int nt = 0; nt < 4; ++nt) {
@@ -391,10 +434,18 @@ __global__ __launch_bounds__(kBlock) void lmhead_p_inplace_kernel(uint16_t* __re
 // C[i][j] = sum_k A[i][k] * B[j][k] for the tile at (tm, tn). PRELOAD: the accumulators start from
 // the fp32 partial sum in c32 (a product continued from an earlier stretch of k). OUT_F32: the sum
 // goes back to c32 (ld32); otherwise it is rounded once to DT and stored to c16 (ld16).
-template <int DT, bool A_MN, bool B_MN, bool PRELOAD, bool OUT_F32>
+//
+// ROWS_OUT (dW: thousands of tiles of a depth of only a few thousand, where the exit of a tile is
+// several percent of its time): the tile is formed transposed (B's rows along the accumulators'
+// register dimension, A's rows along the lanes: the product is symmetric in its operands), so that
+// four consecutive registers of a lane are four consecutive columns j of one row of C, and it
+// leaves through LDS in whole rows. dHidden, one tile per CU over the whole vocabulary, stores
+// from its registers.
+template <int DT, bool A_MN, bool B_MN, bool PRELOAD, bool OUT_F32, bool ROWS_OUT = false>
 __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_gemm_kernel(Operand a, Operand b, float* __restrict__ c32, int64_t ld32,
                                                                       uint16_t* __restrict__ c16, int64_t ld16,
                                                                       uint32_t tiles_m, uint32_t tiles_n) {
+  static_assert(!ROWS_OUT || (!PRELOAD && !OUT_F32), "the row-wise exit is for a 16-bit result of a product begun here");
   extern __shared__ __align__(16) char lds[];
   using E = Elt<DT>;
   const uint32_t n_items = tiles_m * tiles_n;
@@ -427,6 +478,27 @@ __global__ __launch_bounds__(mm::kThreads, 1) void lmhead_gemm_kernel(Operand a,
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+  }
+  if (ROWS_OUT) {
+    // transposed: B's rows along the register dimension, A's rows along the lanes
+    mm::tile_product<DT, B_MN, A_MN, true>(acc, b, a, (int64_t)tn * 256, (int64_t)tm * 256, lds);
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, w_reg = wave & 1u, w_lane = wave >> 1;
+    __syncthreads();  // every wave is done with the slab buffers
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+      const uint32_t row = mm::acc_col(w_lane, nt, lane);
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          deposit4(lds, row, mm::acc_row(w_reg, mt, 4 * g, lane), pack2<DT>(acc[mt][nt][4 * g], acc[mt][nt][4 * g + 1]),
+                   pack2<DT>(acc[mt][nt][4 * g + 2], acc[mt][nt][4 * g + 3]));
+      }
+    }
+    __syncthreads();
+    flush_rows(lds, c16 + (int64_t)tm * 256 * ld16 + (int64_t)tn * 256, ld16, a.rows - (int64_t)tm * 256,
+               b.rows - (int64_t)tn * 256);
+    return;
   }
   mm::tile_product<DT, A_MN, B_MN, !PRELOAD>(acc, a, b, (int64_t)tm * 256, (int64_t)tn * 256, lds);
   const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6, wm = wave & 1u, wn = wave >> 1;
@@ -489,7 +561,7 @@ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 inline unsigned grid_for_items(int64_t items) { return (unsigned)(((items + 7) / 8) * 8); }
 
 template <typename K>
-static hipError_t allow_lds(K kernel, int bytes = mm::kLdsBytes) {
+static hipError_t allow_lds(K kernel, int bytes = kLaunchLds) {
   return hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
 }
 
@@ -557,12 +629,12 @@ static int launch_fwd(const void* hidden, const void* weight, int64_t n_rows, in
   const dim3 grid(grid_for_items(n_tb * n_vt)), block(mm::kThreads);
   const uint32_t kept_tiles = (uint32_t)(kept_cols / 256);
   if (both_t) {
-    if (allow_lds(lmhead_fwd_kernel<DT, true>) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", mm::kLdsBytes);
-    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, true>), grid, block, mm::kLdsBytes, s, w, h, labels, c1, cT, records, x_label,
+    if (allow_lds(lmhead_fwd_kernel<DT, true>) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", lm::kLaunchLds);
+    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, true>), grid, block, lm::kLaunchLds, s, w, h, labels, c1, cT, records, x_label,
                        (uint16_t*)kept, kept_ld, kept_tiles, (uint32_t)n_tb, (uint32_t)n_vt);
   } else {
-    if (allow_lds(lmhead_fwd_kernel<DT, false>) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", mm::kLdsBytes);
-    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, false>), grid, block, mm::kLdsBytes, s, w, h, labels, c1, cT, records, x_label,
+    if (allow_lds(lmhead_fwd_kernel<DT, false>) != hipSuccess) return fail(ORLHF_ERR_LAUNCH, "lmhead_fwd: cannot get %d bytes of LDS", lm::kLaunchLds);
+    hipLaunchKernelGGL((lmhead_fwd_kernel<DT, false>), grid, block, lm::kLaunchLds, s, w, h, labels, c1, cT, records, x_label,
                        (uint16_t*)kept, kept_ld, kept_tiles, (uint32_t)n_tb, (uint32_t)n_vt);
   }
   ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_fwd(tiles)");
@@ -581,8 +653,8 @@ static int launch_dhidden(const Operand& p, const Operand& wt, bool first, bool 
 #define ORLHF_DH(PRE, F32)                                                                                                   \
   {                                                                                                                           \
     if (allow_lds(lmhead_gemm_kernel<DT, false, true, PRE, F32>) != hipSuccess)                                              \
-      return fail(ORLHF_ERR_LAUNCH, "lmhead_bwd: cannot get %d bytes of LDS", mm::kLdsBytes);                                \
-    hipLaunchKernelGGL((lmhead_gemm_kernel<DT, false, true, PRE, F32>), grid, block, mm::kLdsBytes, s, p, wt, dh_acc,        \
+      return fail(ORLHF_ERR_LAUNCH, "lmhead_bwd: cannot get %d bytes of LDS", lm::kLaunchLds);                                \
+    hipLaunchKernelGGL((lmhead_gemm_kernel<DT, false, true, PRE, F32>), grid, block, lm::kLaunchLds, s, p, wt, dh_acc,        \
                        hidden_dim, grad_hidden, grad_hidden_stride, (uint32_t)n_tb, (uint32_t)tiles_h);                      \
   }
   if (first && last) ORLHF_DH(false, false)
@@ -599,9 +671,9 @@ template <int DT>
 static int launch_dweight(const Operand& pt, const Operand& ht, uint16_t* grad_weight, int64_t grad_weight_stride, hipStream_t s) {
   const int64_t tiles_v = (pt.rows + 255) / 256, tiles_h = (ht.rows + 255) / 256;
   const dim3 grid(grid_for_items(tiles_v * tiles_h)), block(mm::kThreads);
-  if (allow_lds(lmhead_gemm_kernel<DT, true, true, false, false>) != hipSuccess)
-    return fail(ORLHF_ERR_LAUNCH, "lmhead_bwd: cannot get %d bytes of LDS", mm::kLdsBytes);
-  hipLaunchKernelGGL((lmhead_gemm_kernel<DT, true, true, false, false>), grid, block, mm::kLdsBytes, s, pt, ht, nullptr, 0,
+  if (allow_lds(lmhead_gemm_kernel<DT, true, true, false, false, true>) != hipSuccess)
+    return fail(ORLHF_ERR_LAUNCH, "lmhead_bwd: cannot get %d bytes of LDS", lm::kLaunchLds);
+  hipLaunchKernelGGL((lmhead_gemm_kernel<DT, true, true, false, false, true>), grid, block, lm::kLaunchLds, s, pt, ht, nullptr, 0,
                      grad_weight, grad_weight_stride, (uint32_t)tiles_v, (uint32_t)tiles_h);
   ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(dW)");
   return ORLHF_OK;
@@ -652,17 +724,17 @@ static int launch_bwd(const void* hidden, const void* weight, int64_t n_rows, in
   }
   if (kept_cols < vpad) {
     if (allow_lds(lmhead_bwd_p_kernel<DT, true>) != hipSuccess || allow_lds(lmhead_bwd_p_kernel<DT, false>) != hipSuccess)
-      return fail(ORLHF_ERR_LAUNCH, "lmhead_bwd: cannot get %d bytes of LDS", mm::kLdsBytes);
+      return fail(ORLHF_ERR_LAUNCH, "lmhead_bwd: cannot get %d bytes of LDS", lm::kLaunchLds);
     const int64_t ldp = p_chunk_ld(chunk_cols);
     for (int64_t v0 = kept_cols; v0 < vpad; v0 += chunk_cols) {
       const int64_t cols_pad = vpad - v0 < chunk_cols ? vpad - v0 : chunk_cols;
       const int64_t ctiles = cols_pad / 256;
       const dim3 grid(grid_for_items(n_tb * ctiles)), block(mm::kThreads);
       if (both_t)
-        hipLaunchKernelGGL((lmhead_bwd_p_kernel<DT, true>), grid, block, mm::kLdsBytes, s, w, h, labels, temperature, g_logprob,
+        hipLaunchKernelGGL((lmhead_bwd_p_kernel<DT, true>), grid, block, lm::kLaunchLds, s, w, h, labels, temperature, g_logprob,
                            g_entropy, row_stats, p_chunk, ldp, v0, (uint32_t)n_tb, (uint32_t)ctiles);
       else
-        hipLaunchKernelGGL((lmhead_bwd_p_kernel<DT, false>), grid, block, mm::kLdsBytes, s, w, h, labels, temperature, g_logprob,
+        hipLaunchKernelGGL((lmhead_bwd_p_kernel<DT, false>), grid, block, lm::kLaunchLds, s, w, h, labels, temperature, g_logprob,
                            g_entropy, row_stats, p_chunk, ldp, v0, (uint32_t)n_tb, (uint32_t)ctiles);
       ORLHF_CHECK_LAUNCH("orlhf_lmhead_logprob_entropy_bwd(P)");
       if (int rc = products(p_chunk, ldp, v0, cols_pad)) return rc;
@@ -797,8 +869,8 @@ extern "C" int orlhf_matrix_tile_product(const void* a, const void* b, int dtype
 #define ORLHF_TP(DT, AM, BM, PRE)                                                                                             \
   {                                                                                                                           \
     if (lm::allow_lds(lm::lmhead_gemm_kernel<DT, AM, BM, PRE, true>) != hipSuccess)                                           \
-      return fail(ORLHF_ERR_LAUNCH, "matrix_tile_product: cannot get %d bytes of LDS", mm::kLdsBytes);                        \
-    hipLaunchKernelGGL((lm::lmhead_gemm_kernel<DT, AM, BM, PRE, true>), grid, block, mm::kLdsBytes, s, oa, ob, c, ldc, nullptr, 0, \
+      return fail(ORLHF_ERR_LAUNCH, "matrix_tile_product: cannot get %d bytes of LDS", lm::kLaunchLds);                        \
+    hipLaunchKernelGGL((lm::lmhead_gemm_kernel<DT, AM, BM, PRE, true>), grid, block, lm::kLaunchLds, s, oa, ob, c, ldc, nullptr, 0, \
                        (uint32_t)tiles_m, (uint32_t)tiles_n);                                                                 \
   }
 #define ORLHF_TP_LAYOUT(DT, PRE)                                    \
@@ -840,8 +912,8 @@ extern "C" int orlhf_matrix_tile_probe(const void* a, const void* b, int dtype, 
 #define ORLHF_PROBE(DT, RES)                                                                                   \
   {                                                                                                            \
     if (lm::allow_lds(lm::matrix_tile_probe_kernel<DT, RES>) != hipSuccess)                                    \
-      return fail(ORLHF_ERR_LAUNCH, "matrix_tile_probe: cannot get %d bytes of LDS", mm::kLdsBytes);           \
-    hipLaunchKernelGGL((lm::matrix_tile_probe_kernel<DT, RES>), grid, block, mm::kLdsBytes, s, oa, ob, tile_sums, (uint32_t)tiles_m, (uint32_t)tiles_n); \
+      return fail(ORLHF_ERR_LAUNCH, "matrix_tile_probe: cannot get %d bytes of LDS", lm::kLaunchLds);           \
+    hipLaunchKernelGGL((lm::matrix_tile_probe_kernel<DT, RES>), grid, block, lm::kLaunchLds, s, oa, ob, tile_sums, (uint32_t)tiles_m, (uint32_t)tiles_n); \
   }
   if (dtype == ORLHF_BF16) {
     if (resident_operands) ORLHF_PROBE(ORLHF_BF16, true) else ORLHF_PROBE(ORLHF_BF16, false)

@@ -275,3 +275,49 @@ def test_lmhead_every_row_masked(cuda):
     # and an empty batch
     lp0, ent0 = lm_head_logprobs_and_entropy(h[:0], w, labels[:0], 1.0)
     assert lp0.shape == (0,) and ent0.shape == (0,)
+
+
+def test_lmhead_outputs_at_any_stride_and_alignment_hold_the_same_bits(cuda):
+    """The weight gradient leaves its tiles in whole rows with 16-byte stores where the array allows
+    it and element by element where it does not (the kept logits must be 16-byte aligned anyway):
+    gradient arrays that start 2 bytes past a 16-byte boundary with odd row strides must hold the
+    same bits as well-aligned ones, and nothing outside them may be written. Through the C entry
+    points, at a shape with ragged tiles in every dimension."""
+    from openrlhf_amd import _lib
+    from openrlhf_amd._lib import call, ptr, stream_of
+
+    n, hdim, vocab, temperature = 300, 328, 1000, 0.7
+    hidden, weight, labels, g_lp, g_ent = _case(n, hdim, vocab, torch.bfloat16, seed=31)
+    hd, wd, lab = hidden.to(cuda), weight.to(cuda), labels.to(cuda)
+    glp, gent = g_lp.to(cuda), g_ent.to(cuda)
+    lib = _lib.load()
+    kept_cols = (vocab + 255) // 256 * 256
+
+    def run(kept_ld, offset, pad):
+        kept = torch.full((n * kept_ld + 8,), float("nan"), dtype=torch.bfloat16, device=cuda)[:n * kept_ld].view(n, kept_ld)
+        lp, ent, stats = torch.empty(n, device=cuda), torch.empty(n, device=cuda), torch.empty(n, 4, device=cuda)
+        ws = torch.empty(lib.orlhf_lmhead_workspace_bytes(n, hdim, vocab, kept_cols, 0), dtype=torch.uint8, device=cuda)
+        call("orlhf_lmhead_logprob_entropy_fwd", ptr(hd), ptr(wd), _lib.BF16, n, hdim, vocab, hdim, hdim, ptr(lab), temperature,
+             ptr(lp), ptr(ent), ptr(stats), ptr(kept), kept_cols, kept_ld, ptr(ws), ws.numel(), stream_of(cuda))
+        logits = kept[:, :vocab].clone()
+        gh_buf = torch.full((n * (hdim + pad) + offset + 8,), float("nan"), dtype=torch.bfloat16, device=cuda)
+        gw_buf = torch.full((vocab * (hdim + pad) + offset + 8,), float("nan"), dtype=torch.bfloat16, device=cuda)
+        gh = gh_buf[offset:offset + n * (hdim + pad)].view(n, hdim + pad)[:, :hdim]
+        gw = gw_buf[offset:offset + vocab * (hdim + pad)].view(vocab, hdim + pad)[:, :hdim]
+        ws2 = torch.empty(lib.orlhf_lmhead_workspace_bytes(n, hdim, vocab, kept_cols, 1), dtype=torch.uint8, device=cuda)
+        call("orlhf_lmhead_logprob_entropy_bwd", ptr(hd), ptr(wd), _lib.BF16, n, hdim, vocab, hdim, hdim, ptr(lab), temperature,
+             ptr(glp), ptr(gent), ptr(stats), ptr(kept), kept_cols, kept_ld, gh.data_ptr(), hdim + pad, gw.data_ptr(), hdim + pad,
+             ptr(ws2), ws2.numel(), stream_of(cuda))
+        torch.cuda.synchronize()
+        # nothing outside the arrays was touched
+        assert torch.isnan(gw_buf[:offset]).all() and torch.isnan(gw_buf[offset + vocab * (hdim + pad):]).all()
+        if pad:
+            assert torch.isnan(gw_buf[offset:offset + vocab * (hdim + pad)].view(vocab, hdim + pad)[:, hdim:]).all()
+        return logits, lp, ent, gh.clone(), gw.clone()
+
+    aligned = run(kept_cols + 64, 0, 0)
+    assert torch.isfinite(aligned[3].float()).all() and torch.isfinite(aligned[4].float()).all()
+    for kept_ld, offset, pad in ((kept_cols + 8, 1, 3), (kept_cols + 72, 3, 1), (kept_cols + 64, 8, 8), (kept_cols, 4, 0)):
+        other = run(kept_ld, offset, pad)
+        for a, b in zip(aligned, other):
+            assert torch.equal(a.view(torch.int16) if a.dtype == torch.bfloat16 else a, b.view(torch.int16) if b.dtype == torch.bfloat16 else b), (kept_ld, offset, pad)
